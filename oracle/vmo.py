@@ -1,0 +1,271 @@
+"""ctypes binding of the CPU oracle's C interface (vm_oracle.h).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by bench.py's cpu_baseline leg and by
+__graft_entry__.smoke(); never by the engine package.
+
+`load("oracle")` opens libvm_oracle.so (the restatement), `load("reference")` opens
+_ref/libvm_ref.so (the reference's own headers behind the same interface) and returns None when that
+library has not been built.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+RING6, NMGRID8 = 0, 1
+SPHERE, CIRCLE = 0, 1
+RECTILINEAR, EQUISOLID, EQUIDISTANT = 0, 1, 2
+SELU, RELU, SOFTMAX, TANH = 0, 1, 2, 3
+ERR_FORMAT, ERR_LENS, ERR_ARG, ERR_CAPACITY = -2, -3, -4, -5
+
+
+def fourcc(s):
+    b = s.encode()
+    assert len(b) == 4
+    return b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24)
+
+
+class Lens(C.Structure):
+    _fields_ = [
+        ("width", C.c_int32),
+        ("height", C.c_int32),
+        ("projection", C.c_int32),
+        ("focal_length", C.c_float),
+        ("centre", C.c_float * 2),
+        ("k", C.c_float * 2),
+        ("fov", C.c_float),
+    ]
+
+
+def make_lens(width, height, projection, focal_length, fov, centre=(0.0, 0.0), k=(0.0, 0.0)):
+    return Lens(width, height, projection, focal_length, (C.c_float * 2)(*centre), (C.c_float * 2)(*k), fov)
+
+
+class _Layer(C.Structure):
+    _fields_ = [
+        ("n_in", C.c_int32),
+        ("n_out", C.c_int32),
+        ("activation", C.c_int32),
+        ("weights", C.POINTER(C.c_float)),
+        ("biases", C.POINTER(C.c_float)),
+    ]
+
+
+class _Network(C.Structure):
+    _fields_ = [("n_groups", C.c_int32), ("group_sizes", C.POINTER(C.c_int32)), ("layers", C.POINTER(_Layer))]
+
+
+def _fp(a):
+    return a.ctypes.data_as(C.POINTER(C.c_float))
+
+
+def _ip(a):
+    return a.ctypes.data_as(C.POINTER(C.c_int32))
+
+
+class Network:
+    """network = list of groups, group = list of (weights[n_in, n_out] float32, biases[n_out], activation)."""
+
+    def __init__(self, groups):
+        self.groups = groups
+        self._keep = []
+        layers = []
+        for g in groups:
+            for (w, b, act) in g:
+                w = np.ascontiguousarray(w, dtype=np.float32)
+                b = np.ascontiguousarray(b, dtype=np.float32)
+                self._keep += [w, b]
+                layers.append(_Layer(w.shape[0], w.shape[1], act, _fp(w), _fp(b)))
+        self._layers = (_Layer * max(len(layers), 1))(*layers)
+        self._sizes = (C.c_int32 * max(len(groups), 1))(*[len(g) for g in groups])
+        self.c = _Network(len(groups), self._sizes, self._layers)
+        self.n_out = groups[-1][-1][0].shape[1] if groups else 4
+
+
+class Oracle:
+    def __init__(self, path):
+        self.lib = L = C.CDLL(path)
+        vp = C.c_void_p
+        L.vmo_name.restype = C.c_char_p
+        L.vmo_mesh_create.restype = vp
+        L.vmo_mesh_create.argtypes = [C.c_int, C.c_int, C.c_float, C.c_float, C.c_float, C.c_float]
+        L.vmo_mesh_destroy.argtypes = [vp]
+        L.vmo_mesh_n_nodes.argtypes = [vp]
+        L.vmo_mesh_n_neighbours.argtypes = [vp]
+        L.vmo_mesh_h.argtypes = [vp]
+        L.vmo_mesh_h.restype = C.c_float
+        L.vmo_mesh_copy.argtypes = [vp, C.POINTER(C.c_float), C.POINTER(C.c_int32)]
+        L.vmo_mesh_lookup.argtypes = [vp, C.POINTER(C.c_float), C.POINTER(Lens), C.POINTER(C.c_int32), C.c_int]
+        L.vmo_visualmesh_create.restype = vp
+        L.vmo_visualmesh_create.argtypes = [C.c_int, C.c_int] + [C.c_float] * 6
+        L.vmo_visualmesh_destroy.argtypes = [vp]
+        L.vmo_visualmesh_n_meshes.argtypes = [vp]
+        L.vmo_visualmesh_mesh.restype = vp
+        L.vmo_visualmesh_mesh.argtypes = [vp, C.c_int]
+        L.vmo_visualmesh_height.restype = vp
+        L.vmo_visualmesh_height.argtypes = [vp, C.c_float]
+        L.vmo_project.argtypes = [vp, C.POINTER(C.c_float), C.POINTER(Lens), C.c_int, C.POINTER(C.c_float),
+                                  C.POINTER(C.c_int32), C.POINTER(C.c_int32)]
+        L.vmo_classify.argtypes = [vp, C.POINTER(C.c_float), C.POINTER(Lens), vp, C.c_uint32, C.POINTER(_Network),
+                                   C.c_int, C.POINTER(C.c_float), C.POINTER(C.c_int32), C.POINTER(C.c_int32),
+                                   C.POINTER(C.c_float)]
+        L.vmo_fn_project.argtypes = [C.POINTER(C.c_float), C.POINTER(Lens), C.POINTER(C.c_float)]
+        L.vmo_fn_unproject.argtypes = [C.POINTER(C.c_float), C.POINTER(Lens), C.POINTER(C.c_float)]
+        L.vmo_fn_interpolate.argtypes = [C.POINTER(C.c_float), vp, C.c_int, C.c_int, C.c_uint32, C.POINTER(C.c_float)]
+        L.vmo_fn_get_pixel.argtypes = [C.c_int, C.c_int, vp, C.c_int, C.c_int, C.c_uint32, C.POINTER(C.c_float)]
+        L.vmo_fn_activation.argtypes = [C.c_int, C.POINTER(C.c_float), C.c_int, C.c_int]
+        L.vmo_fn_shape.restype = C.c_float
+        L.vmo_fn_shape.argtypes = [C.c_int, C.c_float, C.c_int, C.c_float, C.c_float]
+        self.name = L.vmo_name().decode()
+
+    # ---- meshes
+    def mesh(self, model, shape, radius, h, k, max_distance):
+        p = self.lib.vmo_mesh_create(model, shape, radius, h, k, max_distance)
+        if not p:
+            raise RuntimeError("mesh construction failed")
+        return Mesh(self, p, owned=True)
+
+    def visualmesh(self, model, shape, radius, min_h, max_h, k, max_error, max_distance):
+        p = self.lib.vmo_visualmesh_create(model, shape, radius, min_h, max_h, k, max_error, max_distance)
+        if not p:
+            raise RuntimeError("visual mesh construction failed")
+        return VisualMesh(self, p)
+
+    # ---- single functions
+    def fn_project(self, ray, lens):
+        r = np.asarray(ray, dtype=np.float32)
+        o = np.zeros(2, np.float32)
+        self.lib.vmo_fn_project(_fp(r), C.byref(lens), _fp(o))
+        return o
+
+    def fn_unproject(self, px, lens):
+        p = np.asarray(px, dtype=np.float32)
+        o = np.zeros(3, np.float32)
+        self.lib.vmo_fn_unproject(_fp(p), C.byref(lens), _fp(o))
+        return o
+
+    def fn_interpolate(self, px, image, width, height, fcc):
+        p = np.asarray(px, dtype=np.float32)
+        o = np.zeros(4, np.float32)
+        rc = self.lib.vmo_fn_interpolate(_fp(p), image.ctypes.data, width, height, fcc, _fp(o))
+        if rc != 0:
+            raise ValueError("unsupported format (%d)" % rc)
+        return o
+
+    def fn_get_pixel(self, x, y, image, width, height, fcc):
+        o = np.zeros(4, np.float32)
+        rc = self.lib.vmo_fn_get_pixel(x, y, image.ctypes.data, width, height, fcc, _fp(o))
+        if rc != 0:
+            raise ValueError("unsupported format (%d)" % rc)
+        return o
+
+    def fn_activation(self, act, data, dims):
+        d = np.ascontiguousarray(data, dtype=np.float32).copy()
+        self.lib.vmo_fn_activation(act, _fp(d), d.size // dims, dims)
+        return d
+
+    def fn_shape(self, shape, radius, which, a=0.0, b=0.0):
+        return self.lib.vmo_fn_shape(shape, radius, {"phi": 0, "n": 1, "theta": 2, "k": 3, "c": 4}[which], a, b)
+
+
+class Mesh:
+    def __init__(self, oracle, ptr, owned):
+        self.o, self.ptr, self.owned = oracle, ptr, owned
+        L = oracle.lib
+        self.n_nodes = L.vmo_mesh_n_nodes(ptr)
+        self.n_neighbours = L.vmo_mesh_n_neighbours(ptr)
+        self.h = L.vmo_mesh_h(ptr)
+        self._arrays = None
+
+    def __del__(self):
+        if self.owned and self.ptr:
+            self.o.lib.vmo_mesh_destroy(self.ptr)
+            self.ptr = None
+
+    def arrays(self):
+        """(rays[n,3] float32, neighbours[n,nn] int32)"""
+        if self._arrays is None:
+            rays = np.zeros((self.n_nodes, 3), np.float32)
+            nbr = np.zeros((self.n_nodes, self.n_neighbours), np.int32)
+            self.o.lib.vmo_mesh_copy(self.ptr, _fp(rays), _ip(nbr))
+            self._arrays = (rays, nbr)
+        return self._arrays
+
+    def lookup(self, Hoc, lens):
+        H = np.ascontiguousarray(Hoc, dtype=np.float32)
+        cap = 4096
+        while True:
+            r = np.zeros((cap, 2), np.int32)
+            n = self.o.lib.vmo_mesh_lookup(self.ptr, _fp(H), C.byref(lens), _ip(r), cap)
+            if n < 0:
+                raise RuntimeError("lookup failed (%d)" % n)
+            if n <= cap:
+                return r[:n].copy()
+            cap = n
+
+    def project(self, Hoc, lens):
+        """-> dict(px[V,2], nb[V+1,nn], gidx[V])"""
+        H = np.ascontiguousarray(Hoc, dtype=np.float32)
+        ranges = self.lookup(Hoc, lens)
+        cap = int((ranges[:, 1] - ranges[:, 0]).sum()) if len(ranges) else 0
+        px = np.zeros((max(cap, 1), 2), np.float32)
+        nb = np.zeros((cap + 1, self.n_neighbours), np.int32)
+        gidx = np.zeros(max(cap, 1), np.int32)
+        V = self.o.lib.vmo_project(self.ptr, _fp(H), C.byref(lens), cap, _fp(px), _ip(nb), _ip(gidx))
+        if V < 0:
+            raise RuntimeError("project failed (%d)" % V)
+        return dict(px=px[:V].copy(), nb=nb[:V + 1].copy(), gidx=gidx[:V].copy(), ranges=ranges)
+
+    def classify(self, Hoc, lens, image, fcc, network):
+        """-> dict(px, nb, gidx, cls[V+1, n_out]); an empty visible set gives empty arrays (default result)"""
+        H = np.ascontiguousarray(Hoc, dtype=np.float32)
+        ranges = self.lookup(Hoc, lens)
+        cap = int((ranges[:, 1] - ranges[:, 0]).sum()) if len(ranges) else 0
+        n_out = network.n_out
+        px = np.zeros((max(cap, 1), 2), np.float32)
+        nb = np.zeros((cap + 1, self.n_neighbours), np.int32)
+        gidx = np.zeros(max(cap, 1), np.int32)
+        cls = np.zeros((cap + 1, n_out), np.float32)
+        img = np.ascontiguousarray(image)
+        V = self.o.lib.vmo_classify(self.ptr, _fp(H), C.byref(lens), img.ctypes.data, fcc, C.byref(network.c), cap,
+                                    _fp(px), _ip(nb), _ip(gidx), _fp(cls))
+        if V == ERR_FORMAT:
+            raise ValueError("Unsupported image format")
+        if V < 0:
+            raise RuntimeError("classify failed (%d)" % V)
+        if V == 0:
+            return dict(px=px[:0], nb=nb[:0], gidx=gidx[:0], cls=cls[:0], ranges=ranges)
+        return dict(px=px[:V].copy(), nb=nb[:V + 1].copy(), gidx=gidx[:V].copy(), cls=cls[:V + 1].copy(), ranges=ranges)
+
+
+class VisualMesh:
+    def __init__(self, oracle, ptr):
+        self.o, self.ptr = oracle, ptr
+        n = oracle.lib.vmo_visualmesh_n_meshes(ptr)
+        self.meshes = [Mesh(oracle, oracle.lib.vmo_visualmesh_mesh(ptr, i), owned=False) for i in range(n)]
+        self._by_ptr = {m.ptr: m for m in self.meshes}
+
+    def __del__(self):
+        if self.ptr:
+            self.o.lib.vmo_visualmesh_destroy(self.ptr)
+            self.ptr = None
+
+    def height(self, h):
+        return self._by_ptr[self.o.lib.vmo_visualmesh_height(self.ptr, h)]
+
+
+_cache = {}
+
+
+def load(which="oracle"):
+    if which not in _cache:
+        path = os.path.join(HERE, "libvm_oracle.so") if which == "oracle" else os.path.join(HERE, "_ref", "libvm_ref.so")
+        if not os.path.exists(path):
+            if which == "oracle":
+                raise FileNotFoundError(path + " is not built: run `make -C oracle` or __graft_entry__.build()")
+            _cache[which] = None
+        else:
+            _cache[which] = Oracle(path)
+    return _cache[which]

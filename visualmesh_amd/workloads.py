@@ -1,0 +1,141 @@
+"""Seeded synthetic inputs for the Visual Mesh inference path: camera poses, lenses, images and
+Glorot-initialised networks, plus the five benchmark/parity configurations.
+
+Everything here is plain numpy and depends on nothing else in the package, so the same generator
+feeds the HIP engine, the parity tests and the CPU baseline.
+"""
+import math
+
+import numpy as np
+
+RING6, NMGRID8 = 0, 1
+SPHERE, CIRCLE = 0, 1
+RECTILINEAR, EQUISOLID, EQUIDISTANT = 0, 1, 2
+SELU, RELU, SOFTMAX, TANH = 0, 1, 2, 3
+N_NEIGHBOURS = {RING6: 6, NMGRID8: 8}
+
+
+def fourcc(s):
+    b = s.encode()
+    assert len(b) == 4
+    return b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24)
+
+
+def make_hoc(height, pitch, roll=0.0, yaw=0.0):
+    """Camera-to-observation-plane transform, row major 4x4 float32.
+
+    Rotation = Rz(yaw) . Ry(pitch) . Rx(roll); the camera looks along its own x axis (y left, z up), so a
+    positive pitch tilts the optical axis down towards the observation plane. Translation = (0, 0, height).
+    """
+    cy, sy = math.cos(yaw), math.sin(yaw)
+    cp, sp = math.cos(pitch), math.sin(pitch)
+    cr, sr = math.cos(roll), math.sin(roll)
+    Rz = np.array([[cy, -sy, 0], [sy, cy, 0], [0, 0, 1]])
+    Ry = np.array([[cp, 0, sp], [0, 1, 0], [-sp, 0, cp]])
+    Rx = np.array([[1, 0, 0], [0, cr, -sr], [0, sr, cr]])
+    H = np.eye(4)
+    H[:3, :3] = Rz @ Ry @ Rx
+    H[2, 3] = height
+    return H.astype(np.float32)
+
+
+def random_image(rng, width, height, bytes_per_pixel):
+    """iid uniform bytes, shape [height, width * bytes_per_pixel] uint8 (tightly packed rows)."""
+    return rng.integers(0, 256, size=(height, width * bytes_per_pixel), dtype=np.uint8)
+
+
+def glorot_network(rng, widths, n_neighbours, hidden_activation, rgb_input=True, bias_scale=0.1):
+    """One dense layer per graph-convolution group, Glorot-uniform weights.
+
+    widths[0] is the number of image channels the network was "trained" on. With rgb_input (3 channels)
+    the first weight matrix is drawn for (n+1)*3 rows and a zero row is inserted after every third row, the
+    way the reference's exporter pads RGB networks to the engines' fixed 4-channel input
+    (training/export.py:83-89), giving (n+1)*4 rows. Returns a list of groups, each a list of
+    (weights[K, C_out] float32, biases[C_out] float32, activation).
+    """
+    groups = []
+    c_in = widths[0]
+    for li, c_out in enumerate(widths[1:]):
+        last = li == len(widths) - 2
+        fan_in = (n_neighbours + 1) * c_in
+        limit = math.sqrt(6.0 / (fan_in + c_out))
+        w = rng.uniform(-limit, limit, size=(fan_in, c_out)).astype(np.float32)
+        if li == 0 and rgb_input:
+            assert c_in == 3
+            w4 = np.zeros(((n_neighbours + 1) * 4, c_out), np.float32)
+            for s in range(n_neighbours + 1):
+                w4[s * 4:s * 4 + 3] = w[s * 3:s * 3 + 3]
+            w = w4
+        b = rng.uniform(-bias_scale, bias_scale, size=c_out).astype(np.float32)
+        groups.append([(w, b, SOFTMAX if last else hidden_activation)])
+        c_in = c_out
+    return groups
+
+
+class Config:
+    """One of the benchmark configurations, fully materialised from a seed."""
+
+    def __init__(self, name, **kw):
+        self.name = name
+        self.__dict__.update(kw)
+
+    def lens_tuple(self):
+        return (self.width, self.height, self.projection, self.focal_length, self.fov)
+
+
+def _frames(rng, n, width, height, bpp, pitch_range, height_range, yaw_range, roll_range):
+    frames = []
+    for _ in range(n):
+        pitch = math.radians(rng.uniform(*pitch_range))
+        h = rng.uniform(*height_range)
+        roll = math.radians(rng.uniform(*roll_range))
+        yaw = math.radians(rng.uniform(*yaw_range))
+        frames.append(dict(Hoc=make_hoc(h, pitch, roll, yaw), image=random_image(rng, width, height, bpp)))
+    return frames
+
+
+def config(index, n_frames=None, seed=None):
+    """The five parity/benchmark configurations (1-based index).
+
+    Choices the configuration text leaves open are fixed here and stated:
+      * biases are U(-0.1, 0.1); roll is U(-5, 5) degrees everywhere; yaw is U(-5, 5) degrees for
+        configurations 1-3 and U(-180, 180) for 4-5 ("random orientations").
+      * configuration 3's "Cylinder" does not exist in the reference; the reference's Circle(r=0.05)
+        stands in for it and max_distance is 5 m.
+      * configurations 4/5 use focal length 672 px (420 scaled by 2048/1280) and a 180 degree field of view.
+    """
+    seed = 1000 + index if seed is None else seed
+    rng = np.random.default_rng(seed)
+    deg = math.pi / 180.0
+    if index == 1:
+        n = 1 if n_frames is None else n_frames
+        net = glorot_network(rng, [3, 16, 16, 2], 6, SELU)
+        fr = _frames(rng, n, 1280, 1024, 4, (30, 30), (1.2, 1.2), (-5, 5), (-5, 5))
+        return Config("cfg1", model=RING6, shape=SPHERE, radius=0.0949, k=6.0, max_distance=20.0, mesh_h=1.2,
+                      visualmesh=None, width=1280, height=1024, projection=EQUISOLID, focal_length=420.0,
+                      fov=math.pi, fourcc=fourcc("RGBA"), network=net, frames=fr, precision="fp32")
+    if index == 2:
+        n = 16 if n_frames is None else n_frames
+        net = glorot_network(rng, [3, 16, 32, 32, 32, 32, 32, 16, 3], 6, SELU)
+        fr = _frames(rng, n, 1280, 1024, 4, (10, 60), (0.8, 1.5), (-5, 5), (-5, 5))
+        return Config("cfg2", model=RING6, shape=SPHERE, radius=0.0949, k=6.0, max_distance=20.0, mesh_h=None,
+                      visualmesh=dict(min_h=0.8, max_h=1.5, max_error=0.5), width=1280, height=1024,
+                      projection=EQUISOLID, focal_length=420.0, fov=math.pi, fourcc=fourcc("RGBA"), network=net,
+                      frames=fr, precision="fp32")
+    if index == 3:
+        n = 1 if n_frames is None else n_frames
+        net = glorot_network(rng, [3, 24, 24, 24, 24, 4], 8, RELU)
+        fr = _frames(rng, n, 1280, 1024, 1, (30, 30), (1.2, 1.2), (-5, 5), (-5, 5))
+        return Config("cfg3", model=NMGRID8, shape=CIRCLE, radius=0.05, k=8.0, max_distance=5.0, mesh_h=1.2,
+                      visualmesh=None, width=1280, height=1024, projection=RECTILINEAR, focal_length=700.0,
+                      fov=math.pi / 2, fourcc=fourcc("GRBG"), network=net, frames=fr, precision="fp32")
+    if index in (4, 5):
+        n = 64 if n_frames is None else n_frames
+        rng = np.random.default_rng(1004 if seed in (1004, 1005) else seed)  # 5 shares 4's inputs
+        net = glorot_network(rng, [3, 64, 64, 64, 64, 64, 64], 6, SELU)
+        fr = _frames(rng, n, 2048, 1536, 4, (10, 60), (1.2, 1.2), (-180, 180), (-5, 5))
+        return Config("cfg%d" % index, model=RING6, shape=SPHERE, radius=0.0949, k=16.0, max_distance=20.0,
+                      mesh_h=1.2, visualmesh=None, width=2048, height=1536, projection=EQUIDISTANT,
+                      focal_length=672.0, fov=math.pi, fourcc=fourcc("RGBA"), network=net, frames=fr,
+                      precision="fp32" if index == 4 else "bf16")
+    raise ValueError("configurations are numbered 1..5")
