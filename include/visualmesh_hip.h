@@ -1,0 +1,164 @@
+/*
+ * visualmesh_hip.h - C ABI of libvisualmesh_hip.so, the MI355X (gfx950) back end of
+ * visualmesh::engine::hip::Engine.
+ *
+ * The library owns all HIP state. Callers pass plain host pointers and sizes; there are no C++ or
+ * framework types in any signature. All functions return VMHIP_OK (0) or a negative status;
+ * vmhip_last_error() returns the message of the last failure on the calling thread.
+ *
+ * What stays with the caller (host C++): mesh generation and the BSP range lookup
+ * (reference cpp/visualmesh/mesh.hpp:424-467 and :499-595). The caller hands over the mesh's node
+ * table once (vmhip_mesh_upload) and, per frame, the index ranges that lookup returned.
+ *
+ * What the library replaces, per frame (reference cpp/visualmesh/engine/cpu/engine.hpp):
+ *   :97-125   projection of every candidate node, strict on-screen filter, order-preserving compaction
+ *   :127-143  reverse lookup and local neighbourhood table, null row last
+ *   :198-206  image sampling (pixel.hpp:43-144, bayer.hpp:95-158) and the (-1,-1,-1,-1) null row
+ *   :213-264  per convolutional group: neighbour gather + dense layers + activation
+ *   :267-272  result assembly
+ *
+ * Threading: like the reference engines, an engine (and every batch made from it) is used from one
+ * thread at a time. Meshes are immutable and may be shared by engines on different threads.
+ */
+#ifndef VISUALMESH_HIP_H
+#define VISUALMESH_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+    VMHIP_OK = 0,
+    VMHIP_ERR_HIP = -1,      /* a HIP runtime call failed (no device, out of memory, launch failure) */
+    VMHIP_ERR_FORMAT = -2,   /* unsupported fourcc: reference engine/cpu/pixel.hpp:100 throws here */
+    VMHIP_ERR_LENS = -3,     /* unknown lens projection: reference utility/projection.hpp:174 throws */
+    VMHIP_ERR_ARGUMENT = -4, /* null pointer, inconsistent sizes, network does not fit the mesh */
+    VMHIP_ERR_CAPACITY = -5  /* a caller-provided result buffer is too small */
+};
+
+/* Same numbering as the reference's LensProjection (lens.hpp:33). */
+enum { VMHIP_RECTILINEAR = 0, VMHIP_EQUISOLID = 1, VMHIP_EQUIDISTANT = 2 };
+/* Same numbering as the reference's ActivationFunction (network_structure.hpp:34-39). */
+enum { VMHIP_SELU = 0, VMHIP_RELU = 1, VMHIP_SOFTMAX = 2, VMHIP_TANH = 3 };
+/* Arithmetic of the graph-convolution layers. Projection and sampling are always fp32. */
+enum { VMHIP_FP32 = 0, VMHIP_BF16 = 1 };
+
+/* POD mirror of visualmesh::Lens<float> (reference lens.hpp:41-52). */
+typedef struct vmhip_lens {
+    int32_t width, height; /* dimensions[0], dimensions[1] */
+    int32_t projection;
+    float focal_length; /* pixels */
+    float centre[2];
+    float k[2];
+    float fov; /* radians, full angle */
+} vmhip_lens;
+
+/* One dense layer (reference network_structure.hpp:43-47): weights[n_in][n_out] row major, the layout
+ * of NetworkStructure and model.yaml, biases[n_out]. */
+typedef struct vmhip_layer {
+    int32_t n_in, n_out;
+    int32_t activation;
+    const float* weights;
+    const float* biases;
+} vmhip_layer;
+
+/* NetworkStructure flattened: n_groups convolutional groups, group g owning group_sizes[g] consecutive
+ * entries of layers. The first layer of a group consumes (n_neighbours+1) * width_of_previous_output
+ * values (4 for the first group), ordered [self, neighbour 0, ..., neighbour n-1]
+ * (reference engine/cpu/engine.hpp:222-231). */
+typedef struct vmhip_network {
+    int32_t n_groups;
+    const int32_t* group_sizes;
+    const vmhip_layer* layers;
+} vmhip_network;
+
+/* Inputs of one frame. */
+typedef struct vmhip_frame {
+    const struct vmhip_mesh* mesh;
+    float Rco[9];          /* row major; Rco[i][j] = Hoc[j][i] (reference engine/cpu/engine.hpp:95) */
+    vmhip_lens lens;
+    const int32_t* ranges; /* n_ranges pairs (first, one-past-last), ascending and disjoint: Mesh::lookup's output */
+    int32_t n_ranges;
+    const void* image;     /* tightly packed rows, width*height*bytes_per_pixel(fourcc) bytes; NULL when only projecting */
+    uint32_t fourcc;       /* little-endian four character code (reference utility/fourcc.hpp:34-36) */
+} vmhip_frame;
+
+/* Outputs of one frame, in caller-owned buffers. capacity counts nodes: it must be at least the number
+ * of candidate nodes (the sum of the range lengths). n_visible is written by the library.
+ *   pixel_coordinates [capacity][2]              first n_visible rows valid
+ *   global_indices    [capacity]                 first n_visible valid, ascending
+ *   neighbourhood     [capacity+1][n_neighbours] first n_visible+1 rows valid, last one is the null row
+ *   classifications   [capacity+1][n_classes]    first n_visible+1 rows valid; may be NULL when projecting
+ * Any pointer may be NULL to skip that output. If nothing is visible n_visible is 0 and nothing is
+ * written (the reference returns a default-constructed result, engine/cpu/engine.hpp:193). */
+typedef struct vmhip_result {
+    int32_t capacity;
+    int32_t n_visible;
+    float* pixel_coordinates;
+    int32_t* global_indices;
+    int32_t* neighbourhood;
+    float* classifications;
+} vmhip_result;
+
+typedef struct vmhip_engine vmhip_engine;
+typedef struct vmhip_mesh vmhip_mesh;
+typedef struct vmhip_batch vmhip_batch;
+
+const char* vmhip_last_error(void);
+
+/* Replaces the engine constructor (reference engine/cpu/engine.hpp:57-71, engine/opencl/engine.hpp:189):
+ * validates the network, converts the weights to the kernels' layouts and uploads them. net may have
+ * zero groups (projection only, or classification returning the sampled 4-channel input). */
+int vmhip_engine_create(const vmhip_network* net, int32_t n_neighbours, int32_t precision, vmhip_engine** out);
+void vmhip_engine_destroy(vmhip_engine* engine);
+/* Width of the classification rows this engine produces (4 for an empty network). */
+int32_t vmhip_engine_n_classes(const vmhip_engine* engine);
+
+/* Replaces the per-mesh device cache of the reference's OpenCL engine (engine/opencl/engine.hpp:603-625):
+ * rays[n_nodes][3] and neighbours[n_nodes][n_neighbours] (global indices, n_nodes = "no neighbour") are
+ * copied to the device once. The handle is independent of any engine. */
+int vmhip_mesh_upload(const float* rays, const int32_t* neighbours, int32_t n_nodes, int32_t n_neighbours,
+                      vmhip_mesh** out);
+void vmhip_mesh_release(vmhip_mesh* mesh);
+
+/* Replaces cpu::Engine::operator()(mesh, Hoc, lens) (reference engine/cpu/engine.hpp:84-147). */
+int vmhip_project(vmhip_engine* engine, const vmhip_frame* frame, vmhip_result* result);
+/* Replaces cpu::Engine::operator()(mesh, Hoc, lens, image, format) (reference engine/cpu/engine.hpp:180-273). */
+int vmhip_classify(vmhip_engine* engine, const vmhip_frame* frame, vmhip_result* result);
+/* The same for n_frames independent frames in one pass (the reference has no batched call; its
+ * benchmark loops over frames, example/benchmark.cpp:50-58). Frames may use different meshes and lenses. */
+int vmhip_classify_batch(vmhip_engine* engine, const vmhip_frame* frames, int32_t n_frames, vmhip_result* results);
+
+/* Staged form of vmhip_classify_batch for pipelines that keep frames resident on the device:
+ *   stage  copies the frames' inputs to the device (images, poses, lenses, ranges) and sizes the workspace
+ *   run    executes the whole path on the device and waits for it; may be repeated
+ *   fetch  copies the results of the last run into caller buffers
+ * classify != 0 runs sampling and the network, 0 stops after the neighbourhood table. */
+int vmhip_batch_create(vmhip_engine* engine, vmhip_batch** out);
+void vmhip_batch_destroy(vmhip_batch* batch);
+int vmhip_batch_stage(vmhip_batch* batch, const vmhip_frame* frames, int32_t n_frames, int32_t classify);
+int vmhip_batch_run(vmhip_batch* batch);
+/* n_visible[n_frames] of the last run */
+int vmhip_batch_counts(const vmhip_batch* batch, int32_t* n_visible);
+int vmhip_batch_fetch(vmhip_batch* batch, vmhip_result* results);
+
+/* Per-kernel timing of vmhip_batch_run with HIP events on the stream the kernels run on.
+ * enable != 0 brackets every kernel launch of later runs with events. After a run,
+ * vmhip_batch_profile_read returns, for kernel slot i < *n_slots, its name (static string), the
+ * duration in milliseconds of its launch in the last run and the rows (nodes incl. null rows) or
+ * candidates it processed. Slots are in launch order. */
+int vmhip_batch_profile(vmhip_batch* batch, int32_t enable);
+int vmhip_batch_profile_read(vmhip_batch* batch, int32_t max_slots, int32_t* n_slots, const char** names,
+                             float* milliseconds, int64_t* units);
+
+/* Diagnostic with no counterpart in the reference: evaluates on the device, for n floats, the library's
+ * own acosf (which = 0), sinf (1), tanf (2) or sqrtf (3) - the functions the lens projection is built from
+ * and which must return the host C library's bits. x and y are host buffers. */
+int vmhip_selftest_libm(int32_t which, const float* x, float* y, int32_t n);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -294,4 +294,8 @@ float vmo_fn_shape(int shape, float radius, int which, float a, float b) {
     if (shape == VMO_SHAPE_SPHERE) return shape_fn(Sphere<float>(radius), which, a, b);
     return shape_fn(Circle<float>(radius), which, a, b);
 }
+void vmo_fn_libm(int which, const float* x, float* y, int n) {
+    for (int i = 0; i < n; ++i)
+        y[i] = which == 0 ? std::acos(x[i]) : which == 1 ? std::sin(x[i]) : which == 2 ? std::tan(x[i]) : std::sqrt(x[i]);
+}
 }

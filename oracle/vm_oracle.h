@@ -100,6 +100,8 @@ int vmo_fn_get_pixel(int x, int y, const void* image, int width, int height, uin
 void vmo_fn_activation(int activation, float* data, int n_rows, int dims);
 /* shape functions: which = 0 phi(n,h), 1 n(phi,h), 2 theta(n,h), 3 k(h0,h1), 4 c() */
 float vmo_fn_shape(int shape, float radius, int which, float a, float b);
+/* the host C library functions the lens projection is built from: which = 0 acosf, 1 sinf, 2 tanf, 3 sqrtf */
+void vmo_fn_libm(int which, const float* x, float* y, int n);
 
 #ifdef __cplusplus
 }

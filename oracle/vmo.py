@@ -118,6 +118,7 @@ class Oracle:
         L.vmo_fn_activation.argtypes = [C.c_int, C.POINTER(C.c_float), C.c_int, C.c_int]
         L.vmo_fn_shape.restype = C.c_float
         L.vmo_fn_shape.argtypes = [C.c_int, C.c_float, C.c_int, C.c_float, C.c_float]
+        L.vmo_fn_libm.argtypes = [C.c_int, C.POINTER(C.c_float), C.POINTER(C.c_float), C.c_int]
         self.name = L.vmo_name().decode()
 
     # ---- meshes
@@ -165,6 +166,13 @@ class Oracle:
         d = np.ascontiguousarray(data, dtype=np.float32).copy()
         self.lib.vmo_fn_activation(act, _fp(d), d.size // dims, dims)
         return d
+
+    def fn_libm(self, which, x):
+        """host libm: which in acos, sin, tan, sqrt"""
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        y = np.zeros_like(x)
+        self.lib.vmo_fn_libm({"acos": 0, "sin": 1, "tan": 2, "sqrt": 3}[which], _fp(x), _fp(y), x.size)
+        return y
 
     def fn_shape(self, shape, radius, which, a=0.0, b=0.0):
         return self.lib.vmo_fn_shape(shape, radius, {"phi": 0, "n": 1, "theta": 2, "k": 3, "c": 4}[which], a, b)

@@ -1,0 +1,99 @@
+"""HIP engine against the CPU oracle on the benchmark configurations, through the C++ engine and so
+through the C ABI. Gates: visible-node indices and neighbour tables bit-exact, pixel coordinates within
+1e-3 px, fp32 class probabilities within 1e-4 absolute."""
+import numpy as np
+import pytest
+
+from helpers import (PROB_TOL, assert_classification_parity, assert_projection_parity, lens_pair, meshes_for, pick)
+from oracle import vmo
+from visualmesh_amd import engine as eng
+from visualmesh_amd import workloads as wl
+
+pytestmark = pytest.mark.gpu
+
+
+def _run_config(oracle, index, n_frames, batch, check_cls_frames=None):
+    cfg = wl.config(index, n_frames=n_frames)
+    o_lens, e_lens = lens_pair(cfg)
+    o_mesh, e_mesh = meshes_for(cfg, oracle)
+    engine = eng.Engine(cfg.network, cfg.model)
+    net = vmo.Network(cfg.network)
+    if batch:
+        frames = [dict(mesh=e_mesh, Hoc=f["Hoc"], lens=e_lens, image=f["image"], fourcc=cfg.fourcc) for f in cfg.frames]
+        results = engine.classify_batch(frames)
+    else:
+        results = [engine(e_mesh, f["Hoc"], e_lens, f["image"], cfg.fourcc) for f in cfg.frames]
+    for i, f in enumerate(cfg.frames):
+        label = "%s frame %d" % (cfg.name, i)
+        print(label, "V =", len(results[i]["gidx"]), flush=True)
+        if check_cls_frames is None or i in check_cls_frames:
+            want = pick(o_mesh, f["Hoc"]).classify(f["Hoc"], o_lens, f["image"], cfg.fourcc, net)
+            assert_classification_parity(results[i], want, PROB_TOL, label)
+            # the null row is an ordinary row
+            assert results[i]["cls"].shape[0] == len(results[i]["gidx"]) + 1
+        else:
+            want = pick(o_mesh, f["Hoc"]).project(f["Hoc"], o_lens)
+            assert_projection_parity(results[i], want, label)
+
+
+def test_config1_single_frame(oracle):
+    _run_config(oracle, 1, 1, batch=False)
+
+
+def test_config1_projection_only(oracle):
+    cfg = wl.config(1)
+    o_lens, e_lens = lens_pair(cfg)
+    o_mesh, e_mesh = meshes_for(cfg, oracle)
+    engine = eng.Engine([], cfg.model)
+    got = engine(e_mesh, cfg.frames[0]["Hoc"], e_lens)
+    want = o_mesh.project(cfg.frames[0]["Hoc"], o_lens)
+    assert_projection_parity(got, want, "cfg1 projection")
+
+
+def test_config2_batch(oracle):
+    _run_config(oracle, 2, 4, batch=True)
+
+
+def test_config3_bayer(oracle):
+    _run_config(oracle, 3, 1, batch=False)
+
+
+def test_device_libm_matches_host(oracle):
+    """The device's acosf/sinf/tanf/sqrtf must return the host C library's bits (a dense sample here; the
+    same source is compared exhaustively on the CPU in test_libm_exact.py)."""
+    import ctypes as C
+    from visualmesh_amd import native
+    L = native.hip()
+    rng = np.random.default_rng(7)
+    n = 1 << 22
+    cases = {
+        "acos": (0, np.concatenate([rng.uniform(-1, 1, n).astype(np.float32), (1 - np.geomspace(1e-8, 1, 4096)).astype(np.float32),
+                                    np.array([1.0, -1.0, 0.0, 0.5, -0.5], np.float32)])),
+        "sin": (1, np.concatenate([rng.uniform(0, np.pi / 2, n).astype(np.float32), np.geomspace(1e-7, 1.6, 4096).astype(np.float32)])),
+        "tan": (2, np.concatenate([rng.uniform(0, np.pi / 2, n).astype(np.float32), (np.float32(np.pi / 2) - np.geomspace(1e-7, 1, 4096)).astype(np.float32),
+                                   np.array([np.float32(np.pi / 2)], np.float32)])),
+        "sqrt": (3, rng.uniform(0, 4, n).astype(np.float32)),
+    }
+    for name, (which, x) in cases.items():
+        x = np.ascontiguousarray(x)
+        y = np.zeros_like(x)
+        native.hip_check(L.vmhip_selftest_libm(which, x.ctypes.data_as(C.POINTER(C.c_float)), y.ctypes.data_as(C.POINTER(C.c_float)), x.size))
+        want = oracle.fn_libm(name, x)
+        bad = np.flatnonzero(y.view(np.uint32) != want.view(np.uint32))
+        assert bad.size == 0, "%s: %d of %d differ, e.g. x=%r device=%r host=%r" % (name, bad.size, x.size, x[bad[0]], y[bad[0]], want[bad[0]])
+
+
+def test_pixels_and_inputs_bit_exact(oracle):
+    """Beyond the 1e-3 px gate: with the host-exact libm the pixel coordinates, and with them the sampled
+    network inputs, are bit-identical to the CPU engine's (empty network -> classifications = sampled input)."""
+    for index in (1, 3, 4):
+        cfg = wl.config(index, n_frames=1)
+        o_lens, e_lens = lens_pair(cfg)
+        o_mesh, e_mesh = meshes_for(cfg, oracle)
+        engine = eng.Engine([], cfg.model)
+        f = cfg.frames[0]
+        got = engine(e_mesh, f["Hoc"], e_lens, f["image"], cfg.fourcc)
+        want = pick(o_mesh, f["Hoc"]).classify(f["Hoc"], o_lens, f["image"], cfg.fourcc, vmo.Network([]))
+        assert np.array_equal(got["gidx"], want["gidx"])
+        assert np.array_equal(got["px"].view(np.uint32), want["px"].view(np.uint32)), "%s pixel bits" % cfg.name
+        assert np.array_equal(got["cls"].view(np.uint32), want["cls"].view(np.uint32)), "%s sampled input bits" % cfg.name

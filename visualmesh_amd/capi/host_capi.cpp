@@ -1,0 +1,313 @@
+/*
+ * host_capi.cpp - a small C interface over the C++ host code (Mesh, VisualMesh and
+ * visualmesh::engine::hip::Engine), so that Python tests and the benchmark drive exactly the C++ a user
+ * of the engine would write. Built into libvisualmesh_host.so, which links libvisualmesh_hip.so.
+ *
+ * Functions return a count / 0 on success or a negative status (the VMHIP_ERR_* values);
+ * vmh_last_error() holds the message of the last failure on the calling thread.
+ */
+#include <cstring>
+#include <memory>
+#include <stdexcept>
+#include <string>
+#include <system_error>
+#include <vector>
+
+#include "visualmesh/engine/hip/engine.hpp"
+#include "visualmesh/geometry/Circle.hpp"
+#include "visualmesh/geometry/Sphere.hpp"
+#include "visualmesh/mesh.hpp"
+#include "visualmesh/model/nmgrid8.hpp"
+#include "visualmesh/model/ring6.hpp"
+#include "visualmesh/visualmesh.hpp"
+
+using namespace visualmesh;
+using geometry::Circle;
+using geometry::Sphere;
+using model::NMGrid8;
+using model::Ring6;
+typedef engine::hip::Engine<float> HipEngine;
+
+enum { VMH_RING6 = 0, VMH_NMGRID8 = 1 };
+enum { VMH_SPHERE = 0, VMH_CIRCLE = 1 };
+
+struct vmh_mesh {
+    const Mesh<float, Ring6>* r6 = nullptr;
+    const Mesh<float, NMGrid8>* g8 = nullptr;
+    std::unique_ptr<Mesh<float, Ring6>> own_r6;
+    std::unique_ptr<Mesh<float, NMGrid8>> own_g8;
+};
+struct vmh_visualmesh {
+    std::unique_ptr<VisualMesh<float, Ring6>> r6;
+    std::unique_ptr<VisualMesh<float, NMGrid8>> g8;
+    std::vector<std::unique_ptr<vmh_mesh>> views;  // ascending height
+};
+struct vmh_engine {
+    int model;
+    std::unique_ptr<HipEngine> engine;
+    std::vector<ClassifiedMesh<float, 6>> fetched6;
+    std::vector<ClassifiedMesh<float, 8>> fetched8;
+};
+
+namespace {
+thread_local std::string g_error;
+
+int report(const std::exception& e) {
+    g_error = e.what();
+    if (const std::system_error* se = dynamic_cast<const std::system_error*>(&e)) return se->code().value();
+    if (g_error.find("Unsupported image format") != std::string::npos) return VMHIP_ERR_FORMAT;
+    if (g_error.find("lens") != std::string::npos) return VMHIP_ERR_LENS;
+    return VMHIP_ERR_ARGUMENT;
+}
+#define GUARD(...)                      \
+    try {                               \
+        __VA_ARGS__                     \
+    } catch (const std::exception& e) { \
+        return report(e);               \
+    }
+
+Lens<float> to_lens(const vmhip_lens* l) {
+    Lens<float> lens;
+    lens.dimensions = {{l->width, l->height}};
+    lens.projection = LensProjection(l->projection);
+    lens.focal_length = l->focal_length;
+    lens.centre = {{l->centre[0], l->centre[1]}};
+    lens.k = {{l->k[0], l->k[1]}};
+    lens.fov = l->fov;
+    return lens;
+}
+mat4<float> to_hoc(const float* H) {
+    mat4<float> m;
+    for (int i = 0; i < 4; ++i)
+        for (int j = 0; j < 4; ++j) m[i][j] = H[i * 4 + j];
+    return m;
+}
+NetworkStructure<float> to_network(const vmhip_network* net) {
+    NetworkStructure<float> s;
+    int li = 0;
+    for (int g = 0; net && g < net->n_groups; ++g) {
+        s.emplace_back();
+        for (int l = 0; l < net->group_sizes[g]; ++l, ++li) {
+            const vmhip_layer& L = net->layers[li];
+            Layer<float> layer;
+            layer.weights.assign(L.n_in, std::vector<float>(L.n_out));
+            for (int t = 0; t < L.n_in; ++t)
+                for (int j = 0; j < L.n_out; ++j) layer.weights[t][j] = L.weights[size_t(t) * L.n_out + j];
+            layer.biases.assign(L.biases, L.biases + L.n_out);
+            layer.activation = ActivationFunction(L.activation);
+            s.back().push_back(std::move(layer));
+        }
+    }
+    return s;
+}
+
+template <typename M>
+void copy_nodes(const M& mesh, float* rays, int32_t* nbr) {
+    const int nn = M::N_NEIGHBOURS;
+    for (size_t i = 0; i < mesh.nodes.size(); ++i) {
+        if (rays)
+            for (int c = 0; c < 3; ++c) rays[i * 3 + c] = mesh.nodes[i].ray[c];
+        if (nbr)
+            for (int t = 0; t < nn; ++t) nbr[i * nn + t] = mesh.nodes[i].neighbours[t];
+    }
+}
+
+template <typename R>
+int export_result(const R& r, int cap, float* px, int32_t* nb, int32_t* gidx) {
+    const int V = int(r.global_indices.size());
+    if (V > cap) {
+        g_error = "result capacity too small";
+        return VMHIP_ERR_CAPACITY;
+    }
+    if (V == 0) return 0;
+    if (px) std::memcpy(px, r.pixel_coordinates.data(), sizeof(float) * 2 * V);
+    if (gidx) std::memcpy(gidx, r.global_indices.data(), sizeof(int32_t) * V);
+    if (nb) std::memcpy(nb, r.neighbourhood.data(), sizeof(r.neighbourhood[0]) * r.neighbourhood.size());
+    return V;
+}
+}  // namespace
+
+extern "C" {
+
+const char* vmh_last_error(void) { return g_error.c_str(); }
+
+vmh_mesh* vmh_mesh_create(int model, int shape, float radius, float h, float k, float max_distance) {
+    try {
+        std::unique_ptr<vmh_mesh> m(new vmh_mesh());
+        if (model == VMH_RING6) {
+            if (shape == VMH_SPHERE) m->own_r6.reset(new Mesh<float, Ring6>(Sphere<float>(radius), h, k, max_distance));
+            else if (shape == VMH_CIRCLE) m->own_r6.reset(new Mesh<float, Ring6>(Circle<float>(radius), h, k, max_distance));
+            else return nullptr;
+            m->r6 = m->own_r6.get();
+        }
+        else if (model == VMH_NMGRID8) {
+            if (shape == VMH_SPHERE) m->own_g8.reset(new Mesh<float, NMGrid8>(Sphere<float>(radius), h, k, max_distance));
+            else if (shape == VMH_CIRCLE) m->own_g8.reset(new Mesh<float, NMGrid8>(Circle<float>(radius), h, k, max_distance));
+            else return nullptr;
+            m->g8 = m->own_g8.get();
+        }
+        else return nullptr;
+        return m.release();
+    } catch (const std::exception& e) {
+        g_error = e.what();
+        return nullptr;
+    }
+}
+void vmh_mesh_destroy(vmh_mesh* m) { delete m; }
+int vmh_mesh_n_nodes(const vmh_mesh* m) { return m->r6 ? int(m->r6->nodes.size()) : int(m->g8->nodes.size()); }
+int vmh_mesh_n_neighbours(const vmh_mesh* m) { return m->r6 ? 6 : 8; }
+float vmh_mesh_h(const vmh_mesh* m) { return m->r6 ? m->r6->h : m->g8->h; }
+void vmh_mesh_copy(const vmh_mesh* m, float* rays, int32_t* neighbours) {
+    if (m->r6) copy_nodes(*m->r6, rays, neighbours);
+    else copy_nodes(*m->g8, rays, neighbours);
+}
+int vmh_mesh_lookup(const vmh_mesh* m, const float* Hoc16, const vmhip_lens* lens, int32_t* ranges, int cap) {
+    GUARD({
+        const auto r = m->r6 ? m->r6->lookup(to_hoc(Hoc16), to_lens(lens)) : m->g8->lookup(to_hoc(Hoc16), to_lens(lens));
+        for (int i = 0; i < int(r.size()) && i < cap; ++i) {
+            ranges[2 * i] = r[i].first;
+            ranges[2 * i + 1] = r[i].second;
+        }
+        return int(r.size());
+    })
+}
+
+vmh_visualmesh* vmh_visualmesh_create(int model, int shape, float radius, float min_h, float max_h, float k, float max_error,
+                                      float max_distance) {
+    try {
+        std::unique_ptr<vmh_visualmesh> v(new vmh_visualmesh());
+        if (model == VMH_RING6) {
+            if (shape == VMH_SPHERE) v->r6.reset(new VisualMesh<float, Ring6>(Sphere<float>(radius), min_h, max_h, k, max_error, max_distance));
+            else v->r6.reset(new VisualMesh<float, Ring6>(Circle<float>(radius), min_h, max_h, k, max_error, max_distance));
+            for (const auto& kv : v->r6->meshes()) {
+                std::unique_ptr<vmh_mesh> view(new vmh_mesh());
+                view->r6 = &kv.second;
+                v->views.push_back(std::move(view));
+            }
+        }
+        else if (model == VMH_NMGRID8) {
+            if (shape == VMH_SPHERE) v->g8.reset(new VisualMesh<float, NMGrid8>(Sphere<float>(radius), min_h, max_h, k, max_error, max_distance));
+            else v->g8.reset(new VisualMesh<float, NMGrid8>(Circle<float>(radius), min_h, max_h, k, max_error, max_distance));
+            for (const auto& kv : v->g8->meshes()) {
+                std::unique_ptr<vmh_mesh> view(new vmh_mesh());
+                view->g8 = &kv.second;
+                v->views.push_back(std::move(view));
+            }
+        }
+        else return nullptr;
+        return v.release();
+    } catch (const std::exception& e) {
+        g_error = e.what();
+        return nullptr;
+    }
+}
+void vmh_visualmesh_destroy(vmh_visualmesh* v) { delete v; }
+int vmh_visualmesh_n_meshes(const vmh_visualmesh* v) { return int(v->views.size()); }
+const vmh_mesh* vmh_visualmesh_mesh(const vmh_visualmesh* v, int i) { return v->views[i].get(); }
+const vmh_mesh* vmh_visualmesh_height(const vmh_visualmesh* v, float h) {
+    const void* picked = v->r6 ? static_cast<const void*>(&v->r6->height(h)) : static_cast<const void*>(&v->g8->height(h));
+    for (const auto& view : v->views)
+        if (static_cast<const void*>(view->r6) == picked || static_cast<const void*>(view->g8) == picked) return view.get();
+    return nullptr;
+}
+
+int vmh_engine_create(const vmhip_network* net, int model, int precision, vmh_engine** out) {
+    GUARD({
+        std::unique_ptr<vmh_engine> e(new vmh_engine());
+        e->model = model;
+        e->engine.reset(new HipEngine(to_network(net), engine::hip::Precision(precision)));
+        *out = e.release();
+        return 0;
+    })
+}
+void vmh_engine_destroy(vmh_engine* e) { delete e; }
+
+int vmh_engine_project(vmh_engine* e, const vmh_mesh* m, const float* Hoc16, const vmhip_lens* lens, int cap, float* px,
+                       int32_t* nb, int32_t* gidx) {
+    GUARD({
+        if (m->r6) return export_result(e->engine->project(*m->r6, to_hoc(Hoc16), to_lens(lens)), cap, px, nb, gidx);
+        return export_result(e->engine->project(*m->g8, to_hoc(Hoc16), to_lens(lens)), cap, px, nb, gidx);
+    })
+}
+
+int vmh_engine_classify(vmh_engine* e, const vmh_mesh* m, const float* Hoc16, const vmhip_lens* lens, const void* image,
+                        uint32_t fourcc, int cap, float* px, int32_t* nb, int32_t* gidx, float* cls) {
+    GUARD({
+        if (m->r6) {
+            const auto r = (*e->engine)(*m->r6, to_hoc(Hoc16), to_lens(lens), image, fourcc);
+            const int V = export_result(r, cap, px, nb, gidx);
+            if (V > 0 && cls) std::memcpy(cls, r.classifications.data(), sizeof(float) * r.classifications.size());
+            return V;
+        }
+        const auto r = (*e->engine)(*m->g8, to_hoc(Hoc16), to_lens(lens), image, fourcc);
+        const int V = export_result(r, cap, px, nb, gidx);
+        if (V > 0 && cls) std::memcpy(cls, r.classifications.data(), sizeof(float) * r.classifications.size());
+        return V;
+    })
+}
+
+/* staged batch: all frames must use meshes of the engine's model */
+int vmh_engine_stage(vmh_engine* e, int n, const vmh_mesh* const* meshes, const float* Hoc16s, const vmhip_lens* lenses,
+                     const void* const* images, const uint32_t* fourccs) {
+    GUARD({
+        if (e->model == VMH_RING6) {
+            std::vector<HipEngine::Frame<Ring6>> frames(n);
+            for (int i = 0; i < n; ++i) {
+                if (!meshes[i]->r6) throw std::invalid_argument("mesh model does not match the engine");
+                frames[i] = HipEngine::Frame<Ring6>{meshes[i]->r6, to_hoc(Hoc16s + 16 * i), to_lens(lenses + i), images[i], fourccs[i]};
+            }
+            e->engine->stage(frames);
+        }
+        else {
+            std::vector<HipEngine::Frame<NMGrid8>> frames(n);
+            for (int i = 0; i < n; ++i) {
+                if (!meshes[i]->g8) throw std::invalid_argument("mesh model does not match the engine");
+                frames[i] = HipEngine::Frame<NMGrid8>{meshes[i]->g8, to_hoc(Hoc16s + 16 * i), to_lens(lenses + i), images[i], fourccs[i]};
+            }
+            e->engine->stage(frames);
+        }
+        return 0;
+    })
+}
+int vmh_engine_run(vmh_engine* e) {
+    GUARD({
+        e->engine->run();
+        return 0;
+    })
+}
+int vmh_engine_counts(vmh_engine* e, int32_t* visible, int n) {
+    GUARD({
+        const std::vector<int32_t> v = e->engine->visible_counts();
+        for (int i = 0; i < n && i < int(v.size()); ++i) visible[i] = v[i];
+        return int(v.size());
+    })
+}
+/* downloads every frame of the last run into the harness */
+int vmh_engine_fetch(vmh_engine* e) {
+    GUARD({
+        if (e->model == VMH_RING6) {
+            e->fetched6 = e->engine->fetch<Ring6>();
+            return int(e->fetched6.size());
+        }
+        e->fetched8 = e->engine->fetch<NMGrid8>();
+        return int(e->fetched8.size());
+    })
+}
+/* copies frame i of the last fetch */
+int vmh_engine_result(vmh_engine* e, int i, int cap, float* px, int32_t* nb, int32_t* gidx, float* cls) {
+    GUARD({
+        if (e->model == VMH_RING6) {
+            const auto& r = e->fetched6.at(i);
+            const int V = export_result(r, cap, px, nb, gidx);
+            if (V > 0 && cls) std::memcpy(cls, r.classifications.data(), sizeof(float) * r.classifications.size());
+            return V;
+        }
+        const auto& r = e->fetched8.at(i);
+        const int V = export_result(r, cap, px, nb, gidx);
+        if (V > 0 && cls) std::memcpy(cls, r.classifications.data(), sizeof(float) * r.classifications.size());
+        return V;
+    })
+}
+void* vmh_engine_native_batch(vmh_engine* e) { return e->engine->native_batch(); }
+void vmh_engine_clear_cache(vmh_engine* e) { e->engine->clear_cache(); }
+}

@@ -1,0 +1,373 @@
+/*
+ * visualmesh::engine::hip::Engine - the Visual Mesh engine for AMD MI355X (gfx950).
+ *
+ * Same interface as the reference's engines (reference engine/cpu/engine.hpp:49-306,
+ * engine/opencl/engine.hpp:172-572):
+ *
+ *     Engine(const NetworkStructure<Scalar>& structure = {});
+ *     ProjectedMesh  engine(mesh, Hoc, lens);                    // also engine.project(mesh, Hoc, lens)
+ *     ClassifiedMesh engine(mesh, Hoc, lens, image, format);
+ *
+ * with `mesh` either a Mesh<Scalar, Model> or a VisualMesh<Scalar, Model> (which picks the mesh for the
+ * camera height Hoc[2][3]). In addition a batch of frames can be classified in one pass, either in one
+ * call (classify(frames)) or staged (stage / run / fetch) to keep inputs resident on the device.
+ *
+ * This header is host C++14 and contains no device code: it runs Mesh::lookup on the host, flattens the
+ * STL types and calls the C ABI of libvisualmesh_hip.so (include/visualmesh_hip.h). It only uses
+ * `mesh.nodes` and `mesh.lookup(Hoc, lens)`, so it works with any Mesh type that has them.
+ *
+ * Results are those of the reference CPU engine on a fresh engine object: visible-node indices and the
+ * neighbourhood table bit for bit, pixel coordinates to the last bits of acosf/sinf/tanf, class
+ * probabilities to summation order.
+ *
+ * Errors: an unsupported fourcc or lens projection throws std::runtime_error with the reference's
+ * message; any other failure throws std::system_error with hip_error_category(). An empty visible set is
+ * not an error and returns a default-constructed result.
+ *
+ * Like the reference engines an Engine is not thread safe: use one engine per thread; meshes may be
+ * shared.
+ */
+#ifndef VISUALMESH_ENGINE_HIP_ENGINE_HPP
+#define VISUALMESH_ENGINE_HIP_ENGINE_HPP
+
+#include <cstdint>
+#include <cstring>
+#include <map>
+#include <stdexcept>
+#include <string>
+#include <system_error>
+#include <type_traits>
+#include <utility>
+#include <vector>
+
+#include "visualmesh/classified_mesh.hpp"
+#include "visualmesh/lens.hpp"
+#include "visualmesh/mesh.hpp"
+#include "visualmesh/network_structure.hpp"
+#include "visualmesh/projected_mesh.hpp"
+#include "visualmesh/visualmesh.hpp"
+#include "visualmesh_hip.h"
+
+namespace visualmesh {
+namespace engine {
+    namespace hip {
+
+        /// Error category for the status codes of libvisualmesh_hip.so.
+        class error_category_t : public std::error_category {
+        public:
+            const char* name() const noexcept override { return "visualmesh_hip"; }
+            std::string message(int code) const override {
+                switch (code) {
+                    case VMHIP_OK: return "success";
+                    case VMHIP_ERR_HIP: return "HIP runtime failure";
+                    case VMHIP_ERR_FORMAT: return "unsupported image format";
+                    case VMHIP_ERR_LENS: return "unknown lens projection";
+                    case VMHIP_ERR_ARGUMENT: return "invalid argument";
+                    case VMHIP_ERR_CAPACITY: return "result buffer too small";
+                    default: return "unknown error";
+                }
+            }
+        };
+        inline const std::error_category& hip_error_category() {
+            static error_category_t instance;
+            return instance;
+        }
+        inline void throw_on_error(int code) {
+            if (code == VMHIP_OK) return;
+            const std::string what = vmhip_last_error();
+            if (code == VMHIP_ERR_FORMAT || code == VMHIP_ERR_LENS) throw std::runtime_error(what);
+            throw std::system_error(code, hip_error_category(), what);
+        }
+
+        enum class Precision { FP32 = VMHIP_FP32, BF16 = VMHIP_BF16 };
+
+        template <typename Scalar>
+        class Engine {
+            static_assert(std::is_same<Scalar, float>::value, "the HIP engine computes in float");
+
+        public:
+            /// One frame of a batch.
+            template <template <typename> class Model>
+            struct Frame {
+                const Mesh<Scalar, Model>* mesh;
+                mat4<Scalar> Hoc;
+                Lens<Scalar> lens;
+                const void* image;
+                uint32_t format;
+            };
+
+            Engine(const NetworkStructure<Scalar>& structure = {}, Precision precision = Precision::FP32)
+              : precision_(precision) {
+                for (const auto& group : structure) {
+                    group_sizes_.push_back(int32_t(group.size()));
+                    for (const auto& layer : group) {
+                        FlatLayer flat;
+                        flat.n_in = int32_t(layer.weights.size());
+                        flat.n_out = int32_t(layer.biases.size());
+                        flat.activation = int32_t(layer.activation);
+                        flat.weights.reserve(size_t(flat.n_in) * flat.n_out);
+                        for (const auto& row : layer.weights) {
+                            if (int32_t(row.size()) != flat.n_out) throw std::invalid_argument("ragged weight matrix");
+                            flat.weights.insert(flat.weights.end(), row.begin(), row.end());
+                        }
+                        flat.biases = layer.biases;
+                        layers_.push_back(std::move(flat));
+                    }
+                }
+            }
+            ~Engine() { release(); }
+            Engine(const Engine&) = delete;
+            Engine& operator=(const Engine&) = delete;
+            Engine(Engine&& o) noexcept { *this = std::move(o); }
+            Engine& operator=(Engine&& o) noexcept {
+                if (this != &o) {
+                    release();
+                    precision_ = o.precision_;
+                    group_sizes_ = std::move(o.group_sizes_);
+                    layers_ = std::move(o.layers_);
+                    engine_ = o.engine_;
+                    engine_nn_ = o.engine_nn_;
+                    batch_ = o.batch_;
+                    meshes_ = std::move(o.meshes_);
+                    staged_ = std::move(o.staged_);
+                    o.engine_ = nullptr;
+                    o.batch_ = nullptr;
+                    o.meshes_.clear();
+                }
+                return *this;
+            }
+
+            // ------------------------------------------------------------------ projection
+            template <template <typename> class Model>
+            ProjectedMesh<Scalar, Model<Scalar>::N_NEIGHBOURS> operator()(const Mesh<Scalar, Model>& mesh,
+                                                                          const mat4<Scalar>& Hoc,
+                                                                          const Lens<Scalar>& lens) const {
+                constexpr int N = Model<Scalar>::N_NEIGHBOURS;
+                FrameData fd;
+                describe(mesh, Hoc, lens, nullptr, 0, fd);
+                ProjectedMesh<Scalar, N> out;
+                if (fd.candidates == 0) return out;
+                out.pixel_coordinates.resize(fd.candidates);
+                out.global_indices.resize(fd.candidates);
+                out.neighbourhood.resize(size_t(fd.candidates) + 1);
+                vmhip_result r{};
+                r.capacity = fd.candidates;
+                r.pixel_coordinates = reinterpret_cast<float*>(out.pixel_coordinates.data());
+                r.global_indices = out.global_indices.data();
+                r.neighbourhood = reinterpret_cast<int32_t*>(out.neighbourhood.data());
+                throw_on_error(vmhip_project(handle(N), &fd.frame, &r));
+                if (r.n_visible == 0) return ProjectedMesh<Scalar, N>();
+                out.pixel_coordinates.resize(r.n_visible);
+                out.global_indices.resize(r.n_visible);
+                out.neighbourhood.resize(size_t(r.n_visible) + 1);
+                return out;
+            }
+            template <template <typename> class Model>
+            ProjectedMesh<Scalar, Model<Scalar>::N_NEIGHBOURS> operator()(const VisualMesh<Scalar, Model>& mesh,
+                                                                          const mat4<Scalar>& Hoc,
+                                                                          const Lens<Scalar>& lens) const {
+                return operator()(mesh.height(Hoc[2][3]), Hoc, lens);
+            }
+            template <typename AnyMesh>
+            auto project(const AnyMesh& mesh, const mat4<Scalar>& Hoc, const Lens<Scalar>& lens) const
+              -> decltype(this->operator()(mesh, Hoc, lens)) {
+                return operator()(mesh, Hoc, lens);
+            }
+
+            // ------------------------------------------------------------------ classification
+            template <template <typename> class Model>
+            ClassifiedMesh<Scalar, Model<Scalar>::N_NEIGHBOURS> operator()(const Mesh<Scalar, Model>& mesh,
+                                                                           const mat4<Scalar>& Hoc,
+                                                                           const Lens<Scalar>& lens,
+                                                                           const void* image,
+                                                                           const uint32_t& format) const {
+                std::vector<Frame<Model>> one(1, Frame<Model>{&mesh, Hoc, lens, image, format});
+                return std::move(classify(one)[0]);
+            }
+            template <template <typename> class Model>
+            ClassifiedMesh<Scalar, Model<Scalar>::N_NEIGHBOURS> operator()(const VisualMesh<Scalar, Model>& mesh,
+                                                                           const mat4<Scalar>& Hoc,
+                                                                           const Lens<Scalar>& lens,
+                                                                           const void* image,
+                                                                           const uint32_t& format) const {
+                return operator()(mesh.height(Hoc[2][3]), Hoc, lens, image, format);
+            }
+
+            /// Classify a batch of independent frames in one pass over the device.
+            template <template <typename> class Model>
+            std::vector<ClassifiedMesh<Scalar, Model<Scalar>::N_NEIGHBOURS>> classify(const std::vector<Frame<Model>>& frames) const {
+                stage(frames);
+                run();
+                return fetch<Model>();
+            }
+
+            /// Copy the frames' inputs to the device (images, poses, lenses, lookup ranges).
+            template <template <typename> class Model>
+            void stage(const std::vector<Frame<Model>>& frames) const {
+                constexpr int N = Model<Scalar>::N_NEIGHBOURS;
+                staged_.assign(frames.size(), FrameData());
+                std::vector<vmhip_frame> flat(frames.size());
+                for (size_t i = 0; i < frames.size(); ++i) {
+                    describe(*frames[i].mesh, frames[i].Hoc, frames[i].lens, frames[i].image, frames[i].format, staged_[i]);
+                    flat[i] = staged_[i].frame;
+                }
+                vmhip_engine* e = handle(N);
+                if (!batch_) throw_on_error(vmhip_batch_create(e, &batch_));
+                if (!flat.empty()) throw_on_error(vmhip_batch_stage(batch_, flat.data(), int32_t(flat.size()), 1));
+            }
+            /// Run the staged frames on the device and wait; may be called repeatedly.
+            void run() const {
+                if (batch_ && !staged_.empty()) throw_on_error(vmhip_batch_run(batch_));
+            }
+            /// Download the results of the last run.
+            template <template <typename> class Model>
+            std::vector<ClassifiedMesh<Scalar, Model<Scalar>::N_NEIGHBOURS>> fetch() const {
+                constexpr int N = Model<Scalar>::N_NEIGHBOURS;
+                const size_t n = staged_.size();
+                std::vector<ClassifiedMesh<Scalar, N>> out(n);
+                if (n == 0) return out;
+                const int classes = vmhip_engine_n_classes(engine_);
+                std::vector<int32_t> visible(n);
+                throw_on_error(vmhip_batch_counts(batch_, visible.data()));
+                std::vector<vmhip_result> results(n);
+                for (size_t i = 0; i < n; ++i) {
+                    const int V = visible[i];
+                    vmhip_result& r = results[i];
+                    std::memset(&r, 0, sizeof(r));
+                    r.capacity = V;
+                    if (V == 0) continue;
+                    out[i].pixel_coordinates.resize(V);
+                    out[i].global_indices.resize(V);
+                    out[i].neighbourhood.resize(size_t(V) + 1);
+                    out[i].classifications.resize((size_t(V) + 1) * classes);
+                    r.pixel_coordinates = reinterpret_cast<float*>(out[i].pixel_coordinates.data());
+                    r.global_indices = out[i].global_indices.data();
+                    r.neighbourhood = reinterpret_cast<int32_t*>(out[i].neighbourhood.data());
+                    r.classifications = out[i].classifications.data();
+                }
+                throw_on_error(vmhip_batch_fetch(batch_, results.data()));
+                return out;
+            }
+            /// Visible nodes per staged frame after run().
+            std::vector<int32_t> visible_counts() const {
+                std::vector<int32_t> v(staged_.size());
+                if (!v.empty()) throw_on_error(vmhip_batch_counts(batch_, v.data()));
+                return v;
+            }
+            /// The batch object behind stage/run/fetch, for profiling hooks.
+            vmhip_batch* native_batch() const { return batch_; }
+
+            /// Forget the device copies of all meshes (same purpose as the reference OpenCL engine's
+            /// clear_cache, engine/opencl/engine.hpp:559-572). Call it before destroying a mesh this engine
+            /// has seen if another mesh may be created at the same address with the same node count.
+            void clear_cache() {
+                for (auto& kv : meshes_) vmhip_mesh_release(kv.second.device);
+                meshes_.clear();
+            }
+
+        private:
+            struct FlatLayer {
+                int32_t n_in, n_out, activation;
+                std::vector<float> weights, biases;
+            };
+            struct MeshEntry {
+                const void* nodes;
+                size_t count;
+                vmhip_mesh* device;
+            };
+            struct FrameData {
+                vmhip_frame frame;
+                std::vector<int32_t> ranges;
+                int32_t candidates = 0;
+            };
+
+            vmhip_engine* handle(int n_neighbours) const {
+                if (engine_ && engine_nn_ == n_neighbours) return engine_;
+                if (engine_) throw std::invalid_argument("this engine was already used with a different neighbour count");
+                std::vector<vmhip_layer> flat(layers_.size());
+                for (size_t i = 0; i < layers_.size(); ++i)
+                    flat[i] = vmhip_layer{layers_[i].n_in, layers_[i].n_out, layers_[i].activation, layers_[i].weights.data(),
+                                          layers_[i].biases.data()};
+                vmhip_network net{int32_t(group_sizes_.size()), group_sizes_.data(), flat.data()};
+                throw_on_error(vmhip_engine_create(&net, n_neighbours, int32_t(precision_), &engine_));
+                engine_nn_ = n_neighbours;
+                return engine_;
+            }
+
+            template <template <typename> class Model>
+            vmhip_mesh* device_mesh(const Mesh<Scalar, Model>& mesh) const {
+                constexpr int N = Model<Scalar>::N_NEIGHBOURS;
+                auto it = meshes_.find(&mesh);
+                if (it != meshes_.end() && it->second.nodes == mesh.nodes.data() && it->second.count == mesh.nodes.size())
+                    return it->second.device;
+                if (it != meshes_.end()) {  // another mesh now lives at this address
+                    vmhip_mesh_release(it->second.device);
+                    meshes_.erase(it);
+                }
+                const size_t n = mesh.nodes.size();
+                std::vector<float> rays(n * 3);
+                std::vector<int32_t> nbr(n * N);
+                for (size_t i = 0; i < n; ++i) {
+                    for (int c = 0; c < 3; ++c) rays[i * 3 + c] = mesh.nodes[i].ray[c];
+                    for (int t = 0; t < N; ++t) nbr[i * N + t] = mesh.nodes[i].neighbours[t];
+                }
+                vmhip_mesh* dev = nullptr;
+                throw_on_error(vmhip_mesh_upload(rays.data(), nbr.data(), int32_t(n), N, &dev));
+                meshes_[&mesh] = MeshEntry{mesh.nodes.data(), n, dev};
+                return dev;
+            }
+
+            template <template <typename> class Model>
+            void describe(const Mesh<Scalar, Model>& mesh, const mat4<Scalar>& Hoc, const Lens<Scalar>& lens, const void* image,
+                          uint32_t format, FrameData& fd) const {
+                const auto ranges = mesh.lookup(Hoc, lens);  // host side of the path
+                fd.ranges.resize(ranges.size() * 2);
+                fd.candidates = 0;
+                for (size_t i = 0; i < ranges.size(); ++i) {
+                    fd.ranges[2 * i] = ranges[i].first;
+                    fd.ranges[2 * i + 1] = ranges[i].second;
+                    fd.candidates += ranges[i].second - ranges[i].first;
+                }
+                vmhip_frame& f = fd.frame;
+                std::memset(&f, 0, sizeof(f));
+                f.mesh = device_mesh(mesh);
+                for (int i = 0; i < 3; ++i)
+                    for (int j = 0; j < 3; ++j) f.Rco[i * 3 + j] = Hoc[j][i];
+                f.lens.width = lens.dimensions[0];
+                f.lens.height = lens.dimensions[1];
+                f.lens.projection = int32_t(lens.projection);
+                f.lens.focal_length = lens.focal_length;
+                f.lens.centre[0] = lens.centre[0];
+                f.lens.centre[1] = lens.centre[1];
+                f.lens.k[0] = lens.k[0];
+                f.lens.k[1] = lens.k[1];
+                f.lens.fov = lens.fov;
+                f.ranges = fd.ranges.data();
+                f.n_ranges = int32_t(ranges.size());
+                f.image = image;
+                f.fourcc = format;
+            }
+
+            void release() {
+                if (batch_) vmhip_batch_destroy(batch_);
+                batch_ = nullptr;
+                clear_cache();
+                if (engine_) vmhip_engine_destroy(engine_);
+                engine_ = nullptr;
+            }
+
+            Precision precision_ = Precision::FP32;
+            std::vector<int32_t> group_sizes_;
+            std::vector<FlatLayer> layers_;
+            mutable vmhip_engine* engine_ = nullptr;
+            mutable int engine_nn_ = -1;
+            mutable vmhip_batch* batch_ = nullptr;
+            mutable std::map<const void*, MeshEntry> meshes_;
+            mutable std::vector<FrameData> staged_;
+        };
+
+    }  // namespace hip
+}  // namespace engine
+}  // namespace visualmesh
+
+#endif  // VISUALMESH_ENGINE_HIP_ENGINE_HPP

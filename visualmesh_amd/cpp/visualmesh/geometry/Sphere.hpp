@@ -1,0 +1,44 @@
+/*
+ * Sphere of radius r resting on the observation plane: the shape functions a mesh generator needs
+ * (reference geometry/Sphere.hpp:55-134). fp32 only; operand types follow the reference so that the
+ * generated mesh is bit-identical.
+ */
+#ifndef VISUALMESH_GEOMETRY_SPHERE_HPP
+#define VISUALMESH_GEOMETRY_SPHERE_HPP
+
+#include <cmath>
+#include <type_traits>
+
+namespace visualmesh {
+namespace geometry {
+
+    template <typename Scalar>
+    struct Sphere {
+        static_assert(std::is_same<Scalar, float>::value, "the host mesh code is written for float");
+        explicit Sphere(const Scalar& radius) : r(radius) {}
+
+        /// angle from straight down to the centre of the n-th object
+        Scalar phi(const Scalar& n, const Scalar& h) const { return -std::atan(std::sinh(n * std::log1p(-2.0f * r / h))); }
+        /// inverse of phi
+        Scalar n(const Scalar& phi_, const Scalar& h) const { return std::asinh(std::tan(-phi_)) / std::log1p(-2.0f * r / h); }
+        /// ratio of intersections seen from h1 versus h0
+        Scalar k(const Scalar& h0, const Scalar& h1) const {
+            return (std::log(h1 - 2 * r) - std::log(h1)) / (std::log(h0 - 2 * r) - std::log(h0));
+        }
+        /// height of the object's centre above the plane
+        const Scalar& c() const { return r; }
+        /// angular width of the object at ring n. Below n = 0.5 it is interpolated from 2 pi to pi; that arm
+        /// divides in double and both arms meet in double before the result is rounded.
+        Scalar theta(const Scalar& n, const Scalar& h) const {
+            const double v = n <= 0.5 ? double(float(2.0 * M_PI)) / (1.0 + double(n * 2.0f))
+                                      : double(2.0f * std::asin(r / ((h - r) * std::tan(phi(n, h)))));
+            return float(v);
+        }
+
+        Scalar r;
+    };
+
+}  // namespace geometry
+}  // namespace visualmesh
+
+#endif  // VISUALMESH_GEOMETRY_SPHERE_HPP

@@ -1,0 +1,71 @@
+/*
+ * Mesh<Scalar, Model>: a Visual Mesh for one camera height - nodes in cone-tree order plus the tree that
+ * answers "which index ranges can be on screen" (interface of reference mesh.hpp:56-609: constructor
+ * :424-467, lookup :499-595, public members h, max_distance, nodes).
+ *
+ * Generation and lookup stay on the host. The HIP engine uploads `nodes` once per mesh and receives the
+ * lookup ranges per frame.
+ */
+#ifndef VISUALMESH_MESH_HPP
+#define VISUALMESH_MESH_HPP
+
+#include <type_traits>
+#include <utility>
+#include <vector>
+
+#include "detail/cone_tree.hpp"
+#include "types.hpp"
+
+namespace visualmesh {
+
+template <typename Scalar, template <typename> class Model>
+class Mesh {
+    static_assert(std::is_same<Scalar, float>::value, "the host mesh code is written for float");
+
+public:
+    static constexpr int N_NEIGHBOURS = Model<Scalar>::N_NEIGHBOURS;
+    typedef Node<Scalar, N_NEIGHBOURS> node_type;
+
+    /**
+     * @param shape         object the mesh is sized for (Sphere, Circle)
+     * @param h             height of the camera above the observation plane
+     * @param k             number of mesh intersections per object
+     * @param max_distance  how far along the plane the mesh reaches
+     */
+    template <typename Shape>
+    Mesh(const Shape& shape, const Scalar& h, const Scalar& k, const Scalar& max_distance)
+      : h(h), max_distance(max_distance) {
+        std::vector<node_type> generated = Model<Scalar>::generate(shape, h, k, max_distance);
+        const int n = int(generated.size());
+        std::vector<detail::f3> rays(n);
+        for (int i = 0; i < n; ++i) rays[i] = generated[i].ray;
+
+        const std::vector<int> order = tree_.build(rays);
+
+        // generation index -> sorted position; "no neighbour" (n) maps to itself
+        std::vector<int> position(size_t(n) + 1);
+        position[n] = n;
+        for (int i = 0; i < n; ++i) position[order[i]] = i;
+        nodes.resize(n);
+        for (int i = 0; i < n; ++i) {
+            nodes[i].ray = generated[order[i]].ray;
+            for (int t = 0; t < N_NEIGHBOURS; ++t) nodes[i].neighbours[t] = position[generated[order[i]].neighbours[t]];
+        }
+    }
+
+    /// Index ranges [first, last) of nodes that may be on screen, ascending and disjoint.
+    std::vector<std::pair<int, int>> lookup(const mat4<Scalar>& Hoc, const Lens<Scalar>& lens) const {
+        return tree_.visible_ranges([this](int i) -> const detail::f3& { return nodes[i].ray; }, Hoc, lens);
+    }
+
+    Scalar h;                      ///< camera height this mesh was generated for
+    Scalar max_distance;           ///< reach of the mesh
+    std::vector<node_type> nodes;  ///< nodes in cone-tree order
+
+private:
+    detail::ConeTree tree_;
+};
+
+}  // namespace visualmesh
+
+#endif  // VISUALMESH_MESH_HPP

@@ -1,0 +1,677 @@
+/*
+ * api.hip - the C ABI of libvisualmesh_hip.so (include/visualmesh_hip.h): engine, mesh and batch objects,
+ * staging, the launch sequence, the host re-decision of edge-ambiguous candidates, result download.
+ */
+#include <algorithm>
+#include <cstdio>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "visualmesh_hip.h"
+#include "vmhip_internal.h"
+
+namespace {
+
+thread_local std::string g_error;
+
+int fail(int code, const std::string& msg) {
+    g_error = msg;
+    return code;
+}
+#define HIP_TRY(expr)                                                                                  \
+    do {                                                                                               \
+        hipError_t e_ = (expr);                                                                        \
+        if (e_ != hipSuccess)                                                                          \
+            return fail(VMHIP_ERR_HIP, std::string(#expr) + " failed: " + hipGetErrorString(e_));      \
+    } while (0)
+
+/* grow-only device allocation */
+struct DevBuf {
+    void* p = nullptr;
+    size_t cap = 0;
+    bool grew = false;
+    hipError_t reserve(size_t bytes) {
+        grew = false;
+        if (bytes <= cap) return hipSuccess;
+        if (p) {
+            hipError_t e = hipFree(p);
+            p = nullptr;
+            cap = 0;
+            if (e != hipSuccess) return e;
+        }
+        const size_t want = bytes + bytes / 8 + 256;
+        hipError_t e = hipMalloc(&p, want);
+        if (e != hipSuccess) {
+            p = nullptr;
+            return e;
+        }
+        cap = want;
+        grew = true;
+        return hipSuccess;
+    }
+    void release() {
+        if (p) (void) hipFree(p);
+        p = nullptr;
+        cap = 0;
+    }
+    template <typename T>
+    T* as() const {
+        return reinterpret_cast<T*>(p);
+    }
+};
+
+inline uint32_t cc(char a, char b, char c, char d) {
+    return uint32_t(uint8_t(a)) | (uint32_t(uint8_t(b)) << 8) | (uint32_t(uint8_t(c)) << 16) | (uint32_t(uint8_t(d)) << 24);
+}
+/* fourcc -> sampling kind and bytes per pixel; the accepted codes are those of reference
+ * engine/cpu/pixel.hpp:48-97 */
+bool decode_fourcc(uint32_t f, int* fmt, int* bpp) {
+    if (f == cc('R', 'G', 'B', 'A')) return *fmt = VMHIP_FMT_RGBA, *bpp = 4, true;
+    if (f == cc('B', 'G', 'R', 'A')) return *fmt = VMHIP_FMT_BGRA, *bpp = 4, true;
+    if (f == cc('R', 'G', 'B', '3') || f == cc('R', 'G', 'B', '8')) return *fmt = VMHIP_FMT_RGB3, *bpp = 3, true;
+    if (f == cc('B', 'G', 'R', '3') || f == cc('B', 'G', 'R', '8')) return *fmt = VMHIP_FMT_BGR3, *bpp = 3, true;
+    if (f == cc('G', 'R', 'A', 'Y') || f == cc('G', 'R', 'E', 'Y') || f == cc('Y', '8', ' ', ' '))
+        return *fmt = VMHIP_FMT_GRAY, *bpp = 1, true;
+    if (f == cc('G', 'R', 'B', 'G')) return *fmt = VMHIP_FMT_GRBG, *bpp = 1, true;
+    if (f == cc('R', 'G', 'G', 'B')) return *fmt = VMHIP_FMT_RGGB, *bpp = 1, true;
+    if (f == cc('G', 'B', 'R', 'G')) return *fmt = VMHIP_FMT_GBRG, *bpp = 1, true;
+    if (f == cc('B', 'G', 'G', 'R')) return *fmt = VMHIP_FMT_BGGR, *bpp = 1, true;
+    return false;
+}
+std::string fourcc_text(uint32_t f) {
+    char t[5] = {char(f & 0xff), char((f >> 8) & 0xff), char((f >> 16) & 0xff), char((f >> 24) & 0xff), 0};
+    return std::string(t);
+}
+
+inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+}  // namespace
+
+struct vmhip_mesh {
+    float* d_rays = nullptr;
+    int32_t* d_nbr = nullptr;
+    int32_t n_nodes = 0, nn = 0;
+    std::vector<float> h_rays; /* host copy for the re-decision of ambiguous candidates */
+};
+
+struct HostLayer {
+    int32_t c_in, c_out, slots, activation;
+    float* d_w = nullptr;
+    float* d_b = nullptr;
+};
+
+struct vmhip_engine {
+    int32_t nn = 0;
+    int32_t precision = VMHIP_FP32;
+    int32_t n_classes = 4;
+    int32_t max_width = 4;
+    std::vector<HostLayer> layers;
+    hipStream_t stream = nullptr;
+    vmhip_batch* scratch = nullptr; /* used by the one-call entry points */
+};
+
+struct HostFrame {
+    const vmhip_mesh* mesh;
+    std::vector<int32_t> first, prefix; /* host copies of the range table */
+    VmFrame dev;
+    float centre[2];
+};
+
+struct vmhip_batch {
+    vmhip_engine* engine = nullptr;
+    int32_t classify = 0;
+    std::vector<HostFrame> frames;
+    std::vector<int32_t> h_V, h_amb_count;
+    std::vector<int2> h_amb;
+    std::vector<uint64_t> h_force_valid, h_force_keep;
+    bool have_run = false;
+    uint32_t epoch = 0;
+    size_t cand_total = 0, row_total = 0, lookup_total = 0;
+
+    VmBatchDev dev{};
+    DevBuf d_frames, d_ranges, d_images, d_cand_px, d_cand_keep, d_tile_count, d_force_valid, d_force_keep, d_frame_V,
+      d_amb_count, d_amb_list, d_row_px, d_row_gidx, d_row_nb, d_act[2], d_lookup;
+    float* final_act = nullptr;
+
+    /* profiling */
+    bool profile = false;
+    std::vector<hipEvent_t> events;
+    std::vector<const char*> slot_names;
+    std::vector<int64_t> slot_units;
+    int n_slots = 0;
+
+    void release() {
+        DevBuf* all[] = {&d_frames, &d_ranges, &d_images, &d_cand_px, &d_cand_keep, &d_tile_count, &d_force_valid,
+                         &d_force_keep, &d_frame_V, &d_amb_count, &d_amb_list, &d_row_px, &d_row_gidx, &d_row_nb,
+                         &d_act[0], &d_act[1], &d_lookup};
+        for (DevBuf* b : all) b->release();
+        for (hipEvent_t e : events) (void) hipEventDestroy(e);
+        events.clear();
+    }
+};
+
+namespace {
+
+int batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int32_t classify) {
+    vmhip_engine* E = b->engine;
+    if (!frames || n_frames <= 0) return fail(VMHIP_ERR_ARGUMENT, "stage: no frames");
+    b->have_run = false;
+    b->classify = classify ? 1 : 0;
+    b->frames.assign(n_frames, HostFrame());
+
+    /* validate and place */
+    size_t cand_tiles = 0, row_tiles = 0, range_ints = 0, image_bytes = 0, lookup_entries = 0;
+    int32_t nb_stride = 1;
+    for (int f = 0; f < n_frames; ++f) {
+        const vmhip_frame& in = frames[f];
+        HostFrame& hf = b->frames[f];
+        if (!in.mesh) return fail(VMHIP_ERR_ARGUMENT, "stage: frame without a mesh");
+        if (in.lens.projection < VMHIP_RECTILINEAR || in.lens.projection > VMHIP_EQUIDISTANT)
+            return fail(VMHIP_ERR_LENS, "Cannot project: Unknown lens type");
+        if (in.lens.width <= 0 || in.lens.height <= 0) return fail(VMHIP_ERR_ARGUMENT, "stage: empty image dimensions");
+        if (in.n_ranges < 0 || (in.n_ranges > 0 && !in.ranges)) return fail(VMHIP_ERR_ARGUMENT, "stage: bad range table");
+        if (classify && !E->layers.empty() && in.mesh->nn != E->nn)
+            return fail(VMHIP_ERR_ARGUMENT, "stage: the mesh's neighbour count does not match the network");
+        int fmt = VMHIP_FMT_NONE, bpp = 0;
+        if (classify) {
+            if (!decode_fourcc(in.fourcc, &fmt, &bpp)) return fail(VMHIP_ERR_FORMAT, "Unsupported image format " + fourcc_text(in.fourcc));
+            if (!in.image) return fail(VMHIP_ERR_ARGUMENT, "stage: classification needs an image");
+        }
+        hf.mesh = in.mesh;
+        hf.first.resize(in.n_ranges);
+        hf.prefix.resize(size_t(in.n_ranges) + 1);
+        int64_t total = 0;
+        int32_t last_end = 0;
+        for (int r = 0; r < in.n_ranges; ++r) {
+            const int32_t a = in.ranges[2 * r], e = in.ranges[2 * r + 1];
+            if (a < last_end || e < a || e > in.mesh->n_nodes) return fail(VMHIP_ERR_ARGUMENT, "stage: ranges must be ascending, disjoint and inside the mesh");
+            hf.first[r] = a;
+            hf.prefix[r] = int32_t(total);
+            total += e - a;
+            last_end = e;
+        }
+        hf.prefix[in.n_ranges] = int32_t(total);
+        if (total > 0x7fff0000) return fail(VMHIP_ERR_ARGUMENT, "stage: too many candidates");
+
+        VmFrame& d = hf.dev;
+        std::memset(&d, 0, sizeof(d));
+        d.rays = in.mesh->d_rays;
+        d.nbr = in.mesh->d_nbr;
+        d.n_nodes = in.mesh->n_nodes;
+        d.nn = in.mesh->nn;
+        std::memcpy(d.Rco, in.Rco, sizeof(d.Rco));
+        d.focal = in.lens.focal_length;
+        d.centre_x = hf.centre[0] = in.lens.centre[0];
+        d.centre_y = hf.centre[1] = in.lens.centre[1];
+        vm_host_inverse_coefficients(in.lens.k, d.ik);
+        d.width = in.lens.width;
+        d.height = in.lens.height;
+        d.projection = in.lens.projection;
+        d.fmt = fmt;
+        d.n_ranges = in.n_ranges;
+        d.n_cand = int32_t(total);
+        d.cand_tile0 = int32_t(cand_tiles);
+        d.cand_tiles = int32_t((total + VMHIP_TILE - 1) / VMHIP_TILE);
+        d.cand_base = d.cand_tile0 * VMHIP_TILE;
+        d.row_tile0 = int32_t(row_tiles);
+        d.row_tiles = total > 0 ? int32_t((total + 1 + VMHIP_TILE - 1) / VMHIP_TILE) : 0;
+        d.row_base = d.row_tile0 * VMHIP_TILE;
+        cand_tiles += d.cand_tiles;
+        row_tiles += d.row_tiles;
+        if (cand_tiles > 0x7fffff || row_tiles > 0x7fffff) return fail(VMHIP_ERR_ARGUMENT, "stage: batch too large");
+        range_ints += size_t(in.n_ranges) * 2 + 1;
+        if (classify) image_bytes += align_up(size_t(in.lens.width) * in.lens.height * bpp, 256);
+        lookup_entries += size_t(in.mesh->n_nodes) + 1;
+        nb_stride = std::max(nb_stride, in.mesh->nn);
+    }
+    b->cand_total = cand_tiles * VMHIP_TILE;
+    b->row_total = row_tiles * VMHIP_TILE;
+    const size_t words = b->cand_total / 64;
+
+    /* device workspace */
+    HIP_TRY(b->d_frames.reserve(sizeof(VmFrame) * n_frames));
+    HIP_TRY(b->d_ranges.reserve(sizeof(int32_t) * std::max<size_t>(range_ints, 1)));
+    HIP_TRY(b->d_images.reserve(std::max<size_t>(image_bytes, 256)));
+    HIP_TRY(b->d_cand_px.reserve(sizeof(float2) * std::max<size_t>(b->cand_total, 1)));
+    HIP_TRY(b->d_cand_keep.reserve(8 * std::max<size_t>(words, 1)));
+    HIP_TRY(b->d_tile_count.reserve(4 * std::max<size_t>(cand_tiles, 1)));
+    HIP_TRY(b->d_force_valid.reserve(8 * std::max<size_t>(words, 1)));
+    HIP_TRY(b->d_force_keep.reserve(8 * std::max<size_t>(words, 1)));
+    HIP_TRY(b->d_frame_V.reserve(4 * size_t(n_frames)));
+    HIP_TRY(b->d_amb_count.reserve(4 * size_t(n_frames)));
+    HIP_TRY(b->d_amb_list.reserve(sizeof(int2) * size_t(n_frames) * VMHIP_AMB_CAP));
+    HIP_TRY(b->d_row_px.reserve(sizeof(float2) * std::max<size_t>(b->row_total, 1)));
+    HIP_TRY(b->d_row_gidx.reserve(4 * std::max<size_t>(b->row_total, 1)));
+    HIP_TRY(b->d_row_nb.reserve(4 * std::max<size_t>(b->row_total, 1) * nb_stride));
+    if (classify) {
+        for (int i = 0; i < 2; ++i) HIP_TRY(b->d_act[i].reserve(4 * std::max<size_t>(b->row_total, 1) * E->max_width));
+    }
+    HIP_TRY(b->d_lookup.reserve(sizeof(uint2) * lookup_entries));
+    if (b->d_lookup.grew) {
+        /* a fresh reverse-lookup table holds no valid stamp; epochs start above zero */
+        HIP_TRY(hipMemsetAsync(b->d_lookup.p, 0, b->d_lookup.cap, E->stream));
+    }
+    b->lookup_total = lookup_entries;
+
+    /* fill in device pointers and upload */
+    std::vector<int32_t> h_ranges(std::max<size_t>(range_ints, 1));
+    size_t range_off = 0, image_off = 0, lookup_off = 0;
+    std::vector<VmFrame> h_frames(n_frames);
+    for (int f = 0; f < n_frames; ++f) {
+        HostFrame& hf = b->frames[f];
+        VmFrame& d = hf.dev;
+        const int R = d.n_ranges;
+        d.range_first = b->d_ranges.as<int32_t>() + range_off;
+        std::copy(hf.first.begin(), hf.first.end(), h_ranges.begin() + range_off);
+        range_off += R;
+        d.range_prefix = b->d_ranges.as<int32_t>() + range_off;
+        std::copy(hf.prefix.begin(), hf.prefix.end(), h_ranges.begin() + range_off);
+        range_off += size_t(R) + 1;
+        if (classify) {
+            int fmt, bpp;
+            decode_fourcc(frames[f].fourcc, &fmt, &bpp);
+            const size_t bytes = size_t(d.width) * d.height * bpp;
+            d.image = b->d_images.as<uint8_t>() + image_off;
+            HIP_TRY(hipMemcpyAsync(b->d_images.as<uint8_t>() + image_off, frames[f].image, bytes, hipMemcpyHostToDevice, E->stream));
+            image_off += align_up(bytes, 256);
+        }
+        d.r_lookup = b->d_lookup.as<uint2>() + lookup_off;
+        lookup_off += size_t(d.n_nodes) + 1;
+        d.force_valid = b->d_force_valid.as<uint64_t>();
+        d.force_keep = b->d_force_keep.as<uint64_t>();
+        h_frames[f] = d;
+    }
+    HIP_TRY(hipMemcpyAsync(b->d_frames.p, h_frames.data(), sizeof(VmFrame) * n_frames, hipMemcpyHostToDevice, E->stream));
+    HIP_TRY(hipMemcpyAsync(b->d_ranges.p, h_ranges.data(), sizeof(int32_t) * h_ranges.size(), hipMemcpyHostToDevice, E->stream));
+    HIP_TRY(hipMemsetAsync(b->d_force_valid.p, 0, 8 * std::max<size_t>(words, 1), E->stream));
+    HIP_TRY(hipMemsetAsync(b->d_force_keep.p, 0, 8 * std::max<size_t>(words, 1), E->stream));
+    b->h_force_valid.assign(std::max<size_t>(words, 1), 0);
+    b->h_force_keep.assign(std::max<size_t>(words, 1), 0);
+    HIP_TRY(hipStreamSynchronize(E->stream)); /* the host vectors above go out of scope */
+
+    VmBatchDev& D = b->dev;
+    D.frames = b->d_frames.as<VmFrame>();
+    D.n_frames = n_frames;
+    D.n_cand_tiles = int32_t(cand_tiles);
+    D.n_row_tiles = int32_t(row_tiles);
+    D.cand_px = b->d_cand_px.as<float2>();
+    D.cand_keep = b->d_cand_keep.as<uint64_t>();
+    D.tile_count = b->d_tile_count.as<int32_t>();
+    D.frame_V = b->d_frame_V.as<int32_t>();
+    D.amb_count = b->d_amb_count.as<int32_t>();
+    D.amb_list = b->d_amb_list.as<int2>();
+    D.row_px = b->d_row_px.as<float2>();
+    D.row_gidx = b->d_row_gidx.as<int32_t>();
+    D.row_nb = b->d_row_nb.as<int32_t>();
+    D.nb_stride = nb_stride;
+    b->h_V.assign(n_frames, 0);
+    b->h_amb_count.assign(n_frames, 0);
+    return VMHIP_OK;
+}
+
+struct Profiler {
+    vmhip_batch* b;
+    hipStream_t s;
+    int slot = 0;
+    hipError_t begin() {
+        if (!b->profile) return hipSuccess;
+        while (int(b->events.size()) < 2 * (slot + 1)) {
+            hipEvent_t e;
+            hipError_t r = hipEventCreate(&e);
+            if (r != hipSuccess) return r;
+            b->events.push_back(e);
+        }
+        return hipEventRecord(b->events[2 * slot], s);
+    }
+    hipError_t end(const char* name, int64_t units) {
+        if (!b->profile) return hipSuccess;
+        hipError_t r = hipEventRecord(b->events[2 * slot + 1], s);
+        if (int(b->slot_names.size()) <= slot) {
+            b->slot_names.resize(slot + 1);
+            b->slot_units.resize(slot + 1);
+        }
+        b->slot_names[slot] = name;
+        b->slot_units[slot] = units;
+        ++slot;
+        return r;
+    }
+};
+
+int batch_enqueue(vmhip_batch* b) {
+    vmhip_engine* E = b->engine;
+    hipStream_t s = E->stream;
+    VmBatchDev& D = b->dev;
+    D.epoch = b->epoch;
+    Profiler P{b, s};
+    int64_t cands = 0, rows = 0;
+    for (const HostFrame& hf : b->frames) cands += hf.dev.n_cand;
+    rows = cands + int64_t(b->frames.size());
+
+    vm_launch_reset(D, s);
+    HIP_TRY(P.begin());
+    vm_launch_project(D, s);
+    HIP_TRY(P.end("project", cands));
+    HIP_TRY(P.begin());
+    vm_launch_compact(D, b->d_act[0].as<float>(), b->classify, s);
+    HIP_TRY(P.end(b->classify ? "compact_sample" : "compact", cands));
+    HIP_TRY(P.begin());
+    vm_launch_neighbourhood(D, s);
+    HIP_TRY(P.end("neighbourhood", rows));
+
+    int cur = 0;
+    if (b->classify) {
+        for (const HostLayer& L : E->layers) {
+            VmLayerDev ld{L.c_in, L.c_out, L.slots, L.activation, L.d_w, L.d_b};
+            const char* name = "conv";
+            HIP_TRY(P.begin());
+            const int rc = vm_launch_conv(D, ld, b->d_act[cur].as<float>(), b->d_act[cur ^ 1].as<float>(), s, &name);
+            if (rc != 0) return fail(rc, "unsupported layer shape");
+            HIP_TRY(P.end(name, rows));
+            cur ^= 1;
+        }
+        b->final_act = b->d_act[cur].as<float>();
+    }
+    b->n_slots = P.slot;
+    HIP_TRY(hipGetLastError());
+    return VMHIP_OK;
+}
+
+/* Re-decide, with the host's arithmetic, every candidate the device flagged as lying within the
+ * ambiguity band of a screen edge. Returns the number of decisions that differ (those are written
+ * into the force masks), or a negative status. */
+int batch_verify(vmhip_batch* b) {
+    vmhip_engine* E = b->engine;
+    const int n = int(b->frames.size());
+    HIP_TRY(hipMemcpyAsync(b->h_V.data(), b->d_frame_V.p, 4 * size_t(n), hipMemcpyDeviceToHost, E->stream));
+    HIP_TRY(hipMemcpyAsync(b->h_amb_count.data(), b->d_amb_count.p, 4 * size_t(n), hipMemcpyDeviceToHost, E->stream));
+    HIP_TRY(hipStreamSynchronize(E->stream));
+    int changed = 0;
+    for (int f = 0; f < n; ++f) {
+        HostFrame& hf = b->frames[f];
+        const VmFrame& d = hf.dev;
+        if (d.n_cand == 0) {
+            b->h_V[f] = 0;
+            continue;
+        }
+        const int count = b->h_amb_count[f];
+        if (count == 0) continue;
+        const float* rays = hf.mesh->h_rays.data();
+        auto redecide = [&](int p, int gpu_keep, bool force_all) {
+            /* candidate slot -> global index */
+            const int r = int(std::upper_bound(hf.prefix.begin(), hf.prefix.end() - 1, p) - hf.prefix.begin()) - 1;
+            const int g = hf.first[r] + (p - hf.prefix[r]);
+            const int keep = vm_host_on_screen(d.Rco, rays + size_t(g) * 3, d.projection, d.focal, hf.centre, d.ik, d.width, d.height, nullptr);
+            if (keep != gpu_keep || force_all) {
+                const size_t word = (size_t(d.cand_base) + p) >> 6;
+                const uint64_t bit = 1ull << (p & 63);
+                b->h_force_valid[word] |= bit;
+                if (keep) b->h_force_keep[word] |= bit;
+                else b->h_force_keep[word] &= ~bit;
+                if (keep != gpu_keep) ++changed;
+            }
+        };
+        if (count > VMHIP_AMB_CAP) {
+            /* the list overflowed: decide the whole frame on the host (slow, never seen with real lenses) */
+            for (int p = 0; p < d.n_cand; ++p) redecide(p, -1, true);
+        }
+        else {
+            b->h_amb.resize(count);
+            HIP_TRY(hipMemcpy(b->h_amb.data(), b->d_amb_list.as<int2>() + size_t(f) * VMHIP_AMB_CAP, sizeof(int2) * count, hipMemcpyDeviceToHost));
+            for (int i = 0; i < count; ++i) redecide(b->h_amb[i].x, b->h_amb[i].y, false);
+        }
+    }
+    if (changed > 0) {
+        const size_t words = std::max<size_t>(b->cand_total / 64, 1);
+        HIP_TRY(hipMemcpyAsync(b->d_force_valid.p, b->h_force_valid.data(), 8 * words, hipMemcpyHostToDevice, E->stream));
+        HIP_TRY(hipMemcpyAsync(b->d_force_keep.p, b->h_force_keep.data(), 8 * words, hipMemcpyHostToDevice, E->stream));
+        HIP_TRY(hipStreamSynchronize(E->stream));
+    }
+    return changed;
+}
+
+int batch_run(vmhip_batch* b) {
+    if (b->frames.empty()) return fail(VMHIP_ERR_ARGUMENT, "run: nothing staged");
+    for (int attempt = 0; attempt < 4; ++attempt) {
+        ++b->epoch;
+        if (b->epoch == 0) { /* wrapped: old stamps could look current again */
+            HIP_TRY(hipMemsetAsync(b->d_lookup.p, 0, b->d_lookup.cap, b->engine->stream));
+            b->epoch = 1;
+        }
+        int rc = batch_enqueue(b);
+        if (rc != VMHIP_OK) return rc;
+        rc = batch_verify(b);
+        if (rc < 0) return rc;
+        if (rc == 0) {
+            b->have_run = true;
+            return VMHIP_OK;
+        }
+    }
+    return fail(VMHIP_ERR_HIP, "run: edge decisions did not settle");
+}
+
+int batch_fetch(vmhip_batch* b, vmhip_result* results) {
+    if (!b->have_run) return fail(VMHIP_ERR_ARGUMENT, "fetch: no completed run");
+    if (!results) return fail(VMHIP_ERR_ARGUMENT, "fetch: null results");
+    vmhip_engine* E = b->engine;
+    hipStream_t s = E->stream;
+    const int n = int(b->frames.size());
+    const int stride = b->dev.nb_stride;
+    const int C = E->n_classes;
+    for (int f = 0; f < n; ++f) {
+        const VmFrame& d = b->frames[f].dev;
+        vmhip_result& R = results[f];
+        const int V = b->h_V[f];
+        R.n_visible = V;
+        if (V == 0) continue;
+        if (R.capacity < V) return fail(VMHIP_ERR_CAPACITY, "fetch: result capacity is smaller than the visible node count");
+        const size_t base = size_t(d.row_base);
+        if (R.pixel_coordinates)
+            HIP_TRY(hipMemcpyAsync(R.pixel_coordinates, b->dev.row_px + base, sizeof(float2) * V, hipMemcpyDeviceToHost, s));
+        if (R.global_indices)
+            HIP_TRY(hipMemcpyAsync(R.global_indices, b->dev.row_gidx + base, 4 * size_t(V), hipMemcpyDeviceToHost, s));
+        if (R.neighbourhood) {
+            if (stride == d.nn)
+                HIP_TRY(hipMemcpyAsync(R.neighbourhood, b->dev.row_nb + base * stride, 4 * size_t(V + 1) * d.nn, hipMemcpyDeviceToHost, s));
+            else
+                HIP_TRY(hipMemcpy2DAsync(R.neighbourhood, 4 * size_t(d.nn), b->dev.row_nb + base * stride, 4 * size_t(stride),
+                                         4 * size_t(d.nn), size_t(V + 1), hipMemcpyDeviceToHost, s));
+        }
+        if (R.classifications && b->classify)
+            HIP_TRY(hipMemcpyAsync(R.classifications, b->final_act + base * C, 4 * size_t(V + 1) * C, hipMemcpyDeviceToHost, s));
+    }
+    HIP_TRY(hipStreamSynchronize(s));
+    return VMHIP_OK;
+}
+
+int ensure_scratch(vmhip_engine* E) {
+    if (!E->scratch) {
+        E->scratch = new vmhip_batch();
+        E->scratch->engine = E;
+    }
+    return VMHIP_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* vmhip_last_error(void) { return g_error.c_str(); }
+
+int vmhip_engine_create(const vmhip_network* net, int32_t n_neighbours, int32_t precision, vmhip_engine** out) {
+    if (!out) return fail(VMHIP_ERR_ARGUMENT, "engine_create: null output");
+    *out = nullptr;
+    if (n_neighbours < 0 || n_neighbours > 16) return fail(VMHIP_ERR_ARGUMENT, "engine_create: unsupported neighbour count");
+    if (precision != VMHIP_FP32 && precision != VMHIP_BF16) return fail(VMHIP_ERR_ARGUMENT, "engine_create: unknown precision");
+    int n_dev = 0;
+    HIP_TRY(hipGetDeviceCount(&n_dev));
+    if (n_dev <= 0) return fail(VMHIP_ERR_HIP, "engine_create: no HIP device");
+
+    vmhip_engine* E = new vmhip_engine();
+    E->nn = n_neighbours;
+    E->precision = precision;
+    auto bail = [&](int code, const std::string& msg) {
+        vmhip_engine_destroy(E);
+        return fail(code, msg);
+    };
+    int width = 4;
+    int li = 0;
+    for (int g = 0; net && g < net->n_groups; ++g) {
+        if (net->group_sizes[g] <= 0) return bail(VMHIP_ERR_ARGUMENT, "engine_create: empty convolutional group");
+        for (int l = 0; l < net->group_sizes[g]; ++l, ++li) {
+            const vmhip_layer& L = net->layers[li];
+            const int slots = l == 0 ? n_neighbours + 1 : 1;
+            if (L.n_in != slots * width || L.n_out <= 0 || !L.weights || !L.biases)
+                return bail(VMHIP_ERR_ARGUMENT, "engine_create: layer " + std::to_string(li) + " expects " + std::to_string(slots * width)
+                                                  + " inputs, has " + std::to_string(L.n_in));
+            if (L.activation < VMHIP_SELU || L.activation > VMHIP_TANH) return bail(VMHIP_ERR_ARGUMENT, "engine_create: unknown activation");
+            HostLayer H{width, L.n_out, slots, L.activation, nullptr, nullptr};
+            if (hipMalloc(&H.d_w, 4 * size_t(L.n_in) * L.n_out) != hipSuccess || hipMalloc(&H.d_b, 4 * size_t(L.n_out)) != hipSuccess)
+                return bail(VMHIP_ERR_HIP, "engine_create: out of device memory");
+            E->layers.push_back(H);
+            if (hipMemcpy(H.d_w, L.weights, 4 * size_t(L.n_in) * L.n_out, hipMemcpyHostToDevice) != hipSuccess
+                || hipMemcpy(H.d_b, L.biases, 4 * size_t(L.n_out), hipMemcpyHostToDevice) != hipSuccess)
+                return bail(VMHIP_ERR_HIP, "engine_create: weight upload failed");
+            width = L.n_out;
+            E->max_width = std::max(E->max_width, width);
+        }
+    }
+    E->n_classes = width;
+    if (hipStreamCreateWithFlags(&E->stream, hipStreamNonBlocking) != hipSuccess) return bail(VMHIP_ERR_HIP, "engine_create: stream creation failed");
+    *out = E;
+    return VMHIP_OK;
+}
+
+void vmhip_engine_destroy(vmhip_engine* E) {
+    if (!E) return;
+    if (E->scratch) vmhip_batch_destroy(E->scratch);
+    for (HostLayer& L : E->layers) {
+        if (L.d_w) (void) hipFree(L.d_w);
+        if (L.d_b) (void) hipFree(L.d_b);
+    }
+    if (E->stream) (void) hipStreamDestroy(E->stream);
+    delete E;
+}
+
+int32_t vmhip_engine_n_classes(const vmhip_engine* E) { return E ? E->n_classes : 0; }
+
+int vmhip_mesh_upload(const float* rays, const int32_t* neighbours, int32_t n_nodes, int32_t n_neighbours, vmhip_mesh** out) {
+    if (!out) return fail(VMHIP_ERR_ARGUMENT, "mesh_upload: null output");
+    *out = nullptr;
+    if (!rays || !neighbours || n_nodes <= 0 || n_neighbours <= 0 || n_neighbours > 16)
+        return fail(VMHIP_ERR_ARGUMENT, "mesh_upload: bad arguments");
+    for (size_t i = 0; i < size_t(n_nodes) * n_neighbours; ++i)
+        if (neighbours[i] < 0 || neighbours[i] > n_nodes) return fail(VMHIP_ERR_ARGUMENT, "mesh_upload: neighbour index outside [0, n_nodes]");
+    vmhip_mesh* M = new vmhip_mesh();
+    M->n_nodes = n_nodes;
+    M->nn = n_neighbours;
+    M->h_rays.assign(rays, rays + size_t(n_nodes) * 3);
+    const size_t rb = sizeof(float) * 3 * size_t(n_nodes), nb = sizeof(int32_t) * size_t(n_nodes) * n_neighbours;
+    if (hipMalloc(&M->d_rays, rb) != hipSuccess || hipMalloc(&M->d_nbr, nb) != hipSuccess
+        || hipMemcpy(M->d_rays, rays, rb, hipMemcpyHostToDevice) != hipSuccess
+        || hipMemcpy(M->d_nbr, neighbours, nb, hipMemcpyHostToDevice) != hipSuccess) {
+        vmhip_mesh_release(M);
+        return fail(VMHIP_ERR_HIP, "mesh_upload: device allocation or copy failed");
+    }
+    *out = M;
+    return VMHIP_OK;
+}
+
+void vmhip_mesh_release(vmhip_mesh* M) {
+    if (!M) return;
+    if (M->d_rays) (void) hipFree(M->d_rays);
+    if (M->d_nbr) (void) hipFree(M->d_nbr);
+    delete M;
+}
+
+int vmhip_batch_create(vmhip_engine* E, vmhip_batch** out) {
+    if (!E || !out) return fail(VMHIP_ERR_ARGUMENT, "batch_create: null argument");
+    *out = new vmhip_batch();
+    (*out)->engine = E;
+    return VMHIP_OK;
+}
+void vmhip_batch_destroy(vmhip_batch* b) {
+    if (!b) return;
+    if (b->engine && b->engine->stream) (void) hipStreamSynchronize(b->engine->stream);
+    b->release();
+    delete b;
+}
+int vmhip_batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int32_t classify) {
+    if (!b) return fail(VMHIP_ERR_ARGUMENT, "batch_stage: null batch");
+    const int rc = batch_stage(b, frames, n_frames, classify);
+    if (rc != VMHIP_OK) b->frames.clear();
+    return rc;
+}
+int vmhip_batch_run(vmhip_batch* b) {
+    if (!b) return fail(VMHIP_ERR_ARGUMENT, "batch_run: null batch");
+    return batch_run(b);
+}
+int vmhip_batch_counts(const vmhip_batch* b, int32_t* n_visible) {
+    if (!b || !n_visible || !b->have_run) return fail(VMHIP_ERR_ARGUMENT, "batch_counts: no completed run");
+    std::copy(b->h_V.begin(), b->h_V.end(), n_visible);
+    return VMHIP_OK;
+}
+int vmhip_batch_fetch(vmhip_batch* b, vmhip_result* results) {
+    if (!b) return fail(VMHIP_ERR_ARGUMENT, "batch_fetch: null batch");
+    return batch_fetch(b, results);
+}
+int vmhip_batch_profile(vmhip_batch* b, int32_t enable) {
+    if (!b) return fail(VMHIP_ERR_ARGUMENT, "batch_profile: null batch");
+    b->profile = enable != 0;
+    return VMHIP_OK;
+}
+int vmhip_batch_profile_read(vmhip_batch* b, int32_t max_slots, int32_t* n_slots, const char** names, float* milliseconds,
+                             int64_t* units) {
+    if (!b || !n_slots) return fail(VMHIP_ERR_ARGUMENT, "batch_profile_read: null argument");
+    if (!b->profile || !b->have_run) return fail(VMHIP_ERR_ARGUMENT, "batch_profile_read: profiling was not enabled for the last run");
+    const int n = std::min<int>(b->n_slots, max_slots);
+    for (int i = 0; i < n; ++i) {
+        float ms = 0.0f;
+        HIP_TRY(hipEventElapsedTime(&ms, b->events[2 * i], b->events[2 * i + 1]));
+        if (names) names[i] = b->slot_names[i];
+        if (milliseconds) milliseconds[i] = ms;
+        if (units) units[i] = b->slot_units[i];
+    }
+    *n_slots = n;
+    return VMHIP_OK;
+}
+
+int vmhip_selftest_libm(int32_t which, const float* x, float* y, int32_t n) {
+    if (!x || !y || n <= 0 || which < 0 || which > 3) return fail(VMHIP_ERR_ARGUMENT, "selftest_libm: bad arguments");
+    float *dx = nullptr, *dy = nullptr;
+    HIP_TRY(hipMalloc(&dx, 4 * size_t(n)));
+    if (hipMalloc(&dy, 4 * size_t(n)) != hipSuccess) {
+        (void) hipFree(dx);
+        return fail(VMHIP_ERR_HIP, "selftest_libm: out of device memory");
+    }
+    hipError_t e = hipMemcpy(dx, x, 4 * size_t(n), hipMemcpyHostToDevice);
+    if (e == hipSuccess) {
+        vm_launch_libm(which, dx, dy, n, nullptr);
+        e = hipMemcpy(y, dy, 4 * size_t(n), hipMemcpyDeviceToHost);
+    }
+    (void) hipFree(dx);
+    (void) hipFree(dy);
+    if (e != hipSuccess) return fail(VMHIP_ERR_HIP, std::string("selftest_libm: ") + hipGetErrorString(e));
+    return VMHIP_OK;
+}
+
+int vmhip_classify_batch(vmhip_engine* E, const vmhip_frame* frames, int32_t n_frames, vmhip_result* results) {
+    if (!E) return fail(VMHIP_ERR_ARGUMENT, "classify_batch: null engine");
+    ensure_scratch(E);
+    int rc = vmhip_batch_stage(E->scratch, frames, n_frames, 1);
+    if (rc == VMHIP_OK) rc = batch_run(E->scratch);
+    if (rc == VMHIP_OK) rc = batch_fetch(E->scratch, results);
+    return rc;
+}
+int vmhip_classify(vmhip_engine* E, const vmhip_frame* frame, vmhip_result* result) {
+    return vmhip_classify_batch(E, frame, 1, result);
+}
+int vmhip_project(vmhip_engine* E, const vmhip_frame* frame, vmhip_result* result) {
+    if (!E) return fail(VMHIP_ERR_ARGUMENT, "project: null engine");
+    ensure_scratch(E);
+    int rc = vmhip_batch_stage(E->scratch, frame, 1, 0);
+    if (rc == VMHIP_OK) rc = batch_run(E->scratch);
+    if (rc == VMHIP_OK) rc = batch_fetch(E->scratch, result);
+    return rc;
+}
+}

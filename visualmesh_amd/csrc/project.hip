@@ -1,0 +1,369 @@
+/*
+ * project.hip - candidate projection, on-screen filter, order-preserving compaction, image sampling and
+ * the local neighbourhood table, for gfx950 (wave64).
+ *
+ * This file is compiled with -ffp-contract=off: the lens projection and the bilinear weights must be
+ * single IEEE binary32 operations in the reference's order, and acosf/sinf/tanf come from libm_exact.h,
+ * which returns the host C library's bits. Pixel coordinates and sampled inputs are then bit-identical
+ * to the CPU engine's. The ambiguity band below stays as a guard for hosts whose C library differs: a
+ * node within 1/64 px of a screen edge is re-decided on the host, so the visible set cannot diverge.
+ *
+ * Kernels (one launch each per batch, grids over all frames of the batch):
+ *   vm_reset_kernel          clears the per-frame ambiguity counters
+ *   vm_project_kernel        candidate space: global index from the range table, pixel coordinate, keep
+ *                            decision, per-wave keep mask (ballot), per-tile kept count, ambiguity list
+ *   vm_compact_kernel        candidate space: exclusive prefix over tile counts + wave popcount prefix ->
+ *                            ascending local row; writes pixel, global index, reverse lookup stamp and the
+ *                            sampled 4-channel input row; the frame's last tile writes V and the null row
+ *   vm_neighbourhood_kernel  row space: neighbour table through the stamped reverse lookup
+ */
+#include "vmhip_internal.h"
+
+#pragma clang fp contract(off)
+
+#include "libm_exact.h"
+
+#define AMB_EPS 0.015625f /* 1/64 px: far above any device/host libm difference, far below node spacing */
+
+namespace {
+
+__device__ __forceinline__ int find_frame_by_cand_tile(const VmFrame* frames, int n, int tile) {
+    int lo = 0, hi = n - 1;
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (frames[mid].cand_tile0 <= tile) lo = mid;
+        else hi = mid - 1;
+    }
+    return lo;
+}
+__device__ __forceinline__ int find_frame_by_row_tile(const VmFrame* frames, int n, int tile) {
+    int lo = 0, hi = n - 1;
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (frames[mid].row_tile0 <= tile) lo = mid;
+        else hi = mid - 1;
+    }
+    return lo;
+}
+
+/* candidate slot -> global node index: ranges are ascending, prefix[r] <= p < prefix[r+1] */
+__device__ __forceinline__ int cand_to_global(const VmFrame& F, int p) {
+    int lo = 0, hi = F.n_ranges - 1;
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (F.range_prefix[mid] <= p) lo = mid;
+        else hi = mid - 1;
+    }
+    return F.range_first[lo] + (p - F.range_prefix[lo]);
+}
+
+/* Lens projection, reference utility/projection.hpp:162-187 with utility/math.hpp's dot order. */
+__device__ __forceinline__ float2 project_ray(const VmFrame& F, float rx, float ry, float rz) {
+    const float c0 = F.Rco[2] * rz + (F.Rco[1] * ry + F.Rco[0] * rx);
+    const float c1 = F.Rco[5] * rz + (F.Rco[4] * ry + F.Rco[3] * rx);
+    const float c2 = F.Rco[8] * rz + (F.Rco[7] * ry + F.Rco[6] * rx);
+
+    /* vm_acosf / vm_sinf / vm_tanf return the host C library's bits (libm_exact.h) */
+    const float theta = vm_acosf(c0);
+    const float rsin_theta = 1.0f / vm_sqrtf(1.0f - c0 * c0);
+    float r_u;
+    if (F.projection == VMHIP_RECTILINEAR) {
+        r_u = F.focal * vm_tanf(fminf(fmaxf(theta, 0.0f), 1.57079637050628662109375f));
+    }
+    else if (F.projection == VMHIP_EQUISOLID) {
+        r_u = 2.0f * F.focal * vm_sinf(theta * 0.5f);
+    }
+    else {
+        r_u = F.focal * theta;
+    }
+    /* distortion polynomial: a double sum of float terms (the reference's literal 1.0) */
+    const float r2 = r_u * r_u;
+    const double s = 1.0 + (double) (F.ik[0] * r2) + (double) (F.ik[1] * (r2 * r2)) + (double) (F.ik[2] * (r2 * r2) * r2)
+                     + (double) (F.ik[3] * (r2 * r2) * (r2 * r2));
+    const float r_d = (float) ((double) r_u * s);
+
+    float sx = 0.0f, sy = 0.0f;
+    if (!(c0 >= 1.0f)) {
+        sx = r_d * c1 * rsin_theta;
+        sy = r_d * c2 * rsin_theta;
+    }
+    float2 px;
+    px.x = ((float) F.width * 0.5f - sx) - F.centre_x;
+    px.y = ((float) F.height * 0.5f - sy) - F.centre_y;
+    return px;
+}
+
+__global__ void vm_libm_kernel(int which, const float* x, float* y, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float v = x[i];
+    y[i] = which == 0 ? vm_acosf(v) : which == 1 ? vm_sinf(v) : which == 2 ? vm_tanf(v) : vm_sqrtf(v);
+}
+
+__global__ void vm_reset_kernel(VmBatchDev B) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < B.n_frames) B.amb_count[i] = 0;
+}
+
+__global__ __launch_bounds__(VMHIP_TILE) void vm_project_kernel(VmBatchDev B) {
+    __shared__ int wave_count[VMHIP_TILE / 64];
+    const int tile = blockIdx.x;
+    const int f = find_frame_by_cand_tile(B.frames, B.n_frames, tile);
+    const VmFrame& F = B.frames[f];
+    const int p = (tile - F.cand_tile0) * VMHIP_TILE + threadIdx.x;
+    const bool valid = p < F.n_cand;
+
+    bool keep = false;
+    float2 px = make_float2(0.0f, 0.0f);
+    if (valid) {
+        const int g = cand_to_global(F, p);
+        const float* r = F.rays + (size_t) g * 3;
+        px = project_ray(F, r[0], r[1], r[2]);
+        const float W = (float) F.width, H = (float) F.height;
+        /* strict test of the CPU engine, engine/cpu/engine.hpp:116-117 */
+        keep = 0.0f <= px.x && px.x + 1.0f < W && 0.0f <= px.y && px.y + 1.0f < H;
+
+        /* distance to the nearest decision boundary; NaN counts as ambiguous */
+        const float d = fminf(fminf(fabsf(px.x), fabsf(px.x + 1.0f - W)), fminf(fabsf(px.y), fabsf(px.y + 1.0f - H)));
+        const bool ambiguous = !(d >= AMB_EPS);
+
+        const size_t word = (size_t) (F.cand_base + p) >> 6;
+        const uint64_t bit = 1ull << (threadIdx.x & 63);
+        const bool forced = (F.force_valid[word] & bit) != 0;
+        if (forced) { keep = (F.force_keep[word] & bit) != 0; }
+        else if (ambiguous) {
+            const int slot = atomicAdd(&B.amb_count[f], 1);
+            if (slot < VMHIP_AMB_CAP) B.amb_list[(size_t) f * VMHIP_AMB_CAP + slot] = make_int2(p, keep ? 1 : 0);
+        }
+        B.cand_px[(size_t) F.cand_base + p] = px;
+    }
+
+    const uint64_t mask = __ballot(keep);
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) {
+        B.cand_keep[((size_t) F.cand_base >> 6) + (size_t) (tile - F.cand_tile0) * (VMHIP_TILE / 64) + wave] = mask;
+        wave_count[wave] = __popcll(mask);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int total = 0;
+        for (int w = 0; w < VMHIP_TILE / 64; ++w) total += wave_count[w];
+        B.tile_count[tile] = total;
+    }
+}
+
+/* ---- image sampling: reference engine/cpu/pixel.hpp and bayer.hpp ---- */
+#define INV255 0.0039215688593685626983642578125f /* float(1.0 / 255.0) */
+
+__device__ __forceinline__ float4 texel_packed(const VmFrame& F, int x, int y) {
+    const size_t idx = (size_t) y * F.width + x;
+    float4 o;
+    switch (F.fmt) {
+        case VMHIP_FMT_RGBA: {
+            const uint32_t v = reinterpret_cast<const uint32_t*>(F.image)[idx];
+            o = make_float4((float) (v & 0xff) * INV255, (float) ((v >> 8) & 0xff) * INV255,
+                            (float) ((v >> 16) & 0xff) * INV255, (float) (v >> 24) * INV255);
+        } break;
+        case VMHIP_FMT_BGRA: {
+            const uint32_t v = reinterpret_cast<const uint32_t*>(F.image)[idx];
+            o = make_float4((float) ((v >> 16) & 0xff) * INV255, (float) ((v >> 8) & 0xff) * INV255,
+                            (float) (v & 0xff) * INV255, (float) (v >> 24) * INV255);
+        } break;
+        case VMHIP_FMT_RGB3: {
+            const uint8_t* b = F.image + idx * 3;
+            o = make_float4((float) b[0] * INV255, (float) b[1] * INV255, (float) b[2] * INV255, 1.0f);
+        } break;
+        case VMHIP_FMT_BGR3: {
+            const uint8_t* b = F.image + idx * 3;
+            o = make_float4((float) b[2] * INV255, (float) b[1] * INV255, (float) b[0] * INV255, 1.0f);
+        } break;
+        default: { /* GRAY */
+            const float v = (float) F.image[idx] * INV255;
+            o = make_float4(v, v, v, 1.0f);
+        } break;
+    }
+    return o;
+}
+
+/* Malvar-He-Cutler demosaic of the 5x5 patch whose top-left corner is (ox, oy) inside the 6x6 union u.
+ * Integer arithmetic with truncating division by 64 and no clamp (bayer.hpp:95-108). type: 0 R, 1 GR, 2 GB, 3 B */
+template <int OX, int OY>
+__device__ __forceinline__ float4 demosaic_at(const int (&u)[6][6], int type) {
+#define P(r, c) u[OY + (r)][OX + (c)]
+    const int centre = P(2, 2);
+    int red, green, blue;
+    if (type == 0 || type == 3) {
+        const int arms = P(0, 2) + P(2, 0) + P(2, 4) + P(4, 2);
+        const int cross = (-8 * arms + 16 * (P(1, 2) + P(2, 1) + P(2, 3) + P(3, 2)) + 32 * centre) / 64;
+        const int checker = (-12 * arms + 16 * (P(1, 1) + P(1, 3) + P(3, 1) + P(3, 3)) + 48 * centre) / 64;
+        green = cross;
+        red = type == 0 ? centre : checker;
+        blue = type == 0 ? checker : centre;
+    }
+    else {
+        const int diag = P(1, 1) + P(1, 3) + P(3, 1) + P(3, 3);
+        const int horiz = (4 * (P(0, 2) + P(4, 2)) - 8 * diag - 8 * (P(2, 0) + P(2, 4)) + 32 * (P(2, 1) + P(2, 3)) + 40 * centre) / 64;
+        const int vert = (-8 * (P(0, 2) + P(4, 2)) - 8 * diag + 32 * (P(1, 2) + P(3, 2)) + 4 * (P(2, 0) + P(2, 4)) + 40 * centre) / 64;
+        green = centre;
+        red = type == 1 ? horiz : vert;
+        blue = type == 1 ? vert : horiz;
+    }
+#undef P
+    return make_float4((float) red * INV255, (float) green * INV255, (float) blue * INV255, (float) 255 * INV255);
+}
+
+__device__ __forceinline__ int bayer_type(int fmt, int x, int y) {
+    /* pattern letters in (row, col) order: index = row*2 + col; 0 R, 1 GR, 2 GB, 3 B (bayer.hpp:140-155) */
+    const int i = ((y & 1) << 1) | (x & 1);
+    switch (fmt) {
+        case VMHIP_FMT_GRBG: return (0x2301 >> (i * 4)) & 0xf; /* GR R B GB */
+        case VMHIP_FMT_RGGB: return (0x3210 >> (i * 4)) & 0xf; /* R GR GB B */
+        case VMHIP_FMT_GBRG: return (0x1032 >> (i * 4)) & 0xf; /* GB B R GR */
+        default: return (0x0123 >> (i * 4)) & 0xf;             /* BGGR: B GB GR R */
+    }
+}
+
+/* bilinear interpolation of the four surrounding texels, reference engine/cpu/pixel.hpp:115-144. The
+ * on-screen filter guarantees 0 <= x and x + 1 < width, so x2 = x1 + 1 and the reference's division by
+ * (x2 - x1) is a division by one. */
+__device__ __forceinline__ float4 sample_image(const VmFrame& F, float2 px) {
+    const int x1 = max((int) floorf(px.x), 0);
+    const int y1 = max((int) floorf(px.y), 0);
+    const int x2 = min(x1 + 1, F.width - 1);
+    const int y2 = min(y1 + 1, F.height - 1);
+    float4 q1, q2, q3, q4;
+    if (F.fmt >= VMHIP_FMT_GRBG && F.fmt <= VMHIP_FMT_BGGR) {
+        int u[6][6];
+#pragma unroll
+        for (int r = 0; r < 6; ++r) {
+            const int yc = min(max(y1 - 2 + r, 0), F.height - 1);
+#pragma unroll
+            for (int c = 0; c < 6; ++c) {
+                const int xc = min(max(x1 - 2 + c, 0), F.width - 1);
+                u[r][c] = F.image[(size_t) yc * F.width + xc];
+            }
+        }
+        /* x2 == x1 or y2 == y1 only on the last column/row, which the filter excludes; handle anyway */
+        q1 = demosaic_at<0, 0>(u, bayer_type(F.fmt, x1, y1));
+        q2 = x2 > x1 ? demosaic_at<1, 0>(u, bayer_type(F.fmt, x2, y1)) : q1;
+        q3 = y2 > y1 ? demosaic_at<0, 1>(u, bayer_type(F.fmt, x1, y2)) : q1;
+        q4 = (x2 > x1 && y2 > y1) ? demosaic_at<1, 1>(u, bayer_type(F.fmt, x2, y2)) : (x2 > x1 ? q2 : q3);
+    }
+    else {
+        q1 = texel_packed(F, x1, y1);
+        q2 = texel_packed(F, x2, y1);
+        q3 = texel_packed(F, x1, y2);
+        q4 = texel_packed(F, x2, y2);
+    }
+    const float wxa = ((float) x2 - px.x) / (float) (x2 - x1), wxb = (px.x - (float) x1) / (float) (x2 - x1);
+    const float wya = ((float) y2 - px.y) / (float) (y2 - y1), wyb = (px.y - (float) y1) / (float) (y2 - y1);
+    float4 o;
+    {
+        const float r1 = q1.x * wxa + q2.x * wxb, r2 = q3.x * wxa + q4.x * wxb;
+        o.x = r1 * wya + r2 * wyb;
+    }
+    {
+        const float r1 = q1.y * wxa + q2.y * wxb, r2 = q3.y * wxa + q4.y * wxb;
+        o.y = r1 * wya + r2 * wyb;
+    }
+    {
+        const float r1 = q1.z * wxa + q2.z * wxb, r2 = q3.z * wxa + q4.z * wxb;
+        o.z = r1 * wya + r2 * wyb;
+    }
+    {
+        const float r1 = q1.w * wxa + q2.w * wxb, r2 = q3.w * wxa + q4.w * wxb;
+        o.w = r1 * wya + r2 * wyb;
+    }
+    return o;
+}
+
+__global__ __launch_bounds__(VMHIP_TILE) void vm_compact_kernel(VmBatchDev B, float4* feat, int classify) {
+    __shared__ int partial[VMHIP_TILE / 64];
+    __shared__ int wave_count[VMHIP_TILE / 64];
+    const int tile = blockIdx.x;
+    const int f = find_frame_by_cand_tile(B.frames, B.n_frames, tile);
+    const VmFrame& F = B.frames[f];
+    const int t_local = tile - F.cand_tile0;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+
+    /* kept candidates in this frame's earlier tiles */
+    int sum = 0;
+    for (int i = threadIdx.x; i < t_local; i += VMHIP_TILE) sum += B.tile_count[F.cand_tile0 + i];
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
+    const uint64_t mask = B.cand_keep[((size_t) F.cand_base >> 6) + (size_t) t_local * (VMHIP_TILE / 64) + wave];
+    if (lane == 0) {
+        partial[wave] = sum;
+        wave_count[wave] = __popcll(mask);
+    }
+    __syncthreads();
+    int base = 0, before = 0, total = 0;
+#pragma unroll
+    for (int w = 0; w < VMHIP_TILE / 64; ++w) {
+        base += partial[w];
+        if (w < wave) before += wave_count[w];
+        total += wave_count[w];
+    }
+
+    const int p = t_local * VMHIP_TILE + threadIdx.x;
+    if ((mask >> lane) & 1ull) {
+        const int local = base + before + __popcll(mask & ((1ull << lane) - 1ull));
+        const size_t row = (size_t) F.row_base + local;
+        const int g = cand_to_global(F, p);
+        const float2 px = B.cand_px[(size_t) F.cand_base + p];
+        B.row_px[row] = px;
+        B.row_gidx[row] = g;
+        F.r_lookup[g] = make_uint2(B.epoch, (uint32_t) local);
+        if (classify) feat[row] = sample_image(F, px);
+    }
+    if (t_local == F.cand_tiles - 1 && threadIdx.x == 0) {
+        const int V = base + total;
+        B.frame_V[f] = V;
+        /* the off-screen row, engine/cpu/engine.hpp:205-206 */
+        if (classify) feat[(size_t) F.row_base + V] = make_float4(-1.0f, -1.0f, -1.0f, -1.0f);
+    }
+}
+
+/* reference engine/cpu/engine.hpp:127-143: one thread per (row, neighbour) */
+__global__ __launch_bounds__(VMHIP_TILE) void vm_neighbourhood_kernel(VmBatchDev B) {
+    const int tile = blockIdx.x;
+    const int f = find_frame_by_row_tile(B.frames, B.n_frames, tile);
+    const VmFrame& F = B.frames[f];
+    const int V = B.frame_V[f];
+    const int nn = F.nn;
+    const int row0 = (tile - F.row_tile0) * VMHIP_TILE;
+    if (row0 > V) return;
+    const int n_items = min(VMHIP_TILE, V + 1 - row0) * nn;
+    for (int it = threadIdx.x; it < n_items; it += VMHIP_TILE) {
+        const int i = row0 + it / nn;
+        const int j = it - (it / nn) * nn;
+        int out = V;
+        if (i < V) {
+            const int g = B.row_gidx[(size_t) F.row_base + i];
+            const int gn = F.nbr[(size_t) g * nn + j];
+            const uint2 e = F.r_lookup[min(gn, F.n_nodes)];
+            out = e.x == B.epoch ? (int) e.y : V;
+        }
+        B.row_nb[((size_t) F.row_base + i) * B.nb_stride + j] = out;
+    }
+}
+
+}  // namespace
+
+void vm_launch_libm(int which, const float* x, float* y, int n, hipStream_t stream) {
+    hipLaunchKernelGGL(vm_libm_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, which, x, y, n);
+}
+void vm_launch_reset(const VmBatchDev& B, hipStream_t stream) {
+    hipLaunchKernelGGL(vm_reset_kernel, dim3((B.n_frames + 63) / 64), dim3(64), 0, stream, B);
+}
+void vm_launch_project(const VmBatchDev& B, hipStream_t stream) {
+    if (B.n_cand_tiles > 0) hipLaunchKernelGGL(vm_project_kernel, dim3(B.n_cand_tiles), dim3(VMHIP_TILE), 0, stream, B);
+}
+void vm_launch_compact(const VmBatchDev& B, float* feat, int classify, hipStream_t stream) {
+    if (B.n_cand_tiles > 0)
+        hipLaunchKernelGGL(vm_compact_kernel, dim3(B.n_cand_tiles), dim3(VMHIP_TILE), 0, stream, B,
+                           reinterpret_cast<float4*>(feat), classify);
+}
+void vm_launch_neighbourhood(const VmBatchDev& B, hipStream_t stream) {
+    if (B.n_row_tiles > 0) hipLaunchKernelGGL(vm_neighbourhood_kernel, dim3(B.n_row_tiles), dim3(VMHIP_TILE), 0, stream, B);
+}

@@ -1,0 +1,111 @@
+/*
+ * Internal definitions shared by the kernels and the C ABI implementation of libvisualmesh_hip.so.
+ *
+ * Device memory layout of a staged batch
+ * --------------------------------------
+ * Two index spaces, both tiled by TILE (256) and laid out frame after frame:
+ *   candidate space: one slot per node in the frame's lookup ranges (slot p of frame f lives at
+ *                    cand_base[f] + p). Holds the projected pixel and the keep mask.
+ *   row space:       one row per visible node plus the null row (row i of frame f lives at
+ *                    row_base[f] + i). Capacity per frame = candidates + 1 rounded up to TILE, because
+ *                    the visible count is only known on the device. Holds pixel coordinates, global
+ *                    indices, the neighbourhood table and the ping/pong activation matrices.
+ * A tile never straddles two frames, so every block works for exactly one frame and finds it by a
+ * binary search over the frames' first-tile numbers.
+ */
+#ifndef VMHIP_INTERNAL_H
+#define VMHIP_INTERNAL_H
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "visualmesh_hip.h"
+
+#define VMHIP_TILE 256
+#define VMHIP_AMB_CAP 2048 /* ambiguous candidates recorded per frame */
+
+/* image sampling kinds (derived from the fourcc on the host) */
+enum {
+    VMHIP_FMT_RGBA = 0,
+    VMHIP_FMT_BGRA = 1,
+    VMHIP_FMT_RGB3 = 2,
+    VMHIP_FMT_BGR3 = 3,
+    VMHIP_FMT_GRAY = 4,
+    VMHIP_FMT_GRBG = 5,
+    VMHIP_FMT_RGGB = 6,
+    VMHIP_FMT_GBRG = 7,
+    VMHIP_FMT_BGGR = 8,
+    VMHIP_FMT_NONE = 9
+};
+
+struct VmFrame {
+    /* mesh */
+    const float* rays;     /* [n_nodes][3] */
+    const int32_t* nbr;    /* [n_nodes][nn] */
+    uint2* r_lookup;       /* [n_nodes+1] {epoch, local row}; entry n_nodes is never stamped */
+    int32_t n_nodes;
+    int32_t nn;
+    /* pose + lens */
+    float Rco[9];
+    float focal, centre_x, centre_y;
+    float ik[4];           /* inverse distortion coefficients, computed on the host in fp32 */
+    int32_t width, height, projection;
+    /* image */
+    const uint8_t* image;
+    int32_t fmt;
+    /* lookup ranges */
+    const int32_t* range_first;  /* [n_ranges] first global index of each range */
+    const int32_t* range_prefix; /* [n_ranges+1] exclusive prefix sum of range lengths */
+    int32_t n_ranges;
+    int32_t n_cand;
+    /* placement */
+    int32_t cand_base, cand_tile0, cand_tiles;
+    int32_t row_base, row_tile0, row_tiles;
+    /* forced decisions for candidates the host re-decided: bit set in force_valid -> take force_keep */
+    const uint64_t* force_valid; /* indexed like the keep mask: (cand_base + p) / 64 */
+    const uint64_t* force_keep;
+};
+
+struct VmBatchDev {
+    const VmFrame* frames;
+    int32_t n_frames;
+    int32_t n_cand_tiles, n_row_tiles;
+    uint32_t epoch;
+    /* candidate space */
+    float2* cand_px;
+    uint64_t* cand_keep;  /* one 64-bit mask per wave of candidates */
+    int32_t* tile_count;  /* [n_cand_tiles] kept candidates per tile */
+    /* per frame */
+    int32_t* frame_V;     /* [n_frames] visible nodes */
+    int32_t* amb_count;   /* [n_frames] */
+    int2* amb_list;       /* [n_frames][VMHIP_AMB_CAP] {candidate slot, gpu decision} */
+    /* row space */
+    float2* row_px;
+    int32_t* row_gidx;
+    int32_t* row_nb;      /* [rows][nn_max] with the frame's own nn as stride */
+    int32_t nb_stride;
+};
+
+/* Layer descriptor on the device side (host struct, passed by value to launchers). */
+struct VmLayerDev {
+    int32_t c_in;    /* width of one gathered row */
+    int32_t c_out;
+    int32_t slots;   /* nn+1 for the first layer of a group, 1 for the dense layers after it */
+    int32_t activation;
+    const float* w;  /* [slots*c_in][c_out] fp32 row major */
+    const float* b;  /* [c_out] */
+};
+
+/* launchers, one per kernel; all asynchronous on `stream` */
+void vm_launch_libm(int which, const float* x, float* y, int n, hipStream_t stream);
+void vm_launch_reset(const VmBatchDev& B, hipStream_t stream);
+void vm_launch_project(const VmBatchDev& B, hipStream_t stream);
+void vm_launch_compact(const VmBatchDev& B, float* feat, int classify, hipStream_t stream);
+void vm_launch_neighbourhood(const VmBatchDev& B, hipStream_t stream);
+/* in -> out over the row space; returns 0 or a negative status if the shape is unsupported */
+int vm_launch_conv(const VmBatchDev& B, const VmLayerDev& L, const float* in, float* out, hipStream_t stream,
+                   const char** kernel_name);
+
+#include "host_project.h"
+
+#endif

@@ -1,0 +1,202 @@
+"""Python face of the C++ host code: Mesh, VisualMesh and the HIP Engine.
+
+These classes only marshal numpy arrays in and out of libvisualmesh_host.so; mesh generation, the BSP
+lookup and the engine logic are the C++ in visualmesh_amd/cpp, the device work is libvisualmesh_hip.so.
+The call shapes mirror the reference's engine interface: engine(mesh, Hoc, lens) projects,
+engine(mesh, Hoc, lens, image, fourcc) classifies, `mesh` may be a Mesh or a VisualMesh.
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import native
+from .native import Lens, Network, make_lens  # noqa: F401  (re-exported)
+
+
+def _fp(a):
+    return a.ctypes.data_as(C.POINTER(C.c_float))
+
+
+def _ip(a):
+    return a.ctypes.data_as(C.POINTER(C.c_int32))
+
+
+class Mesh:
+    def __init__(self, model=None, shape=None, radius=None, h=None, k=None, max_distance=None, _ptr=None, _owner=None):
+        self._lib = native.host()
+        if _ptr is None:
+            _ptr = self._lib.vmh_mesh_create(model, shape, radius, h, k, max_distance)
+            if not _ptr:
+                raise RuntimeError("mesh construction failed: " + self._lib.vmh_last_error().decode())
+            self._owned = True
+        else:
+            self._owned = False
+        self._owner = _owner  # keeps a VisualMesh alive while one of its meshes is in use
+        self.ptr = _ptr
+        self.n_nodes = self._lib.vmh_mesh_n_nodes(_ptr)
+        self.n_neighbours = self._lib.vmh_mesh_n_neighbours(_ptr)
+        self.h = self._lib.vmh_mesh_h(_ptr)
+        self._arrays = None
+
+    def __del__(self):
+        if getattr(self, "_owned", False) and self.ptr:
+            self._lib.vmh_mesh_destroy(self.ptr)
+            self.ptr = None
+
+    def arrays(self):
+        """(rays[n,3] float32, neighbours[n,nn] int32) in mesh order"""
+        if self._arrays is None:
+            rays = np.zeros((self.n_nodes, 3), np.float32)
+            nbr = np.zeros((self.n_nodes, self.n_neighbours), np.int32)
+            self._lib.vmh_mesh_copy(self.ptr, _fp(rays), _ip(nbr))
+            self._arrays = (rays, nbr)
+        return self._arrays
+
+    def lookup(self, Hoc, lens):
+        H = np.ascontiguousarray(Hoc, dtype=np.float32)
+        cap = 4096
+        while True:
+            r = np.zeros((cap, 2), np.int32)
+            n = native.host_check(self._lib.vmh_mesh_lookup(self.ptr, _fp(H), C.byref(lens), _ip(r), cap))
+            if n <= cap:
+                return r[:n].copy()
+            cap = n
+
+    def height(self, h):
+        return self
+
+
+class VisualMesh:
+    def __init__(self, model, shape, radius, min_h, max_h, k, max_error, max_distance):
+        self._lib = native.host()
+        self.ptr = self._lib.vmh_visualmesh_create(model, shape, radius, min_h, max_h, k, max_error, max_distance)
+        if not self.ptr:
+            raise RuntimeError("visual mesh construction failed: " + self._lib.vmh_last_error().decode())
+        n = self._lib.vmh_visualmesh_n_meshes(self.ptr)
+        self.meshes = [Mesh(_ptr=self._lib.vmh_visualmesh_mesh(self.ptr, i), _owner=None) for i in range(n)]
+        self._by_ptr = {m.ptr: m for m in self.meshes}
+
+    def __del__(self):
+        if getattr(self, "ptr", None):
+            self._lib.vmh_visualmesh_destroy(self.ptr)
+            self.ptr = None
+
+    def height(self, h):
+        return self._by_ptr[self._lib.vmh_visualmesh_height(self.ptr, float(h))]
+
+
+class Engine:
+    """visualmesh::engine::hip::Engine<float> for meshes of one model (0 = Ring6, 1 = NMGrid8)."""
+
+    def __init__(self, network_groups, model, precision=native.FP32):
+        self._lib = native.host()
+        self.network = network_groups if isinstance(network_groups, Network) else Network(network_groups)
+        self.model = model
+        p = C.c_void_p()
+        native.host_check(self._lib.vmh_engine_create(C.byref(self.network.c), model, precision, C.byref(p)))
+        self.ptr = p
+        self._staged = None
+
+    def __del__(self):
+        if getattr(self, "ptr", None):
+            self._lib.vmh_engine_destroy(self.ptr)
+            self.ptr = None
+
+    @staticmethod
+    def _pick(mesh, Hoc):
+        return mesh.height(float(Hoc[2][3]))
+
+    @staticmethod
+    def _cap(mesh, Hoc, lens):
+        r = mesh.lookup(Hoc, lens)
+        return int((r[:, 1] - r[:, 0]).sum()) if len(r) else 0
+
+    def project(self, mesh, Hoc, lens):
+        m = self._pick(mesh, Hoc)
+        H = np.ascontiguousarray(Hoc, dtype=np.float32)
+        cap = self._cap(m, H, lens)
+        px = np.zeros((max(cap, 1), 2), np.float32)
+        nb = np.zeros((cap + 1, m.n_neighbours), np.int32)
+        gidx = np.zeros(max(cap, 1), np.int32)
+        V = native.host_check(self._lib.vmh_engine_project(self.ptr, m.ptr, _fp(H), C.byref(lens), cap, _fp(px), _ip(nb), _ip(gidx)))
+        if V == 0:
+            return dict(px=px[:0], nb=nb[:0], gidx=gidx[:0])
+        return dict(px=px[:V].copy(), nb=nb[:V + 1].copy(), gidx=gidx[:V].copy())
+
+    def classify(self, mesh, Hoc, lens, image, fcc):
+        m = self._pick(mesh, Hoc)
+        H = np.ascontiguousarray(Hoc, dtype=np.float32)
+        cap = self._cap(m, H, lens)
+        n_out = self.network.n_out
+        px = np.zeros((max(cap, 1), 2), np.float32)
+        nb = np.zeros((cap + 1, m.n_neighbours), np.int32)
+        gidx = np.zeros(max(cap, 1), np.int32)
+        cls = np.zeros((cap + 1, n_out), np.float32)
+        img = np.ascontiguousarray(image)
+        V = native.host_check(self._lib.vmh_engine_classify(self.ptr, m.ptr, _fp(H), C.byref(lens), img.ctypes.data, fcc, cap,
+                                                            _fp(px), _ip(nb), _ip(gidx), _fp(cls)))
+        if V == 0:
+            return dict(px=px[:0], nb=nb[:0], gidx=gidx[:0], cls=cls[:0])
+        return dict(px=px[:V].copy(), nb=nb[:V + 1].copy(), gidx=gidx[:V].copy(), cls=cls[:V + 1].copy())
+
+    def __call__(self, mesh, Hoc, lens, image=None, fcc=None):
+        if image is None:
+            return self.project(mesh, Hoc, lens)
+        return self.classify(mesh, Hoc, lens, image, fcc)
+
+    # ---- staged batches
+    def stage(self, frames):
+        """frames: list of dict(mesh=Mesh|VisualMesh, Hoc, lens, image, fourcc); copies the inputs to the device"""
+        n = len(frames)
+        meshes = [self._pick(f["mesh"], f["Hoc"]) for f in frames]
+        mesh_ptrs = (C.c_void_p * n)(*[m.ptr for m in meshes])
+        H = np.ascontiguousarray(np.stack([np.asarray(f["Hoc"], dtype=np.float32) for f in frames]))
+        lenses = (Lens * n)(*[f["lens"] for f in frames])
+        images = [np.ascontiguousarray(f["image"]) for f in frames]
+        image_ptrs = (C.c_void_p * n)(*[im.ctypes.data for im in images])
+        fccs = (C.c_uint32 * n)(*[f["fourcc"] for f in frames])
+        native.host_check(self._lib.vmh_engine_stage(self.ptr, n, mesh_ptrs, _fp(H), lenses, image_ptrs, fccs))
+        self._staged = meshes
+
+    def run(self):
+        native.host_check(self._lib.vmh_engine_run(self.ptr))
+
+    def counts(self):
+        n = len(self._staged)
+        v = np.zeros(n, np.int32)
+        native.host_check(self._lib.vmh_engine_counts(self.ptr, _ip(v), n))
+        return v
+
+    def fetch(self):
+        n = native.host_check(self._lib.vmh_engine_fetch(self.ptr))
+        counts = self.counts()
+        out = []
+        n_out = self.network.n_out
+        for i in range(n):
+            V = int(counts[i])
+            m = self._staged[i]
+            px = np.zeros((max(V, 1), 2), np.float32)
+            nb = np.zeros((V + 1, m.n_neighbours), np.int32)
+            gidx = np.zeros(max(V, 1), np.int32)
+            cls = np.zeros((V + 1, n_out), np.float32)
+            got = native.host_check(self._lib.vmh_engine_result(self.ptr, i, V, _fp(px), _ip(nb), _ip(gidx), _fp(cls)))
+            assert got == V
+            if V == 0:
+                out.append(dict(px=px[:0], nb=nb[:0], gidx=gidx[:0], cls=cls[:0]))
+            else:
+                out.append(dict(px=px, nb=nb, gidx=gidx, cls=cls))
+        return out
+
+    def classify_batch(self, frames):
+        self.stage(frames)
+        self.run()
+        return self.fetch()
+
+    def native_batch(self):
+        return C.c_void_p(self._lib.vmh_engine_native_batch(self.ptr))
+
+    def profile(self, enable=True):
+        native.hip_check(native.hip().vmhip_batch_profile(self.native_batch(), 1 if enable else 0))
+
+    def profile_read(self):
+        return native.profile_read(self.native_batch())

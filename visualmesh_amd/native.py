@@ -1,0 +1,208 @@
+"""ctypes bindings of the two native libraries.
+
+    hip()   libvisualmesh_hip.so   the C ABI of include/visualmesh_hip.h (kernels + device state)
+    host()  libvisualmesh_host.so  the C++ host code (Mesh, VisualMesh, visualmesh::engine::hip::Engine)
+                                   behind a small C interface
+
+There is no fallback: if a library has not been built, loading raises, and every call that needs a GPU
+fails with the library's own error when none is present.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+HIP_LIB = os.path.join(PKG, "lib", "libvisualmesh_hip.so")
+HOST_LIB = os.path.join(PKG, "lib", "libvisualmesh_host.so")
+
+OK, ERR_HIP, ERR_FORMAT, ERR_LENS, ERR_ARGUMENT, ERR_CAPACITY = 0, -1, -2, -3, -4, -5
+FP32, BF16 = 0, 1
+
+# every symbol include/visualmesh_hip.h declares
+HIP_SYMBOLS = [
+    "vmhip_last_error", "vmhip_engine_create", "vmhip_engine_destroy", "vmhip_engine_n_classes", "vmhip_mesh_upload",
+    "vmhip_mesh_release", "vmhip_project", "vmhip_classify", "vmhip_classify_batch", "vmhip_batch_create",
+    "vmhip_batch_destroy", "vmhip_batch_stage", "vmhip_batch_run", "vmhip_batch_counts", "vmhip_batch_fetch",
+    "vmhip_batch_profile", "vmhip_batch_profile_read", "vmhip_selftest_libm",
+]
+
+
+class VisualMeshError(RuntimeError):
+    def __init__(self, code, message):
+        super().__init__("%s (status %d)" % (message, code))
+        self.code = code
+
+
+class Lens(C.Structure):
+    _fields_ = [("width", C.c_int32), ("height", C.c_int32), ("projection", C.c_int32), ("focal_length", C.c_float),
+                ("centre", C.c_float * 2), ("k", C.c_float * 2), ("fov", C.c_float)]
+
+
+def make_lens(width, height, projection, focal_length, fov, centre=(0.0, 0.0), k=(0.0, 0.0)):
+    return Lens(width, height, projection, focal_length, (C.c_float * 2)(*centre), (C.c_float * 2)(*k), fov)
+
+
+class Layer(C.Structure):
+    _fields_ = [("n_in", C.c_int32), ("n_out", C.c_int32), ("activation", C.c_int32), ("weights", C.POINTER(C.c_float)),
+                ("biases", C.POINTER(C.c_float))]
+
+
+class NetworkC(C.Structure):
+    _fields_ = [("n_groups", C.c_int32), ("group_sizes", C.POINTER(C.c_int32)), ("layers", C.POINTER(Layer))]
+
+
+class Frame(C.Structure):
+    _fields_ = [("mesh", C.c_void_p), ("Rco", C.c_float * 9), ("lens", Lens), ("ranges", C.POINTER(C.c_int32)),
+                ("n_ranges", C.c_int32), ("image", C.c_void_p), ("fourcc", C.c_uint32)]
+
+
+class Result(C.Structure):
+    _fields_ = [("capacity", C.c_int32), ("n_visible", C.c_int32), ("pixel_coordinates", C.POINTER(C.c_float)),
+                ("global_indices", C.POINTER(C.c_int32)), ("neighbourhood", C.POINTER(C.c_int32)),
+                ("classifications", C.POINTER(C.c_float))]
+
+
+def _fp(a):
+    return a.ctypes.data_as(C.POINTER(C.c_float))
+
+
+def _ip(a):
+    return a.ctypes.data_as(C.POINTER(C.c_int32))
+
+
+class Network:
+    """list of groups, group = list of (weights[n_in, n_out], biases[n_out], activation) -> vmhip_network"""
+
+    def __init__(self, groups):
+        self.groups = groups
+        self._keep = []
+        layers = []
+        for g in groups:
+            for (w, b, act) in g:
+                w = np.ascontiguousarray(w, dtype=np.float32)
+                b = np.ascontiguousarray(b, dtype=np.float32)
+                self._keep += [w, b]
+                layers.append(Layer(w.shape[0], w.shape[1], act, _fp(w), _fp(b)))
+        self._layers = (Layer * max(len(layers), 1))(*layers)
+        self._sizes = (C.c_int32 * max(len(groups), 1))(*[len(g) for g in groups])
+        self.c = NetworkC(len(groups), self._sizes, self._layers)
+        self.n_out = groups[-1][-1][0].shape[1] if groups else 4
+
+
+_hip = None
+_host = None
+
+
+def hip():
+    """libvisualmesh_hip.so with argument types set."""
+    global _hip
+    if _hip is not None:
+        return _hip
+    if not os.path.exists(HIP_LIB):
+        raise FileNotFoundError(HIP_LIB + " is not built: run `python -m visualmesh_amd.build`")
+    L = C.CDLL(HIP_LIB, mode=C.RTLD_GLOBAL)
+    vp = C.c_void_p
+    L.vmhip_last_error.restype = C.c_char_p
+    L.vmhip_engine_create.argtypes = [C.POINTER(NetworkC), C.c_int32, C.c_int32, C.POINTER(vp)]
+    L.vmhip_engine_destroy.argtypes = [vp]
+    L.vmhip_engine_destroy.restype = None
+    L.vmhip_engine_n_classes.argtypes = [vp]
+    L.vmhip_mesh_upload.argtypes = [C.POINTER(C.c_float), C.POINTER(C.c_int32), C.c_int32, C.c_int32, C.POINTER(vp)]
+    L.vmhip_mesh_release.argtypes = [vp]
+    L.vmhip_mesh_release.restype = None
+    L.vmhip_project.argtypes = [vp, C.POINTER(Frame), C.POINTER(Result)]
+    L.vmhip_classify.argtypes = [vp, C.POINTER(Frame), C.POINTER(Result)]
+    L.vmhip_classify_batch.argtypes = [vp, C.POINTER(Frame), C.c_int32, C.POINTER(Result)]
+    L.vmhip_batch_create.argtypes = [vp, C.POINTER(vp)]
+    L.vmhip_batch_destroy.argtypes = [vp]
+    L.vmhip_batch_destroy.restype = None
+    L.vmhip_batch_stage.argtypes = [vp, C.POINTER(Frame), C.c_int32, C.c_int32]
+    L.vmhip_batch_run.argtypes = [vp]
+    L.vmhip_batch_counts.argtypes = [vp, C.POINTER(C.c_int32)]
+    L.vmhip_batch_fetch.argtypes = [vp, C.POINTER(Result)]
+    L.vmhip_batch_profile.argtypes = [vp, C.c_int32]
+    L.vmhip_batch_profile_read.argtypes = [vp, C.c_int32, C.POINTER(C.c_int32), C.POINTER(C.c_char_p), C.POINTER(C.c_float),
+                                           C.POINTER(C.c_int64)]
+    L.vmhip_selftest_libm.argtypes = [C.c_int32, C.POINTER(C.c_float), C.POINTER(C.c_float), C.c_int32]
+    _hip = L
+    return L
+
+
+def hip_check(rc):
+    if rc < 0:
+        raise VisualMeshError(rc, hip().vmhip_last_error().decode())
+    return rc
+
+
+def profile_read(batch_ptr, max_slots=256):
+    """[(kernel name, milliseconds, units)] of the last profiled run of a vmhip_batch."""
+    L = hip()
+    n = C.c_int32(0)
+    names = (C.c_char_p * max_slots)()
+    ms = (C.c_float * max_slots)()
+    units = (C.c_int64 * max_slots)()
+    hip_check(L.vmhip_batch_profile_read(batch_ptr, max_slots, C.byref(n), names, ms, units))
+    return [(names[i].decode(), float(ms[i]), int(units[i])) for i in range(n.value)]
+
+
+def host():
+    """libvisualmesh_host.so with argument types set."""
+    global _host
+    if _host is not None:
+        return _host
+    hip()  # the host library links against it; load it first so a missing build fails with a clear message
+    if not os.path.exists(HOST_LIB):
+        raise FileNotFoundError(HOST_LIB + " is not built: run `python -m visualmesh_amd.build`")
+    L = C.CDLL(HOST_LIB)
+    vp = C.c_void_p
+    L.vmh_last_error.restype = C.c_char_p
+    L.vmh_mesh_create.restype = vp
+    L.vmh_mesh_create.argtypes = [C.c_int, C.c_int, C.c_float, C.c_float, C.c_float, C.c_float]
+    L.vmh_mesh_destroy.argtypes = [vp]
+    L.vmh_mesh_destroy.restype = None
+    L.vmh_mesh_n_nodes.argtypes = [vp]
+    L.vmh_mesh_n_neighbours.argtypes = [vp]
+    L.vmh_mesh_h.argtypes = [vp]
+    L.vmh_mesh_h.restype = C.c_float
+    L.vmh_mesh_copy.argtypes = [vp, C.POINTER(C.c_float), C.POINTER(C.c_int32)]
+    L.vmh_mesh_copy.restype = None
+    L.vmh_mesh_lookup.argtypes = [vp, C.POINTER(C.c_float), C.POINTER(Lens), C.POINTER(C.c_int32), C.c_int]
+    L.vmh_visualmesh_create.restype = vp
+    L.vmh_visualmesh_create.argtypes = [C.c_int, C.c_int] + [C.c_float] * 6
+    L.vmh_visualmesh_destroy.argtypes = [vp]
+    L.vmh_visualmesh_destroy.restype = None
+    L.vmh_visualmesh_n_meshes.argtypes = [vp]
+    L.vmh_visualmesh_mesh.restype = vp
+    L.vmh_visualmesh_mesh.argtypes = [vp, C.c_int]
+    L.vmh_visualmesh_height.restype = vp
+    L.vmh_visualmesh_height.argtypes = [vp, C.c_float]
+    L.vmh_engine_create.argtypes = [C.POINTER(NetworkC), C.c_int, C.c_int, C.POINTER(vp)]
+    L.vmh_engine_destroy.argtypes = [vp]
+    L.vmh_engine_destroy.restype = None
+    L.vmh_engine_project.argtypes = [vp, vp, C.POINTER(C.c_float), C.POINTER(Lens), C.c_int, C.POINTER(C.c_float),
+                                     C.POINTER(C.c_int32), C.POINTER(C.c_int32)]
+    L.vmh_engine_classify.argtypes = [vp, vp, C.POINTER(C.c_float), C.POINTER(Lens), vp, C.c_uint32, C.c_int,
+                                      C.POINTER(C.c_float), C.POINTER(C.c_int32), C.POINTER(C.c_int32), C.POINTER(C.c_float)]
+    L.vmh_engine_stage.argtypes = [vp, C.c_int, C.POINTER(vp), C.POINTER(C.c_float), C.POINTER(Lens), C.POINTER(vp),
+                                   C.POINTER(C.c_uint32)]
+    L.vmh_engine_run.argtypes = [vp]
+    L.vmh_engine_counts.argtypes = [vp, C.POINTER(C.c_int32), C.c_int]
+    L.vmh_engine_fetch.argtypes = [vp]
+    L.vmh_engine_result.argtypes = [vp, C.c_int, C.c_int, C.POINTER(C.c_float), C.POINTER(C.c_int32), C.POINTER(C.c_int32),
+                                    C.POINTER(C.c_float)]
+    L.vmh_engine_native_batch.restype = vp
+    L.vmh_engine_native_batch.argtypes = [vp]
+    L.vmh_engine_clear_cache.argtypes = [vp]
+    L.vmh_engine_clear_cache.restype = None
+    _host = L
+    return L
+
+
+def host_check(rc):
+    if rc < 0:
+        msg = host().vmh_last_error().decode()
+        if rc == ERR_FORMAT:
+            raise ValueError(msg)
+        raise VisualMeshError(rc, msg)
+    return rc
