@@ -1,0 +1,216 @@
+"""Benchmark of the Visual Mesh inference hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2] [--frames F] [--no-cpu]
+
+A step is one pass of the whole device path (projection, filter/compaction, sampling, neighbourhood, all
+graph-convolution layers) over one staged batch of synthetic frames whose inputs are already resident in
+device memory. Prints one JSON line: nodes classified per second, plus frames per second, the roofline
+position of the dominant kernel (timed live with HIP events on the engine's stream) and the CPU oracle
+timed on the host's cores as a baseline.
+"""
+import argparse
+import json
+import os
+import sys
+import threading
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
+FP32_PEAK_TFLOPS = 157.3   # MI355X dense fp32 matrix
+BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix
+
+# HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, keyed by
+# (workload, kernel); filled in from the summaries under profiles/ (None = not measured).
+MEASURED_TRAFFIC = {}
+
+
+def layer_table(cfg, n_neighbours):
+    """per layer: (c_in, c_out, slots, algorithmic bytes per row, flops per row) for fp32 activations"""
+    out = []
+    c_in = 4
+    for group in cfg.network:
+        for li, (w, b, act) in enumerate(group):
+            slots = n_neighbours + 1 if li == 0 else 1
+            c_out = w.shape[1]
+            nbytes = c_in * 4 + (4 * n_neighbours if li == 0 else 0) + c_out * 4
+            flops = 2 * slots * c_in * c_out
+            out.append((c_in, c_out, slots, nbytes, flops))
+            c_in = c_out
+    return out
+
+
+def cpu_baseline(cfg, threads):
+    """The CPU oracle (a port of the reference CPU engine) on `threads` host threads, one frame per task, a
+    fresh engine state per frame, the mesh shared - the reference benchmark's own pattern."""
+    from oracle import vmo
+    O = vmo.load("oracle")
+    lens = vmo.make_lens(*cfg.lens_tuple())
+    if cfg.visualmesh is None:
+        mesh = O.mesh(cfg.model, cfg.shape, cfg.radius, cfg.mesh_h, cfg.k, cfg.max_distance)
+        pick = lambda H: mesh
+    else:
+        v = cfg.visualmesh
+        vm = O.visualmesh(cfg.model, cfg.shape, cfg.radius, v["min_h"], v["max_h"], cfg.k, v["max_error"], cfg.max_distance)
+        pick = lambda H: vm.height(float(H[2][3]))
+    net = vmo.Network(cfg.network)
+    frames = cfg.frames
+    visible = [0] * len(frames)
+    todo = list(range(len(frames)))
+    lock = threading.Lock()
+
+    def worker():
+        while True:
+            with lock:
+                if not todo:
+                    return
+                i = todo.pop()
+            f = frames[i]
+            r = pick(f["Hoc"]).classify(f["Hoc"], lens, f["image"], cfg.fourcc, net)  # ctypes releases the GIL
+            visible[i] = len(r["gidx"])
+
+    t0 = time.perf_counter()
+    pool = [threading.Thread(target=worker) for _ in range(threads)]
+    for t in pool:
+        t.start()
+    for t in pool:
+        t.join()
+    dt = time.perf_counter() - t0
+    return sum(visible) / dt, len(frames) / dt, dt
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", type=int, default=2, help="workload configuration 1..5 (default 2: batched 1280x1024)")
+    ap.add_argument("--frames", type=int, default=None, help="frames per batch (default: the configuration's own)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run a 1 GiB plain copy kernel (the dispatch of known size that memory counters are scaled by)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (frames would shard across GPUs "
+              "without any exchange); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    from visualmesh_amd import engine as eng
+    from visualmesh_amd import native
+    from visualmesh_amd import workloads as wl
+
+    cfg = wl.config(args.config, n_frames=args.frames)
+    nn = wl.N_NEIGHBOURS[cfg.model]
+    lens = native.make_lens(*cfg.lens_tuple())
+    if cfg.visualmesh is None:
+        mesh = eng.Mesh(cfg.model, cfg.shape, cfg.radius, cfg.mesh_h, cfg.k, cfg.max_distance)
+    else:
+        v = cfg.visualmesh
+        mesh = eng.VisualMesh(cfg.model, cfg.shape, cfg.radius, v["min_h"], v["max_h"], cfg.k, v["max_error"], cfg.max_distance)
+    precision = native.BF16 if cfg.precision == "bf16" else native.FP32
+    engine = eng.Engine(cfg.network, cfg.model, precision)
+    frames = [dict(mesh=mesh, Hoc=f["Hoc"], lens=lens, image=f["image"], fourcc=cfg.fourcc) for f in cfg.frames]
+
+    engine.stage(frames)          # inputs become resident in HBM here, outside the timed region
+    for _ in range(args.warmup):
+        engine.run()
+    visible = engine.counts()
+    nodes = int(visible.sum())
+
+    engine.profile(True)          # HIP events around every kernel launch, on the engine's stream
+    kernel_ms = {}
+    kernel_launches = {}
+    kernel_rows = {}
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        engine.run()              # launches the whole path and waits for it
+        for name, ms, units in engine.profile_read():
+            kernel_ms[name] = kernel_ms.get(name, 0.0) + ms
+            kernel_launches[name] = kernel_launches.get(name, 0) + 1
+            kernel_rows[name] = units
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+    value = nodes * args.steps / elapsed
+
+    # roofline of the dominant graph-convolution kernel
+    rows = nodes + len(frames)    # visible nodes + one null row per frame
+    table = layer_table(cfg, nn)
+    conv = {k: v for k, v in kernel_ms.items() if k.startswith("conv")}
+    dominant = max(conv, key=conv.get) if conv else None
+    roofline = None
+    if dominant:
+        avg_ms = kernel_ms[dominant] / kernel_launches[dominant]
+        # the layer shape is in the kernel name: conv_<kind>_<cin>x<cout>s<slots>
+        shape = dominant.split("_")[-1]
+        c_in, rest = shape.split("x")
+        c_out, slots = rest.split("s")
+        c_in, c_out, slots = int(c_in), int(c_out), int(slots)
+        s_act = 4
+        bytes_per_row = c_in * s_act + 4 * (slots - 1) + c_out * s_act
+        flops_per_row = 2 * slots * c_in * c_out
+        intensity = flops_per_row / bytes_per_row
+        ridge = FP32_PEAK_TFLOPS * 1e12 / (HBM_PEAK_GBS * 1e9)
+        if intensity > ridge:
+            achieved = flops_per_row * rows / (avg_ms * 1e-3) / 1e12
+            roofline = dict(bound="mfma", achieved=achieved, peak=FP32_PEAK_TFLOPS, unit="TFLOP/s", frac=achieved / FP32_PEAK_TFLOPS)
+        else:
+            achieved = bytes_per_row * rows / (avg_ms * 1e-3) / 1e9
+            roofline = dict(bound="hbm", achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s", frac=achieved / HBM_PEAK_GBS)
+        roofline.update(kernel=dominant, avg_launch_ms=avg_ms, launches_per_step=kernel_launches[dominant] // args.steps,
+                        rows_per_launch=rows, algorithmic_bytes_per_row=bytes_per_row, flops_per_row=flops_per_row,
+                        traffic=MEASURED_TRAFFIC.get((cfg.name, dominant)))
+
+    copy_gbs = None
+    if args.copy_probe:
+        nbytes = 1 << 30
+        copy_gbs = 2 * nbytes / (native.copy_probe(nbytes, 5) * 1e-3) / 1e9
+
+    cpu = None
+    if not args.no_cpu:
+        threads = min(16, os.cpu_count() or 1, len(cfg.frames))
+        sample = cfg
+        note = "all %d frames of the batch once, one frame per task" % len(cfg.frames)
+        if args.config in (4, 5):  # a frame costs ~45 s per core: time a stated subset
+            sample = wl.config(args.config, n_frames=min(threads, len(cfg.frames)))
+            note = "the first %d frames of the batch once, one frame per task" % len(sample.frames)
+        nps, fps, dt = cpu_baseline(sample, threads)
+        cpu = dict(value=nps, unit="nodes/s", cores=threads, kind="port", frames_per_s=fps, seconds=dt, sample=note)
+
+    out = {
+        "metric": "mesh nodes classified/sec",
+        "value": value,
+        "unit": "nodes/s",
+        "frames_per_s": len(frames) * args.steps / elapsed,
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16" if cfg.precision == "bf16" else "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "%s: %d frames of %dx%d %s, %s lens, %s mesh, network %s" % (
+                cfg.name, len(frames), cfg.width, cfg.height, "RGBA8" if cfg.fourcc == wl.fourcc("RGBA") else "GRBG8",
+                {0: "rectilinear", 1: "equisolid", 2: "equidistant"}[cfg.projection],
+                {0: "Ring6", 1: "NMGrid8"}[cfg.model], "->".join(["4"] + [str(t[1]) for t in table])),
+            "frames": len(frames),
+            "visible_nodes_per_batch": nodes,
+            "inputs": "resident in HBM before the timed region",
+        },
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "copy_kernel_GBps": copy_gbs,
+        "kernel_ms_per_step": {k: v / args.steps for k, v in sorted(kernel_ms.items())},
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

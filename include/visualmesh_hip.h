@@ -157,6 +157,11 @@ int vmhip_batch_profile_read(vmhip_batch* batch, int32_t max_slots, int32_t* n_s
  * own acosf (which = 0), sinf (1), tanf (2) or sqrtf (3) - the functions the lens projection is built from
  * and which must return the host C library's bits. x and y are host buffers. */
 int vmhip_selftest_libm(int32_t which, const float* x, float* y, int32_t n);
+/* Diagnostic with no counterpart in the reference: runs a plain device-to-device copy kernel of `bytes`
+ * bytes (a multiple of 16) `repeats` times and returns the average milliseconds per launch in *ms. Profilers
+ * use it as the dispatch of known size that hardware memory counters are scaled by; it also gives the
+ * practical copy bandwidth of the device. */
+int vmhip_selftest_copy(int64_t bytes, int32_t repeats, float* ms);
 
 #ifdef __cplusplus
 }

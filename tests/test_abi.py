@@ -1,0 +1,39 @@
+"""The C ABI library loads without a GPU and exports every symbol include/visualmesh_hip.h declares."""
+import ctypes
+import os
+import re
+
+from visualmesh_amd import native
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "visualmesh_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(vmhip_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_header_and_binding_list_agree():
+    assert declared_symbols() == sorted(native.HIP_SYMBOLS)
+
+
+def test_hip_library_exports_every_declared_symbol():
+    lib = ctypes.CDLL(native.HIP_LIB)
+    for name in declared_symbols():
+        assert hasattr(lib, name), name + " is declared in the header but not exported"
+
+
+def test_host_library_loads_and_links_the_hip_library():
+    lib = native.host()
+    for name in ("vmh_mesh_create", "vmh_mesh_lookup", "vmh_visualmesh_create", "vmh_engine_create", "vmh_engine_project",
+                 "vmh_engine_classify", "vmh_engine_stage", "vmh_engine_run", "vmh_engine_fetch", "vmh_engine_result"):
+        assert hasattr(lib, name)
+
+
+def test_struct_layouts_match_the_header():
+    # vmhip_lens: 2 int32 + int32 + float + 2 float + 2 float + float = 36 bytes; vmhip_frame holds it by value
+    assert ctypes.sizeof(native.Lens) == 36
+    assert ctypes.sizeof(native.Layer) == 32
+    assert ctypes.sizeof(native.Result) == 40
+    assert native.Frame.Rco.offset == 8 and native.Frame.lens.offset == 44 and native.Frame.ranges.offset == 80

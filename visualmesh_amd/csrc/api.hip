@@ -655,6 +655,33 @@ int vmhip_selftest_libm(int32_t which, const float* x, float* y, int32_t n) {
     return VMHIP_OK;
 }
 
+int vmhip_selftest_copy(int64_t bytes, int32_t repeats, float* ms) {
+    if (bytes <= 0 || bytes % 16 != 0 || repeats <= 0) return fail(VMHIP_ERR_ARGUMENT, "selftest_copy: bad arguments");
+    void *src = nullptr, *dst = nullptr;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    hipError_t e = hipMalloc(&src, size_t(bytes));
+    if (e == hipSuccess) e = hipMalloc(&dst, size_t(bytes));
+    if (e == hipSuccess) e = hipMemset(src, 1, size_t(bytes));
+    if (e == hipSuccess) e = hipEventCreate(&e0);
+    if (e == hipSuccess) e = hipEventCreate(&e1);
+    if (e == hipSuccess) {
+        vm_launch_copy_probe(src, dst, size_t(bytes), nullptr); /* warm-up */
+        e = hipEventRecord(e0, nullptr);
+        for (int i = 0; i < repeats && e == hipSuccess; ++i) vm_launch_copy_probe(src, dst, size_t(bytes), nullptr);
+        if (e == hipSuccess) e = hipEventRecord(e1, nullptr);
+        if (e == hipSuccess) e = hipEventSynchronize(e1);
+        float total = 0.0f;
+        if (e == hipSuccess) e = hipEventElapsedTime(&total, e0, e1);
+        if (ms) *ms = total / float(repeats);
+    }
+    if (e0) (void) hipEventDestroy(e0);
+    if (e1) (void) hipEventDestroy(e1);
+    if (src) (void) hipFree(src);
+    if (dst) (void) hipFree(dst);
+    if (e != hipSuccess) return fail(VMHIP_ERR_HIP, std::string("selftest_copy: ") + hipGetErrorString(e));
+    return VMHIP_OK;
+}
+
 int vmhip_classify_batch(vmhip_engine* E, const vmhip_frame* frames, int32_t n_frames, vmhip_result* results) {
     if (!E) return fail(VMHIP_ERR_ARGUMENT, "classify_batch: null engine");
     ensure_scratch(E);

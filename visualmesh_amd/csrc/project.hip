@@ -100,6 +100,11 @@ __global__ void vm_libm_kernel(int which, const float* x, float* y, int n) {
     y[i] = which == 0 ? vm_acosf(v) : which == 1 ? vm_sinf(v) : which == 2 ? vm_tanf(v) : vm_sqrtf(v);
 }
 
+/* plain streaming copy of 16-byte words: the yardstick the memory counters are scaled by */
+__global__ __launch_bounds__(256) void vm_copy_probe_kernel(const float4* __restrict__ src, float4* __restrict__ dst, size_t n) {
+    for (size_t i = (size_t) blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t) gridDim.x * blockDim.x) dst[i] = src[i];
+}
+
 __global__ void vm_reset_kernel(VmBatchDev B) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < B.n_frames) B.amb_count[i] = 0;
@@ -352,6 +357,11 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_neighbourhood_kernel(VmBatchDev
 
 void vm_launch_libm(int which, const float* x, float* y, int n, hipStream_t stream) {
     hipLaunchKernelGGL(vm_libm_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, which, x, y, n);
+}
+void vm_launch_copy_probe(const void* src, void* dst, size_t bytes, hipStream_t stream) {
+    const size_t n = bytes / 16;
+    hipLaunchKernelGGL(vm_copy_probe_kernel, dim3(256 * 16), dim3(256), 0, stream, reinterpret_cast<const float4*>(src),
+                       reinterpret_cast<float4*>(dst), n);
 }
 void vm_launch_reset(const VmBatchDev& B, hipStream_t stream) {
     hipLaunchKernelGGL(vm_reset_kernel, dim3((B.n_frames + 63) / 64), dim3(64), 0, stream, B);

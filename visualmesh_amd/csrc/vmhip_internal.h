@@ -98,6 +98,7 @@ struct VmLayerDev {
 
 /* launchers, one per kernel; all asynchronous on `stream` */
 void vm_launch_libm(int which, const float* x, float* y, int n, hipStream_t stream);
+void vm_launch_copy_probe(const void* src, void* dst, size_t bytes, hipStream_t stream);
 void vm_launch_reset(const VmBatchDev& B, hipStream_t stream);
 void vm_launch_project(const VmBatchDev& B, hipStream_t stream);
 void vm_launch_compact(const VmBatchDev& B, float* feat, int classify, hipStream_t stream);

@@ -24,7 +24,7 @@ HIP_SYMBOLS = [
     "vmhip_last_error", "vmhip_engine_create", "vmhip_engine_destroy", "vmhip_engine_n_classes", "vmhip_mesh_upload",
     "vmhip_mesh_release", "vmhip_project", "vmhip_classify", "vmhip_classify_batch", "vmhip_batch_create",
     "vmhip_batch_destroy", "vmhip_batch_stage", "vmhip_batch_run", "vmhip_batch_counts", "vmhip_batch_fetch",
-    "vmhip_batch_profile", "vmhip_batch_profile_read", "vmhip_selftest_libm",
+    "vmhip_batch_profile", "vmhip_batch_profile_read", "vmhip_selftest_libm", "vmhip_selftest_copy",
 ]
 
 
@@ -125,6 +125,7 @@ def hip():
     L.vmhip_batch_profile_read.argtypes = [vp, C.c_int32, C.POINTER(C.c_int32), C.POINTER(C.c_char_p), C.POINTER(C.c_float),
                                            C.POINTER(C.c_int64)]
     L.vmhip_selftest_libm.argtypes = [C.c_int32, C.POINTER(C.c_float), C.POINTER(C.c_float), C.c_int32]
+    L.vmhip_selftest_copy.argtypes = [C.c_int64, C.c_int32, C.POINTER(C.c_float)]
     _hip = L
     return L
 
@@ -133,6 +134,13 @@ def hip_check(rc):
     if rc < 0:
         raise VisualMeshError(rc, hip().vmhip_last_error().decode())
     return rc
+
+
+def copy_probe(nbytes=1 << 30, repeats=5):
+    """average milliseconds of a plain device copy kernel of nbytes (read nbytes + write nbytes)"""
+    ms = C.c_float(0.0)
+    hip_check(hip().vmhip_selftest_copy(nbytes, repeats, C.byref(ms)))
+    return float(ms.value)
 
 
 def profile_read(batch_ptr, max_slots=256):
