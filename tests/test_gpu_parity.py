@@ -97,3 +97,54 @@ def test_pixels_and_inputs_bit_exact(oracle):
         assert np.array_equal(got["gidx"], want["gidx"])
         assert np.array_equal(got["px"].view(np.uint32), want["px"].view(np.uint32)), "%s pixel bits" % cfg.name
         assert np.array_equal(got["cls"].view(np.uint32), want["cls"].view(np.uint32)), "%s sampled input bits" % cfg.name
+
+
+def test_config4_geometry_projection(oracle):
+    """Configuration 4's mesh (849k nodes), lens and image size: indices, neighbourhood and pixels on three of
+    its random poses (the 64-wide network on this geometry costs the oracle ~45 s per frame, so the
+    probabilities are checked on the smaller geometry below)."""
+    cfg = wl.config(4, n_frames=3)
+    o_lens, e_lens = lens_pair(cfg)
+    o_mesh, e_mesh = meshes_for(cfg, oracle)
+    engine = eng.Engine([], cfg.model)
+    for i, f in enumerate(cfg.frames):
+        got = engine(e_mesh, f["Hoc"], e_lens)
+        want = o_mesh.project(f["Hoc"], o_lens)
+        print("cfg4 frame", i, "V =", len(want["gidx"]), flush=True)
+        assert_projection_parity(got, want, "cfg4 frame %d" % i)
+
+
+def test_config4_network_on_config1_geometry(oracle):
+    """The 6 x 64-wide network of configuration 4 (matrix-core kernels, 64-wide softmax) on configuration 1's
+    geometry, two frames in one batch."""
+    cfg = wl.config(1, n_frames=2)
+    net = wl.config(4, n_frames=1).network
+    o_lens, e_lens = lens_pair(cfg)
+    o_mesh, e_mesh = meshes_for(cfg, oracle)
+    engine = eng.Engine(net, cfg.model)
+    frames = [dict(mesh=e_mesh, Hoc=f["Hoc"], lens=e_lens, image=f["image"], fourcc=cfg.fourcc) for f in cfg.frames]
+    results = engine.classify_batch(frames)
+    for i, f in enumerate(cfg.frames):
+        want = o_mesh.classify(f["Hoc"], o_lens, f["image"], cfg.fourcc, vmo.Network(net))
+        assert_classification_parity(results[i], want, PROB_TOL, "64-wide frame %d" % i)
+
+
+@pytest.mark.parametrize("kernel", ["rows", "mfma"])
+def test_both_convolution_kernels_agree_with_the_oracle(oracle, kernel, monkeypatch):
+    """Every layer shape of configuration 2 through the one-row-per-lane kernel and through the matrix-core
+    kernel (selected per engine with VMHIP_CONV_KERNEL)."""
+    monkeypatch.setenv("VMHIP_CONV_KERNEL", kernel)
+    cfg = wl.config(2, n_frames=2)
+    o_lens, e_lens = lens_pair(cfg)
+    o_mesh, e_mesh = meshes_for(cfg, oracle)
+    engine = eng.Engine(cfg.network, cfg.model)
+    frames = [dict(mesh=e_mesh, Hoc=f["Hoc"], lens=e_lens, image=f["image"], fourcc=cfg.fourcc) for f in cfg.frames]
+    engine.profile(False)
+    results = engine.classify_batch(frames)
+    engine.profile(True)
+    engine.run()
+    names = [n for n, _, _ in engine.profile_read() if n.startswith("conv")]
+    assert all(("mfma" in n) == (kernel == "mfma") or n.endswith("x3s7") for n in names), names
+    for i, f in enumerate(cfg.frames):
+        want = pick(o_mesh, f["Hoc"]).classify(f["Hoc"], o_lens, f["image"], cfg.fourcc, vmo.Network(cfg.network))
+        assert_classification_parity(results[i], want, PROB_TOL, "%s frame %d" % (kernel, i))

@@ -47,7 +47,7 @@ def _headers():
     out = [os.path.join(INCLUDE, "visualmesh_hip.h")]
     for d in (CSRC, CPP):
         for base, _, files in os.walk(d):
-            out += [os.path.join(base, f) for f in files if f.endswith((".h", ".hpp"))]
+            out += [os.path.join(base, f) for f in files if f.endswith((".h", ".hpp", ".inc"))]
     return out
 
 
@@ -60,6 +60,7 @@ def build_hip(force=False):
         # project.hip reproduces the reference's operation order: no FMA contraction in that file
         ("project.hip", HIP_FLAGS + ["-ffp-contract=off"]),
         ("conv.hip", HIP_FLAGS),
+        ("conv_mfma.hip", HIP_FLAGS),
         ("api.hip", HIP_FLAGS),
     ]
     for name, flags in units:

@@ -4,6 +4,7 @@
  */
 #include <algorithm>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <string>
 #include <vector>
@@ -99,6 +100,7 @@ struct HostLayer {
     int32_t c_in, c_out, slots, activation;
     float* d_w = nullptr;
     float* d_b = nullptr;
+    float* d_w_mfma = nullptr;
 };
 
 struct vmhip_engine {
@@ -362,11 +364,13 @@ int batch_enqueue(vmhip_batch* b) {
     int cur = 0;
     if (b->classify) {
         for (const HostLayer& L : E->layers) {
-            VmLayerDev ld{L.c_in, L.c_out, L.slots, L.activation, L.d_w, L.d_b};
+            VmLayerDev ld{L.c_in, L.c_out, L.slots, L.activation, L.d_w, L.d_b, L.d_w_mfma};
             const char* name = "conv";
             HIP_TRY(P.begin());
-            const int rc = vm_launch_conv(D, ld, b->d_act[cur].as<float>(), b->d_act[cur ^ 1].as<float>(), s, &name);
-            if (rc != 0) return fail(rc, "unsupported layer shape");
+            int rc = -1;
+            if (L.d_w_mfma) rc = vm_launch_conv_mfma(D, ld, b->d_act[cur].as<float>(), b->d_act[cur ^ 1].as<float>(), s, &name);
+            if (rc != 0) rc = vm_launch_conv(D, ld, b->d_act[cur].as<float>(), b->d_act[cur ^ 1].as<float>(), s, &name);
+            if (rc != 0) return fail(VMHIP_ERR_ARGUMENT, "unsupported layer shape");
             HIP_TRY(P.end(name, rows));
             cur ^= 1;
         }
@@ -525,13 +529,25 @@ int vmhip_engine_create(const vmhip_network* net, int32_t n_neighbours, int32_t 
                 return bail(VMHIP_ERR_ARGUMENT, "engine_create: layer " + std::to_string(li) + " expects " + std::to_string(slots * width)
                                                   + " inputs, has " + std::to_string(L.n_in));
             if (L.activation < VMHIP_SELU || L.activation > VMHIP_TANH) return bail(VMHIP_ERR_ARGUMENT, "engine_create: unknown activation");
-            HostLayer H{width, L.n_out, slots, L.activation, nullptr, nullptr};
+            HostLayer H{width, L.n_out, slots, L.activation, nullptr, nullptr, nullptr};
             if (hipMalloc(&H.d_w, 4 * size_t(L.n_in) * L.n_out) != hipSuccess || hipMalloc(&H.d_b, 4 * size_t(L.n_out)) != hipSuccess)
                 return bail(VMHIP_ERR_HIP, "engine_create: out of device memory");
             E->layers.push_back(H);
             if (hipMemcpy(H.d_w, L.weights, 4 * size_t(L.n_in) * L.n_out, hipMemcpyHostToDevice) != hipSuccess
                 || hipMemcpy(H.d_b, L.biases, 4 * size_t(L.n_out), hipMemcpyHostToDevice) != hipSuccess)
                 return bail(VMHIP_ERR_HIP, "engine_create: weight upload failed");
+            /* VMHIP_CONV_KERNEL=rows keeps every layer on the one-row-per-lane kernel (for A/B timing) */
+            const char* pick = getenv("VMHIP_CONV_KERNEL");
+            const bool rows_only = pick && std::string(pick) == "rows";
+            if (!rows_only && precision == VMHIP_FP32 && vm_mfma_supported(width, L.n_out, slots)) {
+                std::vector<float> wp(vm_mfma_weight_floats(width, L.n_out, slots));
+                vm_mfma_permute_weights(L.weights, width, L.n_out, slots, wp.data());
+                float* d = nullptr;
+                if (hipMalloc(&d, 4 * wp.size()) != hipSuccess) return bail(VMHIP_ERR_HIP, "engine_create: out of device memory");
+                E->layers.back().d_w_mfma = d;
+                if (hipMemcpy(d, wp.data(), 4 * wp.size(), hipMemcpyHostToDevice) != hipSuccess)
+                    return bail(VMHIP_ERR_HIP, "engine_create: weight upload failed");
+            }
             width = L.n_out;
             E->max_width = std::max(E->max_width, width);
         }
@@ -548,6 +564,7 @@ void vmhip_engine_destroy(vmhip_engine* E) {
     for (HostLayer& L : E->layers) {
         if (L.d_w) (void) hipFree(L.d_w);
         if (L.d_b) (void) hipFree(L.d_b);
+        if (L.d_w_mfma) (void) hipFree(L.d_w_mfma);
     }
     if (E->stream) (void) hipStreamDestroy(E->stream);
     delete E;

@@ -94,6 +94,7 @@ struct VmLayerDev {
     int32_t activation;
     const float* w;  /* [slots*c_in][c_out] fp32 row major */
     const float* b;  /* [c_out] */
+    const float* w_mfma; /* the same weights in the matrix-core kernel's consumption order, or null */
 };
 
 /* launchers, one per kernel; all asynchronous on `stream` */
@@ -106,6 +107,13 @@ void vm_launch_neighbourhood(const VmBatchDev& B, hipStream_t stream);
 /* in -> out over the row space; returns 0 or a negative status if the shape is unsupported */
 int vm_launch_conv(const VmBatchDev& B, const VmLayerDev& L, const float* in, float* out, hipStream_t stream,
                    const char** kernel_name);
+
+/* matrix-core variant (conv_mfma.hip); launch returns a negative value if the shape has no instantiation */
+bool vm_mfma_supported(int c_in, int c_out, int slots);
+size_t vm_mfma_weight_floats(int c_in, int c_out, int slots);
+void vm_mfma_permute_weights(const float* w, int c_in, int c_out, int slots, float* wp);
+int vm_launch_conv_mfma(const VmBatchDev& B, const VmLayerDev& L, const float* in, float* out, hipStream_t stream,
+                        const char** kernel_name);
 
 #include "host_project.h"
 

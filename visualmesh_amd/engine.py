@@ -196,6 +196,8 @@ class Engine:
         return C.c_void_p(self._lib.vmh_engine_native_batch(self.ptr))
 
     def profile(self, enable=True):
+        if not self.native_batch():
+            return  # nothing staged yet: profiling is switched on per batch object
         native.hip_check(native.hip().vmhip_batch_profile(self.native_batch(), 1 if enable else 0))
 
     def profile_read(self):
