@@ -20,6 +20,8 @@
  * rows a tile gathers - which lie in nearby tiles, mesh order being spatially coherent - are found in the
  * same L2 instead of being fetched by every XCD.
  */
+#include <cstdlib>
+
 #include "vmhip_internal.h"
 
 namespace {
@@ -129,22 +131,23 @@ __global__ __launch_bounds__(NW * 64) void vm_conv_mfma_kernel(VmBatchDev B, VmL
         const int V = B.frame_V[f];
         const int wave_row0 = (tile - F.row_tile0) * VMHIP_TILE + wave * (RB * 16);
         if (wave_row0 > V) continue; /* whole wave beyond the null row (wave-uniform) */
-        const size_t base = (size_t) F.row_base;
+        const uint32_t base = (uint32_t) F.row_base;
 
-        /* source rows of this lane's rows: slot 0 is the row itself */
-        size_t src[RB][SLOTS];
+        /* source rows of this lane's rows: slot 0 is the row itself. Lanes past the null row compute on the
+         * null row's data (always valid memory, branch-free) and skip the store. */
+        uint32_t src[RB][SLOTS]; /* row numbers in the batch's row space */
         bool valid[RB];
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb) {
             const int i = wave_row0 + rb * 16 + r16;
             valid[rb] = i <= V;
-            const size_t row = base + i;
+            const uint32_t row = base + (uint32_t) min(i, V);
             src[rb][0] = row;
             if constexpr (NN > 0) {
                 int nb[NN];
-                if (valid[rb]) load_run<NN>(B.row_nb + row * B.nb_stride, nb);
+                load_run<NN>(B.row_nb + (size_t) row * B.nb_stride, nb);
 #pragma unroll
-                for (int s = 0; s < NN; ++s) src[rb][s + 1] = valid[rb] ? base + nb[s] : row;
+                for (int s = 0; s < NN; ++s) src[rb][s + 1] = base + (uint32_t) nb[s];
             }
         }
 
@@ -156,15 +159,18 @@ __global__ __launch_bounds__(NW * 64) void vm_conv_mfma_kernel(VmBatchDev B, VmL
 
         float x[2][RB][KQ];
 #pragma unroll
-        for (int rb = 0; rb < RB; ++rb) load_run<KQ>(in + src[rb][0] * C_IN + q * KQ, x[0][rb]);
+        for (int rb = 0; rb < RB; ++rb) load_run<KQ>(in + (size_t) src[rb][0] * C_IN + q * KQ, x[0][rb]);
 
 #pragma unroll
         for (int s = 0; s < SLOTS; ++s) {
             const int cur = s & 1;
             if (s + 1 < SLOTS) {
 #pragma unroll
-                for (int rb = 0; rb < RB; ++rb) load_run<KQ>(in + src[rb][s + 1] * C_IN + q * KQ, x[cur ^ 1][rb]);
+                for (int rb = 0; rb < RB; ++rb) load_run<KQ>(in + (size_t) src[rb][s + 1] * C_IN + q * KQ, x[cur ^ 1][rb]);
             }
+            /* keep the next slot's gathers ahead of this slot's matrix instructions: without the fence the
+             * scheduler sinks each load next to its first use and every slot stalls on memory latency */
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int j = 0; j < KQ; ++j) {
 #pragma unroll
@@ -208,7 +214,7 @@ __global__ __launch_bounds__(NW * 64) void vm_conv_mfma_kernel(VmBatchDev B, VmL
                     }
             }
             if (valid[rb]) {
-                float* __restrict__ y = out + src[rb][0] * C_OUT;
+                float* __restrict__ y = out + (size_t) src[rb][0] * C_OUT; /* valid => src[rb][0] is the lane's own row */
 #pragma unroll
                 for (int cb = 0; cb < CB; ++cb) {
                     const int o = cb * 16 + q * 4;
@@ -242,6 +248,7 @@ int launch_mfma(const VmBatchDev& B, const VmLayerDev& L, const float* in, float
     /* blocks per CU limited by LDS (160 KB per CU) and registers; 8 XCDs x 32 CUs */
     int per_cu = int((160 * 1024) / (lds + 512));
     per_cu = per_cu < 1 ? 1 : per_cu > (NW == 4 ? 3 : 2) ? (NW == 4 ? 3 : 2) : per_cu;
+    if (const char* e = getenv("VMHIP_MFMA_BLOCKS_PER_CU")) per_cu = atoi(e) > 0 ? atoi(e) : per_cu;
     int grid = 256 * per_cu;
     const int need = ((B.n_row_tiles + 7) / 8) * 8;
     if (grid > need) grid = need;
@@ -252,7 +259,7 @@ int launch_mfma(const VmBatchDev& B, const VmLayerDev& L, const float* in, float
 template <int C_IN, int C_OUT, int SLOTS>
 int launch_pick(const VmBatchDev& B, const VmLayerDev& L, const float* in, float* out, hipStream_t stream) {
     /* wide layers: 8 waves x 2 row blocks keep the accumulators and the double-buffered inputs in registers */
-    if constexpr (C_IN * C_OUT >= 4096) return launch_mfma<C_IN, C_OUT, SLOTS, 8, 2>(B, L, in, out, stream);
+    if constexpr (C_IN * C_OUT >= 1024) return launch_mfma<C_IN, C_OUT, SLOTS, 8, 2>(B, L, in, out, stream);
     else return launch_mfma<C_IN, C_OUT, SLOTS, 4, 4>(B, L, in, out, stream);
 }
 
