@@ -10,10 +10,14 @@
  *   D:         lane l holds out channels 4 * (l / 16) + {0,1,2,3} of row l % 16   -> one 16-byte store per lane
  * The reduction index is free to be permuted as long as both operands agree, so lane group q = l / 16 takes
  * the q-th quarter of every gathered row: a lane's inputs for one gather slot are C_IN / 4 consecutive floats
- * of one source row, loaded straight from global memory into registers with 16-byte loads (no staging), and
- * MFMA step j of slot s uses element j of that run. The weights are stored once, in exactly the order the
- * lanes consume them ([slot][j][column block][lane]), and live in LDS for the life of a block; one LDS read
- * feeds RB MFMAs (RB row blocks per wave).
+ * of one source row, and MFMA step j of slot s uses element j of that run. The weights are stored once, in
+ * exactly the order the lanes consume them ([slot][j][column block][lane]), and live in LDS for the life of a
+ * block; one LDS read feeds RB MFMAs (RB row blocks per wave).
+ *
+ * The gathered rows go straight from global memory into registers in operand layout (16-byte loads, no
+ * staging). Mesh order is spatially coherent (about 88 % of a row's neighbours lie in the same 256-row tile),
+ * so after the XCD-aware tile walk below nearly all of these loads hit in L1/L2 and the HBM traffic is the
+ * algorithmic minimum; what the loads still cost is issue slots next to the matrix instructions.
  *
  * Blocks are persistent and XCD aware: hardware deals consecutive workgroups round-robin to the 8 XCDs, each
  * with its own L2. Block b therefore walks a contiguous eighth of the tiles (xcd = b % 8), so the neighbour
@@ -89,7 +93,16 @@ __device__ __forceinline__ void load_run(const int32_t* __restrict__ p, int (&v)
     }
 }
 
-/* NW waves per block, RB row blocks of 16 rows per wave: NW * RB * 16 == VMHIP_TILE */
+/* Gather-from-global variant. NW waves per block, RB row blocks of 16 rows per wave: NW * RB * 16 == VMHIP_TILE.
+ *
+ * Each wave walks its tiles with a software pipeline, because the per-tile chain "which frame -> how many rows
+ * -> neighbour table -> source rows" is four dependent memory round trips and the waves that share a SIMD tend
+ * to run in lockstep (the matrix pipe is served round-robin), so a chain left in the open idles the pipe for
+ * every wave at once:
+ *   - the frame lookup and the neighbour-table loads of tile t+1 are issued before the matrix work of tile t;
+ *   - the slot-0 rows of tile t+1 are requested during the last slot of tile t, ahead of tile t's epilogue;
+ *   - inside a tile, slot s+1's rows are requested before slot s's matrix instructions (fenced so the
+ *     scheduler cannot sink the loads back next to their uses). */
 template <int C_IN, int C_OUT, int SLOTS, int NW, int RB>
 __global__ __launch_bounds__(NW * 64) void vm_conv_mfma_kernel(VmBatchDev B, VmLayerDev L, const float* __restrict__ in,
                                                                float* __restrict__ out) {
@@ -98,6 +111,7 @@ __global__ __launch_bounds__(NW * 64) void vm_conv_mfma_kernel(VmBatchDev B, VmL
     constexpr int KQ = C_IN / 4;              /* floats per lane per slot */
     constexpr int CB = (C_OUT + 15) / 16;     /* column blocks of 16 output channels */
     constexpr int NN = SLOTS - 1;
+    constexpr int NBV = NN > 0 ? NN : 1;
     constexpr int W_FLOATS = SLOTS * KQ * CB * 64;
 
     extern __shared__ float w_lds[];
@@ -108,8 +122,8 @@ __global__ __launch_bounds__(NW * 64) void vm_conv_mfma_kernel(VmBatchDev B, VmL
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int q = lane >> 4;   /* quarter of the gathered row / group of 4 output channels */
     const int r16 = lane & 15; /* row within a row block / output channel within a column block */
+    const int activation = L.activation;
 
-    /* bias of this lane's output channels */
     v4f bias[CB];
 #pragma unroll
     for (int cb = 0; cb < CB; ++cb) {
@@ -125,31 +139,67 @@ __global__ __launch_bounds__(NW * 64) void vm_conv_mfma_kernel(VmBatchDev B, VmL
     const int xcd = blockIdx.x & 7, lb = blockIdx.x >> 3, gx = gridDim.x >> 3;
     const int per_xcd = (n_tiles + 7) >> 3;
     const int t_end = min(n_tiles, (xcd + 1) * per_xcd);
-    for (int tile = xcd * per_xcd + lb; tile < t_end; tile += gx) {
+
+    /* wave-uniform description of a tile: the frame's first row, its visible count, the wave's first row */
+    struct Info {
+        uint32_t base;
+        int V;
+        int row0;
+    };
+    auto describe = [&](int tile) {
         const int f = find_frame_by_row_tile(B.frames, B.n_frames, tile);
         const VmFrame& F = B.frames[f];
-        const int V = B.frame_V[f];
-        const int wave_row0 = (tile - F.row_tile0) * VMHIP_TILE + wave * (RB * 16);
-        if (wave_row0 > V) continue; /* whole wave beyond the null row (wave-uniform) */
-        const uint32_t base = (uint32_t) F.row_base;
-
-        /* source rows of this lane's rows: slot 0 is the row itself. Lanes past the null row compute on the
-         * null row's data (always valid memory, branch-free) and skip the store. */
-        uint32_t src[RB][SLOTS]; /* row numbers in the batch's row space */
-        bool valid[RB];
+        Info t;
+        t.base = (uint32_t) F.row_base;
+        t.V = B.frame_V[f];
+        t.row0 = (tile - F.row_tile0) * VMHIP_TILE + wave * (RB * 16);
+        return t;
+    };
+    /* the lane's rows of a tile, clamped to the null row (lanes past it compute on its data and skip the store) */
+    auto request_neighbours = [&](const Info& t, int (&nb)[RB][NBV]) {
+        if constexpr (NN > 0) {
 #pragma unroll
-        for (int rb = 0; rb < RB; ++rb) {
-            const int i = wave_row0 + rb * 16 + r16;
-            valid[rb] = i <= V;
-            const uint32_t row = base + (uint32_t) min(i, V);
-            src[rb][0] = row;
-            if constexpr (NN > 0) {
-                int nb[NN];
-                load_run<NN>(B.row_nb + (size_t) row * B.nb_stride, nb);
-#pragma unroll
-                for (int s = 0; s < NN; ++s) src[rb][s + 1] = base + (uint32_t) nb[s];
+            for (int rb = 0; rb < RB; ++rb) {
+                const uint32_t row = t.base + (uint32_t) max(0, min(t.row0 + rb * 16 + r16, t.V));
+                load_run<NN>(B.row_nb + (size_t) row * B.nb_stride, nb[rb]);
             }
         }
+    };
+    auto resolve = [&](const Info& t, const int (&nb)[RB][NBV], uint32_t (&src)[RB][SLOTS], bool (&valid)[RB]) {
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+            const int i = t.row0 + rb * 16 + r16;
+            valid[rb] = i <= t.V;
+            src[rb][0] = t.base + (uint32_t) max(0, min(i, t.V));
+#pragma unroll
+            for (int s = 0; s < NN; ++s) src[rb][s + 1] = t.base + (uint32_t) nb[rb][s];
+        }
+    };
+
+    int tile = xcd * per_xcd + lb;
+    if (tile >= t_end) return;
+
+    Info cur = describe(tile);
+    int nb[RB][NBV];
+    request_neighbours(cur, nb);
+    uint32_t src[RB][SLOTS];
+    bool valid[RB];
+    resolve(cur, nb, src, valid);
+    float x[2][RB][KQ];
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) load_run<KQ>(in + (size_t) src[rb][0] * C_IN + q * KQ, x[0][rb]);
+
+    int next = tile + gx;
+    Info nxt = cur;
+    if (next < t_end) {
+        nxt = describe(next);
+        request_neighbours(nxt, nb);
+    }
+
+    while (true) {
+        const bool has_next = next < t_end;
+        uint32_t src_next[RB][SLOTS];
+        bool valid_next[RB];
 
         v4f acc[RB][CB];
 #pragma unroll
@@ -157,19 +207,19 @@ __global__ __launch_bounds__(NW * 64) void vm_conv_mfma_kernel(VmBatchDev B, VmL
 #pragma unroll
             for (int cb = 0; cb < CB; ++cb) acc[rb][cb] = bias[cb];
 
-        float x[2][RB][KQ];
-#pragma unroll
-        for (int rb = 0; rb < RB; ++rb) load_run<KQ>(in + (size_t) src[rb][0] * C_IN + q * KQ, x[0][rb]);
-
 #pragma unroll
         for (int s = 0; s < SLOTS; ++s) {
-            const int cur = s & 1;
+            const int cur_buf = s & 1;
             if (s + 1 < SLOTS) {
 #pragma unroll
-                for (int rb = 0; rb < RB; ++rb) load_run<KQ>(in + (size_t) src[rb][s + 1] * C_IN + q * KQ, x[cur ^ 1][rb]);
+                for (int rb = 0; rb < RB; ++rb) load_run<KQ>(in + (size_t) src[rb][s + 1] * C_IN + q * KQ, x[cur_buf ^ 1][rb]);
             }
-            /* keep the next slot's gathers ahead of this slot's matrix instructions: without the fence the
-             * scheduler sinks each load next to its first use and every slot stalls on memory latency */
+            else if (has_next) {
+                /* last slot: the other buffer is free; fill it with the next tile's slot 0 */
+                resolve(nxt, nb, src_next, valid_next);
+#pragma unroll
+                for (int rb = 0; rb < RB; ++rb) load_run<KQ>(in + (size_t) src_next[rb][0] * C_IN + q * KQ, x[cur_buf ^ 1][rb]);
+            }
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int j = 0; j < KQ; ++j) {
@@ -178,15 +228,24 @@ __global__ __launch_bounds__(NW * 64) void vm_conv_mfma_kernel(VmBatchDev B, VmL
                     const float a = w_lds[((s * KQ + j) * CB + cb) * 64 + lane];
 #pragma unroll
                     for (int rb = 0; rb < RB; ++rb)
-                        acc[rb][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, x[cur][rb][j], acc[rb][cb], 0, 0, 0);
+                        acc[rb][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, x[cur_buf][rb][j], acc[rb][cb], 0, 0, 0);
                 }
             }
         }
 
+        /* look one more tile ahead before the epilogue: frame lookup + neighbour table of tile t+2 */
+        const int after = next + gx;
+        Info nxt2 = nxt;
+        if (has_next && after < t_end) {
+            nxt2 = describe(after);
+            request_neighbours(nxt2, nb);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+
         /* activation and store: lane holds channels cb*16 + q*4 + {0..3} of row rb*16 + r16 */
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb) {
-            if (L.activation == VMHIP_SOFTMAX) {
+            if (activation == VMHIP_SOFTMAX) {
                 float sum = 0.0f;
 #pragma unroll
                 for (int cb = 0; cb < CB; ++cb)
@@ -210,7 +269,7 @@ __global__ __launch_bounds__(NW * 64) void vm_conv_mfma_kernel(VmBatchDev B, VmL
 #pragma unroll
                     for (int v = 0; v < 4; ++v) {
                         const float a = acc[rb][cb][v];
-                        acc[rb][cb][v] = L.activation == VMHIP_SELU ? selu(a) : L.activation == VMHIP_RELU ? fmaxf(a, 0.0f) : tanhf(a);
+                        acc[rb][cb][v] = activation == VMHIP_SELU ? selu(a) : activation == VMHIP_RELU ? fmaxf(a, 0.0f) : tanhf(a);
                     }
             }
             if (valid[rb]) {
@@ -229,8 +288,26 @@ __global__ __launch_bounds__(NW * 64) void vm_conv_mfma_kernel(VmBatchDev B, VmL
                 }
             }
         }
+
+        if (!has_next) break;
+        /* rotate: the next tile becomes current; its slot 0 sits in the buffer the last slot left free */
+        constexpr int LAST = (SLOTS - 1) & 1;
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+            valid[rb] = valid_next[rb];
+#pragma unroll
+            for (int s = 0; s < SLOTS; ++s) src[rb][s] = src_next[rb][s];
+            if (LAST == 0) {
+#pragma unroll
+                for (int j = 0; j < KQ; ++j) x[0][rb][j] = x[1][rb][j];
+            }
+        }
+        tile = next;
+        next = after;
+        nxt = nxt2;
     }
 }
+
 
 template <int C_IN, int C_OUT, int SLOTS, int NW, int RB>
 int launch_mfma(const VmBatchDev& B, const VmLayerDev& L, const float* in, float* out, hipStream_t stream) {
@@ -258,9 +335,9 @@ int launch_mfma(const VmBatchDev& B, const VmLayerDev& L, const float* in, float
 
 template <int C_IN, int C_OUT, int SLOTS>
 int launch_pick(const VmBatchDev& B, const VmLayerDev& L, const float* in, float* out, hipStream_t stream) {
-    /* wide layers: 8 waves x 2 row blocks keep the accumulators and the double-buffered inputs in registers */
-    if constexpr (C_IN * C_OUT >= 1024) return launch_mfma<C_IN, C_OUT, SLOTS, 8, 2>(B, L, in, out, stream);
-    else return launch_mfma<C_IN, C_OUT, SLOTS, 4, 4>(B, L, in, out, stream);
+    /* 8 waves x 2 row blocks: 16 accumulator registers and two 16-register input buffers per lane leave room
+     * for four waves per SIMD on the 32-wide layers */
+    return launch_mfma<C_IN, C_OUT, SLOTS, 8, 2>(B, L, in, out, stream);
 }
 
 }  // namespace
