@@ -150,14 +150,19 @@ def main():
         c_in, rest = shape.split("x")
         c_out, slots = rest.split("s")
         c_in, c_out, slots = int(c_in), int(c_out), int(slots)
-        s_act = 4
-        bytes_per_row = c_in * s_act + 4 * (slots - 1) + c_out * s_act
+        # storage and arithmetic are in the kernel name too (conv_bf16x2*: bf16 rows in, conv_*_tobf16: bf16 rows
+        # out, conv_bf16*: bf16 matrix instructions); flops are the layer's algorithmic ones, not the hi/lo extras
+        bf16_arith = dominant.startswith("conv_bf16")
+        s_in = 2 if dominant.startswith("conv_bf16x2") else 4
+        s_out = 2 if "_tobf16_" in dominant else (4 if not dominant.startswith("conv_bf16x2") or "_tof32_" in dominant else 2)
+        bytes_per_row = c_in * s_in + 4 * (slots - 1) + c_out * s_out
         flops_per_row = 2 * slots * c_in * c_out
         intensity = flops_per_row / bytes_per_row
-        ridge = FP32_PEAK_TFLOPS * 1e12 / (HBM_PEAK_GBS * 1e9)
+        matrix_peak = BF16_PEAK_TFLOPS if bf16_arith else FP32_PEAK_TFLOPS
+        ridge = matrix_peak * 1e12 / (HBM_PEAK_GBS * 1e9)
         if intensity > ridge:
             achieved = flops_per_row * rows / (avg_ms * 1e-3) / 1e12
-            roofline = dict(bound="mfma", achieved=achieved, peak=FP32_PEAK_TFLOPS, unit="TFLOP/s", frac=achieved / FP32_PEAK_TFLOPS)
+            roofline = dict(bound="mfma", achieved=achieved, peak=matrix_peak, unit="TFLOP/s", frac=achieved / matrix_peak)
         else:
             achieved = bytes_per_row * rows / (avg_ms * 1e-3) / 1e9
             roofline = dict(bound="hbm", achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s", frac=achieved / HBM_PEAK_GBS)

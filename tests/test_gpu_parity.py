@@ -4,9 +4,10 @@ through the C ABI. Gates: visible-node indices and neighbour tables bit-exact, p
 import numpy as np
 import pytest
 
-from helpers import (PROB_TOL, assert_classification_parity, assert_projection_parity, lens_pair, meshes_for, pick)
+from helpers import (BF16_TOL, PROB_TOL, assert_classification_parity, assert_projection_parity, lens_pair, meshes_for, pick)
 from oracle import vmo
 from visualmesh_amd import engine as eng
+from visualmesh_amd import native
 from visualmesh_amd import workloads as wl
 
 pytestmark = pytest.mark.gpu
@@ -127,6 +128,61 @@ def test_config4_network_on_config1_geometry(oracle):
     for i, f in enumerate(cfg.frames):
         want = o_mesh.classify(f["Hoc"], o_lens, f["image"], cfg.fourcc, vmo.Network(net))
         assert_classification_parity(results[i], want, PROB_TOL, "64-wide frame %d" % i)
+
+
+def test_config4_and_5_full_size_frame(oracle):
+    """One frame of configurations 4 and 5 at their real size (2048x1536, ~4.5e5 visible nodes, 6 x 64 network):
+    the fp32 engine within 1e-4 and the bf16 engine within 1e-2 of the same oracle result (~45 s of CPU)."""
+    cfg = wl.config(4, n_frames=1)
+    o_lens, e_lens = lens_pair(cfg)
+    o_mesh, e_mesh = meshes_for(cfg, oracle)
+    f = cfg.frames[0]
+    print("cfg4/5 full-size frame: oracle running", flush=True)
+    want = o_mesh.classify(f["Hoc"], o_lens, f["image"], cfg.fourcc, vmo.Network(cfg.network))
+    print("cfg4/5 full-size frame: V =", len(want["gidx"]), flush=True)
+    for precision, tol, label in ((native.FP32, PROB_TOL, "cfg4 fp32"), (native.BF16, BF16_TOL, "cfg5 bf16")):
+        engine = eng.Engine(cfg.network, cfg.model, precision=precision)
+        got = engine(e_mesh, f["Hoc"], e_lens, f["image"], cfg.fourcc)
+        print(label, "worst absolute probability error: %.3e" % float(np.abs(got["cls"] - want["cls"]).max()), flush=True)
+        assert_classification_parity(got, want, tol, label)
+
+
+def test_bf16_engine(oracle):
+    """The bf16 engine (configuration 5's precision and 6 x 64 network) against the fp32 oracle on configuration
+    1's geometry: geometry bit-exact, probabilities within 1e-2. The kernel names prove that the bf16
+    matrix-instruction kernels were the ones that ran, the error that bf16 rows were really stored."""
+    cfg = wl.config(1, n_frames=2)
+    net = wl.config(5, n_frames=1).network
+    o_lens, e_lens = lens_pair(cfg)
+    o_mesh, e_mesh = meshes_for(cfg, oracle)
+    engine = eng.Engine(net, cfg.model, precision=native.BF16)
+    frames = [dict(mesh=e_mesh, Hoc=f["Hoc"], lens=e_lens, image=f["image"], fourcc=cfg.fourcc) for f in cfg.frames]
+    results = engine.classify_batch(frames)
+    engine.profile(True)
+    engine.run()
+    names = [n for n, _, _ in engine.profile_read() if n.startswith("conv")]
+    assert names == ["conv_mfma_4x64s7", "conv_bf16x3_tobf16_64x64s7", "conv_bf16x2_tof32_64x64s7", "conv_bf16x3_tobf16_64x64s7",
+                     "conv_bf16x2_tof32_64x64s7", "conv_bf16x3_64x64s7"], names
+    worst = 0.0
+    for i, f in enumerate(cfg.frames):
+        want = o_mesh.classify(f["Hoc"], o_lens, f["image"], cfg.fourcc, vmo.Network(net))
+        assert_classification_parity(results[i], want, BF16_TOL, "bf16 frame %d" % i)
+        worst = max(worst, float(np.abs(results[i]["cls"] - want["cls"]).max()))
+    print("bf16 worst absolute probability error: %.3e" % worst, flush=True)
+    assert worst > PROB_TOL  # two boundaries are stored as bf16: an error this small would mean they were not
+
+
+def test_bf16_engine_keeps_narrow_networks_in_fp32(oracle):
+    """Rows narrower than 64 channels are not worth bf16 storage (one rounding already costs ~1e-2 on a 3-class
+    softmax): a bf16 engine built on configuration 2's network meets the fp32 gate."""
+    cfg = wl.config(2, n_frames=1)
+    o_lens, e_lens = lens_pair(cfg)
+    o_mesh, e_mesh = meshes_for(cfg, oracle)
+    engine = eng.Engine(cfg.network, cfg.model, precision=native.BF16)
+    f = cfg.frames[0]
+    got = engine(e_mesh, f["Hoc"], e_lens, f["image"], cfg.fourcc)
+    want = pick(o_mesh, f["Hoc"]).classify(f["Hoc"], o_lens, f["image"], cfg.fourcc, vmo.Network(cfg.network))
+    assert_classification_parity(got, want, PROB_TOL, "bf16 engine, narrow network")
 
 
 @pytest.mark.parametrize("kernel", ["rows", "mfma"])

@@ -100,7 +100,9 @@ struct HostLayer {
     int32_t c_in, c_out, slots, activation;
     float* d_w = nullptr;
     float* d_b = nullptr;
-    float* d_w_mfma = nullptr;
+    void* d_w_mfma = nullptr;
+    int32_t in_bf16 = 0, out_bf16 = 0, arith_bf16 = 0;
+    std::vector<float> h_w; /* kept until the row types are planned */
 };
 
 struct vmhip_engine {
@@ -364,13 +366,14 @@ int batch_enqueue(vmhip_batch* b) {
     int cur = 0;
     if (b->classify) {
         for (const HostLayer& L : E->layers) {
-            VmLayerDev ld{L.c_in, L.c_out, L.slots, L.activation, L.d_w, L.d_b, L.d_w_mfma};
+            VmLayerDev ld{L.c_in, L.c_out, L.slots, L.activation, L.d_w, L.d_b, L.d_w_mfma, L.in_bf16, L.out_bf16, L.arith_bf16};
             const char* name = "conv";
             HIP_TRY(P.begin());
             int rc = -1;
-            if (L.d_w_mfma) rc = vm_launch_conv_mfma(D, ld, b->d_act[cur].as<float>(), b->d_act[cur ^ 1].as<float>(), s, &name);
-            if (rc != 0) rc = vm_launch_conv(D, ld, b->d_act[cur].as<float>(), b->d_act[cur ^ 1].as<float>(), s, &name);
-            if (rc != 0) return fail(VMHIP_ERR_ARGUMENT, "unsupported layer shape");
+            if (L.d_w_mfma) rc = vm_launch_conv_mfma(D, ld, b->d_act[cur].p, b->d_act[cur ^ 1].p, s, &name);
+            /* the one-row-per-lane kernels only know fp32 rows */
+            if (rc != 0 && !L.in_bf16 && !L.out_bf16) rc = vm_launch_conv(D, ld, b->d_act[cur].as<float>(), b->d_act[cur ^ 1].as<float>(), s, &name);
+            if (rc != 0) return fail(VMHIP_ERR_HIP, "no kernel could be launched for a layer");
             HIP_TRY(P.end(name, rows));
             cur ^= 1;
         }
@@ -529,30 +532,70 @@ int vmhip_engine_create(const vmhip_network* net, int32_t n_neighbours, int32_t 
                 return bail(VMHIP_ERR_ARGUMENT, "engine_create: layer " + std::to_string(li) + " expects " + std::to_string(slots * width)
                                                   + " inputs, has " + std::to_string(L.n_in));
             if (L.activation < VMHIP_SELU || L.activation > VMHIP_TANH) return bail(VMHIP_ERR_ARGUMENT, "engine_create: unknown activation");
-            HostLayer H{width, L.n_out, slots, L.activation, nullptr, nullptr, nullptr};
+            HostLayer H;
+            H.c_in = width, H.c_out = L.n_out, H.slots = slots, H.activation = L.activation;
+            H.h_w.assign(L.weights, L.weights + size_t(L.n_in) * L.n_out);
             if (hipMalloc(&H.d_w, 4 * size_t(L.n_in) * L.n_out) != hipSuccess || hipMalloc(&H.d_b, 4 * size_t(L.n_out)) != hipSuccess)
                 return bail(VMHIP_ERR_HIP, "engine_create: out of device memory");
             E->layers.push_back(H);
             if (hipMemcpy(H.d_w, L.weights, 4 * size_t(L.n_in) * L.n_out, hipMemcpyHostToDevice) != hipSuccess
                 || hipMemcpy(H.d_b, L.biases, 4 * size_t(L.n_out), hipMemcpyHostToDevice) != hipSuccess)
                 return bail(VMHIP_ERR_HIP, "engine_create: weight upload failed");
-            /* VMHIP_CONV_KERNEL=rows keeps every layer on the one-row-per-lane kernel (for A/B timing) */
-            const char* pick = getenv("VMHIP_CONV_KERNEL");
-            const bool rows_only = pick && std::string(pick) == "rows";
-            if (!rows_only && precision == VMHIP_FP32 && vm_mfma_supported(width, L.n_out, slots)) {
-                std::vector<float> wp(vm_mfma_weight_floats(width, L.n_out, slots));
-                vm_mfma_permute_weights(L.weights, width, L.n_out, slots, wp.data());
-                float* d = nullptr;
-                if (hipMalloc(&d, 4 * wp.size()) != hipSuccess) return bail(VMHIP_ERR_HIP, "engine_create: out of device memory");
-                E->layers.back().d_w_mfma = d;
-                if (hipMemcpy(d, wp.data(), 4 * wp.size(), hipMemcpyHostToDevice) != hipSuccess)
-                    return bail(VMHIP_ERR_HIP, "engine_create: weight upload failed");
-            }
             width = L.n_out;
             E->max_width = std::max(E->max_width, width);
         }
     }
     E->n_classes = width;
+
+    /* Row types and arithmetic per layer. fp32 engine: everything fp32. bf16 engine: layers reading rows at
+     * least 64 wide run on the bf16 matrix instructions (fp32 accumulation, weights as hi + lo pairs of bf16).
+     * Such a layer reads either bf16 rows, which costs one bf16 rounding of its inputs against the fp32 result,
+     * or fp32 rows split into hi + lo in registers, which costs nothing measurable. Each rounding moves the
+     * final probabilities of a 6 x 64 network by up to ~4.6e-3, so to stay inside the 1e-2 gate with margin
+     * only every second eligible boundary is stored as bf16 (the 2nd, 4th, ...); the others stay fp32. A choice
+     * is only made where the kernels on both sides of the boundary exist for it. */
+    {
+        const char* pick = getenv("VMHIP_CONV_KERNEL"); /* "rows" keeps every layer on the one-row-per-lane kernel (A/B timing) */
+        const bool rows_only = pick && std::string(pick) == "rows";
+        const int n = int(E->layers.size());
+        std::vector<int> bf(n + 1, 0); /* bf[l] = rows entering layer l are bf16; bf[n] = final output (never) */
+        std::vector<int> ar(n, 0);     /* ar[l] = layer l uses the bf16 matrix instructions */
+        if (precision == VMHIP_BF16 && !rows_only) {
+            int eligible = 0;
+            for (int l = 0; l < n; ++l) ar[l] = (E->layers[l].c_in >= 64 && E->layers[l].c_in % 32 == 0) ? 1 : 0;
+            for (int l = 1; l < n; ++l)
+                if (ar[l] && (++eligible % 2) == 0) bf[l] = 1;
+        }
+        auto ok = [&](int l) {
+            const HostLayer& H = E->layers[l];
+            return vm_mfma_supported(H.c_in, H.c_out, H.slots, bf[l], bf[l + 1], ar[l]);
+        };
+        for (bool changed = true; changed;) {
+            changed = false;
+            for (int l = 0; l < n; ++l) {
+                if (ok(l) || (!bf[l] && !bf[l + 1] && !ar[l])) continue;
+                /* give up bf16 storage around the layer first, then its bf16 arithmetic */
+                if (bf[l] || bf[l + 1]) bf[l] = 0, bf[l + 1] = 0;
+                else ar[l] = 0;
+                bf[n] = 0;
+                changed = true;
+            }
+        }
+        auto arith = [&](int l) { return ar[l]; };
+        for (int l = 0; l < n; ++l) {
+            HostLayer& H = E->layers[l];
+            H.in_bf16 = bf[l], H.out_bf16 = bf[l + 1], H.arith_bf16 = arith(l);
+            if (!rows_only && vm_mfma_supported(H.c_in, H.c_out, H.slots, H.in_bf16, H.out_bf16, H.arith_bf16)) {
+                std::vector<unsigned char> wp(vm_mfma_weight_bytes(H.c_in, H.c_out, H.slots, H.arith_bf16));
+                vm_mfma_permute_weights(H.h_w.data(), H.c_in, H.c_out, H.slots, H.arith_bf16, wp.data());
+                if (hipMalloc(&H.d_w_mfma, wp.size()) != hipSuccess) return bail(VMHIP_ERR_HIP, "engine_create: out of device memory");
+                if (hipMemcpy(H.d_w_mfma, wp.data(), wp.size(), hipMemcpyHostToDevice) != hipSuccess)
+                    return bail(VMHIP_ERR_HIP, "engine_create: weight upload failed");
+            }
+            H.h_w.clear();
+            H.h_w.shrink_to_fit();
+        }
+    }
     if (hipStreamCreateWithFlags(&E->stream, hipStreamNonBlocking) != hipSuccess) return bail(VMHIP_ERR_HIP, "engine_create: stream creation failed");
     *out = E;
     return VMHIP_OK;

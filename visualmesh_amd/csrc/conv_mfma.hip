@@ -1,36 +1,53 @@
 /*
- * conv_mfma.hip - graph-convolution layers on the matrix cores of gfx950 (v_mfma_f32_16x16x4_f32, fp32 in,
- * fp32 accumulate): neighbour gather + dense + bias + activation in one kernel
- * (reference engine/cpu/engine.hpp:213-264, apply_activation.hpp:34-84).
+ * conv_mfma.hip - graph-convolution layers on the matrix cores of gfx950: neighbour gather + dense + bias +
+ * activation in one kernel (reference engine/cpu/engine.hpp:213-264, apply_activation.hpp:34-84).
  *
  * Shape of the contraction: out[row][o] = b[o] + sum_{s, c} in[src(row, s)][c] * W[s*C_IN + c][o].
- * One MFMA computes a 16 (output channels) x 16 (rows) block over 4 values of the reduction index:
+ * One MFMA computes a 16 (output channels) x 16 (rows) block over a few values of the reduction index:
  *   A operand: lane l supplies W[k(l / 16)][o = l % 16]
  *   B operand: lane l supplies in[src(row = l % 16)][k(l / 16)]
- *   D:         lane l holds out channels 4 * (l / 16) + {0,1,2,3} of row l % 16   -> one 16-byte store per lane
+ *   D:         lane l holds out channels 4 * (l / 16) + {0,1,2,3} of row l % 16   -> one vector store per lane
+ * Two arithmetics share the kernel:
+ *   fp32  v_mfma_f32_16x16x4_f32    one float per lane and step, 4 reduction values per instruction
+ *   bf16  v_mfma_f32_16x16x32_bf16  eight bf16 per lane and step, 32 reduction values, fp32 accumulation,
+ *         with the weights (and, for rows stored as fp32, the inputs) carried as hi + lo pairs of bf16
  * The reduction index is free to be permuted as long as both operands agree, so lane group q = l / 16 takes
- * the q-th quarter of every gathered row: a lane's inputs for one gather slot are C_IN / 4 consecutive floats
- * of one source row, and MFMA step j of slot s uses element j of that run. The weights are stored once, in
- * exactly the order the lanes consume them ([slot][j][column block][lane]), and live in LDS for the life of a
- * block; one LDS read feeds RB MFMAs (RB row blocks per wave).
+ * the q-th quarter of every gathered row: a lane's inputs for one gather slot are C_IN / 4 consecutive values
+ * of one source row, and step j of slot s uses the j-th register of that run. The weights are stored once, in
+ * exactly the order the lanes consume them ([slot][step][column block][lane]), and live in LDS for the life of
+ * a block; one LDS read feeds RB MFMAs (RB row blocks per wave).
+ *
+ * Activations may be stored as fp32 or bf16 independently of the arithmetic: the bf16 engine chooses per
+ * layer boundary, and only a boundary stored as bf16 costs accuracy.
  *
  * The gathered rows go straight from global memory into registers in operand layout (16-byte loads, no
  * staging). Mesh order is spatially coherent (about 88 % of a row's neighbours lie in the same 256-row tile),
- * so after the XCD-aware tile walk below nearly all of these loads hit in L1/L2 and the HBM traffic is the
- * algorithmic minimum; what the loads still cost is issue slots next to the matrix instructions.
+ * so with the XCD-aware tile walk nearly all of these loads hit in L1/L2 and the HBM traffic is the algorithmic
+ * minimum; what the loads still cost is issue slots next to the matrix instructions.
  *
  * Blocks are persistent and XCD aware: hardware deals consecutive workgroups round-robin to the 8 XCDs, each
  * with its own L2. Block b therefore walks a contiguous eighth of the tiles (xcd = b % 8), so the neighbour
- * rows a tile gathers - which lie in nearby tiles, mesh order being spatially coherent - are found in the
- * same L2 instead of being fetched by every XCD.
+ * rows a tile gathers are found in the same L2 instead of being fetched by every XCD.
+ *
+ * Each wave walks its tiles with a software pipeline, because the per-tile chain "which frame -> how many rows
+ * -> neighbour table -> source rows" is four dependent memory round trips:
+ *   - the frame lookup and the neighbour-table loads of tile t+2 are issued before the epilogue of tile t;
+ *   - the slot-0 rows of tile t+1 are requested during the last slot of tile t;
+ *   - inside a tile, slot s+1's rows are requested before slot s's matrix instructions (fenced so the
+ *     scheduler cannot sink the loads back next to their uses).
  */
+#include <cmath>
 #include <cstdlib>
+#include <cstring>
+#include <type_traits>
 
 #include "vmhip_internal.h"
 
 namespace {
 
 typedef float v4f __attribute__((ext_vector_type(4)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef __bf16 v4bf __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ int find_frame_by_row_tile(const VmFrame* frames, int n, int tile) {
     int lo = 0, hi = n - 1;
@@ -48,42 +65,24 @@ __device__ __forceinline__ float selu(float s) {
     return lambda * (s >= 0.0f ? s : alpha * expf(s) - alpha);
 }
 
-/* loads N consecutive 32-bit words with the widest loads their count allows (the caller guarantees the
- * matching alignment: rows are multiples of 16, 8 or 4 bytes accordingly) */
-template <int N>
-__device__ __forceinline__ void load_run(const float* __restrict__ p, float (&v)[N]) {
+/* N consecutive 32-bit words with the widest loads their count allows (the caller guarantees the matching
+ * alignment: runs start at multiples of 16, 8 or 4 bytes accordingly) */
+template <typename T, int N>
+__device__ __forceinline__ void load_words(const T* __restrict__ p, T (&v)[N]) {
+    static_assert(sizeof(T) == 4, "32-bit words");
     if constexpr (N % 4 == 0) {
+        typedef T vec4 __attribute__((ext_vector_type(4)));
 #pragma unroll
         for (int i = 0; i < N; i += 4) {
-            const float4 t = *reinterpret_cast<const float4*>(p + i);
+            const vec4 t = *reinterpret_cast<const vec4*>(p + i);
             v[i] = t.x, v[i + 1] = t.y, v[i + 2] = t.z, v[i + 3] = t.w;
         }
     }
     else if constexpr (N % 2 == 0) {
+        typedef T vec2 __attribute__((ext_vector_type(2)));
 #pragma unroll
         for (int i = 0; i < N; i += 2) {
-            const float2 t = *reinterpret_cast<const float2*>(p + i);
-            v[i] = t.x, v[i + 1] = t.y;
-        }
-    }
-    else {
-#pragma unroll
-        for (int i = 0; i < N; ++i) v[i] = p[i];
-    }
-}
-template <int N>
-__device__ __forceinline__ void load_run(const int32_t* __restrict__ p, int (&v)[N]) {
-    if constexpr (N % 4 == 0) {
-#pragma unroll
-        for (int i = 0; i < N; i += 4) {
-            const int4 t = *reinterpret_cast<const int4*>(p + i);
-            v[i] = t.x, v[i + 1] = t.y, v[i + 2] = t.z, v[i + 3] = t.w;
-        }
-    }
-    else if constexpr (N % 2 == 0) {
-#pragma unroll
-        for (int i = 0; i < N; i += 2) {
-            const int2 t = *reinterpret_cast<const int2*>(p + i);
+            const vec2 t = *reinterpret_cast<const vec2*>(p + i);
             v[i] = t.x, v[i + 1] = t.y;
         }
     }
@@ -93,31 +92,135 @@ __device__ __forceinline__ void load_run(const int32_t* __restrict__ p, int (&v)
     }
 }
 
-/* Gather-from-global variant. NW waves per block, RB row blocks of 16 rows per wave: NW * RB * 16 == VMHIP_TILE.
- *
- * Each wave walks its tiles with a software pipeline, because the per-tile chain "which frame -> how many rows
- * -> neighbour table -> source rows" is four dependent memory round trips and the waves that share a SIMD tend
- * to run in lockstep (the matrix pipe is served round-robin), so a chain left in the open idles the pipe for
- * every wave at once:
- *   - the frame lookup and the neighbour-table loads of tile t+1 are issued before the matrix work of tile t;
- *   - the slot-0 rows of tile t+1 are requested during the last slot of tile t, ahead of tile t's epilogue;
- *   - inside a tile, slot s+1's rows are requested before slot s's matrix instructions (fenced so the
- *     scheduler cannot sink the loads back next to their uses). */
-template <int C_IN, int C_OUT, int SLOTS, int NW, int RB>
-__global__ __launch_bounds__(NW * 64) void vm_conv_mfma_kernel(VmBatchDev B, VmLayerDev L, const float* __restrict__ in,
-                                                               float* __restrict__ out) {
-    static_assert(C_IN % 4 == 0, "a lane group takes a quarter of each gathered row");
+/* ---- operand policies: how a lane fetches its quarter of a gathered row (load: raw registers, no dependent
+ * arithmetic, so that the request can be issued a slot ahead), how the raw registers become matrix operands
+ * (prepare: runs when the slot is consumed) and what one reduction step issues (accumulate) ---- */
+
+/* fp32 arithmetic on fp32 rows */
+template <int C_IN>
+struct OperandF32 {
+    static constexpr int STEPS = C_IN / 4;
+    static constexpr int PARTS = 1;
+    static constexpr int RAW = STEPS;
+    typedef float areg_t;
+    typedef float raw_t;
+    typedef float op_t;
+    static __device__ __forceinline__ void load(const void* __restrict__ in, uint32_t row, int q, raw_t (&x)[RAW]) {
+        load_words<float, RAW>(reinterpret_cast<const float*>(in) + (size_t) row * C_IN + q * RAW, x);
+    }
+    static __device__ __forceinline__ void prepare(const raw_t (&x)[RAW], op_t (&b)[STEPS]) {
+#pragma unroll
+        for (int j = 0; j < STEPS; ++j) b[j] = x[j];
+    }
+    static __device__ __forceinline__ v4f accumulate(int, areg_t a, op_t b, v4f c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
+};
+
+/* bf16 matrix instructions with fp32 accumulation. Every weight is held as two bf16, w = hi + lo with
+ * hi = bf16(w) and lo = bf16(w - hi), one part each in LDS, so the products carry the weights to about 16
+ * significant bits. Rows stored as bf16 are used as they are (two instructions per step: hi and lo weights);
+ * the only rounding such a layer adds to the fp32 result is the storage of its input rows. */
+template <int C_IN>
+struct OperandBF16 {
+    static_assert(C_IN % 32 == 0, "one step consumes 8 bf16 from each of the four lane groups");
+    static constexpr int STEPS = C_IN / 32;
+    static constexpr int PARTS = 2;
+    static constexpr int RAW = STEPS;
+    typedef v8bf areg_t;
+    typedef v8bf raw_t;
+    typedef v8bf op_t;
+    static __device__ __forceinline__ void load(const void* __restrict__ in, uint32_t row, int q, raw_t (&x)[RAW]) {
+        const uint16_t* p = reinterpret_cast<const uint16_t*>(in) + (size_t) row * C_IN + q * (C_IN / 4);
+#pragma unroll
+        for (int j = 0; j < STEPS; ++j) x[j] = *reinterpret_cast<const v8bf*>(p + j * 8);
+    }
+    static __device__ __forceinline__ void prepare(const raw_t (&x)[RAW], op_t (&b)[STEPS]) {
+#pragma unroll
+        for (int j = 0; j < STEPS; ++j) b[j] = x[j];
+    }
+    static __device__ __forceinline__ v4f accumulate(int, areg_t a, op_t b, v4f c) { return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0); }
+};
+
+/* The same bf16 matrix instructions on rows stored as fp32: each value is split in registers into
+ * hi = bf16(x) and lo = bf16(x - hi) and a step issues hi*w_hi + lo*w_hi + hi*w_lo. What is dropped (lo*w_lo
+ * and the rounding of lo) is about 2^-17 of a product, so this layer adds no bf16-sized error at all while the
+ * matrix pipe still runs at the bf16 rate (3 instructions of K=32 against 8 fp32 instructions of K=4). */
+template <int C_IN>
+struct OperandBF16FromF32 {
+    static_assert(C_IN % 32 == 0, "one step consumes 8 values from each of the four lane groups");
+    static constexpr int STEPS = C_IN / 32;
+    static constexpr int PARTS = 2;
+    static constexpr int RAW = C_IN / 4;
+    typedef v8bf areg_t;
+    typedef float raw_t;
+    struct op_t {
+        v8bf hi, lo;
+    };
+    static __device__ __forceinline__ void load(const void* __restrict__ in, uint32_t row, int q, raw_t (&x)[RAW]) {
+        load_words<float, RAW>(reinterpret_cast<const float*>(in) + (size_t) row * C_IN + q * RAW, x);
+    }
+    static __device__ __forceinline__ void prepare(const raw_t (&x)[RAW], op_t (&b)[STEPS]) {
+#pragma unroll
+        for (int j = 0; j < STEPS; ++j) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float v = x[j * 8 + e];
+                const __bf16 h = (__bf16) v; /* round to nearest even */
+                b[j].hi[e] = h;
+                b[j].lo[e] = (__bf16) (v - (float) h); /* the difference is exact in fp32 */
+            }
+        }
+    }
+    static __device__ __forceinline__ v4f accumulate(int part, areg_t a, const op_t& b, v4f c) {
+        c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b.hi, c, 0, 0, 0);
+        if (part == 0) c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b.lo, c, 0, 0, 0);
+        return c;
+    }
+};
+
+/* four consecutive output channels of one row; OUT_T is float or uint16_t (bf16 bits) */
+template <typename OUT_T, int C_OUT>
+__device__ __forceinline__ void store4(void* __restrict__ out, uint32_t row, int o, v4f v) {
+    if constexpr (sizeof(OUT_T) == 4) {
+        float* y = reinterpret_cast<float*>(out) + (size_t) row * C_OUT + o;
+        if constexpr (C_OUT % 4 == 0) {
+            if (o < C_OUT) *reinterpret_cast<float4*>(y) = make_float4(v[0], v[1], v[2], v[3]);
+        }
+        else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (o + i < C_OUT) y[i] = v[i];
+        }
+    }
+    else {
+        static_assert(sizeof(OUT_T) == 4 || C_OUT % 4 == 0, "bf16 rows are written four channels at a time");
+        if (o < C_OUT) {
+            v4bf h;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) h[i] = (__bf16) v[i]; /* round to nearest even */
+            *reinterpret_cast<v4bf*>(reinterpret_cast<uint16_t*>(out) + (size_t) row * C_OUT + o) = h;
+        }
+    }
+}
+
+/* NW waves per block, RB row blocks of 16 rows per wave: NW * RB * 16 == VMHIP_TILE. */
+template <class OP, int C_OUT, int SLOTS, typename OUT_T, int NW, int RB>
+__global__ __launch_bounds__(NW * 64) void vm_conv_mfma_kernel(VmBatchDev B, VmLayerDev L, const void* __restrict__ in, void* __restrict__ out) {
     static_assert(NW * RB * 16 == VMHIP_TILE, "a block covers one tile");
-    constexpr int KQ = C_IN / 4;              /* floats per lane per slot */
-    constexpr int CB = (C_OUT + 15) / 16;     /* column blocks of 16 output channels */
+    constexpr int STEPS = OP::STEPS;
+    constexpr int CB = (C_OUT + 15) / 16; /* column blocks of 16 output channels */
     constexpr int NN = SLOTS - 1;
     constexpr int NBV = NN > 0 ? NN : 1;
-    constexpr int W_FLOATS = SLOTS * KQ * CB * 64;
+    constexpr int PARTS = OP::PARTS;
+    constexpr int W_BYTES = SLOTS * STEPS * CB * PARTS * 64 * (int) sizeof(typename OP::areg_t);
+    constexpr int RAW = OP::RAW;
+    typedef typename OP::areg_t areg_t;
+    typedef typename OP::raw_t raw_t;
+    typedef typename OP::op_t op_t;
 
-    extern __shared__ float w_lds[];
-    for (int i = threadIdx.x * 4; i < W_FLOATS; i += NW * 64 * 4)
-        *reinterpret_cast<float4*>(w_lds + i) = *reinterpret_cast<const float4*>(L.w_mfma + i);
+    extern __shared__ float4 w_lds4[];
+    for (int i = threadIdx.x; i < W_BYTES / 16; i += NW * 64) w_lds4[i] = reinterpret_cast<const float4*>(L.w_mfma)[i];
     __syncthreads();
+    const areg_t* w_lds = reinterpret_cast<const areg_t*>(w_lds4);
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int q = lane >> 4;   /* quarter of the gathered row / group of 4 output channels */
@@ -161,7 +264,7 @@ __global__ __launch_bounds__(NW * 64) void vm_conv_mfma_kernel(VmBatchDev B, VmL
 #pragma unroll
             for (int rb = 0; rb < RB; ++rb) {
                 const uint32_t row = t.base + (uint32_t) max(0, min(t.row0 + rb * 16 + r16, t.V));
-                load_run<NN>(B.row_nb + (size_t) row * B.nb_stride, nb[rb]);
+                load_words<int, NN>(B.row_nb + (size_t) row * B.nb_stride, nb[rb]);
             }
         }
     };
@@ -185,9 +288,9 @@ __global__ __launch_bounds__(NW * 64) void vm_conv_mfma_kernel(VmBatchDev B, VmL
     uint32_t src[RB][SLOTS];
     bool valid[RB];
     resolve(cur, nb, src, valid);
-    float x[2][RB][KQ];
+    raw_t x[2][RB][RAW];
 #pragma unroll
-    for (int rb = 0; rb < RB; ++rb) load_run<KQ>(in + (size_t) src[rb][0] * C_IN + q * KQ, x[0][rb]);
+    for (int rb = 0; rb < RB; ++rb) OP::load(in, src[rb][0], q, x[0][rb]);
 
     int next = tile + gx;
     Info nxt = cur;
@@ -212,23 +315,28 @@ __global__ __launch_bounds__(NW * 64) void vm_conv_mfma_kernel(VmBatchDev B, VmL
             const int cur_buf = s & 1;
             if (s + 1 < SLOTS) {
 #pragma unroll
-                for (int rb = 0; rb < RB; ++rb) load_run<KQ>(in + (size_t) src[rb][s + 1] * C_IN + q * KQ, x[cur_buf ^ 1][rb]);
+                for (int rb = 0; rb < RB; ++rb) OP::load(in, src[rb][s + 1], q, x[cur_buf ^ 1][rb]);
             }
             else if (has_next) {
                 /* last slot: the other buffer is free; fill it with the next tile's slot 0 */
                 resolve(nxt, nb, src_next, valid_next);
 #pragma unroll
-                for (int rb = 0; rb < RB; ++rb) load_run<KQ>(in + (size_t) src_next[rb][0] * C_IN + q * KQ, x[cur_buf ^ 1][rb]);
+                for (int rb = 0; rb < RB; ++rb) OP::load(in, src_next[rb][0], q, x[cur_buf ^ 1][rb]);
             }
             __builtin_amdgcn_sched_barrier(0);
+            op_t b[RB][STEPS];
 #pragma unroll
-            for (int j = 0; j < KQ; ++j) {
+            for (int rb = 0; rb < RB; ++rb) OP::prepare(x[cur_buf][rb], b[rb]);
+#pragma unroll
+            for (int j = 0; j < STEPS; ++j) {
 #pragma unroll
                 for (int cb = 0; cb < CB; ++cb) {
-                    const float a = w_lds[((s * KQ + j) * CB + cb) * 64 + lane];
 #pragma unroll
-                    for (int rb = 0; rb < RB; ++rb)
-                        acc[rb][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, x[cur_buf][rb][j], acc[rb][cb], 0, 0, 0);
+                    for (int part = 0; part < PARTS; ++part) {
+                        const areg_t a = w_lds[(((s * STEPS + j) * CB + cb) * PARTS + part) * 64 + lane];
+#pragma unroll
+                        for (int rb = 0; rb < RB; ++rb) acc[rb][cb] = OP::accumulate(part, a, b[rb][j], acc[rb][cb]);
+                    }
                 }
             }
         }
@@ -272,20 +380,9 @@ __global__ __launch_bounds__(NW * 64) void vm_conv_mfma_kernel(VmBatchDev B, VmL
                         acc[rb][cb][v] = activation == VMHIP_SELU ? selu(a) : activation == VMHIP_RELU ? fmaxf(a, 0.0f) : tanhf(a);
                     }
             }
-            if (valid[rb]) {
-                float* __restrict__ y = out + (size_t) src[rb][0] * C_OUT; /* valid => src[rb][0] is the lane's own row */
+            if (valid[rb]) { /* valid => src[rb][0] is the lane's own row */
 #pragma unroll
-                for (int cb = 0; cb < CB; ++cb) {
-                    const int o = cb * 16 + q * 4;
-                    if (C_OUT % 4 == 0) {
-                        if (o < C_OUT) *reinterpret_cast<float4*>(y + o) = make_float4(acc[rb][cb][0], acc[rb][cb][1], acc[rb][cb][2], acc[rb][cb][3]);
-                    }
-                    else {
-#pragma unroll
-                        for (int v = 0; v < 4; ++v)
-                            if (o + v < C_OUT) y[o + v] = acc[rb][cb][v];
-                    }
-                }
+                for (int cb = 0; cb < CB; ++cb) store4<OUT_T, C_OUT>(out, src[rb][0], cb * 16 + q * 4, acc[rb][cb]);
             }
         }
 
@@ -299,7 +396,7 @@ __global__ __launch_bounds__(NW * 64) void vm_conv_mfma_kernel(VmBatchDev B, VmL
             for (int s = 0; s < SLOTS; ++s) src[rb][s] = src_next[rb][s];
             if (LAST == 0) {
 #pragma unroll
-                for (int j = 0; j < KQ; ++j) x[0][rb][j] = x[1][rb][j];
+                for (int j = 0; j < RAW; ++j) x[0][rb][j] = x[1][rb][j];
             }
         }
         tile = next;
@@ -308,12 +405,17 @@ __global__ __launch_bounds__(NW * 64) void vm_conv_mfma_kernel(VmBatchDev B, VmL
     }
 }
 
-
-template <int C_IN, int C_OUT, int SLOTS, int NW, int RB>
-int launch_mfma(const VmBatchDev& B, const VmLayerDev& L, const float* in, float* out, hipStream_t stream) {
-    constexpr int KQ = C_IN / 4, CB = (C_OUT + 15) / 16;
-    constexpr size_t lds = size_t(SLOTS) * KQ * CB * 64 * sizeof(float);
-    auto kernel = vm_conv_mfma_kernel<C_IN, C_OUT, SLOTS, NW, RB>;
+template <class OP, int C_OUT, int SLOTS, typename OUT_T>
+int launch_mfma(const VmBatchDev& B, const VmLayerDev& L, const void* in, void* out, hipStream_t stream) {
+    constexpr int CB = (C_OUT + 15) / 16;
+    constexpr size_t lds = size_t(SLOTS) * OP::STEPS * CB * OP::PARTS * 64 * sizeof(typename OP::areg_t);
+    /* 8 waves x 2 row blocks: 16 accumulator registers per pair of column blocks and two input buffers per
+     * lane leave room for four waves per SIMD on the 32-wide layers, two blocks per CU. Where the weights
+     * allow only one block per CU and the kernel lives on hiding gather latency (bf16), one block of 16 waves
+     * keeps the same four waves per SIMD. */
+    constexpr bool one_big_block = OP::PARTS > 1 && lds > 80 * 1024;
+    constexpr int NW = one_big_block ? 16 : 8, RB = VMHIP_TILE / (16 * NW);
+    auto kernel = vm_conv_mfma_kernel<OP, C_OUT, SLOTS, OUT_T, NW, RB>;
     static bool configured = false;
     if (!configured) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, int(lds)) != hipSuccess) {
@@ -322,9 +424,9 @@ int launch_mfma(const VmBatchDev& B, const VmLayerDev& L, const float* in, float
         }
         configured = true;
     }
-    /* blocks per CU limited by LDS (160 KB per CU) and registers; 8 XCDs x 32 CUs */
+    /* resident blocks per CU: limited by LDS (160 KB per CU) and by four waves per SIMD; 8 XCDs x 32 CUs */
     int per_cu = int((160 * 1024) / (lds + 512));
-    per_cu = per_cu < 1 ? 1 : per_cu > (NW == 4 ? 3 : 2) ? (NW == 4 ? 3 : 2) : per_cu;
+    per_cu = per_cu < 1 ? 1 : per_cu > 2 ? 2 : per_cu;
     if (const char* e = getenv("VMHIP_MFMA_BLOCKS_PER_CU")) per_cu = atoi(e) > 0 ? atoi(e) : per_cu;
     int grid = 256 * per_cu;
     const int need = ((B.n_row_tiles + 7) / 8) * 8;
@@ -333,48 +435,109 @@ int launch_mfma(const VmBatchDev& B, const VmLayerDev& L, const float* in, float
     return 0;
 }
 
-template <int C_IN, int C_OUT, int SLOTS>
-int launch_pick(const VmBatchDev& B, const VmLayerDev& L, const float* in, float* out, hipStream_t stream) {
-    /* 8 waves x 2 row blocks: 16 accumulator registers and two 16-register input buffers per lane leave room
-     * for four waves per SIMD on the 32-wide layers */
-    return launch_mfma<C_IN, C_OUT, SLOTS, 8, 2>(B, L, in, out, stream);
+uint16_t bf16_round(float f) {
+    uint32_t u;
+    std::memcpy(&u, &f, 4);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return uint16_t((u >> 16) | 0x40); /* NaN stays NaN */
+    u += 0x7fffu + ((u >> 16) & 1u);                                         /* round to nearest even */
+    return uint16_t(u >> 16);
+}
+
+template <int CI, int CO, int SL, int IB, int OB, int AB>
+int launch_variant(const VmBatchDev& B, const VmLayerDev& L, const void* in, void* out, hipStream_t stream) {
+    typedef typename std::conditional<OB != 0, uint16_t, float>::type out_t;
+    static_assert(AB != 0 || IB == 0, "fp32 arithmetic reads fp32 rows");
+    if constexpr (AB != 0 && IB != 0) return launch_mfma<OperandBF16<CI>, CO, SL, out_t>(B, L, in, out, stream);
+    else if constexpr (AB != 0) return launch_mfma<OperandBF16FromF32<CI>, CO, SL, out_t>(B, L, in, out, stream);
+    else return launch_mfma<OperandF32<CI>, CO, SL, out_t>(B, L, in, out, stream);
 }
 
 }  // namespace
 
-/* Permuted weight layout the kernel consumes: [slot][j][column block][lane = q*16 + o] with
- * value W[slot*C_IN + q*(C_IN/4) + j][cb*16 + o], zero for padded output channels. */
-size_t vm_mfma_weight_floats(int c_in, int c_out, int slots) { return size_t(slots) * (c_in / 4) * ((c_out + 15) / 16) * 64; }
-void vm_mfma_permute_weights(const float* w, int c_in, int c_out, int slots, float* wp) {
-    const int KQ = c_in / 4, CB = (c_out + 15) / 16;
+/* Weight layouts the kernel consumes, [slot][step][column block][part][lane = q*16 + o] with, per lane,
+ *   fp32 arithmetic: one part, one float,   W[slot*C_IN + q*(C_IN/4) + step][cb*16 + o]
+ *   bf16 arithmetic: two parts (hi, lo), eight bf16 each, of W[slot*C_IN + q*(C_IN/4) + step*8 + e][cb*16 + o], e = 0..7
+ * and zeros for padded output channels. */
+size_t vm_mfma_weight_bytes(int c_in, int c_out, int slots, int arith_bf16) {
+    const size_t cb = (c_out + 15) / 16;
+    return arith_bf16 ? size_t(slots) * (c_in / 32) * cb * 2 * 64 * 16 : size_t(slots) * (c_in / 4) * cb * 64 * 4;
+}
+void vm_mfma_permute_weights(const float* w, int c_in, int c_out, int slots, int arith_bf16, void* wp) {
+    const int CB = (c_out + 15) / 16;
+    const int quarter = c_in / 4;
+    if (!arith_bf16) {
+        float* dst = reinterpret_cast<float*>(wp);
+        for (int s = 0; s < slots; ++s)
+            for (int j = 0; j < quarter; ++j)
+                for (int cb = 0; cb < CB; ++cb)
+                    for (int q = 0; q < 4; ++q)
+                        for (int o = 0; o < 16; ++o) {
+                            const int col = cb * 16 + o;
+                            const int k = s * c_in + q * quarter + j;
+                            dst[((size_t(s) * quarter + j) * CB + cb) * 64 + q * 16 + o] = col < c_out ? w[size_t(k) * c_out + col] : 0.0f;
+                        }
+        return;
+    }
+    uint16_t* dst = reinterpret_cast<uint16_t*>(wp);
+    const int steps = c_in / 32;
     for (int s = 0; s < slots; ++s)
-        for (int j = 0; j < KQ; ++j)
+        for (int j = 0; j < steps; ++j)
             for (int cb = 0; cb < CB; ++cb)
                 for (int q = 0; q < 4; ++q)
-                    for (int o = 0; o < 16; ++o) {
-                        const int col = cb * 16 + o;
-                        const int k = s * c_in + q * KQ + j;
-                        wp[((size_t(s) * KQ + j) * CB + cb) * 64 + q * 16 + o] = col < c_out ? w[size_t(k) * c_out + col] : 0.0f;
-                    }
+                    for (int o = 0; o < 16; ++o)
+                        for (int e = 0; e < 8; ++e) {
+                            const int col = cb * 16 + o;
+                            const int k = s * c_in + q * quarter + j * 8 + e;
+                            const float v = col < c_out ? w[size_t(k) * c_out + col] : 0.0f;
+                            const uint16_t hi = bf16_round(v);
+                            const uint32_t hi_bits = uint32_t(hi) << 16;
+                            float hi_f;
+                            std::memcpy(&hi_f, &hi_bits, 4);
+                            const uint16_t lo = std::isfinite(v) ? bf16_round(v - hi_f) : uint16_t(0);
+                            const size_t at = ((size_t(s) * steps + j) * CB + cb) * 2;
+                            dst[((at + 0) * 64 + q * 16 + o) * 8 + e] = hi;
+                            dst[((at + 1) * 64 + q * 16 + o) * 8 + e] = lo;
+                        }
 }
 
-bool vm_mfma_supported(int c_in, int c_out, int slots) {
-#define MFMA_SHAPE(CI, CO, SL) \
-    if (c_in == CI && c_out == CO && slots == SL) return true;
-#include "conv_mfma_shapes.inc"
-#undef MFMA_SHAPE
+/* Instantiated combinations: (C_in, C_out, gather slots, bf16 rows in, bf16 rows out, bf16 arithmetic). */
+#define VM_FOR_EACH_MFMA_VARIANT(X)                                \
+    /* fp32 rows in and out, fp32 arithmetic */                    \
+    X(4, 16, 7, 0, 0, 0)                                           \
+    X(16, 16, 7, 0, 0, 0)                                          \
+    X(16, 32, 7, 0, 0, 0)                                          \
+    X(32, 32, 7, 0, 0, 0)                                          \
+    X(32, 16, 7, 0, 0, 0)                                          \
+    X(4, 64, 7, 0, 0, 0)                                           \
+    X(64, 64, 7, 0, 0, 0)                                          \
+    X(4, 24, 9, 0, 0, 0)                                           \
+    X(24, 24, 9, 0, 0, 0)                                          \
+    /* bf16 engine: bf16 matrix instructions; rows fp32 -> fp32, fp32 -> bf16, bf16 -> fp32 (bf16 storage is \
+     * only ever chosen for every second boundary, so bf16 -> bf16 does not occur) */                          \
+    X(64, 64, 7, 0, 0, 1)                                          \
+    X(64, 64, 7, 0, 1, 1)                                          \
+    X(64, 64, 7, 1, 0, 1)
+
+bool vm_mfma_supported(int c_in, int c_out, int slots, int in_bf16, int out_bf16, int arith_bf16) {
+#define X(CI, CO, SL, IB, OB, AB) \
+    if (c_in == CI && c_out == CO && slots == SL && in_bf16 == IB && out_bf16 == OB && arith_bf16 == AB) return true;
+    VM_FOR_EACH_MFMA_VARIANT(X)
+#undef X
     return false;
 }
 
-int vm_launch_conv_mfma(const VmBatchDev& B, const VmLayerDev& L, const float* in, float* out, hipStream_t stream,
-                        const char** kernel_name) {
+int vm_launch_conv_mfma(const VmBatchDev& B, const VmLayerDev& L, const void* in, void* out, hipStream_t stream, const char** kernel_name) {
     if (B.n_row_tiles <= 0) return 0;
-#define MFMA_SHAPE(CI, CO, SL)                                                                 \
-    if (L.c_in == CI && L.c_out == CO && L.slots == SL) {                                      \
-        if (kernel_name) *kernel_name = "conv_mfma_" #CI "x" #CO "s" #SL;                      \
-        return launch_pick<CI, CO, SL>(B, L, in, out, stream);                                 \
+#define X(CI, CO, SL, IB, OB, AB)                                                                                      \
+    if (L.c_in == CI && L.c_out == CO && L.slots == SL && L.in_bf16 == IB && L.out_bf16 == OB && L.arith_bf16 == AB) { \
+        if (kernel_name)                                                                                               \
+            *kernel_name = AB && IB   ? (OB ? "conv_bf16x2_" #CI "x" #CO "s" #SL : "conv_bf16x2_tof32_" #CI "x" #CO "s" #SL)  \
+                           : AB       ? (OB ? "conv_bf16x3_tobf16_" #CI "x" #CO "s" #SL : "conv_bf16x3_" #CI "x" #CO "s" #SL) \
+                           : OB       ? "conv_mfma_tobf16_" #CI "x" #CO "s" #SL                                        \
+                                      : "conv_mfma_" #CI "x" #CO "s" #SL;                                              \
+        return launch_variant<CI, CO, SL, IB, OB, AB>(B, L, in, out, stream);                                          \
     }
-#include "conv_mfma_shapes.inc"
-#undef MFMA_SHAPE
+    VM_FOR_EACH_MFMA_VARIANT(X)
+#undef X
     return -1;
 }

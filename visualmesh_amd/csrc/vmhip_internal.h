@@ -94,7 +94,10 @@ struct VmLayerDev {
     int32_t activation;
     const float* w;  /* [slots*c_in][c_out] fp32 row major */
     const float* b;  /* [c_out] */
-    const float* w_mfma; /* the same weights in the matrix-core kernel's consumption order, or null */
+    const void* w_mfma; /* the same weights in the matrix-core kernel's consumption order, or null */
+    int32_t in_bf16;    /* input rows are stored as bf16 */
+    int32_t out_bf16;   /* output rows are stored as bf16 */
+    int32_t arith_bf16; /* bf16 products with fp32 accumulation (weights in w_mfma are bf16 then) */
 };
 
 /* launchers, one per kernel; all asynchronous on `stream` */
@@ -108,11 +111,11 @@ void vm_launch_neighbourhood(const VmBatchDev& B, hipStream_t stream);
 int vm_launch_conv(const VmBatchDev& B, const VmLayerDev& L, const float* in, float* out, hipStream_t stream,
                    const char** kernel_name);
 
-/* matrix-core variant (conv_mfma.hip); launch returns a negative value if the shape has no instantiation */
-bool vm_mfma_supported(int c_in, int c_out, int slots);
-size_t vm_mfma_weight_floats(int c_in, int c_out, int slots);
-void vm_mfma_permute_weights(const float* w, int c_in, int c_out, int slots, float* wp);
-int vm_launch_conv_mfma(const VmBatchDev& B, const VmLayerDev& L, const float* in, float* out, hipStream_t stream,
+/* matrix-core variant (conv_mfma.hip); launch returns a negative value if the combination has no instantiation */
+bool vm_mfma_supported(int c_in, int c_out, int slots, int in_bf16, int out_bf16, int arith_bf16);
+size_t vm_mfma_weight_bytes(int c_in, int c_out, int slots, int arith_bf16);
+void vm_mfma_permute_weights(const float* w, int c_in, int c_out, int slots, int arith_bf16, void* wp);
+int vm_launch_conv_mfma(const VmBatchDev& B, const VmLayerDev& L, const void* in, void* out, hipStream_t stream,
                         const char** kernel_name);
 
 #include "host_project.h"
