@@ -161,7 +161,7 @@ def test_bf16_engine(oracle):
     engine.profile(True)
     engine.run()
     names = [n for n, _, _ in engine.profile_read() if n.startswith("conv")]
-    assert names == ["conv_mfma_4x64s7", "conv_bf16x3_tobf16_64x64s7", "conv_bf16x2_tof32_64x64s7", "conv_bf16x3_tobf16_64x64s7",
+    assert names == ["conv_lds_4x64s7", "conv_bf16x3_tobf16_64x64s7", "conv_bf16x2_tof32_64x64s7", "conv_bf16x3_tobf16_64x64s7",
                      "conv_bf16x2_tof32_64x64s7", "conv_bf16x3_64x64s7"], names
     worst = 0.0
     for i, f in enumerate(cfg.frames):
@@ -185,10 +185,11 @@ def test_bf16_engine_keeps_narrow_networks_in_fp32(oracle):
     assert_classification_parity(got, want, PROB_TOL, "bf16 engine, narrow network")
 
 
-@pytest.mark.parametrize("kernel", ["rows", "mfma"])
-def test_both_convolution_kernels_agree_with_the_oracle(oracle, kernel, monkeypatch):
-    """Every layer shape of configuration 2 through the one-row-per-lane kernel and through the matrix-core
-    kernel (selected per engine with VMHIP_CONV_KERNEL)."""
+@pytest.mark.parametrize("kernel", ["rows", "mfma", "lds"])
+def test_every_convolution_kernel_agrees_with_the_oracle(oracle, kernel, monkeypatch):
+    """Every layer shape of configuration 2 through the one-row-per-lane kernel, the matrix-core kernel that
+    gathers into registers and the matrix-core kernel that gathers from LDS (VMHIP_CONV_KERNEL, read when the
+    engine is built)."""
     monkeypatch.setenv("VMHIP_CONV_KERNEL", kernel)
     cfg = wl.config(2, n_frames=2)
     o_lens, e_lens = lens_pair(cfg)
@@ -200,7 +201,30 @@ def test_both_convolution_kernels_agree_with_the_oracle(oracle, kernel, monkeypa
     engine.profile(True)
     engine.run()
     names = [n for n, _, _ in engine.profile_read() if n.startswith("conv")]
-    assert all(("mfma" in n) == (kernel == "mfma") or n.endswith("x3s7") for n in names), names
+    assert len(names) == 8, names
+    if kernel == "mfma":
+        assert all(n.startswith("conv_mfma_") or n == "conv_rows_16x3s7" for n in names), names
+    else:
+        assert all(n.startswith("conv_%s_" % kernel) for n in names), names
     for i, f in enumerate(cfg.frames):
         want = pick(o_mesh, f["Hoc"]).classify(f["Hoc"], o_lens, f["image"], cfg.fourcc, vmo.Network(cfg.network))
         assert_classification_parity(results[i], want, PROB_TOL, "%s frame %d" % (kernel, i))
+
+
+@pytest.mark.parametrize("index", [2, 3])
+def test_rows_beyond_the_halo_capacity(oracle, index, monkeypatch):
+    """With only 8 halo slots per tile most out-of-tile neighbours are marked as not staged and the LDS kernel
+    reads them from global memory: same results (configuration 2's Ring6 and 3's NMGrid8 networks)."""
+    monkeypatch.setenv("VMHIP_HALO_CAP", "8")
+    cfg = wl.config(index, n_frames=1)
+    o_lens, e_lens = lens_pair(cfg)
+    o_mesh, e_mesh = meshes_for(cfg, oracle)
+    engine = eng.Engine(cfg.network, cfg.model)
+    f = cfg.frames[0]
+    got = engine(e_mesh, f["Hoc"], e_lens, f["image"], cfg.fourcc)
+    engine.profile(True)
+    engine.run()
+    names = [n for n, _, _ in engine.profile_read() if n.startswith("conv")]
+    assert all(n.startswith("conv_lds_") for n in names), names
+    want = pick(o_mesh, f["Hoc"]).classify(f["Hoc"], o_lens, f["image"], cfg.fourcc, vmo.Network(cfg.network))
+    assert_classification_parity(got, want, PROB_TOL, "halo cap 8, cfg%d" % index)

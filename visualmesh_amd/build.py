@@ -61,6 +61,7 @@ def build_hip(force=False):
         ("project.hip", HIP_FLAGS + ["-ffp-contract=off"]),
         ("conv.hip", HIP_FLAGS),
         ("conv_mfma.hip", HIP_FLAGS),
+        ("conv_lds.hip", HIP_FLAGS),
         ("api.hip", HIP_FLAGS),
     ]
     for name, flags in units:

@@ -102,10 +102,13 @@ struct HostLayer {
     float* d_b = nullptr;
     void* d_w_mfma = nullptr;
     int32_t in_bf16 = 0, out_bf16 = 0, arith_bf16 = 0;
+    bool use_lds = false, use_mfma = false; /* which matrix-core kernels may take the layer */
     std::vector<float> h_w; /* kept until the row types are planned */
 };
 
 struct vmhip_engine {
+    bool use_lds = false;                /* some layer gathers through the tile-local tables */
+    int32_t halo_cap = VMHIP_HALO_MAX;   /* VMHIP_HALO_CAP lowers it to exercise the not-staged path */
     int32_t nn = 0;
     int32_t precision = VMHIP_FP32;
     int32_t n_classes = 4;
@@ -135,7 +138,7 @@ struct vmhip_batch {
 
     VmBatchDev dev{};
     DevBuf d_frames, d_ranges, d_images, d_cand_px, d_cand_keep, d_tile_count, d_force_valid, d_force_keep, d_frame_V,
-      d_amb_count, d_amb_list, d_row_px, d_row_gidx, d_row_nb, d_act[2], d_lookup;
+      d_amb_count, d_amb_list, d_row_px, d_row_gidx, d_row_nb, d_row_nbl, d_tile_halo, d_tile_desc, d_act[2], d_lookup;
     float* final_act = nullptr;
 
     /* profiling */
@@ -148,6 +151,7 @@ struct vmhip_batch {
     void release() {
         DevBuf* all[] = {&d_frames, &d_ranges, &d_images, &d_cand_px, &d_cand_keep, &d_tile_count, &d_force_valid,
                          &d_force_keep, &d_frame_V, &d_amb_count, &d_amb_list, &d_row_px, &d_row_gidx, &d_row_nb,
+                         &d_row_nbl, &d_tile_halo, &d_tile_desc,
                          &d_act[0], &d_act[1], &d_lookup};
         for (DevBuf* b : all) b->release();
         for (hipEvent_t e : events) (void) hipEventDestroy(e);
@@ -248,8 +252,15 @@ int batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int
     HIP_TRY(b->d_row_px.reserve(sizeof(float2) * std::max<size_t>(b->row_total, 1)));
     HIP_TRY(b->d_row_gidx.reserve(4 * std::max<size_t>(b->row_total, 1)));
     HIP_TRY(b->d_row_nb.reserve(4 * std::max<size_t>(b->row_total, 1) * nb_stride));
+    const bool local_tables = classify && E->use_lds && nb_stride <= VMHIP_NBL_STRIDE;
     if (classify) {
         for (int i = 0; i < 2; ++i) HIP_TRY(b->d_act[i].reserve(4 * std::max<size_t>(b->row_total, 1) * E->max_width));
+    }
+    if (local_tables) {
+        const size_t row_tiles = std::max<size_t>(b->row_total / VMHIP_TILE, 1);
+        HIP_TRY(b->d_row_nbl.reserve(2 * std::max<size_t>(b->row_total, 1) * VMHIP_NBL_STRIDE));
+        HIP_TRY(b->d_tile_halo.reserve(4 * row_tiles * VMHIP_HALO_MAX));
+        HIP_TRY(b->d_tile_desc.reserve(sizeof(int4) * row_tiles));
     }
     HIP_TRY(b->d_lookup.reserve(sizeof(uint2) * lookup_entries));
     if (b->d_lookup.grew) {
@@ -309,6 +320,10 @@ int batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int
     D.row_gidx = b->d_row_gidx.as<int32_t>();
     D.row_nb = b->d_row_nb.as<int32_t>();
     D.nb_stride = nb_stride;
+    D.row_nbl = local_tables ? b->d_row_nbl.as<uint16_t>() : nullptr;
+    D.tile_halo = local_tables ? b->d_tile_halo.as<uint32_t>() : nullptr;
+    D.tile_desc = local_tables ? b->d_tile_desc.as<int4>() : nullptr;
+    D.halo_cap = E->halo_cap;
     b->h_V.assign(n_frames, 0);
     b->h_amb_count.assign(n_frames, 0);
     return VMHIP_OK;
@@ -370,7 +385,8 @@ int batch_enqueue(vmhip_batch* b) {
             const char* name = "conv";
             HIP_TRY(P.begin());
             int rc = -1;
-            if (L.d_w_mfma) rc = vm_launch_conv_mfma(D, ld, b->d_act[cur].p, b->d_act[cur ^ 1].p, s, &name);
+            if (L.use_lds && D.row_nbl) rc = vm_launch_conv_lds(D, ld, b->d_act[cur].as<float>(), b->d_act[cur ^ 1].as<float>(), s, &name);
+            if (rc != 0 && L.d_w_mfma && L.use_mfma) rc = vm_launch_conv_mfma(D, ld, b->d_act[cur].p, b->d_act[cur ^ 1].p, s, &name);
             /* the one-row-per-lane kernels only know fp32 rows */
             if (rc != 0 && !L.in_bf16 && !L.out_bf16) rc = vm_launch_conv(D, ld, b->d_act[cur].as<float>(), b->d_act[cur ^ 1].as<float>(), s, &name);
             if (rc != 0) return fail(VMHIP_ERR_HIP, "no kernel could be launched for a layer");
@@ -555,8 +571,13 @@ int vmhip_engine_create(const vmhip_network* net, int32_t n_neighbours, int32_t 
      * only every second eligible boundary is stored as bf16 (the 2nd, 4th, ...); the others stay fp32. A choice
      * is only made where the kernels on both sides of the boundary exist for it. */
     {
-        const char* pick = getenv("VMHIP_CONV_KERNEL"); /* "rows" keeps every layer on the one-row-per-lane kernel (A/B timing) */
+        /* VMHIP_CONV_KERNEL selects the kernel family for A/B runs: "rows" = one row per lane, "mfma" = matrix
+         * cores gathering into registers, "lds" (default) = matrix cores gathering from LDS where the shape
+         * has an instantiation and the register-gather kernel elsewhere */
+        const char* pick = getenv("VMHIP_CONV_KERNEL");
         const bool rows_only = pick && std::string(pick) == "rows";
+        const bool allow_lds = !rows_only && !(pick && std::string(pick) == "mfma");
+        if (const char* cap = getenv("VMHIP_HALO_CAP")) E->halo_cap = std::min(std::max(atoi(cap), 0), VMHIP_HALO_MAX);
         const int n = int(E->layers.size());
         std::vector<int> bf(n + 1, 0); /* bf[l] = rows entering layer l are bf16; bf[n] = final output (never) */
         std::vector<int> ar(n, 0);     /* ar[l] = layer l uses the bf16 matrix instructions */
@@ -585,7 +606,11 @@ int vmhip_engine_create(const vmhip_network* net, int32_t n_neighbours, int32_t 
         for (int l = 0; l < n; ++l) {
             HostLayer& H = E->layers[l];
             H.in_bf16 = bf[l], H.out_bf16 = bf[l + 1], H.arith_bf16 = arith(l);
-            if (!rows_only && vm_mfma_supported(H.c_in, H.c_out, H.slots, H.in_bf16, H.out_bf16, H.arith_bf16)) {
+            const bool plain = !H.in_bf16 && !H.out_bf16 && !H.arith_bf16;
+            H.use_mfma = !rows_only && vm_mfma_supported(H.c_in, H.c_out, H.slots, H.in_bf16, H.out_bf16, H.arith_bf16);
+            H.use_lds = allow_lds && plain && H.slots - 1 <= VMHIP_NBL_STRIDE && vm_lds_supported(H.c_in, H.c_out, H.slots);
+            E->use_lds = E->use_lds || H.use_lds;
+            if (H.use_mfma || H.use_lds) {
                 std::vector<unsigned char> wp(vm_mfma_weight_bytes(H.c_in, H.c_out, H.slots, H.arith_bf16));
                 vm_mfma_permute_weights(H.h_w.data(), H.c_in, H.c_out, H.slots, H.arith_bf16, wp.data());
                 if (hipMalloc(&H.d_w_mfma, wp.size()) != hipSuccess) return bail(VMHIP_ERR_HIP, "engine_create: out of device memory");

@@ -1,0 +1,494 @@
+/*
+ * conv_lds.hip - graph-convolution layers on the matrix cores with both operands fed from LDS: neighbour gather +
+ * dense + bias + activation in one kernel (reference engine/cpu/engine.hpp:213-264, apply_activation.hpp:34-84).
+ *
+ * The contraction and the operand layout are those of conv_mfma.hip (v_mfma_f32_16x16x4_f32, lane group q takes
+ * the q-th quarter of every gathered row, weights stored in consumption order). What differs is where the
+ * gathered rows come from. A row tile's sources are its own 256 rows plus about 100 distinct rows of other tiles
+ * (tile_halo, at most VMHIP_HALO_MAX), and row_nbl names every neighbour as a position in that list. So a block
+ *   1. copies the tile's rows (one contiguous run of global memory) and its halo rows into LDS with coalesced
+ *      16-byte loads: every row is requested once per tile instead of once per gather slot;
+ *   2. gathers matrix operands from LDS with ds_read, the weights next to them: no vector-memory instruction
+ *      sits between the matrix instructions, which is what held the register-gather kernel near 57 % of the
+ *      matrix peak;
+ *   3. applies the activation and writes the output rows.
+ * The global loads of tile t+1 (rows, halo rows, neighbour positions) are issued before the matrix work of tile
+ * t and land in registers; they are written to LDS after the barrier that ends tile t. Halo row numbers and tile
+ * descriptors are requested two tiles ahead because the row loads depend on them.
+ *
+ * A kernel stages as many halo rows as its LDS budget allows (144 to 256 depending on the layer shape). A
+ * neighbour beyond that, or marked VMHIP_NBL_FAR in row_nbl, is not staged: a wave that holds such an entry
+ * takes a side path that reads that row from global memory (a few per cent of the tiles of the benchmark
+ * meshes have more than 144 halo rows).
+ *
+ * Blocks are persistent and XCD aware exactly as in conv_mfma.hip.
+ */
+#include <cstdlib>
+#include <type_traits>
+
+#include "vmhip_internal.h"
+
+/* Build with -DVM_LDS_TIMING to count, per phase of the tile loop, the shader clock cycles every wave spends in
+ * it (first wave of every block, layers with C_IN = C_OUT = VM_LDS_TIMING; slot 7 counts tiles);
+ * vm_lds_timing_read() returns and clears the sums. A development aid, compiled out otherwise. */
+#ifdef VM_LDS_TIMING
+__device__ unsigned long long vm_lds_timing[10];
+#define VM_T_DECL unsigned long long t_acc[10] = {}, t_last = __builtin_readcyclecounter();
+#define VM_T_MARK(i)                                              \
+    {                                                             \
+        const unsigned long long t_now = __builtin_readcyclecounter(); \
+        t_acc[i] += t_now - t_last;                               \
+        t_last = t_now;                                           \
+    }
+#define VM_T_FLUSH                                                 \
+    if (threadIdx.x == 0 && C_IN == VM_LDS_TIMING && C_OUT == VM_LDS_TIMING) { /* wave 0 of every block, one layer shape */ \
+        for (int i = 0; i < 10; ++i) atomicAdd(&vm_lds_timing[i], t_acc[i]); \
+    }
+extern "C" int vm_lds_timing_read(unsigned long long* out) {
+    unsigned long long zero[10] = {};
+    if (hipMemcpyFromSymbol(out, HIP_SYMBOL(vm_lds_timing), sizeof(zero)) != hipSuccess) return -1;
+    return hipMemcpyToSymbol(HIP_SYMBOL(vm_lds_timing), zero, sizeof(zero)) == hipSuccess ? 0 : -1;
+}
+#else
+#define VM_T_DECL
+#define VM_T_MARK(i)
+#define VM_T_FLUSH
+#endif
+
+namespace {
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float selu(float s) {
+    const float lambda = 1.0507009873554804934193349852946f;
+    const float alpha = 1.6732632423543772848170429916717f;
+    return lambda * (s >= 0.0f ? s : alpha * expf(s) - alpha);
+}
+
+/* N consecutive floats with the widest loads their count allows (the caller guarantees matching alignment) */
+template <int N>
+__device__ __forceinline__ void load_floats(const float* __restrict__ p, float (&v)[N]) {
+    if constexpr (N % 4 == 0) {
+#pragma unroll
+        for (int i = 0; i < N; i += 4) {
+            const float4 t = *reinterpret_cast<const float4*>(p + i);
+            v[i] = t.x, v[i + 1] = t.y, v[i + 2] = t.z, v[i + 3] = t.w;
+        }
+    }
+    else if constexpr (N % 2 == 0) {
+#pragma unroll
+        for (int i = 0; i < N; i += 2) {
+            const float2 t = *reinterpret_cast<const float2*>(p + i);
+            v[i] = t.x, v[i + 1] = t.y;
+        }
+    }
+    else {
+#pragma unroll
+        for (int i = 0; i < N; ++i) v[i] = p[i];
+    }
+}
+
+template <int C_OUT>
+__device__ __forceinline__ void store4(float* __restrict__ out, uint32_t row, int o, v4f v) {
+    float* y = out + (size_t) row * C_OUT + o;
+    if constexpr (C_OUT % 4 == 0) {
+        if (o < C_OUT) *reinterpret_cast<float4*>(y) = make_float4(v[0], v[1], v[2], v[3]);
+    }
+    else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (o + i < C_OUT) y[i] = v[i];
+    }
+}
+
+/* the k-th 16-bit entry of a row of the tile-local neighbour table */
+__device__ __forceinline__ uint32_t nbl_entry(const uint4& t, int k) {
+    const uint32_t w = (k >> 1) == 0 ? t.x : (k >> 1) == 1 ? t.y : (k >> 1) == 2 ? t.z : t.w;
+    return (k & 1) ? (w >> 16) : (w & 0xffffu);
+}
+
+/* How staged rows are spread over the LDS banks. 128-byte rows (C_IN = 32) keep their size and XOR the position
+ * of each 16-byte piece with the low bits of the row number; 64-byte and 16-byte rows need nothing (consecutive
+ * rows already rotate through the banks); other widths get 16 bytes of padding per row. */
+__host__ __device__ constexpr bool row_swizzled(int c_in) { return c_in == 32; }
+__host__ __device__ constexpr int row_stride(int c_in) { return (c_in == 32 || c_in == 16 || c_in == 4) ? c_in : c_in + 4; }
+__host__ __device__ constexpr size_t lds_bytes(int c_in, int c_out, int slots, int halo) {
+    return (size_t(slots) * (c_in / 4) * ((c_out + 15) / 16) * 64 + size_t((c_out + 15) / 16) * 16 + size_t(VMHIP_TILE + halo) * row_stride(c_in)) * 4;
+}
+/* Halo rows a block stages: all VMHIP_HALO_MAX if two blocks then still fit a CU's 160 KB of LDS (two blocks
+ * overlap one's activation/store/staging phase with the other's matrix work), else 192 or 128
+ * if that lets two fit, else everything in one block per CU. */
+__host__ __device__ constexpr int halo_rows(int c_in, int c_out, int slots) {
+    for (int h = VMHIP_HALO_MAX; h >= 128; h -= 64)
+        if (2 * lds_bytes(c_in, c_out, slots, h) <= 160 * 1024) return h;
+    return VMHIP_HALO_MAX;
+}
+
+/* NW waves per block, RB row blocks of 16 rows per wave: NW * RB * 16 == VMHIP_TILE. */
+template <int C_IN, int C_OUT, int SLOTS, int NW, int HALO>
+__global__ __launch_bounds__(NW * 64, 4) void vm_conv_lds_kernel(VmBatchDev B, VmLayerDev L, const float* __restrict__ in, float* __restrict__ out) {
+    constexpr int RB = VMHIP_TILE / (16 * NW);
+    static_assert(NW * RB * 16 == VMHIP_TILE, "a block covers one tile");
+    static_assert(C_IN % 4 == 0, "rows are staged in 16-byte pieces");
+    constexpr int NT = NW * 64;
+    constexpr int STEPS = C_IN / 4; /* matrix steps per slot = floats in a lane's quarter row */
+    constexpr int CB = (C_OUT + 15) / 16;
+    constexpr int NN = SLOTS - 1;
+    static_assert(NN <= VMHIP_NBL_STRIDE, "the tile-local neighbour table holds 8 entries per row");
+    constexpr int RS = row_stride(C_IN);
+    constexpr bool SWZ = row_swizzled(C_IN);
+    constexpr uint32_t FAR_FROM = VMHIP_TILE + HALO; /* positions from here on are not staged by this kernel */
+    constexpr int Q4 = C_IN / 4; /* 16-byte pieces per row */
+    constexpr int W_FLOATS = SLOTS * STEPS * CB * 64;
+    constexpr int G = STEPS % 4 == 0 ? 4 : STEPS % 2 == 0 ? 2 : 1; /* weights fetched per LDS read */
+    constexpr int N_MAIN = (VMHIP_TILE * Q4 + NT - 1) / NT;      /* pieces of the tile's rows per thread */
+    constexpr int N_HALO = (HALO * Q4 + NT - 1) / NT;  /* pieces of halo rows per thread */
+
+    extern __shared__ float4 lds4[];
+    float* const w_lds = reinterpret_cast<float*>(lds4);
+    float* const b_lds = w_lds + W_FLOATS; /* CB * 16 biases, zero for padded channels */
+    float* const rows = b_lds + CB * 16;
+    for (int i = threadIdx.x; i < CB * 16; i += NT) b_lds[i] = i < C_OUT ? L.b[i] : 0.0f;
+    /* Weights: global order is [slot][step][column block][lane]; in LDS a lane's G consecutive steps sit together,
+     * [slot][column block][step / G][lane][G], so that one ds_read fetches G of them. */
+    for (int i = threadIdx.x; i < W_FLOATS; i += NT) {
+        const int e = i % G, l = (i / G) % 64, jg = (i / (G * 64)) % (STEPS / G), cb = (i / (G * 64 * (STEPS / G))) % CB, sl = i / (STEPS * 64 * CB);
+        w_lds[i] = reinterpret_cast<const float*>(L.w_mfma)[((sl * STEPS + jg * G + e) * CB + cb) * 64 + l];
+    }
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int q = lane >> 4, r16 = lane & 15;
+    const int activation = L.activation;
+    const v4f* __restrict__ in4 = reinterpret_cast<const v4f*>(in);
+
+    const int n_tiles = B.n_row_tiles;
+    const int xcd = blockIdx.x & 7, lb = blockIdx.x >> 3, gx = gridDim.x >> 3;
+    const int per_xcd = (n_tiles + 7) >> 3;
+    const int t_end = min(n_tiles, (xcd + 1) * per_xcd);
+    int tile = xcd * per_xcd + lb;
+    if (tile >= t_end) return; /* the whole block leaves: no barrier is left waiting */
+
+    /* ---- staging helpers: thread-private pieces of the next tile ---- */
+    v4f st_main[N_MAIN] = {}, st_halo[N_HALO] = {};
+    uint32_t hrow[N_HALO] = {};
+    auto request_halo_rows = [&](int t) {
+#pragma unroll
+        for (int k = 0; k < N_HALO; ++k) {
+            const int idx = threadIdx.x + k * NT;
+            const int h = idx / Q4;
+            hrow[k] = h < HALO ? B.tile_halo[(size_t) t * VMHIP_HALO_MAX + h] : 0u; /* entries past the tile's count are not used */
+        }
+    };
+    auto request_rows = [&](const int4& d) {
+#pragma unroll
+        for (int k = 0; k < N_MAIN; ++k) {
+            const int idx = threadIdx.x + k * NT;
+            if (idx < VMHIP_TILE * Q4 && d.y > 0) st_main[k] = in4[(size_t) d.x * Q4 + idx];
+        }
+#pragma unroll
+        for (int k = 0; k < N_HALO; ++k) {
+            const int idx = threadIdx.x + k * NT;
+            const int h = idx / Q4, c = idx - h * Q4;
+            if (h < min(d.z, HALO)) st_halo[k] = in4[(size_t) hrow[k] * Q4 + c];
+        }
+    };
+    auto write_rows = [&](const int4& d) {
+        v4f* rows4 = reinterpret_cast<v4f*>(rows);
+#pragma unroll
+        for (int k = 0; k < N_MAIN; ++k) {
+            const int idx = threadIdx.x + k * NT;
+            const int r = idx / Q4, c = idx - r * Q4;
+            if (idx < VMHIP_TILE * Q4 && d.y > 0) rows4[(r * RS) / 4 + (SWZ ? (c ^ (r & 7)) : c)] = st_main[k];
+        }
+#pragma unroll
+        for (int k = 0; k < N_HALO; ++k) {
+            const int idx = threadIdx.x + k * NT;
+            const int h = idx / Q4, c = idx - h * Q4;
+            if (h < min(d.z, HALO)) rows4[((VMHIP_TILE + h) * RS) / 4 + (SWZ ? (c ^ (h & 7)) : c)] = st_halo[k];
+        }
+    };
+    /* the lane's rows of a tile: rows past the tile's count compute on its last row (the frame's null row) and
+     * skip the store */
+    auto own_row = [&](const int4& d, int rb) { return max(0, min(wave * (RB * 16) + rb * 16 + r16, d.y - 1)); };
+    auto request_positions = [&](const int4& d, uint4 (&nbl)[RB]) {
+        if constexpr (NN > 0) {
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb)
+                if (d.y > 0) nbl[rb] = *reinterpret_cast<const uint4*>(B.row_nbl + (size_t) (d.x + own_row(d, rb)) * VMHIP_NBL_STRIDE);
+        }
+    };
+
+    /* Tile descriptors are wave-uniform but must not be fetched with scalar loads: scalar loads return out of
+     * order on the counter that LDS reads use too, so one descriptor in flight would turn every LDS wait of the
+     * matrix loop into a wait for that (global-latency) load. A buffer load is a vector-memory instruction. */
+    const __amdgpu_buffer_rsrc_t desc_rsrc = __builtin_amdgcn_make_buffer_rsrc(B.tile_desc, 0, n_tiles * 16, 0x00020000);
+    auto load_desc = [&](int t) {
+        typedef int v4i __attribute__((ext_vector_type(4)));
+        const v4i d = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(desc_rsrc, t * 16, 0, 0));
+        return make_int4(d.x, d.y, d.z, d.w);
+    };
+    auto uniform = [](const int4& d) {
+        return make_int4(__builtin_amdgcn_readfirstlane(d.x), __builtin_amdgcn_readfirstlane(d.y), __builtin_amdgcn_readfirstlane(d.z),
+                         __builtin_amdgcn_readfirstlane(d.w));
+    };
+
+    /* ---- prologue: everything tile `tile` needs, then the look-ahead for the next one ---- */
+    int4 d_cur = uniform(load_desc(tile));
+    int next = tile + gx;
+    int4 d_next = make_int4(0, 0, 0, 0), d_after = make_int4(0, 0, 0, 0);
+    uint4 nbl[RB], nbl_next[RB];
+    request_halo_rows(tile);
+    request_rows(d_cur);
+    request_positions(d_cur, nbl);
+    if (next < t_end) {
+        d_next = load_desc(next);
+        request_halo_rows(next);
+    }
+
+    VM_T_DECL
+    while (true) {
+        write_rows(d_cur);
+        VM_T_MARK(0)
+        __syncthreads(); /* rows (and, the first time, weights) are in LDS */
+        VM_T_MARK(1)
+
+        const bool has_next = next < t_end;
+        const int after = next + gx;
+        if (has_next) {
+            request_rows(d_next);
+            if (after < t_end) {
+                d_after = load_desc(after);
+                request_halo_rows(after);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        VM_T_MARK(2)
+
+        if (d_cur.y > 0) {
+            uint32_t li[RB][SLOTS];
+            bool valid[RB];
+            bool far = false;
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb) {
+                valid[rb] = wave * (RB * 16) + rb * 16 + r16 < d_cur.y;
+                li[rb][0] = (uint32_t) own_row(d_cur, rb);
+#pragma unroll
+                for (int s = 0; s < NN; ++s) {
+                    li[rb][s + 1] = nbl_entry(nbl[rb], s);
+                    far |= li[rb][s + 1] >= FAR_FROM;
+                }
+            }
+            const bool any_far = __any(far);
+
+            v4f acc[RB][CB];
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) {
+                const v4f bias = *reinterpret_cast<const v4f*>(b_lds + cb * 16 + q * 4);
+#pragma unroll
+                for (int rb = 0; rb < RB; ++rb) acc[rb][cb] = bias;
+            }
+
+            /* The matrix work, compiled twice: the usual tile touches nothing but LDS here; a tile with
+             * not-staged neighbours (wave-uniform choice) patches those lanes' operands from global memory. */
+            auto contract = [&](auto far_tag) {
+                constexpr bool FAR = decltype(far_tag)::value;
+                /* chunk = G consecutive steps of one slot: the lane's G inputs per row block ... */
+                auto gather = [&](int chunk, float (&x)[RB][G]) {
+                    const int sl = chunk / (STEPS / G), jg = chunk % (STEPS / G);
+#pragma unroll
+                    for (int rb = 0; rb < RB; ++rb) {
+                        const uint32_t at = (FAR && li[rb][sl] >= FAR_FROM) ? 0u : li[rb][sl];
+                        if constexpr (SWZ) {
+                            /* the lane's quarter row is pieces 2q and 2q+1, each moved by the row's low bits */
+                            static_assert(STEPS == 8 && G == 4, "swizzled rows are 8 pieces of 16 bytes");
+                            load_floats<G>(rows + at * RS + (((2 * q + jg) ^ (at & 7)) << 2), x[rb]);
+                        }
+                        else {
+                            load_floats<G>(rows + at * RS + q * STEPS + jg * G, x[rb]);
+                        }
+                    }
+                    if constexpr (FAR && NN > 0) {
+                        if (sl > 0) {
+#pragma unroll
+                            for (int rb = 0; rb < RB; ++rb) {
+                                if (li[rb][sl] >= FAR_FROM) {
+                                    const int g = B.row_nb[(size_t) (d_cur.x + li[rb][0]) * B.nb_stride + (sl - 1)];
+                                    load_floats<G>(in + (size_t) (d_cur.w + g) * C_IN + q * STEPS + jg * G, x[rb]);
+                                }
+                            }
+                        }
+                    }
+                };
+                /* ... and the weights of those steps, all column blocks */
+                auto weights = [&](int chunk, float (&a)[CB][G]) {
+                    const int sl = chunk / (STEPS / G), jg = chunk % (STEPS / G);
+#pragma unroll
+                    for (int cb = 0; cb < CB; ++cb) load_floats<G>(w_lds + (((sl * CB + cb) * (STEPS / G) + jg) * 64 + lane) * G, a[cb]);
+                };
+                /* Software pipeline: chunk c+1's operands are requested before chunk c's matrix instructions. The
+                 * side path runs unpipelined: it is rare, and its extra address registers would otherwise push the
+                 * staged rows of the next tile out of the register file. */
+                constexpr int CHUNKS = SLOTS * (STEPS / G);
+                constexpr int NBUF = FAR ? 1 : 2;
+                float x[NBUF][RB][G], a[NBUF][CB][G];
+                if constexpr (!FAR) {
+                    gather(0, x[0]);
+                    weights(0, a[0]);
+                }
+#pragma unroll
+                for (int c = 0; c < CHUNKS; ++c) {
+                    const int cur = FAR ? 0 : (c & 1);
+                    if constexpr (FAR) {
+                        gather(c, x[0]);
+                        weights(c, a[0]);
+                    }
+                    else if (c + 1 < CHUNKS) {
+                        gather(c + 1, x[cur ^ 1]);
+                        weights(c + 1, a[cur ^ 1]);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int e = 0; e < G; ++e)
+#pragma unroll
+                        for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+                            for (int rb = 0; rb < RB; ++rb)
+                                acc[rb][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[cur][cb][e], x[cur][rb][e], acc[rb][cb], 0, 0, 0);
+                    if constexpr (FAR) __builtin_amdgcn_sched_barrier(0);
+                }
+            };
+            VM_T_MARK(3)
+            if (any_far) contract(std::true_type());
+            else contract(std::false_type());
+            VM_T_MARK(4)
+            /* the next tile's neighbour positions: requested only now, when the operand registers are free */
+            if (has_next) request_positions(d_next, nbl_next);
+
+            /* activation: lane holds channels cb*16 + q*4 + {0..3} of row rb*16 + r16; one uniform branch */
+            auto for_each_value = [&](auto fn) {
+#pragma unroll
+                for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+                    for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+                        for (int v = 0; v < 4; ++v) acc[rb][cb][v] = fn(acc[rb][cb][v]);
+            };
+            if (activation == VMHIP_SELU) {
+                for_each_value([](float a) { return selu(a); });
+            }
+            else if (activation == VMHIP_RELU) {
+                for_each_value([](float a) { return fmaxf(a, 0.0f); });
+            }
+            else if (activation == VMHIP_TANH) {
+                for_each_value([](float a) { return tanhf(a); });
+            }
+            else {
+#pragma unroll
+                for (int rb = 0; rb < RB; ++rb) {
+                    float sum = 0.0f;
+#pragma unroll
+                    for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+                        for (int v = 0; v < 4; ++v) {
+                            const bool real = cb * 16 + q * 4 + v < C_OUT;
+                            const float e = real ? expf(acc[rb][cb][v]) : 0.0f;
+                            acc[rb][cb][v] = e;
+                            sum += e;
+                        }
+                    sum += __shfl_xor(sum, 16);
+                    sum += __shfl_xor(sum, 32);
+#pragma unroll
+                    for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+                        for (int v = 0; v < 4; ++v) acc[rb][cb][v] = acc[rb][cb][v] / sum;
+                }
+            }
+            VM_T_MARK(8)
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb) {
+                if (valid[rb]) {
+#pragma unroll
+                    for (int cb = 0; cb < CB; ++cb) store4<C_OUT>(out, (uint32_t) d_cur.x + li[rb][0], cb * 16 + q * 4, acc[rb][cb]);
+                }
+            }
+        }
+
+        VM_T_MARK(5)
+#ifdef VM_LDS_TIMING
+        t_acc[7] += 1;
+#endif
+        if (!has_next) break;
+        __syncthreads(); /* every wave is done reading this tile's rows */
+        VM_T_MARK(6)
+        d_cur = uniform(d_next);
+        d_next = d_after;
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) nbl[rb] = nbl_next[rb];
+        tile = next;
+        next = after;
+    }
+    VM_T_FLUSH
+}
+
+template <int C_IN, int C_OUT, int SLOTS>
+int launch_lds(const VmBatchDev& B, const VmLayerDev& L, const float* in, float* out, hipStream_t stream) {
+    constexpr int HALO = halo_rows(C_IN, C_OUT, SLOTS);
+    constexpr size_t lds = lds_bytes(C_IN, C_OUT, SLOTS, HALO);
+    static_assert(lds <= 160 * 1024, "weights and staged rows must fit the CU's LDS");
+    /* Two or more blocks of 8 waves per CU where LDS allows (registers are capped at 128 per lane, four waves
+     * per SIMD); otherwise one block of 16 waves. */
+    constexpr bool single = 2 * lds > 160 * 1024;
+    constexpr int NW = single ? 16 : 8;
+    auto kernel = vm_conv_lds_kernel<C_IN, C_OUT, SLOTS, NW, HALO>;
+    static bool configured = false;
+    if (!configured) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, int(lds)) != hipSuccess) {
+            (void) hipGetLastError();
+            return -1;
+        }
+        configured = true;
+    }
+    int per_cu = single ? 1 : 2;
+    if (const char* e = getenv("VMHIP_LDS_BLOCKS_PER_CU")) per_cu = atoi(e) > 0 ? atoi(e) : per_cu;
+    int grid = 256 * per_cu;
+    const int need = ((B.n_row_tiles + 7) / 8) * 8;
+    if (grid > need) grid = need;
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(NW * 64), lds, stream, B, L, in, out);
+    return 0;
+}
+
+}  // namespace
+
+#define VM_FOR_EACH_LDS_SHAPE(X) \
+    X(4, 16, 7)                  \
+    X(16, 16, 7)                 \
+    X(16, 32, 7)                 \
+    X(32, 32, 7)                 \
+    X(32, 16, 7)                 \
+    X(16, 3, 7)                  \
+    X(16, 2, 7)                  \
+    X(4, 64, 7)                  \
+    X(4, 24, 9)                  \
+    X(24, 24, 9)                 \
+    X(24, 4, 9)
+
+bool vm_lds_supported(int c_in, int c_out, int slots) {
+#define X(CI, CO, SL) \
+    if (c_in == CI && c_out == CO && slots == SL) return true;
+    VM_FOR_EACH_LDS_SHAPE(X)
+#undef X
+    return false;
+}
+
+int vm_launch_conv_lds(const VmBatchDev& B, const VmLayerDev& L, const float* in, float* out, hipStream_t stream, const char** kernel_name) {
+    if (B.n_row_tiles <= 0) return 0;
+    if (!B.row_nbl || !B.tile_halo || !B.tile_desc || !L.w_mfma || L.in_bf16 || L.out_bf16 || L.arith_bf16) return -1;
+#define X(CI, CO, SL)                                                       \
+    if (L.c_in == CI && L.c_out == CO && L.slots == SL) {                   \
+        if (kernel_name) *kernel_name = "conv_lds_" #CI "x" #CO "s" #SL;    \
+        return launch_lds<CI, CO, SL>(B, L, in, out, stream);               \
+    }
+    VM_FOR_EACH_LDS_SHAPE(X)
+#undef X
+    return -1;
+}

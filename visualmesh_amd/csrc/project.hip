@@ -329,16 +329,39 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_compact_kernel(VmBatchDev B, fl
     }
 }
 
-/* reference engine/cpu/engine.hpp:127-143: one thread per (row, neighbour) */
+/* reference engine/cpu/engine.hpp:127-143: one thread per (row, neighbour).
+ *
+ * When the batch carries tile-local tables the block also builds them for its tile: the neighbours that live in
+ * other tiles are deduplicated through an open-addressing hash in LDS, numbered densely in table order (the
+ * halo slots), and every neighbour is rewritten as a position in "own tile rows, then halo slots". Which row
+ * gets which halo slot depends on the order the atomics land in and may differ from run to run; the rows that a
+ * slot stands for, and so every result computed through the tables, do not. */
+#define NB_HASH 4096
 __global__ __launch_bounds__(VMHIP_TILE) void vm_neighbourhood_kernel(VmBatchDev B) {
+    __shared__ uint32_t h_key[NB_HASH];
+    __shared__ uint16_t h_dense[NB_HASH];
+    __shared__ int wave_total[VMHIP_TILE / 64];
+
     const int tile = blockIdx.x;
     const int f = find_frame_by_row_tile(B.frames, B.n_frames, tile);
     const VmFrame& F = B.frames[f];
     const int V = B.frame_V[f];
     const int nn = F.nn;
     const int row0 = (tile - F.row_tile0) * VMHIP_TILE;
-    if (row0 > V) return;
-    const int n_items = min(VMHIP_TILE, V + 1 - row0) * nn;
+    const bool tables = B.row_nbl != nullptr;
+    const int n_rows = max(0, min(VMHIP_TILE, V + 1 - row0));
+    if (n_rows == 0) {
+        if (tables && threadIdx.x == 0) B.tile_desc[tile] = make_int4(F.row_base + row0, 0, 0, F.row_base);
+        return;
+    }
+    constexpr uint32_t EMPTY = 0xffffffffu;
+    auto hash = [](uint32_t key) { return (key * 2654435761u) >> 20; }; /* 12 bits */
+    if (tables) {
+        for (int e = threadIdx.x; e < NB_HASH; e += VMHIP_TILE) h_key[e] = EMPTY;
+        __syncthreads();
+    }
+
+    const int n_items = n_rows * nn;
     for (int it = threadIdx.x; it < n_items; it += VMHIP_TILE) {
         const int i = row0 + it / nn;
         const int j = it - (it / nn) * nn;
@@ -350,6 +373,66 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_neighbourhood_kernel(VmBatchDev
             out = e.x == B.epoch ? (int) e.y : V;
         }
         B.row_nb[((size_t) F.row_base + i) * B.nb_stride + j] = out;
+        if (tables && (out < row0 || out >= row0 + VMHIP_TILE)) {
+            uint32_t slot = hash((uint32_t) out);
+            while (true) {
+                const uint32_t prev = atomicCAS(&h_key[slot], EMPTY, (uint32_t) out);
+                if (prev == EMPTY || prev == (uint32_t) out) break;
+                slot = (slot + 1) & (NB_HASH - 1);
+            }
+        }
+    }
+    if (!tables) return;
+    __syncthreads();
+
+    /* dense numbering of the occupied hash entries, in table order: 16 entries per thread, block-wide scan */
+    constexpr int PER = NB_HASH / VMHIP_TILE;
+    int mine = 0;
+#pragma unroll
+    for (int k = 0; k < PER; ++k) mine += h_key[threadIdx.x * PER + k] != EMPTY;
+    int scan = mine;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const int up = __shfl_up(scan, d);
+        if ((int) (threadIdx.x & 63) >= d) scan += up;
+    }
+    if ((threadIdx.x & 63) == 63) wave_total[threadIdx.x >> 6] = scan;
+    __syncthreads();
+    int before = scan - mine, total = 0;
+#pragma unroll
+    for (int w = 0; w < VMHIP_TILE / 64; ++w) {
+        if (w < (int) (threadIdx.x >> 6)) before += wave_total[w];
+        total += wave_total[w];
+    }
+    const int cap = B.halo_cap;
+#pragma unroll
+    for (int k = 0; k < PER; ++k) {
+        const int e = threadIdx.x * PER + k;
+        const uint32_t key = h_key[e];
+        if (key != EMPTY) {
+            h_dense[e] = (uint16_t) min(before, 0xffff);
+            if (before < cap) B.tile_halo[(size_t) tile * VMHIP_HALO_MAX + before] = (uint32_t) F.row_base + key;
+            ++before;
+        }
+    }
+    if (threadIdx.x == 0) B.tile_desc[tile] = make_int4(F.row_base + row0, n_rows, min(total, cap), F.row_base);
+    __syncthreads();
+
+    for (int it = threadIdx.x; it < n_items; it += VMHIP_TILE) {
+        const int i = row0 + it / nn;
+        const int j = it - (it / nn) * nn;
+        const int out = B.row_nb[((size_t) F.row_base + i) * B.nb_stride + j]; /* written above by this thread */
+        uint32_t local;
+        if (out >= row0 && out < row0 + VMHIP_TILE) {
+            local = (uint32_t) (out - row0);
+        }
+        else {
+            uint32_t slot = hash((uint32_t) out);
+            while (h_key[slot] != (uint32_t) out) slot = (slot + 1) & (NB_HASH - 1);
+            const int dense = h_dense[slot];
+            local = dense < cap ? (uint32_t) (VMHIP_TILE + dense) : VMHIP_NBL_FAR;
+        }
+        B.row_nbl[((size_t) F.row_base + i) * VMHIP_NBL_STRIDE + j] = (uint16_t) local;
     }
 }
 

@@ -12,6 +12,13 @@
  *                    indices, the neighbourhood table and the ping/pong activation matrices.
  * A tile never straddles two frames, so every block works for exactly one frame and finds it by a
  * binary search over the frames' first-tile numbers.
+ *
+ * Tile-local gather tables (built once per run next to the neighbourhood table, used by every layer):
+ * mesh order is spatially coherent, so most of a row's neighbours live in the row's own tile and the rest
+ * of a tile's neighbours are ~100 distinct rows of other tiles (its halo). tile_halo lists those rows,
+ * row_nbl holds every neighbour as a position in "the tile's 256 rows followed by its halo rows", and
+ * tile_desc describes the tile in one 16-byte word. A layer kernel copies tile + halo rows into LDS with
+ * coalesced loads and gathers from there.
  */
 #ifndef VMHIP_INTERNAL_H
 #define VMHIP_INTERNAL_H
@@ -23,6 +30,9 @@
 
 #define VMHIP_TILE 256
 #define VMHIP_AMB_CAP 2048 /* ambiguous candidates recorded per frame */
+#define VMHIP_HALO_MAX 256 /* rows of other tiles that a row tile can stage next to its own 256 rows */
+#define VMHIP_NBL_STRIDE 8 /* tile-local neighbour table: 8 x uint16 per row */
+#define VMHIP_NBL_FAR 0xffffu /* tile-local neighbour entry: not staged, read the row from global memory */
 
 /* image sampling kinds (derived from the fourcc on the host) */
 enum {
@@ -84,6 +94,11 @@ struct VmBatchDev {
     int32_t* row_gidx;
     int32_t* row_nb;      /* [rows][nn_max] with the frame's own nn as stride */
     int32_t nb_stride;
+    /* tile-local gather tables (null unless the batch classifies and nn <= VMHIP_NBL_STRIDE) */
+    uint16_t* row_nbl;    /* [rows][VMHIP_NBL_STRIDE]: 0..255 own tile, 256+h halo slot h, VMHIP_NBL_FAR not staged */
+    uint32_t* tile_halo;  /* [n_row_tiles][VMHIP_HALO_MAX] batch-global row of each halo slot */
+    int4* tile_desc;      /* [n_row_tiles] {first batch-global row, rows in use (0..256), halo rows, frame's row_base} */
+    int32_t halo_cap;     /* halo slots handed out per tile, <= VMHIP_HALO_MAX (smaller only to test the far path) */
 };
 
 /* Layer descriptor on the device side (host struct, passed by value to launchers). */
@@ -106,7 +121,7 @@ void vm_launch_copy_probe(const void* src, void* dst, size_t bytes, hipStream_t 
 void vm_launch_reset(const VmBatchDev& B, hipStream_t stream);
 void vm_launch_project(const VmBatchDev& B, hipStream_t stream);
 void vm_launch_compact(const VmBatchDev& B, float* feat, int classify, hipStream_t stream);
-void vm_launch_neighbourhood(const VmBatchDev& B, hipStream_t stream);
+void vm_launch_neighbourhood(const VmBatchDev& B, hipStream_t stream); /* also the tile-local tables if B.row_nbl */
 /* in -> out over the row space; returns 0 or a negative status if the shape is unsupported */
 int vm_launch_conv(const VmBatchDev& B, const VmLayerDev& L, const float* in, float* out, hipStream_t stream,
                    const char** kernel_name);
@@ -117,6 +132,12 @@ size_t vm_mfma_weight_bytes(int c_in, int c_out, int slots, int arith_bf16);
 void vm_mfma_permute_weights(const float* w, int c_in, int c_out, int slots, int arith_bf16, void* wp);
 int vm_launch_conv_mfma(const VmBatchDev& B, const VmLayerDev& L, const void* in, void* out, hipStream_t stream,
                         const char** kernel_name);
+
+/* matrix-core variant gathering from LDS through the tile-local tables (conv_lds.hip); fp32 rows and arithmetic,
+ * weights in vm_mfma_permute_weights' fp32 order */
+bool vm_lds_supported(int c_in, int c_out, int slots);
+int vm_launch_conv_lds(const VmBatchDev& B, const VmLayerDev& L, const float* in, float* out, hipStream_t stream,
+                       const char** kernel_name);
 
 #include "host_project.h"
 
