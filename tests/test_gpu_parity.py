@@ -161,7 +161,7 @@ def test_bf16_engine(oracle):
     engine.profile(True)
     engine.run()
     names = [n for n, _, _ in engine.profile_read() if n.startswith("conv")]
-    assert names == ["conv_lds_4x64s7", "conv_bf16x3_tobf16_64x64s7", "conv_bf16x2_tof32_64x64s7", "conv_bf16x3_tobf16_64x64s7",
+    assert names == ["conv_mfma_4x64s7", "conv_bf16x3_tobf16_64x64s7", "conv_bf16x2_tof32_64x64s7", "conv_bf16x3_tobf16_64x64s7",
                      "conv_bf16x2_tof32_64x64s7", "conv_bf16x3_64x64s7"], names
     worst = 0.0
     for i, f in enumerate(cfg.frames):
@@ -216,6 +216,7 @@ def test_rows_beyond_the_halo_capacity(oracle, index, monkeypatch):
     """With only 8 halo slots per tile most out-of-tile neighbours are marked as not staged and the LDS kernel
     reads them from global memory: same results (configuration 2's Ring6 and 3's NMGrid8 networks)."""
     monkeypatch.setenv("VMHIP_HALO_CAP", "8")
+    monkeypatch.setenv("VMHIP_CONV_KERNEL", "lds")
     cfg = wl.config(index, n_frames=1)
     o_lens, e_lens = lens_pair(cfg)
     o_mesh, e_mesh = meshes_for(cfg, oracle)

@@ -572,11 +572,13 @@ int vmhip_engine_create(const vmhip_network* net, int32_t n_neighbours, int32_t 
      * is only made where the kernels on both sides of the boundary exist for it. */
     {
         /* VMHIP_CONV_KERNEL selects the kernel family for A/B runs: "rows" = one row per lane, "mfma" = matrix
-         * cores gathering into registers, "lds" (default) = matrix cores gathering from LDS where the shape
-         * has an instantiation and the register-gather kernel elsewhere */
+         * cores gathering into registers, "lds" = matrix cores gathering from LDS
+         * wherever the shape has an instantiation; unset = the register-gather kernel where it has an
+         * instantiation, one row per lane elsewhere */
         const char* pick = getenv("VMHIP_CONV_KERNEL");
         const bool rows_only = pick && std::string(pick) == "rows";
         const bool allow_lds = !rows_only && !(pick && std::string(pick) == "mfma");
+        const bool force_lds = pick && std::string(pick) == "lds";
         if (const char* cap = getenv("VMHIP_HALO_CAP")) E->halo_cap = std::min(std::max(atoi(cap), 0), VMHIP_HALO_MAX);
         const int n = int(E->layers.size());
         std::vector<int> bf(n + 1, 0); /* bf[l] = rows entering layer l are bf16; bf[n] = final output (never) */
@@ -609,6 +611,9 @@ int vmhip_engine_create(const vmhip_network* net, int32_t n_neighbours, int32_t 
             const bool plain = !H.in_bf16 && !H.out_bf16 && !H.arith_bf16;
             H.use_mfma = !rows_only && vm_mfma_supported(H.c_in, H.c_out, H.slots, H.in_bf16, H.out_bf16, H.arith_bf16);
             H.use_lds = allow_lds && plain && H.slots - 1 <= VMHIP_NBL_STRIDE && vm_lds_supported(H.c_in, H.c_out, H.slots);
+            /* Measured on the 16-frame 1280x1024 workload: the LDS gather wins only on the 4-channel first layer
+             * (34 us against 45 us) and building its tables costs 40 us per run, so it is opt-in for now. */
+            if (!force_lds) H.use_lds = false;
             E->use_lds = E->use_lds || H.use_lds;
             if (H.use_mfma || H.use_lds) {
                 std::vector<unsigned char> wp(vm_mfma_weight_bytes(H.c_in, H.c_out, H.slots, H.arith_bf16));
