@@ -88,21 +88,9 @@ __device__ __forceinline__ void load_floats(const float* __restrict__ p, float (
     }
 }
 
-template <int C_OUT>
-__device__ __forceinline__ void store4(float* __restrict__ out, uint32_t row, int o, v4f v) {
-    float* y = out + (size_t) row * C_OUT + o;
-    if constexpr (C_OUT % 4 == 0) {
-        if (o < C_OUT) *reinterpret_cast<float4*>(y) = make_float4(v[0], v[1], v[2], v[3]);
-    }
-    else {
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-            if (o + i < C_OUT) y[i] = v[i];
-    }
-}
-
 /* the k-th 16-bit entry of a row of the tile-local neighbour table */
-__device__ __forceinline__ uint32_t nbl_entry(const uint4& t, int k) {
+typedef uint32_t v4u32 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint32_t nbl_entry(const v4u32& t, int k) {
     const uint32_t w = (k >> 1) == 0 ? t.x : (k >> 1) == 1 ? t.y : (k >> 1) == 2 ? t.z : t.w;
     return (k & 1) ? (w >> 16) : (w & 0xffffu);
 }
@@ -159,7 +147,6 @@ __global__ __launch_bounds__(NW * 64, 4) void vm_conv_lds_kernel(VmBatchDev B, V
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int q = lane >> 4, r16 = lane & 15;
     const int activation = L.activation;
-    const v4f* __restrict__ in4 = reinterpret_cast<const v4f*>(in);
 
     const int n_tiles = B.n_row_tiles;
     const int xcd = blockIdx.x & 7, lb = blockIdx.x >> 3, gx = gridDim.x >> 3;
@@ -168,113 +155,119 @@ __global__ __launch_bounds__(NW * 64, 4) void vm_conv_lds_kernel(VmBatchDev B, V
     int tile = xcd * per_xcd + lb;
     if (tile >= t_end) return; /* the whole block leaves: no barrier is left waiting */
 
-    /* ---- staging helpers: thread-private pieces of the next tile ---- */
-    v4f st_main[N_MAIN] = {}, st_halo[N_HALO] = {};
-    uint32_t hrow[N_HALO] = {};
+    /* ---- staging: thread-private pieces of the next tile ----
+     * Every global read of the tile loop is an unconditional buffer load with a 32-bit offset: out-of-range
+     * offsets (stale halo entries, tiles past the end) read zeros instead of faulting, so there are no branches
+     * around the loads and the compiler can wait for exactly the loads it needs (vector-memory operations retire
+     * in order; a branch would force it to wait for all of them, stores included). */
+    typedef uint32_t v4u __attribute__((ext_vector_type(4)));
+    const uint32_t total_rows = (uint32_t) n_tiles * VMHIP_TILE;
+    auto make_rsrc = [](const void* p, uint64_t bytes) {
+        return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int) (bytes > 0xffffffffull ? 0xffffffffu : (uint32_t) bytes), 0x00020000);
+    };
+    const __amdgpu_buffer_rsrc_t in_rsrc = make_rsrc(in, (uint64_t) total_rows * C_IN * 4);
+    const __amdgpu_buffer_rsrc_t nbl_rsrc = make_rsrc(B.row_nbl, (uint64_t) total_rows * VMHIP_NBL_STRIDE * 2);
+    const __amdgpu_buffer_rsrc_t halo_rsrc = make_rsrc(B.tile_halo, (uint64_t) n_tiles * VMHIP_HALO_MAX * 4);
+    const __amdgpu_buffer_rsrc_t desc_rsrc = make_rsrc(B.tile_desc, (uint64_t) n_tiles * 16);
+
+    v4u st_main[N_MAIN], st_halo[N_HALO];
+    uint32_t hrow[N_HALO];
     auto request_halo_rows = [&](int t) {
 #pragma unroll
         for (int k = 0; k < N_HALO; ++k) {
-            const int idx = threadIdx.x + k * NT;
-            const int h = idx / Q4;
-            hrow[k] = h < HALO ? B.tile_halo[(size_t) t * VMHIP_HALO_MAX + h] : 0u; /* entries past the tile's count are not used */
+            const int h = (threadIdx.x + k * NT) / Q4; /* entries past the tile's count are stale and unused */
+            hrow[k] = __builtin_amdgcn_raw_buffer_load_b32(halo_rsrc, (t * VMHIP_HALO_MAX + h) * 4, 0, 0);
         }
     };
+    /* d = {first row, rows in use, halo rows, frame's first row}, still in vector registers */
     auto request_rows = [&](const int4& d) {
 #pragma unroll
-        for (int k = 0; k < N_MAIN; ++k) {
-            const int idx = threadIdx.x + k * NT;
-            if (idx < VMHIP_TILE * Q4 && d.y > 0) st_main[k] = in4[(size_t) d.x * Q4 + idx];
-        }
+        for (int k = 0; k < N_MAIN; ++k) st_main[k] = __builtin_amdgcn_raw_buffer_load_b128(in_rsrc, (d.x * Q4 + (int) threadIdx.x + k * NT) * 16, 0, 0);
 #pragma unroll
         for (int k = 0; k < N_HALO; ++k) {
             const int idx = threadIdx.x + k * NT;
-            const int h = idx / Q4, c = idx - h * Q4;
-            if (h < min(d.z, HALO)) st_halo[k] = in4[(size_t) hrow[k] * Q4 + c];
+            const int c = idx % Q4;
+            st_halo[k] = __builtin_amdgcn_raw_buffer_load_b128(in_rsrc, (hrow[k] * Q4 + c) * 16, 0, 0);
         }
     };
-    auto write_rows = [&](const int4& d) {
-        v4f* rows4 = reinterpret_cast<v4f*>(rows);
+    auto write_rows = [&]() {
+        v4u* rows4 = reinterpret_cast<v4u*>(rows);
 #pragma unroll
         for (int k = 0; k < N_MAIN; ++k) {
             const int idx = threadIdx.x + k * NT;
             const int r = idx / Q4, c = idx - r * Q4;
-            if (idx < VMHIP_TILE * Q4 && d.y > 0) rows4[(r * RS) / 4 + (SWZ ? (c ^ (r & 7)) : c)] = st_main[k];
+            if (N_MAIN * NT == VMHIP_TILE * Q4 || idx < VMHIP_TILE * Q4) rows4[(r * RS) / 4 + (SWZ ? (c ^ (r & 7)) : c)] = st_main[k];
         }
 #pragma unroll
         for (int k = 0; k < N_HALO; ++k) {
             const int idx = threadIdx.x + k * NT;
             const int h = idx / Q4, c = idx - h * Q4;
-            if (h < min(d.z, HALO)) rows4[((VMHIP_TILE + h) * RS) / 4 + (SWZ ? (c ^ (h & 7)) : c)] = st_halo[k];
+            if (N_HALO * NT == HALO * Q4 || h < HALO) rows4[((VMHIP_TILE + h) * RS) / 4 + (SWZ ? (c ^ (h & 7)) : c)] = st_halo[k];
         }
     };
     /* the lane's rows of a tile: rows past the tile's count compute on its last row (the frame's null row) and
      * skip the store */
-    auto own_row = [&](const int4& d, int rb) { return max(0, min(wave * (RB * 16) + rb * 16 + r16, d.y - 1)); };
-    auto request_positions = [&](const int4& d, uint4 (&nbl)[RB]) {
+    auto own_row = [&](int rows_in_use, int rb) { return max(0, min(wave * (RB * 16) + rb * 16 + r16, rows_in_use - 1)); };
+    auto request_positions = [&](const int4& d, v4u (&nbl)[RB]) {
         if constexpr (NN > 0) {
 #pragma unroll
-            for (int rb = 0; rb < RB; ++rb)
-                if (d.y > 0) nbl[rb] = *reinterpret_cast<const uint4*>(B.row_nbl + (size_t) (d.x + own_row(d, rb)) * VMHIP_NBL_STRIDE);
+            for (int rb = 0; rb < RB; ++rb) nbl[rb] = __builtin_amdgcn_raw_buffer_load_b128(nbl_rsrc, (d.x + own_row(d.y, rb)) * (VMHIP_NBL_STRIDE * 2), 0, 0);
         }
     };
-
     /* Tile descriptors are wave-uniform but must not be fetched with scalar loads: scalar loads return out of
      * order on the counter that LDS reads use too, so one descriptor in flight would turn every LDS wait of the
-     * matrix loop into a wait for that (global-latency) load. A buffer load is a vector-memory instruction. */
-    const __amdgpu_buffer_rsrc_t desc_rsrc = __builtin_amdgcn_make_buffer_rsrc(B.tile_desc, 0, n_tiles * 16, 0x00020000);
+     * matrix loop into a wait for that (global-latency) load. */
     auto load_desc = [&](int t) {
-        typedef int v4i __attribute__((ext_vector_type(4)));
-        const v4i d = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(desc_rsrc, t * 16, 0, 0));
-        return make_int4(d.x, d.y, d.z, d.w);
+        const v4u d = __builtin_amdgcn_raw_buffer_load_b128(desc_rsrc, t * 16, 0, 0);
+        return make_int4((int) d.x, (int) d.y, (int) d.z, (int) d.w);
     };
-    auto uniform = [](const int4& d) {
+    /* to scalar registers; the empty asm keeps the compiler from doing this (and so waiting for the load) early */
+    auto uniform = [](int4 d) {
+        asm volatile("" : "+v"(d.x), "+v"(d.y), "+v"(d.z), "+v"(d.w));
         return make_int4(__builtin_amdgcn_readfirstlane(d.x), __builtin_amdgcn_readfirstlane(d.y), __builtin_amdgcn_readfirstlane(d.z),
                          __builtin_amdgcn_readfirstlane(d.w));
     };
 
-    /* ---- prologue: everything tile `tile` needs, then the look-ahead for the next one ---- */
+    /* ---- prologue: everything tile `tile` needs, then the look-ahead for the next one. Tiles past the end of
+     * the block's share are clamped to its last tile: their loads are redundant, never wrong. ---- */
+    const int t_last = t_end - 1;
     int4 d_cur = uniform(load_desc(tile));
     int next = tile + gx;
-    int4 d_next = make_int4(0, 0, 0, 0), d_after = make_int4(0, 0, 0, 0);
-    uint4 nbl[RB], nbl_next[RB];
+    v4u nbl[RB], nbl_next[RB];
     request_halo_rows(tile);
     request_rows(d_cur);
     request_positions(d_cur, nbl);
-    if (next < t_end) {
-        d_next = load_desc(next);
-        request_halo_rows(next);
-    }
+    int4 d_next = load_desc(min(next, t_last)), d_after = d_next;
+    request_halo_rows(min(next, t_last));
 
     VM_T_DECL
     while (true) {
-        write_rows(d_cur);
+        write_rows();
         VM_T_MARK(0)
         __syncthreads(); /* rows (and, the first time, weights) are in LDS */
         VM_T_MARK(1)
 
         const bool has_next = next < t_end;
         const int after = next + gx;
-        if (has_next) {
-            request_rows(d_next);
-            if (after < t_end) {
-                d_after = load_desc(after);
-                request_halo_rows(after);
-            }
-        }
+        request_rows(d_next);
+        d_after = load_desc(min(after, t_last));
+        request_halo_rows(min(after, t_last));
         __builtin_amdgcn_sched_barrier(0);
         VM_T_MARK(2)
 
-        if (d_cur.y > 0) {
+        {
+            /* an empty tile (no rows in use) runs the same code on position 0 and stores nothing */
+            const bool in_use = d_cur.y > 0;
             uint32_t li[RB][SLOTS];
             bool valid[RB];
             bool far = false;
 #pragma unroll
             for (int rb = 0; rb < RB; ++rb) {
                 valid[rb] = wave * (RB * 16) + rb * 16 + r16 < d_cur.y;
-                li[rb][0] = (uint32_t) own_row(d_cur, rb);
+                li[rb][0] = (uint32_t) own_row(d_cur.y, rb);
 #pragma unroll
                 for (int s = 0; s < NN; ++s) {
-                    li[rb][s + 1] = nbl_entry(nbl[rb], s);
+                    li[rb][s + 1] = in_use ? nbl_entry(nbl[rb], s) : 0u;
                     far |= li[rb][s + 1] >= FAR_FROM;
                 }
             }
@@ -330,21 +323,28 @@ __global__ __launch_bounds__(NW * 64, 4) void vm_conv_lds_kernel(VmBatchDev B, V
                  * staged rows of the next tile out of the register file. */
                 constexpr int CHUNKS = SLOTS * (STEPS / G);
                 constexpr int NBUF = FAR ? 1 : 2;
-                float x[NBUF][RB][G], a[NBUF][CB][G];
+                /* weights are double-buffered only where registers allow (16 accumulator registers leave no room) */
+                constexpr int ABUF = (FAR || RB * CB * 4 >= 16) ? 1 : 2;
+                float x[NBUF][RB][G], a[ABUF][CB][G];
                 if constexpr (!FAR) {
                     gather(0, x[0]);
-                    weights(0, a[0]);
+                    if constexpr (ABUF == 2) weights(0, a[0]);
                 }
 #pragma unroll
                 for (int c = 0; c < CHUNKS; ++c) {
                     const int cur = FAR ? 0 : (c & 1);
+                    const int acur = ABUF == 2 ? (c & 1) : 0;
                     if constexpr (FAR) {
                         gather(c, x[0]);
-                        weights(c, a[0]);
                     }
                     else if (c + 1 < CHUNKS) {
                         gather(c + 1, x[cur ^ 1]);
-                        weights(c + 1, a[cur ^ 1]);
+                    }
+                    if constexpr (ABUF == 1) {
+                        weights(c, a[0]);
+                    }
+                    else if (c + 1 < CHUNKS) {
+                        weights(c + 1, a[acur ^ 1]);
                     }
                     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -353,16 +353,15 @@ __global__ __launch_bounds__(NW * 64, 4) void vm_conv_lds_kernel(VmBatchDev B, V
                         for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
                             for (int rb = 0; rb < RB; ++rb)
-                                acc[rb][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[cur][cb][e], x[cur][rb][e], acc[rb][cb], 0, 0, 0);
-                    if constexpr (FAR) __builtin_amdgcn_sched_barrier(0);
+                                acc[rb][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[acur][cb][e], x[cur][rb][e], acc[rb][cb], 0, 0, 0);
+                    if constexpr (FAR || ABUF == 1) __builtin_amdgcn_sched_barrier(0);
                 }
             };
-            VM_T_MARK(3)
             if (any_far) contract(std::true_type());
             else contract(std::false_type());
             VM_T_MARK(4)
             /* the next tile's neighbour positions: requested only now, when the operand registers are free */
-            if (has_next) request_positions(d_next, nbl_next);
+            request_positions(d_next, nbl_next);
 
             /* activation: lane holds channels cb*16 + q*4 + {0..3} of row rb*16 + r16; one uniform branch */
             auto for_each_value = [&](auto fn) {
@@ -404,11 +403,25 @@ __global__ __launch_bounds__(NW * 64, 4) void vm_conv_lds_kernel(VmBatchDev B, V
                 }
             }
             VM_T_MARK(8)
+            /* buffer stores relative to the tile's first output row; lanes without a row get an out-of-range
+             * offset, which the hardware drops: no branch around the stores either */
+            const __amdgpu_buffer_rsrc_t out_rsrc = make_rsrc(out + (size_t) d_cur.x * C_OUT, (uint64_t) VMHIP_TILE * C_OUT * 4);
 #pragma unroll
             for (int rb = 0; rb < RB; ++rb) {
-                if (valid[rb]) {
 #pragma unroll
-                    for (int cb = 0; cb < CB; ++cb) store4<C_OUT>(out, (uint32_t) d_cur.x + li[rb][0], cb * 16 + q * 4, acc[rb][cb]);
+                for (int cb = 0; cb < CB; ++cb) {
+                    const int o = cb * 16 + q * 4;
+                    const uint32_t at = (li[rb][0] * C_OUT + o) * 4;
+                    if constexpr (C_OUT % 4 == 0) {
+                        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, acc[rb][cb]), out_rsrc, (valid[rb] && o < C_OUT) ? at : 0xffffffffu, 0, 0);
+                    }
+                    else {
+#pragma unroll
+                        for (int v = 0; v < 4; ++v)
+                            if (cb * 16 + v < C_OUT) /* compile-time: some lane group holds a real channel here */
+                                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(acc[rb][cb][v]), out_rsrc,
+                                                                      (valid[rb] && o + v < C_OUT) ? at + v * 4 : 0xffffffffu, 0, 0);
+                    }
                 }
             }
         }
@@ -435,6 +448,8 @@ int launch_lds(const VmBatchDev& B, const VmLayerDev& L, const float* in, float*
     constexpr int HALO = halo_rows(C_IN, C_OUT, SLOTS);
     constexpr size_t lds = lds_bytes(C_IN, C_OUT, SLOTS, HALO);
     static_assert(lds <= 160 * 1024, "weights and staged rows must fit the CU's LDS");
+    /* the kernel addresses its input rows with 32-bit byte offsets */
+    if ((uint64_t) B.n_row_tiles * VMHIP_TILE * C_IN * 4 > 0xffffffffull) return -1;
     /* Two or more blocks of 8 waves per CU where LDS allows (registers are capped at 128 per lane, four waves
      * per SIMD); otherwise one block of 16 waves. */
     constexpr bool single = 2 * lds > 160 * 1024;
