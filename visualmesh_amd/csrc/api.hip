@@ -573,8 +573,7 @@ int vmhip_engine_create(const vmhip_network* net, int32_t n_neighbours, int32_t 
     {
         /* VMHIP_CONV_KERNEL selects the kernel family for A/B runs: "rows" = one row per lane, "mfma" = matrix
          * cores gathering into registers, "lds" = matrix cores gathering from LDS
-         * wherever the shape has an instantiation; unset = the register-gather kernel where it has an
-         * instantiation, one row per lane elsewhere */
+         * wherever the shape has an instantiation; unset = the fastest measured kernel per layer shape */
         const char* pick = getenv("VMHIP_CONV_KERNEL");
         const bool rows_only = pick && std::string(pick) == "rows";
         const bool allow_lds = !rows_only && !(pick && std::string(pick) == "mfma");
@@ -611,9 +610,10 @@ int vmhip_engine_create(const vmhip_network* net, int32_t n_neighbours, int32_t 
             const bool plain = !H.in_bf16 && !H.out_bf16 && !H.arith_bf16;
             H.use_mfma = !rows_only && vm_mfma_supported(H.c_in, H.c_out, H.slots, H.in_bf16, H.out_bf16, H.arith_bf16);
             H.use_lds = allow_lds && plain && H.slots - 1 <= VMHIP_NBL_STRIDE && vm_lds_supported(H.c_in, H.c_out, H.slots);
-            /* Measured on the 16-frame 1280x1024 workload: the LDS gather wins only on the 4-channel first layer
-             * (34 us against 45 us) and building its tables costs 40 us per run, so it is opt-in for now. */
-            if (!force_lds) H.use_lds = false;
+            /* Measured on the 16-frame 1280x1024 workload: the LDS gather is the faster matrix-core kernel on every
+             * shape it has (32->32: 157 us against 166 us, 32->16: 89 against 122, 4->16: 29 against 44); only the
+             * 2- and 3-class output layers are quicker with one row per lane (46 us against 56 us). */
+            if (H.use_lds && !force_lds && H.c_out < 4) H.use_lds = false;
             E->use_lds = E->use_lds || H.use_lds;
             if (H.use_mfma || H.use_lds) {
                 std::vector<unsigned char> wp(vm_mfma_weight_bytes(H.c_in, H.c_out, H.slots, H.arith_bf16));
