@@ -338,7 +338,7 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_compact_kernel(VmBatchDev B, fl
  * slot stands for, and so every result computed through the tables, do not. */
 #define NB_HASH 4096
 __global__ __launch_bounds__(VMHIP_TILE) void vm_neighbourhood_kernel(VmBatchDev B) {
-    __shared__ uint32_t h_key[NB_HASH];
+    __shared__ __align__(16) uint32_t h_key[NB_HASH];
     __shared__ uint16_t h_dense[NB_HASH];
     __shared__ int wave_total[VMHIP_TILE / 64];
 
@@ -357,12 +357,16 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_neighbourhood_kernel(VmBatchDev
     constexpr uint32_t EMPTY = 0xffffffffu;
     auto hash = [](uint32_t key) { return (key * 2654435761u) >> 20; }; /* 12 bits */
     if (tables) {
-        for (int e = threadIdx.x; e < NB_HASH; e += VMHIP_TILE) h_key[e] = EMPTY;
+        for (int e = threadIdx.x * 4; e < NB_HASH; e += VMHIP_TILE * 4) *reinterpret_cast<uint4*>(&h_key[e]) = make_uint4(EMPTY, EMPTY, EMPTY, EMPTY);
         __syncthreads();
     }
 
+    /* (row, neighbour) items are dealt round-robin to the threads; a thread keeps its items' results in registers
+     * between the passes (the tables are only built for nn <= VMHIP_NBL_STRIDE, so at most 8 items per thread) */
     const int n_items = n_rows * nn;
-    for (int it = threadIdx.x; it < n_items; it += VMHIP_TILE) {
+    constexpr int MAX_ITEMS = VMHIP_NBL_STRIDE;
+    int outs[MAX_ITEMS];
+    auto resolve = [&](int it) {
         const int i = row0 + it / nn;
         const int j = it - (it / nn) * nn;
         int out = V;
@@ -373,23 +377,42 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_neighbourhood_kernel(VmBatchDev
             out = e.x == B.epoch ? (int) e.y : V;
         }
         B.row_nb[((size_t) F.row_base + i) * B.nb_stride + j] = out;
-        if (tables && (out < row0 || out >= row0 + VMHIP_TILE)) {
-            uint32_t slot = hash((uint32_t) out);
-            while (true) {
-                const uint32_t prev = atomicCAS(&h_key[slot], EMPTY, (uint32_t) out);
-                if (prev == EMPTY || prev == (uint32_t) out) break;
-                slot = (slot + 1) & (NB_HASH - 1);
+        return out;
+    };
+    if (!tables) {
+        for (int it = threadIdx.x; it < n_items; it += VMHIP_TILE) resolve(it);
+        return;
+    }
+#pragma unroll
+    for (int k = 0; k < MAX_ITEMS; ++k) {
+        const int it = threadIdx.x + k * VMHIP_TILE;
+        outs[k] = -1;
+        if (it < n_items) {
+            const int out = resolve(it);
+            outs[k] = out;
+            if (out < row0 || out >= row0 + VMHIP_TILE) {
+                uint32_t slot = hash((uint32_t) out);
+                while (true) {
+                    const uint32_t prev = atomicCAS(&h_key[slot], EMPTY, (uint32_t) out);
+                    if (prev == EMPTY || prev == (uint32_t) out) break;
+                    slot = (slot + 1) & (NB_HASH - 1);
+                }
             }
         }
     }
-    if (!tables) return;
     __syncthreads();
 
     /* dense numbering of the occupied hash entries, in table order: 16 entries per thread, block-wide scan */
     constexpr int PER = NB_HASH / VMHIP_TILE;
+    uint32_t keys[PER];
+#pragma unroll
+    for (int k = 0; k < PER; k += 4) {
+        const uint4 t = *reinterpret_cast<const uint4*>(&h_key[threadIdx.x * PER + k]);
+        keys[k] = t.x, keys[k + 1] = t.y, keys[k + 2] = t.z, keys[k + 3] = t.w;
+    }
     int mine = 0;
 #pragma unroll
-    for (int k = 0; k < PER; ++k) mine += h_key[threadIdx.x * PER + k] != EMPTY;
+    for (int k = 0; k < PER; ++k) mine += keys[k] != EMPTY;
     int scan = mine;
 #pragma unroll
     for (int d = 1; d < 64; d <<= 1) {
@@ -405,34 +428,38 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_neighbourhood_kernel(VmBatchDev
         total += wave_total[w];
     }
     const int cap = B.halo_cap;
+    if (mine > 0) {
 #pragma unroll
-    for (int k = 0; k < PER; ++k) {
-        const int e = threadIdx.x * PER + k;
-        const uint32_t key = h_key[e];
-        if (key != EMPTY) {
-            h_dense[e] = (uint16_t) min(before, 0xffff);
-            if (before < cap) B.tile_halo[(size_t) tile * VMHIP_HALO_MAX + before] = (uint32_t) F.row_base + key;
-            ++before;
+        for (int k = 0; k < PER; ++k) {
+            if (keys[k] != EMPTY) {
+                h_dense[threadIdx.x * PER + k] = (uint16_t) min(before, 0xffff);
+                if (before < cap) B.tile_halo[(size_t) tile * VMHIP_HALO_MAX + before] = (uint32_t) F.row_base + keys[k];
+                ++before;
+            }
         }
     }
     if (threadIdx.x == 0) B.tile_desc[tile] = make_int4(F.row_base + row0, n_rows, min(total, cap), F.row_base);
     __syncthreads();
 
-    for (int it = threadIdx.x; it < n_items; it += VMHIP_TILE) {
-        const int i = row0 + it / nn;
-        const int j = it - (it / nn) * nn;
-        const int out = B.row_nb[((size_t) F.row_base + i) * B.nb_stride + j]; /* written above by this thread */
-        uint32_t local;
-        if (out >= row0 && out < row0 + VMHIP_TILE) {
-            local = (uint32_t) (out - row0);
+#pragma unroll
+    for (int k = 0; k < MAX_ITEMS; ++k) {
+        const int it = threadIdx.x + k * VMHIP_TILE;
+        const int out = outs[k];
+        if (out >= 0) {
+            uint32_t local;
+            if (out >= row0 && out < row0 + VMHIP_TILE) {
+                local = (uint32_t) (out - row0);
+            }
+            else {
+                uint32_t slot = hash((uint32_t) out);
+                while (h_key[slot] != (uint32_t) out) slot = (slot + 1) & (NB_HASH - 1);
+                const int dense = h_dense[slot];
+                local = dense < cap ? (uint32_t) (VMHIP_TILE + dense) : VMHIP_NBL_FAR;
+            }
+            const int i = row0 + it / nn;
+            const int j = it - (it / nn) * nn;
+            B.row_nbl[((size_t) F.row_base + i) * VMHIP_NBL_STRIDE + j] = (uint16_t) local;
         }
-        else {
-            uint32_t slot = hash((uint32_t) out);
-            while (h_key[slot] != (uint32_t) out) slot = (slot + 1) & (NB_HASH - 1);
-            const int dense = h_dense[slot];
-            local = dense < cap ? (uint32_t) (VMHIP_TILE + dense) : VMHIP_NBL_FAR;
-        }
-        B.row_nbl[((size_t) F.row_base + i) * VMHIP_NBL_STRIDE + j] = (uint16_t) local;
     }
 }
 
