@@ -145,10 +145,12 @@ int vmhip_batch_counts(const vmhip_batch* batch, int32_t* n_visible);
 int vmhip_batch_fetch(vmhip_batch* batch, vmhip_result* results);
 
 /* Per-kernel timing of vmhip_batch_run with HIP events on the stream the kernels run on.
- * enable != 0 brackets every kernel launch of later runs with events. After a run,
- * vmhip_batch_profile_read returns, for kernel slot i < *n_slots, its name (static string), the
+ * enable = 1 brackets every kernel launch of later runs with events (an event pair between two
+ * kernels costs a few microseconds of idle GPU); enable = 2, valid after a run made with enable = 1,
+ * brackets only the launches of the kernel that took longest in that run; 0 switches timing off.
+ * After a run, vmhip_batch_profile_read returns, for kernel slot i < *n_slots, its name (static string), the
  * duration in milliseconds of its launch in the last run and the rows (nodes incl. null rows) or
- * candidates it processed. Slots are in launch order. */
+ * candidates it processed. Slots are in launch order (with enable = 2: the bracketed launches only). */
 int vmhip_batch_profile(vmhip_batch* batch, int32_t enable);
 int vmhip_batch_profile_read(vmhip_batch* batch, int32_t max_slots, int32_t* n_slots, const char** names,
                              float* milliseconds, int64_t* units);

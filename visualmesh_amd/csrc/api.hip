@@ -6,6 +6,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <map>
 #include <string>
 #include <vector>
 
@@ -131,6 +132,11 @@ struct vmhip_batch {
     std::vector<HostFrame> frames;
     std::vector<int32_t> h_V, h_amb_count;
     std::vector<int2> h_amb;
+    /* pinned landing area of the per-run download: V[n], ambiguity count[n], then the first AMB_HEAD entries of
+     * every frame's ambiguity list, so that one wait per run covers everything the host normally needs */
+    static constexpr int AMB_HEAD = 64;
+    void* h_pin = nullptr;
+    size_t h_pin_cap = 0;
     std::vector<uint64_t> h_force_valid, h_force_keep;
     bool have_run = false;
     uint32_t epoch = 0;
@@ -138,11 +144,12 @@ struct vmhip_batch {
 
     VmBatchDev dev{};
     DevBuf d_frames, d_ranges, d_images, d_cand_px, d_cand_keep, d_tile_count, d_force_valid, d_force_keep, d_frame_V,
-      d_amb_count, d_amb_list, d_row_px, d_row_gidx, d_row_nb, d_row_nbl, d_tile_halo, d_tile_desc, d_act[2], d_lookup;
+      d_amb_list, d_row_px, d_row_gidx, d_row_nb, d_row_nbl, d_tile_halo, d_tile_desc, d_act[2], d_lookup;
     float* final_act = nullptr;
 
     /* profiling */
-    bool profile = false;
+    int profile = 0; /* 0 off, 1 every kernel, 2 only the launches of the kernel that took longest in the last mode-1 run */
+    std::vector<char> slot_wanted; /* mode 2: which launch slots are bracketed */
     std::vector<hipEvent_t> events;
     std::vector<const char*> slot_names;
     std::vector<int64_t> slot_units;
@@ -150,10 +157,12 @@ struct vmhip_batch {
 
     void release() {
         DevBuf* all[] = {&d_frames, &d_ranges, &d_images, &d_cand_px, &d_cand_keep, &d_tile_count, &d_force_valid,
-                         &d_force_keep, &d_frame_V, &d_amb_count, &d_amb_list, &d_row_px, &d_row_gidx, &d_row_nb,
+                         &d_force_keep, &d_frame_V, &d_amb_list, &d_row_px, &d_row_gidx, &d_row_nb,
                          &d_row_nbl, &d_tile_halo, &d_tile_desc,
                          &d_act[0], &d_act[1], &d_lookup};
         for (DevBuf* b : all) b->release();
+        if (h_pin) (void) hipHostFree(h_pin);
+        h_pin = nullptr, h_pin_cap = 0;
         for (hipEvent_t e : events) (void) hipEventDestroy(e);
         events.clear();
     }
@@ -246,8 +255,16 @@ int batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int
     HIP_TRY(b->d_tile_count.reserve(4 * std::max<size_t>(cand_tiles, 1)));
     HIP_TRY(b->d_force_valid.reserve(8 * std::max<size_t>(words, 1)));
     HIP_TRY(b->d_force_keep.reserve(8 * std::max<size_t>(words, 1)));
-    HIP_TRY(b->d_frame_V.reserve(4 * size_t(n_frames)));
-    HIP_TRY(b->d_amb_count.reserve(4 * size_t(n_frames)));
+    HIP_TRY(b->d_frame_V.reserve(8 * size_t(n_frames))); /* visible counts, then ambiguity counts */
+    {
+        const size_t need = 8 * size_t(n_frames) + sizeof(int2) * size_t(n_frames) * vmhip_batch::AMB_HEAD;
+        if (need > b->h_pin_cap) {
+            if (b->h_pin) HIP_TRY(hipHostFree(b->h_pin));
+            b->h_pin = nullptr, b->h_pin_cap = 0;
+            HIP_TRY(hipHostMalloc(&b->h_pin, need, hipHostMallocDefault));
+            b->h_pin_cap = need;
+        }
+    }
     HIP_TRY(b->d_amb_list.reserve(sizeof(int2) * size_t(n_frames) * VMHIP_AMB_CAP));
     HIP_TRY(b->d_row_px.reserve(sizeof(float2) * std::max<size_t>(b->row_total, 1)));
     HIP_TRY(b->d_row_gidx.reserve(4 * std::max<size_t>(b->row_total, 1)));
@@ -314,7 +331,7 @@ int batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int
     D.cand_keep = b->d_cand_keep.as<uint64_t>();
     D.tile_count = b->d_tile_count.as<int32_t>();
     D.frame_V = b->d_frame_V.as<int32_t>();
-    D.amb_count = b->d_amb_count.as<int32_t>();
+    D.amb_count = b->d_frame_V.as<int32_t>() + n_frames;
     D.amb_list = b->d_amb_list.as<int2>();
     D.row_px = b->d_row_px.as<float2>();
     D.row_gidx = b->d_row_gidx.as<int32_t>();
@@ -333,8 +350,9 @@ struct Profiler {
     vmhip_batch* b;
     hipStream_t s;
     int slot = 0;
+    bool wanted() const { return b->profile == 1 || (b->profile == 2 && slot < int(b->slot_wanted.size()) && b->slot_wanted[slot]); }
     hipError_t begin() {
-        if (!b->profile) return hipSuccess;
+        if (!wanted()) return hipSuccess;
         while (int(b->events.size()) < 2 * (slot + 1)) {
             hipEvent_t e;
             hipError_t r = hipEventCreate(&e);
@@ -345,7 +363,7 @@ struct Profiler {
     }
     hipError_t end(const char* name, int64_t units) {
         if (!b->profile) return hipSuccess;
-        hipError_t r = hipEventRecord(b->events[2 * slot + 1], s);
+        hipError_t r = wanted() ? hipEventRecord(b->events[2 * slot + 1], s) : hipSuccess;
         if (int(b->slot_names.size()) <= slot) {
             b->slot_names.resize(slot + 1);
             b->slot_units.resize(slot + 1);
@@ -406,9 +424,15 @@ int batch_enqueue(vmhip_batch* b) {
 int batch_verify(vmhip_batch* b) {
     vmhip_engine* E = b->engine;
     const int n = int(b->frames.size());
-    HIP_TRY(hipMemcpyAsync(b->h_V.data(), b->d_frame_V.p, 4 * size_t(n), hipMemcpyDeviceToHost, E->stream));
-    HIP_TRY(hipMemcpyAsync(b->h_amb_count.data(), b->d_amb_count.p, 4 * size_t(n), hipMemcpyDeviceToHost, E->stream));
+    constexpr int HEAD = vmhip_batch::AMB_HEAD;
+    int32_t* pin_counts = reinterpret_cast<int32_t*>(b->h_pin);
+    int2* pin_amb = reinterpret_cast<int2*>(pin_counts + 2 * n);
+    HIP_TRY(hipMemcpyAsync(pin_counts, b->d_frame_V.p, 8 * size_t(n), hipMemcpyDeviceToHost, E->stream));
+    HIP_TRY(hipMemcpy2DAsync(pin_amb, sizeof(int2) * HEAD, b->d_amb_list.p, sizeof(int2) * VMHIP_AMB_CAP, sizeof(int2) * HEAD, n,
+                             hipMemcpyDeviceToHost, E->stream));
     HIP_TRY(hipStreamSynchronize(E->stream));
+    std::copy(pin_counts, pin_counts + n, b->h_V.begin());
+    std::copy(pin_counts + n, pin_counts + 2 * n, b->h_amb_count.begin());
     int changed = 0;
     for (int f = 0; f < n; ++f) {
         HostFrame& hf = b->frames[f];
@@ -439,9 +463,13 @@ int batch_verify(vmhip_batch* b) {
             for (int p = 0; p < d.n_cand; ++p) redecide(p, -1, true);
         }
         else {
-            b->h_amb.resize(count);
-            HIP_TRY(hipMemcpy(b->h_amb.data(), b->d_amb_list.as<int2>() + size_t(f) * VMHIP_AMB_CAP, sizeof(int2) * count, hipMemcpyDeviceToHost));
-            for (int i = 0; i < count; ++i) redecide(b->h_amb[i].x, b->h_amb[i].y, false);
+            const int2* list = pin_amb + size_t(f) * HEAD;
+            if (count > HEAD) { /* more than the head that came with the counts */
+                b->h_amb.resize(count);
+                HIP_TRY(hipMemcpy(b->h_amb.data(), b->d_amb_list.as<int2>() + size_t(f) * VMHIP_AMB_CAP, sizeof(int2) * count, hipMemcpyDeviceToHost));
+                list = b->h_amb.data();
+            }
+            for (int i = 0; i < count; ++i) redecide(list[i].x, list[i].y, false);
         }
     }
     if (changed > 0) {
@@ -707,20 +735,38 @@ int vmhip_batch_fetch(vmhip_batch* b, vmhip_result* results) {
 }
 int vmhip_batch_profile(vmhip_batch* b, int32_t enable) {
     if (!b) return fail(VMHIP_ERR_ARGUMENT, "batch_profile: null batch");
-    b->profile = enable != 0;
+    if (enable < 0 || enable > 2) return fail(VMHIP_ERR_ARGUMENT, "batch_profile: mode must be 0, 1 or 2");
+    if (enable == 2) {
+        if (b->profile != 1 || !b->have_run) return fail(VMHIP_ERR_ARGUMENT, "batch_profile: mode 2 follows a run profiled in mode 1");
+        std::map<std::string, float> total;
+        for (int i = 0; i < b->n_slots; ++i) {
+            float ms = 0.0f;
+            HIP_TRY(hipEventElapsedTime(&ms, b->events[2 * i], b->events[2 * i + 1]));
+            total[b->slot_names[i]] += ms;
+        }
+        std::string longest;
+        float best = -1.0f;
+        for (const auto& kv : total)
+            if (kv.second > best) best = kv.second, longest = kv.first;
+        b->slot_wanted.assign(b->n_slots, 0);
+        for (int i = 0; i < b->n_slots; ++i) b->slot_wanted[i] = longest == b->slot_names[i];
+    }
+    b->profile = enable;
     return VMHIP_OK;
 }
 int vmhip_batch_profile_read(vmhip_batch* b, int32_t max_slots, int32_t* n_slots, const char** names, float* milliseconds,
                              int64_t* units) {
     if (!b || !n_slots) return fail(VMHIP_ERR_ARGUMENT, "batch_profile_read: null argument");
     if (!b->profile || !b->have_run) return fail(VMHIP_ERR_ARGUMENT, "batch_profile_read: profiling was not enabled for the last run");
-    const int n = std::min<int>(b->n_slots, max_slots);
-    for (int i = 0; i < n; ++i) {
+    int n = 0;
+    for (int i = 0; i < b->n_slots && n < max_slots; ++i) {
+        if (b->profile == 2 && !b->slot_wanted[i]) continue;
         float ms = 0.0f;
         HIP_TRY(hipEventElapsedTime(&ms, b->events[2 * i], b->events[2 * i + 1]));
-        if (names) names[i] = b->slot_names[i];
-        if (milliseconds) milliseconds[i] = ms;
-        if (units) units[i] = b->slot_units[i];
+        if (names) names[n] = b->slot_names[i];
+        if (milliseconds) milliseconds[n] = ms;
+        if (units) units[n] = b->slot_units[i];
+        ++n;
     }
     *n_slots = n;
     return VMHIP_OK;

@@ -196,9 +196,10 @@ class Engine:
         return C.c_void_p(self._lib.vmh_engine_native_batch(self.ptr))
 
     def profile(self, enable=True):
+        """0/False off, 1/True every kernel, 2 only the kernel that took longest in the last fully profiled run"""
         if not self.native_batch():
             return  # nothing staged yet: profiling is switched on per batch object
-        native.hip_check(native.hip().vmhip_batch_profile(self.native_batch(), 1 if enable else 0))
+        native.hip_check(native.hip().vmhip_batch_profile(self.native_batch(), int(enable)))
 
     def profile_read(self):
         return native.profile_read(self.native_batch())
