@@ -95,6 +95,8 @@ def main():
     ap.add_argument("--config", type=int, default=2, help="workload configuration 1..5 (default 2: batched 1280x1024)")
     ap.add_argument("--frames", type=int, default=None, help="frames per batch (default: the configuration's own)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--no-events", action="store_true",
+                    help="no HIP events in the timed passes (they then replay the captured HIP graph); no roofline is reported")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a 1 GiB plain copy kernel (the dispatch of known size that memory counters are scaled by)")
     args = ap.parse_args()
@@ -134,12 +136,14 @@ def main():
     kernel_ms_per_step = {}
     for name, ms, units in engine.profile_read():
         kernel_ms_per_step[name] = kernel_ms_per_step.get(name, 0.0) + ms
-    engine.profile(2)
+    engine.profile(0 if args.no_events else 2)   # --no-events: the timed passes replay the captured HIP graph
     kernel_ms = {}
     kernel_launches = {}
     t0 = time.perf_counter()
     for _ in range(args.steps):
         engine.run()              # launches the whole path and waits for it
+        if args.no_events:
+            continue
         for name, ms, units in engine.profile_read():
             kernel_ms[name] = kernel_ms.get(name, 0.0) + ms
             kernel_launches[name] = kernel_launches.get(name, 0) + 1

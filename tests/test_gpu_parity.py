@@ -229,3 +229,27 @@ def test_rows_beyond_the_halo_capacity(oracle, index, monkeypatch):
     assert all(n.startswith("conv_lds_") for n in names), names
     want = pick(o_mesh, f["Hoc"]).classify(f["Hoc"], o_lens, f["image"], cfg.fourcc, vmo.Network(cfg.network))
     assert_classification_parity(got, want, PROB_TOL, "halo cap 8, cfg%d" % index)
+
+
+def test_graph_replays_match_eager_runs(oracle, monkeypatch):
+    """A staged batch launches its first run kernel by kernel, captures the second into a HIP graph and replays it
+    afterwards. Every replay, with eager work of another engine and synchronisations in between, must reproduce
+    the eager results bit for bit (two batches through the same engine, so the graph is rebuilt after restaging)."""
+    cfg = wl.config(2, n_frames=3)
+    _, e_lens = lens_pair(cfg)
+    _, e_mesh = meshes_for(cfg, oracle)
+    frames = [dict(mesh=e_mesh, Hoc=f["Hoc"], lens=e_lens, image=f["image"], fourcc=cfg.fourcc) for f in cfg.frames]
+    monkeypatch.setenv("VMHIP_GRAPH", "0")
+    eager = eng.Engine(cfg.network, cfg.model)
+    monkeypatch.setenv("VMHIP_GRAPH", "1")
+    graphed = eng.Engine(cfg.network, cfg.model)
+    for batch in (frames, frames[:2][::-1]):
+        want = eager.classify_batch(batch)
+        graphed.stage(batch)
+        for replay in range(5):
+            graphed.run()
+            got = graphed.fetch()
+            eager.run()  # unrelated eager work between the replays
+            for i in range(len(batch)):
+                for key in ("px", "gidx", "nb", "cls"):
+                    assert np.array_equal(got[i][key], want[i][key]), "run %d frame %d %s" % (replay, i, key)

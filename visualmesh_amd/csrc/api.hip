@@ -108,6 +108,7 @@ struct HostLayer {
 };
 
 struct vmhip_engine {
+    bool use_graph = true;               /* VMHIP_GRAPH=0: launch every run kernel by kernel */
     bool use_lds = false;                /* some layer gathers through the tile-local tables */
     int32_t halo_cap = VMHIP_HALO_MAX;   /* VMHIP_HALO_CAP lowers it to exercise the not-staged path */
     int32_t nn = 0;
@@ -139,12 +140,21 @@ struct vmhip_batch {
     size_t h_pin_cap = 0;
     std::vector<uint64_t> h_force_valid, h_force_keep;
     bool have_run = false;
-    uint32_t epoch = 0;
+    uint32_t epoch = 0; /* host mirror of the device run stamp */
+    /* the kernel sequence of a run, captured once per staged batch and replayed (no profiling, VMHIP_GRAPH != 0) */
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t graph_exec = nullptr;
+    int eager_runs = 0; /* runs since the last stage: the first one is launched eagerly, then captured */
+    void drop_graph() {
+        if (graph_exec) (void) hipGraphExecDestroy(graph_exec);
+        if (graph) (void) hipGraphDestroy(graph);
+        graph_exec = nullptr, graph = nullptr, eager_runs = 0;
+    }
     size_t cand_total = 0, row_total = 0, lookup_total = 0;
 
     VmBatchDev dev{};
     DevBuf d_frames, d_ranges, d_images, d_cand_px, d_cand_keep, d_tile_count, d_force_valid, d_force_keep, d_frame_V,
-      d_amb_list, d_row_px, d_row_gidx, d_row_nb, d_row_nbl, d_tile_halo, d_tile_desc, d_act[2], d_lookup;
+      d_amb_list, d_row_px, d_row_gidx, d_row_nb, d_row_nbl, d_tile_halo, d_tile_desc, d_act[2], d_lookup, d_epoch;
     float* final_act = nullptr;
 
     /* profiling */
@@ -158,8 +168,9 @@ struct vmhip_batch {
     void release() {
         DevBuf* all[] = {&d_frames, &d_ranges, &d_images, &d_cand_px, &d_cand_keep, &d_tile_count, &d_force_valid,
                          &d_force_keep, &d_frame_V, &d_amb_list, &d_row_px, &d_row_gidx, &d_row_nb,
-                         &d_row_nbl, &d_tile_halo, &d_tile_desc,
+                         &d_row_nbl, &d_tile_halo, &d_tile_desc, &d_epoch,
                          &d_act[0], &d_act[1], &d_lookup};
+        drop_graph();
         for (DevBuf* b : all) b->release();
         if (h_pin) (void) hipHostFree(h_pin);
         h_pin = nullptr, h_pin_cap = 0;
@@ -285,6 +296,12 @@ int batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int
         HIP_TRY(hipMemsetAsync(b->d_lookup.p, 0, b->d_lookup.cap, E->stream));
     }
     b->lookup_total = lookup_entries;
+    if (!b->d_epoch.p) {
+        HIP_TRY(b->d_epoch.reserve(256));
+        HIP_TRY(hipMemsetAsync(b->d_epoch.p, 0, 256, E->stream));
+        b->epoch = 0;
+    }
+    b->drop_graph(); /* pointers and sizes baked into a captured run are no longer valid */
 
     /* fill in device pointers and upload */
     std::vector<int32_t> h_ranges(std::max<size_t>(range_ints, 1));
@@ -341,6 +358,7 @@ int batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int
     D.tile_halo = local_tables ? b->d_tile_halo.as<uint32_t>() : nullptr;
     D.tile_desc = local_tables ? b->d_tile_desc.as<int4>() : nullptr;
     D.halo_cap = E->halo_cap;
+    D.epoch = b->d_epoch.as<uint32_t>();
     b->h_V.assign(n_frames, 0);
     b->h_amb_count.assign(n_frames, 0);
     return VMHIP_OK;
@@ -379,7 +397,6 @@ int batch_enqueue(vmhip_batch* b) {
     vmhip_engine* E = b->engine;
     hipStream_t s = E->stream;
     VmBatchDev& D = b->dev;
-    D.epoch = b->epoch;
     Profiler P{b, s};
     int64_t cands = 0, rows = 0;
     for (const HostFrame& hf : b->frames) cands += hf.dev.n_cand;
@@ -483,13 +500,32 @@ int batch_verify(vmhip_batch* b) {
 
 int batch_run(vmhip_batch* b) {
     if (b->frames.empty()) return fail(VMHIP_ERR_ARGUMENT, "run: nothing staged");
+    vmhip_engine* E = b->engine;
     for (int attempt = 0; attempt < 4; ++attempt) {
-        ++b->epoch;
-        if (b->epoch == 0) { /* wrapped: old stamps could look current again */
-            HIP_TRY(hipMemsetAsync(b->d_lookup.p, 0, b->d_lookup.cap, b->engine->stream));
-            b->epoch = 1;
+        if (b->epoch == 0xffffffffu) { /* the device stamp is about to wrap: old stamps could look current again */
+            HIP_TRY(hipMemsetAsync(b->d_lookup.p, 0, b->d_lookup.cap, E->stream));
+            HIP_TRY(hipMemsetAsync(b->d_epoch.p, 0, 4, E->stream));
+            b->epoch = 0;
         }
-        int rc = batch_enqueue(b);
+        ++b->epoch; /* the reset kernel does the same on the device */
+        int rc = VMHIP_OK;
+        if (E->use_graph && !b->profile && b->eager_runs >= 1) {
+            if (!b->graph_exec) {
+                /* Capture the kernel sequence (kernels only: the clears are a kernel too, no memset nodes). The
+                 * first run after staging was eager, so every kernel's one-time attribute set-up is done. */
+                HIP_TRY(hipStreamBeginCapture(E->stream, hipStreamCaptureModeThreadLocal));
+                rc = batch_enqueue(b);
+                hipError_t e = hipStreamEndCapture(E->stream, &b->graph);
+                if (rc != VMHIP_OK) return rc;
+                HIP_TRY(e);
+                HIP_TRY(hipGraphInstantiate(&b->graph_exec, b->graph, nullptr, nullptr, 0));
+            }
+            HIP_TRY(hipGraphLaunch(b->graph_exec, E->stream));
+        }
+        else {
+            rc = batch_enqueue(b);
+            ++b->eager_runs;
+        }
         if (rc != VMHIP_OK) return rc;
         rc = batch_verify(b);
         if (rc < 0) return rc;
@@ -606,6 +642,7 @@ int vmhip_engine_create(const vmhip_network* net, int32_t n_neighbours, int32_t 
         const bool rows_only = pick && std::string(pick) == "rows";
         const bool allow_lds = !rows_only && !(pick && std::string(pick) == "mfma");
         const bool force_lds = pick && std::string(pick) == "lds";
+        if (const char* g = getenv("VMHIP_GRAPH")) E->use_graph = atoi(g) != 0;
         if (const char* cap = getenv("VMHIP_HALO_CAP")) E->halo_cap = std::min(std::max(atoi(cap), 0), VMHIP_HALO_MAX);
         const int n = int(E->layers.size());
         std::vector<int> bf(n + 1, 0); /* bf[l] = rows entering layer l are bf16; bf[n] = final output (never) */

@@ -191,8 +191,9 @@ __global__ __launch_bounds__(NW * 64, 4) void vm_conv_lds_kernel(VmBatchDev B, V
 #pragma unroll
         for (int k = 0; k < N_HALO; ++k) {
             const int idx = threadIdx.x + k * NT;
-            const int c = idx % Q4;
-            st_halo[k] = __builtin_amdgcn_raw_buffer_load_b128(in_rsrc, (hrow[k] * Q4 + c) * 16, 0, 0);
+            const int h = idx / Q4, c = idx % Q4;
+            /* slots past the tile's halo count: an out-of-range offset reads zeros without touching memory */
+            st_halo[k] = __builtin_amdgcn_raw_buffer_load_b128(in_rsrc, h < d.z ? (hrow[k] * Q4 + c) * 16 : 0xffffffffu, 0, 0);
         }
     };
     auto write_rows = [&]() {

@@ -9,7 +9,7 @@
  * node within 1/64 px of a screen edge is re-decided on the host, so the visible set cannot diverge.
  *
  * Kernels (one launch each per batch, grids over all frames of the batch):
- *   vm_reset_kernel          clears the per-frame ambiguity counters
+ *   vm_reset_kernel          clears the per-frame ambiguity counters, advances the run stamp
  *   vm_project_kernel        candidate space: global index from the range table, pixel coordinate, keep
  *                            decision, per-wave keep mask (ballot), per-tile kept count, ambiguity list
  *   vm_compact_kernel        candidate space: exclusive prefix over tile counts + wave popcount prefix ->
@@ -108,6 +108,7 @@ __global__ __launch_bounds__(256) void vm_copy_probe_kernel(const float4* __rest
 __global__ void vm_reset_kernel(VmBatchDev B) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < B.n_frames) B.amb_count[i] = 0;
+    if (i == 0) *B.epoch += 1; /* a new run: stamps of earlier runs stop matching */
 }
 
 __global__ __launch_bounds__(VMHIP_TILE) void vm_project_kernel(VmBatchDev B) {
@@ -318,7 +319,7 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_compact_kernel(VmBatchDev B, fl
         const float2 px = B.cand_px[(size_t) F.cand_base + p];
         B.row_px[row] = px;
         B.row_gidx[row] = g;
-        F.r_lookup[g] = make_uint2(B.epoch, (uint32_t) local);
+        F.r_lookup[g] = make_uint2(*B.epoch, (uint32_t) local);
         if (classify) feat[row] = sample_image(F, px);
     }
     if (t_local == F.cand_tiles - 1 && threadIdx.x == 0) {
@@ -349,6 +350,7 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_neighbourhood_kernel(VmBatchDev
     const int nn = F.nn;
     const int row0 = (tile - F.row_tile0) * VMHIP_TILE;
     const bool tables = B.row_nbl != nullptr;
+    const uint32_t epoch = *B.epoch;
     const int n_rows = max(0, min(VMHIP_TILE, V + 1 - row0));
     if (n_rows == 0) {
         if (tables && threadIdx.x == 0) B.tile_desc[tile] = make_int4(F.row_base + row0, 0, 0, F.row_base);
@@ -374,7 +376,7 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_neighbourhood_kernel(VmBatchDev
             const int g = B.row_gidx[(size_t) F.row_base + i];
             const int gn = F.nbr[(size_t) g * nn + j];
             const uint2 e = F.r_lookup[min(gn, F.n_nodes)];
-            out = e.x == B.epoch ? (int) e.y : V;
+            out = e.x == epoch ? (int) e.y : V;
         }
         B.row_nb[((size_t) F.row_base + i) * B.nb_stride + j] = out;
         return out;

@@ -80,7 +80,7 @@ struct VmBatchDev {
     const VmFrame* frames;
     int32_t n_frames;
     int32_t n_cand_tiles, n_row_tiles;
-    uint32_t epoch;
+    uint32_t* epoch;      /* device word: the run's stamp for the reverse lookup; the reset kernel increments it */
     /* candidate space */
     float2* cand_px;
     uint64_t* cand_keep;  /* one 64-bit mask per wave of candidates */
