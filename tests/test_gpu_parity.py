@@ -185,11 +185,11 @@ def test_bf16_engine_keeps_narrow_networks_in_fp32(oracle):
     assert_classification_parity(got, want, PROB_TOL, "bf16 engine, narrow network")
 
 
-@pytest.mark.parametrize("kernel", ["rows", "mfma", "lds"])
+@pytest.mark.parametrize("kernel", ["rows", "mfma", "lds", "dma"])
 def test_every_convolution_kernel_agrees_with_the_oracle(oracle, kernel, monkeypatch):
     """Every layer shape of configuration 2 through the one-row-per-lane kernel, the matrix-core kernel that
-    gathers into registers and the matrix-core kernel that gathers from LDS (VMHIP_CONV_KERNEL, read when the
-    engine is built)."""
+    gathers into registers and the two matrix-core kernels that gather from LDS (rows staged through registers /
+    loaded straight into LDS), selected with VMHIP_CONV_KERNEL when the engine is built."""
     monkeypatch.setenv("VMHIP_CONV_KERNEL", kernel)
     cfg = wl.config(2, n_frames=2)
     o_lens, e_lens = lens_pair(cfg)
@@ -211,12 +211,13 @@ def test_every_convolution_kernel_agrees_with_the_oracle(oracle, kernel, monkeyp
         assert_classification_parity(results[i], want, PROB_TOL, "%s frame %d" % (kernel, i))
 
 
+@pytest.mark.parametrize("kernel", ["lds", "dma"])
 @pytest.mark.parametrize("index", [2, 3])
-def test_rows_beyond_the_halo_capacity(oracle, index, monkeypatch):
+def test_rows_beyond_the_halo_capacity(oracle, index, kernel, monkeypatch):
     """With only 8 halo slots per tile most out-of-tile neighbours are marked as not staged and the LDS kernel
     reads them from global memory: same results (configuration 2's Ring6 and 3's NMGrid8 networks)."""
     monkeypatch.setenv("VMHIP_HALO_CAP", "8")
-    monkeypatch.setenv("VMHIP_CONV_KERNEL", "lds")
+    monkeypatch.setenv("VMHIP_CONV_KERNEL", kernel)
     cfg = wl.config(index, n_frames=1)
     o_lens, e_lens = lens_pair(cfg)
     o_mesh, e_mesh = meshes_for(cfg, oracle)
@@ -226,9 +227,9 @@ def test_rows_beyond_the_halo_capacity(oracle, index, monkeypatch):
     engine.profile(True)
     engine.run()
     names = [n for n, _, _ in engine.profile_read() if n.startswith("conv")]
-    assert all(n.startswith("conv_lds_") for n in names), names
+    assert all(n.startswith("conv_%s_" % kernel) for n in names), names
     want = pick(o_mesh, f["Hoc"]).classify(f["Hoc"], o_lens, f["image"], cfg.fourcc, vmo.Network(cfg.network))
-    assert_classification_parity(got, want, PROB_TOL, "halo cap 8, cfg%d" % index)
+    assert_classification_parity(got, want, PROB_TOL, "halo cap 8, cfg%d, %s" % (index, kernel))
 
 
 def test_graph_replays_match_eager_runs(oracle, monkeypatch):

@@ -62,6 +62,7 @@ def build_hip(force=False):
         ("conv.hip", HIP_FLAGS),
         ("conv_mfma.hip", HIP_FLAGS),
         ("conv_lds.hip", HIP_FLAGS),
+        ("conv_dma.hip", HIP_FLAGS),
         ("api.hip", HIP_FLAGS),
     ]
     for name, flags in units:

@@ -103,7 +103,7 @@ struct HostLayer {
     float* d_b = nullptr;
     void* d_w_mfma = nullptr;
     int32_t in_bf16 = 0, out_bf16 = 0, arith_bf16 = 0;
-    bool use_lds = false, use_mfma = false; /* which matrix-core kernels may take the layer */
+    bool use_lds = false, use_mfma = false, use_dma = false; /* which matrix-core kernels may take the layer */
     std::vector<float> h_w; /* kept until the row types are planned */
 };
 
@@ -420,7 +420,8 @@ int batch_enqueue(vmhip_batch* b) {
             const char* name = "conv";
             HIP_TRY(P.begin());
             int rc = -1;
-            if (L.use_lds && D.row_nbl) rc = vm_launch_conv_lds(D, ld, b->d_act[cur].as<float>(), b->d_act[cur ^ 1].as<float>(), s, &name);
+            if (L.use_dma && D.row_nbl) rc = vm_launch_conv_dma(D, ld, b->d_act[cur].as<float>(), b->d_act[cur ^ 1].as<float>(), s, &name);
+            if (rc != 0 && L.use_lds && D.row_nbl) rc = vm_launch_conv_lds(D, ld, b->d_act[cur].as<float>(), b->d_act[cur ^ 1].as<float>(), s, &name);
             if (rc != 0 && L.d_w_mfma && L.use_mfma) rc = vm_launch_conv_mfma(D, ld, b->d_act[cur].p, b->d_act[cur ^ 1].p, s, &name);
             /* the one-row-per-lane kernels only know fp32 rows */
             if (rc != 0 && !L.in_bf16 && !L.out_bf16) rc = vm_launch_conv(D, ld, b->d_act[cur].as<float>(), b->d_act[cur ^ 1].as<float>(), s, &name);
@@ -642,6 +643,7 @@ int vmhip_engine_create(const vmhip_network* net, int32_t n_neighbours, int32_t 
         const bool rows_only = pick && std::string(pick) == "rows";
         const bool allow_lds = !rows_only && !(pick && std::string(pick) == "mfma");
         const bool force_lds = pick && std::string(pick) == "lds";
+        const bool force_dma = pick && std::string(pick) == "dma";
         if (const char* g = getenv("VMHIP_GRAPH")) E->use_graph = atoi(g) != 0;
         if (const char* cap = getenv("VMHIP_HALO_CAP")) E->halo_cap = std::min(std::max(atoi(cap), 0), VMHIP_HALO_MAX);
         const int n = int(E->layers.size());
@@ -679,8 +681,9 @@ int vmhip_engine_create(const vmhip_network* net, int32_t n_neighbours, int32_t 
              * shape it has (32->32: 157 us against 166 us, 32->16: 89 against 122, 4->16: 29 against 44); only the
              * 2- and 3-class output layers are quicker with one row per lane (46 us against 56 us). */
             if (H.use_lds && !force_lds && H.c_out < 4) H.use_lds = false;
-            E->use_lds = E->use_lds || H.use_lds;
-            if (H.use_mfma || H.use_lds) {
+            H.use_dma = force_dma && plain && H.slots - 1 <= VMHIP_NBL_STRIDE && vm_dma_supported(H.c_in, H.c_out, H.slots);
+            E->use_lds = E->use_lds || H.use_lds || H.use_dma;
+            if (H.use_mfma || H.use_lds || H.use_dma) {
                 std::vector<unsigned char> wp(vm_mfma_weight_bytes(H.c_in, H.c_out, H.slots, H.arith_bf16));
                 vm_mfma_permute_weights(H.h_w.data(), H.c_in, H.c_out, H.slots, H.arith_bf16, wp.data());
                 if (hipMalloc(&H.d_w_mfma, wp.size()) != hipSuccess) return bail(VMHIP_ERR_HIP, "engine_create: out of device memory");

@@ -139,6 +139,11 @@ bool vm_lds_supported(int c_in, int c_out, int slots);
 int vm_launch_conv_lds(const VmBatchDev& B, const VmLayerDev& L, const float* in, float* out, hipStream_t stream,
                        const char** kernel_name);
 
+/* the same with rows brought into LDS by buffer_load ... lds and two alternating row buffers (conv_dma.hip) */
+bool vm_dma_supported(int c_in, int c_out, int slots);
+int vm_launch_conv_dma(const VmBatchDev& B, const VmLayerDev& L, const float* in, float* out, hipStream_t stream,
+                       const char** kernel_name);
+
 #include "host_project.h"
 
 #endif
