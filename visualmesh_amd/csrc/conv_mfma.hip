@@ -254,13 +254,30 @@ __global__ __launch_bounds__(NW * 64) void vm_conv_mfma_kernel(VmBatchDev B, VmL
         int V;
         int row0;
     };
+    /* With the tile descriptors at hand (built next to the neighbourhood table) a tile is described by one 16-byte
+     * buffer load: vector memory on purpose, because a scalar load in flight shares its counter with the LDS
+     * reads of the weights and would turn each of their waits into a wait for global memory. The values stay in
+     * vector registers (all lanes equal). Without descriptors: frame search and visible count by scalar loads. */
+    const bool have_desc = B.tile_desc != nullptr;
+    const __amdgpu_buffer_rsrc_t desc_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<int4*>(B.tile_desc), 0, have_desc ? n_tiles * 16 : 0, 0x00020000);
     auto describe = [&](int tile) {
-        const int f = find_frame_by_row_tile(B.frames, B.n_frames, tile);
-        const VmFrame& F = B.frames[f];
         Info t;
-        t.base = (uint32_t) F.row_base;
-        t.V = B.frame_V[f];
-        t.row0 = (tile - F.row_tile0) * VMHIP_TILE + wave * (RB * 16);
+        if (have_desc) {
+            typedef uint32_t v4u __attribute__((ext_vector_type(4)));
+            const v4u d = __builtin_amdgcn_raw_buffer_load_b128(desc_rsrc, tile * 16, 0, 0); /* {first row, rows in use, -, frame's first row} */
+            const int tile_row0 = (int) d.x - (int) d.w;
+            t.base = d.w;
+            t.V = tile_row0 + (int) d.y - 1; /* the last row in use: equals V in the frame's last tile, never clamps elsewhere */
+            t.row0 = tile_row0 + wave * (RB * 16);
+        }
+        else {
+            const int f = find_frame_by_row_tile(B.frames, B.n_frames, tile);
+            const VmFrame& F = B.frames[f];
+            t.base = (uint32_t) F.row_base;
+            t.V = B.frame_V[f];
+            t.row0 = (tile - F.row_tile0) * VMHIP_TILE + wave * (RB * 16);
+        }
         return t;
     };
     /* the lane's rows of a tile, clamped to the null row (lanes past it compute on its data and skip the store) */
