@@ -337,11 +337,12 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_compact_kernel(VmBatchDev B, fl
  * halo slots), and every neighbour is rewritten as a position in "own tile rows, then halo slots". Which row
  * gets which halo slot depends on the order the atomics land in and may differ from run to run; the rows that a
  * slot stands for, and so every result computed through the tables, do not. */
-#define NB_HASH 4096
+#define NB_HASH 2048 /* >= the most out-of-tile neighbours a tile can have (256 rows x 8) */
 __global__ __launch_bounds__(VMHIP_TILE) void vm_neighbourhood_kernel(VmBatchDev B) {
     __shared__ __align__(16) uint32_t h_key[NB_HASH];
     __shared__ uint16_t h_dense[NB_HASH];
     __shared__ int wave_total[VMHIP_TILE / 64];
+    __shared__ __align__(16) uint16_t nbl_rows[VMHIP_TILE][VMHIP_NBL_STRIDE]; /* the tile's positions, stored row by row at the end */
 
     const int tile = blockIdx.x;
     const int f = find_frame_by_row_tile(B.frames, B.n_frames, tile);
@@ -357,7 +358,7 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_neighbourhood_kernel(VmBatchDev
         return;
     }
     constexpr uint32_t EMPTY = 0xffffffffu;
-    auto hash = [](uint32_t key) { return (key * 2654435761u) >> 20; }; /* 12 bits */
+    auto hash = [](uint32_t key) { return (key * 2654435761u) >> 21; }; /* 11 bits */
     if (tables) {
         for (int e = threadIdx.x * 4; e < NB_HASH; e += VMHIP_TILE * 4) *reinterpret_cast<uint4*>(&h_key[e]) = make_uint4(EMPTY, EMPTY, EMPTY, EMPTY);
         __syncthreads();
@@ -458,11 +459,13 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_neighbourhood_kernel(VmBatchDev
                 const int dense = h_dense[slot];
                 local = dense < cap ? (uint32_t) (VMHIP_TILE + dense) : VMHIP_NBL_FAR;
             }
-            const int i = row0 + it / nn;
-            const int j = it - (it / nn) * nn;
-            B.row_nbl[((size_t) F.row_base + i) * VMHIP_NBL_STRIDE + j] = (uint16_t) local;
+            nbl_rows[it / nn][it - (it / nn) * nn] = (uint16_t) local;
         }
     }
+    __syncthreads();
+    /* one 16-byte store per row (entries past nn are never read) */
+    if ((int) threadIdx.x < n_rows)
+        *reinterpret_cast<uint4*>(B.row_nbl + ((size_t) F.row_base + row0 + threadIdx.x) * VMHIP_NBL_STRIDE) = *reinterpret_cast<const uint4*>(nbl_rows[threadIdx.x]);
 }
 
 }  // namespace
