@@ -147,6 +147,25 @@ def test_config4_and_5_full_size_frame(oracle):
         assert_classification_parity(got, want, tol, label)
 
 
+def test_class_layers_use_the_4x4_matrix_instruction(oracle):
+    """The output layers of configurations 1 to 3 (16 -> 2, 16 -> 3, 24 -> 4) run on the kernel built on
+    v_mfma_f32_4x4x1 by default; their probabilities are covered by the configuration tests above, this one pins
+    the kernel choice those tests exercised."""
+    for index, last in ((1, "conv_narrow_16x2s7"), (2, "conv_narrow_16x3s7"), (3, "conv_narrow_24x4s9")):
+        cfg = wl.config(index, n_frames=1)
+        _, e_lens = lens_pair(cfg)
+        _, e_mesh = meshes_for(cfg, oracle)
+        engine = eng.Engine(cfg.network, cfg.model)
+        f = cfg.frames[0]
+        engine(e_mesh, f["Hoc"], e_lens, f["image"], cfg.fourcc)
+        frames = [dict(mesh=e_mesh, Hoc=f["Hoc"], lens=e_lens, image=f["image"], fourcc=cfg.fourcc)]
+        engine.stage(frames)
+        engine.profile(True)
+        engine.run()
+        names = [n for n, _, _ in engine.profile_read() if n.startswith("conv")]
+        assert names[-1] == last, names
+
+
 def test_bf16_engine(oracle):
     """The bf16 engine (configuration 5's precision and 6 x 64 network) against the fp32 oracle on configuration
     1's geometry: geometry bit-exact, probabilities within 1e-2. The kernel names prove that the bf16

@@ -103,7 +103,7 @@ struct HostLayer {
     float* d_b = nullptr;
     void* d_w_mfma = nullptr;
     int32_t in_bf16 = 0, out_bf16 = 0, arith_bf16 = 0;
-    bool use_lds = false, use_mfma = false, use_dma = false; /* which matrix-core kernels may take the layer */
+    bool use_lds = false, use_mfma = false, use_dma = false, use_narrow = false; /* which matrix-core kernels may take the layer */
     std::vector<float> h_w; /* kept until the row types are planned */
 };
 
@@ -420,7 +420,8 @@ int batch_enqueue(vmhip_batch* b) {
             const char* name = "conv";
             HIP_TRY(P.begin());
             int rc = -1;
-            if (L.use_dma && D.row_nbl) rc = vm_launch_conv_dma(D, ld, b->d_act[cur].as<float>(), b->d_act[cur ^ 1].as<float>(), s, &name);
+            if (L.use_narrow && D.row_nbl) rc = vm_launch_conv_narrow(D, ld, b->d_act[cur].as<float>(), b->d_act[cur ^ 1].as<float>(), s, &name);
+            if (rc != 0 && L.use_dma && D.row_nbl) rc = vm_launch_conv_dma(D, ld, b->d_act[cur].as<float>(), b->d_act[cur ^ 1].as<float>(), s, &name);
             if (rc != 0 && L.use_lds && D.row_nbl) rc = vm_launch_conv_lds(D, ld, b->d_act[cur].as<float>(), b->d_act[cur ^ 1].as<float>(), s, &name);
             if (rc != 0 && L.d_w_mfma && L.use_mfma) rc = vm_launch_conv_mfma(D, ld, b->d_act[cur].p, b->d_act[cur ^ 1].p, s, &name);
             /* the one-row-per-lane kernels only know fp32 rows */
@@ -682,7 +683,10 @@ int vmhip_engine_create(const vmhip_network* net, int32_t n_neighbours, int32_t 
              * 2- and 3-class output layers are quicker with one row per lane (46 us against 56 us). */
             if (H.use_lds && !force_lds && H.c_out < 4) H.use_lds = false;
             H.use_dma = force_dma && plain && H.slots - 1 <= VMHIP_NBL_STRIDE && vm_dma_supported(H.c_in, H.c_out, H.slots);
-            E->use_lds = E->use_lds || H.use_lds || H.use_dma;
+            /* class layers (at most four output channels): the 4x4x1 matrix instruction, unless a family is forced */
+            H.use_narrow = allow_lds && !force_lds && !force_dma && plain && H.slots - 1 <= VMHIP_NBL_STRIDE
+                           && vm_narrow_supported(H.c_in, H.c_out, H.slots);
+            E->use_lds = E->use_lds || H.use_lds || H.use_dma || H.use_narrow;
             if (H.use_mfma || H.use_lds || H.use_dma) {
                 std::vector<unsigned char> wp(vm_mfma_weight_bytes(H.c_in, H.c_out, H.slots, H.arith_bf16));
                 vm_mfma_permute_weights(H.h_w.data(), H.c_in, H.c_out, H.slots, H.arith_bf16, wp.data());

@@ -144,6 +144,12 @@ bool vm_dma_supported(int c_in, int c_out, int slots);
 int vm_launch_conv_dma(const VmBatchDev& B, const VmLayerDev& L, const float* in, float* out, hipStream_t stream,
                        const char** kernel_name);
 
+/* layers with at most four output channels on v_mfma_f32_4x4x1 (64 rows x 4 channels per instruction), staged like
+ * conv_dma.hip (conv_narrow.hip); reads the plain row-major weights */
+bool vm_narrow_supported(int c_in, int c_out, int slots);
+int vm_launch_conv_narrow(const VmBatchDev& B, const VmLayerDev& L, const float* in, float* out, hipStream_t stream,
+                          const char** kernel_name);
+
 #include "host_project.h"
 
 #endif
