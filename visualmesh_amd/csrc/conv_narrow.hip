@@ -10,8 +10,7 @@
  * written with one store. Per row that is 8 matrix-pipe cycles for every 64 x 4 x 1 products: no waste against
  * the 16-column instruction, which spends 5.3 times more on a 3-channel layer.
  *
- * Staging is that of conv_dma.hip: rows travel from global memory straight into one of two alternating LDS buffers
- * (buffer_load ... lds), one barrier per tile, tile-local tables, XCD-aware persistent tile walk, a side path for
+ * Staging follows conv_dma.hip: rows travel from global memory straight into LDS (buffer_load ... lds), tile-local tables, XCD-aware persistent tile walk, a side path for
  * neighbours that are not staged. A lane reads its whole source row from LDS per gather slot.
  */
 #include <cstdlib>
@@ -68,8 +67,11 @@ __host__ __device__ constexpr bool row_swizzled(int c_in) { return c_in == 16; }
 __host__ __device__ constexpr int row_stride(int c_in) { return c_in == 16 ? c_in : c_in + 4; }
 constexpr int HALO = VMHIP_HALO_MAX;
 constexpr int NW = 4; /* 64 rows per wave */
+/* Row buffers per block. Two (tile t+1 lands while t is worked on, two blocks of four waves per CU) measured
+ * faster than one (four blocks per CU, each waiting for its own next tile): 39 us against 43 us on 16 -> 3. */
+constexpr int NBUFS = 2;
 __host__ __device__ constexpr size_t narrow_lds_bytes(int c_in, int slots) {
-    return (size_t(slots) * c_in * 4 + 4 + 2 * size_t(VMHIP_TILE + HALO) * row_stride(c_in)) * 4;
+    return (size_t(slots) * c_in * 4 + 4 + NBUFS * size_t(VMHIP_TILE + HALO) * row_stride(c_in)) * 4;
 }
 
 template <int C_IN, int C_OUT, int SLOTS>
@@ -172,25 +174,33 @@ __global__ __launch_bounds__(NW * 64) void vm_conv_narrow_kernel(VmBatchDev B, V
     };
     auto wait_all_loads = [] { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
 
-    /* ---- prologue: tiles t and t+1 on their way into the two buffers, t+2 described ---- */
+    /* ---- prologue: the first tile (and, with two buffers, the second) on its way into LDS, the next ones described.
+     * With two buffers the loop stages tile t+2 while t+1 waits in the other buffer; with one it stages t+1 into
+     * the buffer tile t has just left and meets it again at the top of the loop. ---- */
     int t1 = tile + gx, t2 = tile + 2 * gx;
     int4 d_cur = load_desc(tile), d_n1 = load_desc(min(t1, t_last)), d_n2 = load_desc(min(t2, t_last));
     v4u nbl = {0, 0, 0, 0}, nbl_n1 = nbl, nbl_n2 = nbl;
     request_halo_rows(tile);
     stage(d_cur, buf0);
     nbl = request_positions(d_cur);
-    if (t1 < t_end) {
+    if (NBUFS == 2 && t1 < t_end) {
         request_halo_rows(t1);
         stage(d_n1, buf0 + BUF_FLOATS);
         nbl_n1 = request_positions(d_n1);
     }
-    request_halo_rows(min(t2, t_last));
+    request_halo_rows(min(NBUFS == 2 ? t2 : t1, t_last));
     d_cur = uniform(d_cur);
-    wait_all_loads();
-    __syncthreads(); /* weights, biases and the first tile are in LDS */
+    if (NBUFS == 2) {
+        wait_all_loads();
+        __syncthreads(); /* weights, biases and the first tile are in LDS */
+    }
 
     int cur = 0;
     while (true) {
+        if (NBUFS == 1) {
+            wait_all_loads();
+            __syncthreads(); /* this tile (and, the first time, weights and biases) is in LDS */
+        }
         const float* rows = buf0 + cur * BUF_FLOATS;
         const bool in_use = d_cur.y > 0;
         const bool valid = (int) threadIdx.x < d_cur.y;
@@ -261,18 +271,25 @@ __global__ __launch_bounds__(NW * 64) void vm_conv_narrow_kernel(VmBatchDev B, V
         if (any_far) contract(std::true_type());
         else contract(std::false_type());
 
-        /* ---- the tile's only barrier (see conv_dma.hip) ---- */
-        wait_all_loads();
+        /* ---- every wave is done reading this buffer (with two buffers also: the next tile is complete and visible,
+         * see conv_dma.hip) ---- */
+        if (NBUFS == 2) wait_all_loads();
         __syncthreads();
 
         const bool has_next = t1 < t_end;
-        if (t2 < t_end) { /* uniform */
-            stage(d_n2, buf0 + cur * BUF_FLOATS); /* tile t+2 into the buffer tile t just left */
-            nbl_n2 = request_positions(d_n2);
-        }
         const int t3 = t2 + gx;
+        if (NBUFS == 2) {
+            if (t2 < t_end) { /* uniform */
+                stage(d_n2, buf0 + cur * BUF_FLOATS); /* tile t+2 into the buffer tile t just left */
+                nbl_n2 = request_positions(d_n2);
+            }
+        }
+        else if (has_next) {
+            stage(d_n1, buf0); /* tile t+1 into the one buffer; the activation below overlaps its flight */
+            nbl_n1 = request_positions(d_n1);
+        }
         const int4 d_n3 = load_desc(min(t3, t_last));
-        request_halo_rows(min(t3, t_last));
+        request_halo_rows(min(NBUFS == 2 ? t3 : t2, t_last));
         __builtin_amdgcn_sched_barrier(0);
 
         /* activation: the lane holds its row's channels 0..3 */
@@ -313,7 +330,7 @@ __global__ __launch_bounds__(NW * 64) void vm_conv_narrow_kernel(VmBatchDev B, V
         tile = t1;
         t1 = t2;
         t2 = t3;
-        cur ^= 1;
+        if (NBUFS == 2) cur ^= 1;
     }
     wait_all_loads(); /* no LDS load may outlive the wave */
 }
