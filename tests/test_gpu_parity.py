@@ -273,3 +273,51 @@ def test_graph_replays_match_eager_runs(oracle, monkeypatch):
             for i in range(len(batch)):
                 for key in ("px", "gidx", "nb", "cls"):
                     assert np.array_equal(got[i][key], want[i][key]), "run %d frame %d %s" % (replay, i, key)
+
+
+def _example_network():
+    import json
+    import os
+    here = os.path.dirname(os.path.abspath(__file__))
+    fixture = np.load(os.path.join(here, "golden", "example_model.npz"))
+    meta = json.load(open(os.path.join(here, "golden", "example_poses.json")))
+    network = []
+    for g, l, act in fixture["activations"]:
+        while len(network) <= g:
+            network.append([])
+        network[g].append((fixture["w_%d_%d" % (g, l)], fixture["b_%d_%d" % (g, l)], int(act)))
+    return network, meta
+
+
+def test_reference_example_network_on_its_dataset_poses(oracle):
+    """The reference's exported example network (example/model.yaml: 4->16, 16->16 x5, 16->8, 8->8 x5, 8->5) on the
+    lens and camera pose of its dataset elements (example/images/lens*.yaml, rectilinear 1280x1024), with synthetic
+    BGRA images: projection on all 30 poses, probabilities on 3 of them in one batch."""
+    network, meta = _example_network()
+    assert meta["mesh"] == "RING6" and meta["shape"] == "SPHERE"
+    heights = [p["Hoc"][2][3] for p in meta["poses"]]  # 0.78 m to 1.2 m: one mesh per height band, as the reference does
+    mesh_args = (wl.RING6, wl.SPHERE, meta["radius"], min(heights), max(heights), 6.0, 0.5, 15.0)
+    o_mesh = oracle.visualmesh(*mesh_args)
+    e_mesh = eng.VisualMesh(*mesh_args)
+    engine = eng.Engine(network, wl.RING6)
+    rng = np.random.default_rng(77)
+    projections = {"RECTILINEAR": wl.RECTILINEAR, "EQUISOLID": wl.EQUISOLID, "EQUIDISTANT": wl.EQUIDISTANT}
+    views = []
+    for p in meta["poses"]:
+        args = (p["width"], p["height"], projections[p["projection"]], p["focal_length"], p["fov"], tuple(p["centre"]), tuple(p["k"]))
+        views.append((np.array(p["Hoc"], np.float32), vmo.make_lens(*args), native.make_lens(*args), p))
+    for Hoc, o_lens, e_lens, p in views:
+        assert_projection_parity(engine(e_mesh, Hoc, e_lens), pick(o_mesh, Hoc).project(Hoc, o_lens), "example pose " + p["number"])
+    chosen = [views[i] for i in (0, 11, 29)]
+    images = [wl.random_image(rng, p["width"], p["height"], 4) for _, _, _, p in chosen]
+    frames = [dict(mesh=e_mesh, Hoc=H, lens=el, image=im, fourcc=wl.fourcc("BGRA")) for (H, _, el, _), im in zip(chosen, images)]
+    results = engine.classify_batch(frames)
+    engine.profile(True)
+    engine.run()
+    names = [n for n, _, _ in engine.profile_read() if n.startswith("conv")]
+    assert len(names) == 13 and all(n.startswith("conv_lds_") for n in names), names
+    for (H, ol, _, p), im, got in zip(chosen, images, results):
+        want = pick(o_mesh, H).classify(H, ol, im, wl.fourcc("BGRA"), vmo.Network(network))
+        print("example pose", p["number"], "V =", len(want["gidx"]), flush=True)
+        assert got["cls"].shape[1] == 5
+        assert_classification_parity(got, want, PROB_TOL, "example pose " + p["number"])

@@ -19,6 +19,7 @@
 #include "visualmesh/mesh.hpp"
 #include "visualmesh/model/nmgrid8.hpp"
 #include "visualmesh/model/ring6.hpp"
+#include "visualmesh/utility/load_model.hpp"
 #include "visualmesh/visualmesh.hpp"
 
 using namespace visualmesh;
@@ -41,6 +42,9 @@ struct vmh_visualmesh {
     std::unique_ptr<VisualMesh<float, Ring6>> r6;
     std::unique_ptr<VisualMesh<float, NMGrid8>> g8;
     std::vector<std::unique_ptr<vmh_mesh>> views;  // ascending height
+};
+struct vmh_model {
+    ModelFile<float> file;
 };
 struct vmh_engine {
     int model;
@@ -310,4 +314,60 @@ int vmh_engine_result(vmh_engine* e, int i, int cap, float* px, int32_t* nb, int
 }
 void* vmh_engine_native_batch(vmh_engine* e) { return e->engine->native_batch(); }
 void vmh_engine_clear_cache(vmh_engine* e) { e->engine->clear_cache(); }
+
+/* ---- exported networks and dataset lens files (visualmesh/utility/load_model.hpp) ---- */
+vmh_model* vmh_model_load(const char* path) {
+    try {
+        std::unique_ptr<vmh_model> m(new vmh_model());
+        m->file = load_model_file<float>(path);
+        return m.release();
+    } catch (const std::exception& e) {
+        report(e);
+        return nullptr;
+    }
+}
+void vmh_model_free(vmh_model* m) { delete m; }
+/* names are copied into caller buffers of `cap` bytes */
+int vmh_model_info(const vmh_model* m, char* mesh, char* shape, int cap, float* radius, float* intersections) {
+    GUARD({
+        if (cap <= 0) throw std::invalid_argument("model_info: no room for the names");
+        std::strncpy(mesh, m->file.mesh.c_str(), size_t(cap) - 1);
+        std::strncpy(shape, m->file.shape.c_str(), size_t(cap) - 1);
+        mesh[cap - 1] = shape[cap - 1] = 0;
+        *radius = m->file.radius;
+        *intersections = m->file.intersections;
+        return int(m->file.network.size());
+    })
+}
+int vmh_model_group_size(const vmh_model* m, int group) {
+    GUARD({ return int(m->file.network.at(group).size()); })
+}
+/* sizes of a layer; weights (row major [n_in][n_out]) and biases are copied when the pointers are not null */
+int vmh_model_layer(const vmh_model* m, int group, int layer, int* n_in, int* n_out, int* activation, float* weights, float* biases) {
+    GUARD({
+        const Layer<float>& l = m->file.network.at(group).at(layer);
+        *n_in = int(l.weights.size());
+        *n_out = int(l.biases.size());
+        *activation = int(l.activation);
+        if (weights)
+            for (size_t r = 0; r < l.weights.size(); ++r) std::memcpy(weights + r * l.biases.size(), l.weights[r].data(), sizeof(float) * l.biases.size());
+        if (biases) std::memcpy(biases, l.biases.data(), sizeof(float) * l.biases.size());
+        return 0;
+    })
+}
+int vmh_lens_load(const char* path, int width, int height, vmhip_lens* lens, float* Hoc16) {
+    GUARD({
+        const LensFile<float> f = load_lens<float>(path, width, height);
+        lens->width = width;
+        lens->height = height;
+        lens->projection = int(f.lens.projection);
+        lens->focal_length = f.lens.focal_length;
+        lens->centre[0] = f.lens.centre[0], lens->centre[1] = f.lens.centre[1];
+        lens->k[0] = f.lens.k[0], lens->k[1] = f.lens.k[1];
+        lens->fov = f.lens.fov;
+        for (int r = 0; r < 4; ++r)
+            for (int c = 0; c < 4; ++c) Hoc16[r * 4 + c] = f.Hoc[r][c];
+        return 0;
+    })
+}
 }

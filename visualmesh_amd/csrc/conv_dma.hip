@@ -435,7 +435,11 @@ int launch_dma(const VmBatchDev& B, const VmLayerDev& L, const float* in, float*
     X(4, 64, 7)                  \
     X(4, 24, 9)                  \
     X(24, 24, 9)                 \
-    X(24, 4, 9)
+    X(24, 4, 9)                  \
+    /* the reference's example network: 4->16, 16->16 x5, 16->8, 8->8 x5, 8->5 */ \
+    X(16, 8, 7)                  \
+    X(8, 8, 7)                   \
+    X(8, 5, 7)
 
 bool vm_dma_supported(int c_in, int c_out, int slots) {
 #define X(CI, CO, SL) \

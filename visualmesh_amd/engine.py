@@ -203,3 +203,41 @@ class Engine:
 
     def profile_read(self):
         return native.profile_read(self.native_batch())
+
+
+def load_model(path):
+    """An exported model file through the C++ reader (visualmesh::load_model_file): dict(mesh, shape, radius,
+    intersections, network) with network = list of groups of (weights[n_in, n_out], biases[n_out], activation)."""
+    lib = native.host()
+    handle = lib.vmh_model_load(str(path).encode())
+    if not handle:
+        raise RuntimeError("load_model: " + lib.vmh_last_error().decode())
+    try:
+        mesh = C.create_string_buffer(64)
+        shape = C.create_string_buffer(64)
+        radius, intersections = C.c_float(), C.c_float()
+        n_groups = native.host_check(lib.vmh_model_info(handle, mesh, shape, 64, C.byref(radius), C.byref(intersections)))
+        network = []
+        for g in range(n_groups):
+            group = []
+            for l in range(native.host_check(lib.vmh_model_group_size(handle, g))):
+                n_in, n_out, act = C.c_int(), C.c_int(), C.c_int()
+                native.host_check(lib.vmh_model_layer(handle, g, l, C.byref(n_in), C.byref(n_out), C.byref(act), None, None))
+                w = np.zeros((n_in.value, n_out.value), np.float32)
+                b = np.zeros(n_out.value, np.float32)
+                native.host_check(lib.vmh_model_layer(handle, g, l, C.byref(n_in), C.byref(n_out), C.byref(act), _fp(w), _fp(b)))
+                group.append((w, b, act.value))
+            network.append(group)
+        return dict(mesh=mesh.value.decode(), shape=shape.value.decode(), radius=radius.value,
+                    intersections=intersections.value, network=network)
+    finally:
+        lib.vmh_model_free(handle)
+
+
+def load_lens(path, width, height):
+    """One dataset lens file through the C++ reader: (Lens, Hoc[4, 4] float32)."""
+    lib = native.host()
+    lens = Lens()
+    Hoc = np.zeros((4, 4), np.float32)
+    native.host_check(lib.vmh_lens_load(str(path).encode(), width, height, C.byref(lens), _fp(Hoc)))
+    return lens, Hoc

@@ -203,6 +203,15 @@ def host():
     L.vmh_engine_native_batch.argtypes = [vp]
     L.vmh_engine_clear_cache.argtypes = [vp]
     L.vmh_engine_clear_cache.restype = None
+    L.vmh_model_load.restype = vp
+    L.vmh_model_load.argtypes = [C.c_char_p]
+    L.vmh_model_free.argtypes = [vp]
+    L.vmh_model_free.restype = None
+    L.vmh_model_info.argtypes = [vp, C.c_char_p, C.c_char_p, C.c_int, C.POINTER(C.c_float), C.POINTER(C.c_float)]
+    L.vmh_model_group_size.argtypes = [vp, C.c_int]
+    L.vmh_model_layer.argtypes = [vp, C.c_int, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_int),
+                                  C.POINTER(C.c_float), C.POINTER(C.c_float)]
+    L.vmh_lens_load.argtypes = [C.c_char_p, C.c_int, C.c_int, C.POINTER(Lens), C.POINTER(C.c_float)]
     _host = L
     return L
 
