@@ -321,3 +321,38 @@ def test_reference_example_network_on_its_dataset_poses(oracle):
         print("example pose", p["number"], "V =", len(want["gidx"]), flush=True)
         assert got["cls"].shape[1] == 5
         assert_classification_parity(got, want, PROB_TOL, "example pose " + p["number"])
+
+
+def test_mesh_cache_is_bounded_and_keeps_staged_meshes(oracle):
+    """The device mesh cache releases least recently used meshes beyond its byte limit, never one the staged batch
+    uses, and a mesh that comes back is uploaded again with unchanged results."""
+    cfg = wl.config(1, n_frames=1)
+    o_lens, e_lens = lens_pair(cfg)
+    f = cfg.frames[0]
+    heights = (1.2, 1.0, 0.9)
+    args = [(cfg.model, cfg.shape, cfg.radius, h, cfg.k, cfg.max_distance) for h in heights]
+    meshes = [eng.Mesh(*a) for a in args]
+    engine = eng.Engine(cfg.network, cfg.model)
+    Hocs = []
+    for h in heights:
+        H = np.array(f["Hoc"], np.float32).copy()
+        H[2][3] = h
+        Hocs.append(H)
+    one = meshes[0].n_nodes * (12 + 4 * meshes[0].n_neighbours)
+    engine.set_cache_limit(int(2.5 * one))  # room for two of the three (they are of similar size)
+    want = [oracle.mesh(*a).project(H, o_lens) for a, H in zip(args, Hocs)]
+    for m, H, w in zip(meshes, Hocs, want):
+        assert_projection_parity(engine(m, H, e_lens), w, "first visit")
+    n, nbytes = engine.cache_info()
+    assert n == 2 and nbytes <= 2.5 * one, (n, nbytes)
+    assert_projection_parity(engine(meshes[0], Hocs[0], e_lens), want[0], "mesh that had been released")
+    # a staged batch pins its mesh whatever the limit
+    engine.stage([dict(mesh=meshes[1], Hoc=Hocs[1], lens=e_lens, image=f["image"], fourcc=cfg.fourcc)])
+    engine.set_cache_limit(1)
+    engine(meshes[0], Hocs[0], e_lens)
+    engine(meshes[2], Hocs[2], e_lens)
+    engine.run()
+    got = engine.fetch()[0]
+    assert_projection_parity(got, want[1], "staged mesh after other meshes went through a full cache")
+    n, _ = engine.cache_info()
+    assert n == 2, n  # the staged mesh and the last one used

@@ -30,6 +30,7 @@
 #ifndef VISUALMESH_ENGINE_HIP_ENGINE_HPP
 #define VISUALMESH_ENGINE_HIP_ENGINE_HPP
 
+#include <algorithm>
 #include <cstdint>
 #include <cstring>
 #include <map>
@@ -205,12 +206,21 @@ namespace engine {
             template <template <typename> class Model>
             void stage(const std::vector<Frame<Model>>& frames) const {
                 constexpr int N = Model<Scalar>::N_NEIGHBOURS;
+                staged_since_ = ++clock_;
                 staged_.assign(frames.size(), FrameData());
                 std::vector<vmhip_frame> flat(frames.size());
-                for (size_t i = 0; i < frames.size(); ++i) {
-                    describe(*frames[i].mesh, frames[i].Hoc, frames[i].lens, frames[i].image, frames[i].format, staged_[i]);
-                    flat[i] = staged_[i].frame;
+                staging_ = true;  // meshes described from here on belong to the staged batch
+                try {
+                    for (size_t i = 0; i < frames.size(); ++i) {
+                        describe(*frames[i].mesh, frames[i].Hoc, frames[i].lens, frames[i].image, frames[i].format, staged_[i]);
+                        flat[i] = staged_[i].frame;
+                    }
+                } catch (...) {
+                    staging_ = false;
+                    staged_.clear();
+                    throw;
                 }
+                staging_ = false;
                 vmhip_engine* e = handle(N);
                 if (!batch_) throw_on_error(vmhip_batch_create(e, &batch_));
                 if (!flat.empty()) throw_on_error(vmhip_batch_stage(batch_, flat.data(), int32_t(flat.size()), 1));
@@ -258,12 +268,22 @@ namespace engine {
             vmhip_batch* native_batch() const { return batch_; }
 
             /// Forget the device copies of all meshes (same purpose as the reference OpenCL engine's
-            /// clear_cache, engine/opencl/engine.hpp:559-572). Call it before destroying a mesh this engine
-            /// has seen if another mesh may be created at the same address with the same node count.
+            /// clear_cache, engine/opencl/engine.hpp:559-572). Not needed for correctness: a cached copy is only
+            /// reused for a mesh with the same address, node storage, node count and content fingerprint, so a
+            /// different mesh that the allocator places where an old one lived is uploaded afresh (the reference
+            /// OpenCL engine keys its cache on the address alone, engine/opencl/engine.hpp:603-625).
             void clear_cache() {
                 for (auto& kv : meshes_) vmhip_mesh_release(kv.second.device);
                 meshes_.clear();
+                cache_bytes_ = 0;
+                staged_.clear();  // a staged batch would point at released meshes
             }
+            /// Device memory the mesh cache may hold before the least recently used meshes are released (meshes of
+            /// the currently staged batch are never released). Default 8 GiB: a VisualMesh of many heights stays
+            /// resident, an unbounded stream of distinct meshes does not grow without limit.
+            void set_cache_limit(size_t bytes) { cache_limit_ = bytes; }
+            size_t cache_bytes() const { return cache_bytes_; }
+            size_t cached_meshes() const { return meshes_.size(); }
 
         private:
             struct FlatLayer {
@@ -273,7 +293,11 @@ namespace engine {
             struct MeshEntry {
                 const void* nodes;
                 size_t count;
+                uint64_t fingerprint;
                 vmhip_mesh* device;
+                size_t bytes;
+                uint64_t last_use;
+                uint64_t pinned_by;  ///< the staging (staged_since_) that last used the mesh
             };
             struct FrameData {
                 vmhip_frame frame;
@@ -294,17 +318,44 @@ namespace engine {
                 return engine_;
             }
 
+            /// Over the limit: release least recently used meshes, but none that the staged batch or the running
+            /// call (stamped `now`) uses.
+            void trim_cache(uint64_t now) const {
+                while (cache_bytes_ > cache_limit_) {
+                    auto victim = meshes_.end();
+                    for (auto e = meshes_.begin(); e != meshes_.end(); ++e) {
+                        const bool staged = !staged_.empty() && e->second.pinned_by == staged_since_;
+                        if (!staged && e->second.last_use < now && (victim == meshes_.end() || e->second.last_use < victim->second.last_use)) victim = e;
+                    }
+                    if (victim == meshes_.end()) break;
+                    vmhip_mesh_release(victim->second.device);
+                    cache_bytes_ -= victim->second.bytes;
+                    meshes_.erase(victim);
+                }
+            }
+
             template <template <typename> class Model>
             vmhip_mesh* device_mesh(const Mesh<Scalar, Model>& mesh) const {
                 constexpr int N = Model<Scalar>::N_NEIGHBOURS;
+                const size_t n = mesh.nodes.size();
+                /* FNV-1a over 64 evenly spaced nodes: tells meshes apart that share address, storage and size */
+                uint64_t fingerprint = 1469598103934665603ull;
+                for (size_t k = 0; k < 64 && n > 0; ++k) {
+                    const unsigned char* bytes = reinterpret_cast<const unsigned char*>(&mesh.nodes[(k * (n - 1)) / 63]);
+                    for (size_t b = 0; b < sizeof(mesh.nodes[0]); ++b) fingerprint = (fingerprint ^ bytes[b]) * 1099511628211ull;
+                }
                 auto it = meshes_.find(&mesh);
-                if (it != meshes_.end() && it->second.nodes == mesh.nodes.data() && it->second.count == mesh.nodes.size())
+                if (it != meshes_.end() && it->second.nodes == mesh.nodes.data() && it->second.count == n && it->second.fingerprint == fingerprint) {
+                    it->second.last_use = ++clock_;
+                    if (staging_) it->second.pinned_by = staged_since_;
+                    trim_cache(it->second.last_use);
                     return it->second.device;
+                }
                 if (it != meshes_.end()) {  // another mesh now lives at this address
                     vmhip_mesh_release(it->second.device);
+                    cache_bytes_ -= it->second.bytes;
                     meshes_.erase(it);
                 }
-                const size_t n = mesh.nodes.size();
                 std::vector<float> rays(n * 3);
                 std::vector<int32_t> nbr(n * N);
                 for (size_t i = 0; i < n; ++i) {
@@ -313,7 +364,11 @@ namespace engine {
                 }
                 vmhip_mesh* dev = nullptr;
                 throw_on_error(vmhip_mesh_upload(rays.data(), nbr.data(), int32_t(n), N, &dev));
-                meshes_[&mesh] = MeshEntry{mesh.nodes.data(), n, dev};
+                const size_t bytes = n * (3 * sizeof(float) + N * sizeof(int32_t));
+                const uint64_t now = ++clock_;
+                meshes_[&mesh] = MeshEntry{mesh.nodes.data(), n, fingerprint, dev, bytes, now, staging_ ? staged_since_ : 0};
+                cache_bytes_ += bytes;
+                trim_cache(now);
                 return dev;
             }
 
@@ -363,6 +418,9 @@ namespace engine {
             mutable int engine_nn_ = -1;
             mutable vmhip_batch* batch_ = nullptr;
             mutable std::map<const void*, MeshEntry> meshes_;
+            mutable uint64_t clock_ = 0, staged_since_ = 0;
+            mutable bool staging_ = false;
+            mutable size_t cache_bytes_ = 0, cache_limit_ = size_t(8) << 30;
             mutable std::vector<FrameData> staged_;
         };
 

@@ -192,6 +192,15 @@ class Engine:
         self.run()
         return self.fetch()
 
+    def set_cache_limit(self, nbytes):
+        self._lib.vmh_engine_set_cache_limit(self.ptr, int(nbytes))
+
+    def cache_info(self):
+        """(meshes resident on the device, their bytes)"""
+        nbytes = C.c_uint64()
+        n = self._lib.vmh_engine_cache_info(self.ptr, C.byref(nbytes))
+        return n, nbytes.value
+
     def native_batch(self):
         return C.c_void_p(self._lib.vmh_engine_native_batch(self.ptr))
 

@@ -203,6 +203,9 @@ def host():
     L.vmh_engine_native_batch.argtypes = [vp]
     L.vmh_engine_clear_cache.argtypes = [vp]
     L.vmh_engine_clear_cache.restype = None
+    L.vmh_engine_set_cache_limit.argtypes = [vp, C.c_uint64]
+    L.vmh_engine_set_cache_limit.restype = None
+    L.vmh_engine_cache_info.argtypes = [vp, C.POINTER(C.c_uint64)]
     L.vmh_model_load.restype = vp
     L.vmh_model_load.argtypes = [C.c_char_p]
     L.vmh_model_free.argtypes = [vp]
