@@ -204,11 +204,11 @@ def test_bf16_engine_keeps_narrow_networks_in_fp32(oracle):
     assert_classification_parity(got, want, PROB_TOL, "bf16 engine, narrow network")
 
 
-@pytest.mark.parametrize("kernel", ["rows", "mfma", "lds", "dma"])
+@pytest.mark.parametrize("kernel", ["rows", "mfma", "lds", "dma", "flow"])
 def test_every_convolution_kernel_agrees_with_the_oracle(oracle, kernel, monkeypatch):
     """Every layer shape of configuration 2 through the one-row-per-lane kernel, the matrix-core kernel that
-    gathers into registers and the two matrix-core kernels that gather from LDS (rows staged through registers /
-    loaded straight into LDS), selected with VMHIP_CONV_KERNEL when the engine is built."""
+    gathers into registers and the matrix-core kernels that gather from LDS (rows staged through registers /
+    loaded straight into LDS / the same without barriers in the tile loop), selected with VMHIP_CONV_KERNEL when the engine is built."""
     monkeypatch.setenv("VMHIP_CONV_KERNEL", kernel)
     cfg = wl.config(2, n_frames=2)
     o_lens, e_lens = lens_pair(cfg)
@@ -223,14 +223,19 @@ def test_every_convolution_kernel_agrees_with_the_oracle(oracle, kernel, monkeyp
     assert len(names) == 8, names
     if kernel == "mfma":
         assert all(n.startswith("conv_mfma_") or n == "conv_rows_16x3s7" for n in names), names
+    elif kernel == "flow":  # instantiated for the layers that are bound by the matrix pipe; the rest stay on "lds"
+        pre = "conv_%s_" % kernel
+        assert [n for n in names if n.startswith(pre)] == [pre + "16x32s7"] + [pre + "32x32s7"] * 4 + [pre + "32x16s7"], names
+        assert all(n.startswith((pre, "conv_lds_", "conv_narrow_")) for n in names), names
     else:
         assert all(n.startswith("conv_%s_" % kernel) for n in names), names
     for i, f in enumerate(cfg.frames):
         want = pick(o_mesh, f["Hoc"]).classify(f["Hoc"], o_lens, f["image"], cfg.fourcc, vmo.Network(cfg.network))
         assert_classification_parity(results[i], want, PROB_TOL, "%s frame %d" % (kernel, i))
+    assert native.hip().vm_flow_timeouts_read() == 0  # no wave of the barrier-free kernel ever ran out of polls
 
 
-@pytest.mark.parametrize("kernel", ["lds", "dma"])
+@pytest.mark.parametrize("kernel", ["lds", "dma", "flow"])
 @pytest.mark.parametrize("index", [2, 3])
 def test_rows_beyond_the_halo_capacity(oracle, index, kernel, monkeypatch):
     """With only 8 halo slots per tile most out-of-tile neighbours are marked as not staged and the LDS kernel
@@ -246,9 +251,12 @@ def test_rows_beyond_the_halo_capacity(oracle, index, kernel, monkeypatch):
     engine.profile(True)
     engine.run()
     names = [n for n, _, _ in engine.profile_read() if n.startswith("conv")]
-    assert all(n.startswith("conv_%s_" % kernel) for n in names), names
+    assert all(n.startswith(("conv_%s_" % kernel, "conv_lds_", "conv_narrow_") if kernel == "flow" else "conv_%s_" % kernel) for n in names), names
+    if not (kernel == "flow" and index == 3):  # that kernel has no instantiation for the 24-wide NMGrid8 network
+        assert any(n.startswith("conv_%s_" % kernel) for n in names), names
     want = pick(o_mesh, f["Hoc"]).classify(f["Hoc"], o_lens, f["image"], cfg.fourcc, vmo.Network(cfg.network))
     assert_classification_parity(got, want, PROB_TOL, "halo cap 8, cfg%d, %s" % (index, kernel))
+    assert native.hip().vm_flow_timeouts_read() == 0
 
 
 def test_graph_replays_match_eager_runs(oracle, monkeypatch):

@@ -63,6 +63,7 @@ def build_hip(force=False):
         ("conv_mfma.hip", HIP_FLAGS),
         ("conv_lds.hip", HIP_FLAGS),
         ("conv_dma.hip", HIP_FLAGS),
+        ("conv_flow.hip", HIP_FLAGS),
         ("conv_narrow.hip", HIP_FLAGS),
         ("api.hip", HIP_FLAGS),
     ]

@@ -165,7 +165,7 @@ __global__ __launch_bounds__(NW * 64, 4) void vm_conv_dma_kernel(VmBatchDev B, V
     auto request_positions = [&](const int4& d, v4u (&nbl)[RB]) {
         if constexpr (NN > 0) {
 #pragma unroll
-            for (int rb = 0; rb < RB; ++rb) nbl[rb] = __builtin_amdgcn_raw_buffer_load_b128(nbl_rsrc, (d.x + own_row(d.y, rb)) * (VMHIP_NBL_STRIDE * 2), 0, 0);
+            for (int rb = 0; rb < RB; ++rb) nbl[rb] = vm_load_nbl_row<NN>(nbl_rsrc, (d.x + own_row(d.y, rb)) * (VMHIP_NBL_STRIDE * 2));
         }
     };
     /* descriptors travel through vector memory: a scalar load in flight would turn every LDS wait into a full wait */

@@ -217,7 +217,7 @@ __global__ __launch_bounds__(NW * 64, 4) void vm_conv_lds_kernel(VmBatchDev B, V
     auto request_positions = [&](const int4& d, v4u (&nbl)[RB]) {
         if constexpr (NN > 0) {
 #pragma unroll
-            for (int rb = 0; rb < RB; ++rb) nbl[rb] = __builtin_amdgcn_raw_buffer_load_b128(nbl_rsrc, (d.x + own_row(d.y, rb)) * (VMHIP_NBL_STRIDE * 2), 0, 0);
+            for (int rb = 0; rb < RB; ++rb) nbl[rb] = vm_load_nbl_row<NN>(nbl_rsrc, (d.x + own_row(d.y, rb)) * (VMHIP_NBL_STRIDE * 2));
         }
     };
     /* Tile descriptors are wave-uniform but must not be fetched with scalar loads: scalar loads return out of

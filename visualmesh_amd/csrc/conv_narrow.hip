@@ -161,7 +161,7 @@ __global__ __launch_bounds__(NW * 64) void vm_conv_narrow_kernel(VmBatchDev B, V
      * the store */
     auto own_row = [&](int rows_in_use) { return max(0, min((int) threadIdx.x, rows_in_use - 1)); };
     auto request_positions = [&](const int4& d) {
-        return __builtin_amdgcn_raw_buffer_load_b128(nbl_rsrc, (d.x + own_row(d.y)) * (VMHIP_NBL_STRIDE * 2), 0, 0);
+        return vm_load_nbl_row<NN>(nbl_rsrc, (d.x + own_row(d.y)) * (VMHIP_NBL_STRIDE * 2));
     };
     auto load_desc = [&](int t) {
         const v4u d = __builtin_amdgcn_raw_buffer_load_b128(desc_rsrc, t * 16, 0, 0);

@@ -139,10 +139,39 @@ bool vm_lds_supported(int c_in, int c_out, int slots);
 int vm_launch_conv_lds(const VmBatchDev& B, const VmLayerDev& L, const float* in, float* out, hipStream_t stream,
                        const char** kernel_name);
 
+/* A row of the tile-local neighbour table, read with a load exactly as wide as the NN entries in use. A wider load
+ * leaves dead result registers; the compiler reuses them at once, and that reuse must wait for the load - and for every
+ * load issued before it - to return. */
+template <int NN>
+__device__ __forceinline__ __attribute__((ext_vector_type(4))) uint32_t vm_load_nbl_row(__amdgpu_buffer_rsrc_t rsrc, int byte_offset) {
+    typedef uint32_t u2 __attribute__((ext_vector_type(2)));
+    typedef uint32_t u3 __attribute__((ext_vector_type(3)));
+    typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+    if constexpr (NN <= 2) {
+        return u4{__builtin_amdgcn_raw_buffer_load_b32(rsrc, byte_offset, 0, 0), 0u, 0u, 0u};
+    }
+    else if constexpr (NN <= 4) {
+        const u2 t = __builtin_amdgcn_raw_buffer_load_b64(rsrc, byte_offset, 0, 0);
+        return u4{t.x, t.y, 0u, 0u};
+    }
+    else if constexpr (NN <= 6) {
+        const u3 t = __builtin_amdgcn_raw_buffer_load_b96(rsrc, byte_offset, 0, 0);
+        return u4{t.x, t.y, t.z, 0u};
+    }
+    else {
+        return __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_offset, 0, 0);
+    }
+}
+
 /* the same with rows brought into LDS by buffer_load ... lds and two alternating row buffers (conv_dma.hip) */
 bool vm_dma_supported(int c_in, int c_out, int slots);
 int vm_launch_conv_dma(const VmBatchDev& B, const VmLayerDev& L, const float* in, float* out, hipStream_t stream,
                        const char** kernel_name);
+/* the same with LDS counters in place of the tile loop's barriers, so that the waves of a block run freely between
+ * "my tile is staged" and "my buffer may be refilled" (conv_flow.hip) */
+bool vm_flow_supported(int c_in, int c_out, int slots);
+int vm_launch_conv_flow(const VmBatchDev& B, const VmLayerDev& L, const float* in, float* out, hipStream_t stream,
+                        const char** kernel_name);
 
 /* layers with at most four output channels on v_mfma_f32_4x4x1 (64 rows x 4 channels per instruction), staged like
  * conv_dma.hip (conv_narrow.hip); reads the plain row-major weights */
