@@ -8,19 +8,26 @@
  * What differs is how the 16 waves of a block stay in step. A barrier makes all of them change phase together, so
  * the matrix pipe idles whenever the block applies activations, stores or waits for the barrier itself. Here two
  * counters per row buffer, kept in LDS, take its place:
- *   staged[b]   += 1 by every wave once its own share of a tile's loads has landed in buffer b,
+ *   staged[b]   += 1 by every loader once its share of a tile's loads has landed in buffer b,
  *   consumed[b] += 1 by every wave once it has read the last operand of the tile in buffer b.
- * A wave starts to contract tile k when staged[k & 1] has reached 16 per tile staged there so far, and issues its
- * share of the loads of tile k+2 into that buffer when consumed[k & 1] has. It reports its share of tile k+1 (requested
- * a tile earlier) right after it has contracted tile k. Between those points it runs freely: while one wave applies the activation and stores, the others on its SIMD keep the matrix pipe busy, and
- * a wave that is done early goes on with the next tile, which already lies in the other buffer.
+ * A wave starts to contract tile k when staged[k & 1] says the tile is complete, and otherwise runs freely: while
+ * one wave applies the activation and stores, the others on its SIMD keep the matrix pipe busy, and a wave that is
+ * done early goes on with the next tile, which already lies in the other buffer.
+ * The first four waves of the block (one per SIMD, and the ones the SIMDs serve first) are the loaders. Besides
+ * contracting their rows like everyone else they bring in all data: a tile's rows, its rows of the neighbour table
+ * and its descriptor go into the buffer; the descriptor and the halo row numbers of the tile after go into a slot
+ * of the loader's own, from which it works out, right after a contraction, where each piece of that tile lies. It
+ * issues those loads into buffer k & 1 once consumed[k & 1] says every wave is done with tile k, and reports its
+ * loads of tile k+1 (issued a tile earlier) just before.
  * Everything a wave waits for at step k depends only on what all waves do at step k-1, so the waits cannot form a
  * cycle; each is nevertheless bounded by a poll count, after which the wave goes on (and counts the event in
  * vm_flow_timeouts) rather than hang.
- * Loads are counted, not drained: a wave knows how many vector memory instructions it has issued after the ones it
- * needs (they complete in order) and waits with s_waitcnt vmcnt(that many), so the loads of tile k+1, in flight
- * behind them, are not waited for. For that count to be a constant every load and store of the loop is issued
- * unconditionally, with an out-of-range offset where there is nothing to move.
+ * Loads are counted, not drained: a loader knows how many vector memory instructions it has issued after the ones
+ * it needs (they complete in order) and waits with s_waitcnt vmcnt(that many), so the loads of the next tile, in
+ * flight behind them, are not waited for. For that count to be a constant every load and store of the loop is
+ * issued unconditionally, with an out-of-range offset where there is nothing to move, and no load of the loop
+ * returns into a register: the compiler would wait for such a register by its own count, which misses the loads
+ * written as assembly below.
  * A wave never ends with LDS loads in flight (the LDS could already belong to another block).
  */
 #include <cstdlib>
@@ -104,12 +111,24 @@ __host__ __device__ constexpr size_t dma_lds_bytes(int c_in, int c_out, int slot
 }
 
 constexpr int FLOW_WAVES = 16;
-constexpr int FLOW_LOADERS = 4;
-constexpr int FLOW_HALO = 224; /* halo rows staged per tile: rows and neighbour tables of two tiles fit beside the weights */
+constexpr int FLOW_LOADERS = 4; /* measured: 8 loaders 2 % slower, every wave loading its own sixteenth 12 % slower */
+/* wave priorities (s_setprio): contracting a tile while the tile before is still being read by others / contracting
+ * the oldest unread tile / everything else. Measured on the 32 -> 32 layer: without the rule 152 us, with it 147 us;
+ * "everything else" at 1 instead of 3: 158 us. */
+#define FLOW_PRIO_AHEAD 0
+#define FLOW_PRIO_BEHIND 2
+#define FLOW_PRIO_REST 3
+#define FLOW_SLEEP 1
+constexpr int FLOW_HALO = 192; /* halo rows staged per tile: two tiles, their neighbour tables and the loaders' slots fit beside the weights */
 constexpr int FLOW_POLLS = 1 << 18;
+/* rounds of NT loads that fill a buffer's rows, and how many of them reach into the halo rows */
+__host__ __device__ constexpr int flow_rounds(int c_in) { return ((VMHIP_TILE + FLOW_HALO) * (row_stride(c_in) / 4) + FLOW_WAVES * 64 - 1) / (FLOW_WAVES * 64); }
+__host__ __device__ constexpr int flow_halo_rounds(int c_in) { return flow_rounds(c_in) - VMHIP_TILE * (row_stride(c_in) / 4) / (FLOW_WAVES * 64); }
+/* words of a loader's slot: a descriptor, then one halo row number per lane and load it will issue */
+__host__ __device__ constexpr int flow_slot_words(int c_in) { return 4 + (FLOW_WAVES / FLOW_LOADERS) * flow_halo_rounds(c_in) * 64; }
 __host__ __device__ constexpr size_t flow_lds_bytes(int c_in, int c_out, int slots) {
     return (size_t(slots) * (c_in / 4) * ((c_out + 15) / 16) * 64 + size_t((c_out + 15) / 16) * 16
-            + 2 * (size_t(VMHIP_TILE + FLOW_HALO) * row_stride(c_in) + VMHIP_TILE * 4 + 4) + 4 + 4 * FLOW_LOADERS) * 4;
+            + 2 * (size_t(VMHIP_TILE + FLOW_HALO) * row_stride(c_in) + VMHIP_TILE * 4 + 4) + 4 + size_t(FLOW_LOADERS) * flow_slot_words(c_in)) * 4;
 }
 
 /* polls an LDS counter until it has reached target (wrap-safe); false when the polls ran out. The read is spelled
@@ -120,7 +139,7 @@ __device__ __forceinline__ bool wait_counter(const uint32_t* counter, uint32_t t
         uint32_t v;
         asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(at) : "memory");
         if ((int32_t) (__builtin_amdgcn_readfirstlane(v) - target) >= 0) return true;
-        __builtin_amdgcn_s_sleep(1);
+        __builtin_amdgcn_s_sleep(FLOW_SLEEP);
     }
     return false;
 }
@@ -183,6 +202,8 @@ __global__ __launch_bounds__(FLOW_WAVES * 64) void vm_conv_flow_kernel(VmBatchDe
     constexpr int N_AHEAD = 1 + SHARE * N_HALO;
     constexpr int N_STORE = RB * CB;
     static_assert(N_STORE + 2 * N_FILL + N_AHEAD < 64, "the counts must fit s_waitcnt vmcnt");
+    static_assert(N_DMA == flow_rounds(C_IN) && N_HALO == flow_halo_rounds(C_IN), "the LDS size is computed from the same rounds");
+    constexpr int SLOT_WORDS = flow_slot_words(C_IN);
 
 #ifdef VM_FLOW_TIMING
     const unsigned long long t_kernel = clock64();
@@ -203,7 +224,8 @@ __global__ __launch_bounds__(FLOW_WAVES * 64) void vm_conv_flow_kernel(VmBatchDe
     const int wave = __builtin_amdgcn_readfirstlane((int) (threadIdx.x >> 6));
     const int q = lane >> 4, r16 = lane & 15;
     const int activation = L.activation;
-    uint32_t* const desc_slot = counters + 4 + 4 * (wave % LOADERS); /* a loader's copy of the descriptor of the tile it stages next */
+    const int lw = wave; /* which loader this wave is, if it is one */
+    uint32_t* const slot = counters + 4 + SLOT_WORDS * (wave % LOADERS); /* a loader's notes on the tile it stages next */
 
     const int n_tiles = B.n_row_tiles;
     const int xcd = blockIdx.x & 7, lb = blockIdx.x >> 3, gx = gridDim.x >> 3;
@@ -222,34 +244,42 @@ __global__ __launch_bounds__(FLOW_WAVES * 64) void vm_conv_flow_kernel(VmBatchDe
     const v4u nbl_rsrc = raw_rsrc(B.row_nbl, (uint64_t) total_rows * VMHIP_NBL_STRIDE * 2);
     const v4u desc_lds_rsrc = raw_rsrc(B.tile_desc, (uint64_t) n_tiles * 16);
     const __amdgpu_buffer_rsrc_t halo_rsrc = make_rsrc(B.tile_halo, (uint64_t) n_tiles * VMHIP_HALO_MAX * 4);
+    const v4u halo_lds_rsrc = raw_rsrc(B.tile_halo, (uint64_t) n_tiles * VMHIP_HALO_MAX * 4);
     const __amdgpu_buffer_rsrc_t desc_rsrc = make_rsrc(B.tile_desc, (uint64_t) n_tiles * 16);
 
     /* Piece p of a buffer = 16 bytes at LDS row p / RSP, position p % RSP. Round r fills pieces first_piece(r) + t for
-     * t = 0..NT-1; a loader plays threads (wave * SHARE + v) * 64 + lane, v < SHARE. */
+     * t = 0..NT-1; a loader plays threads (lw * SHARE + v) * 64 + lane, v < SHARE. */
     auto first_piece = [](int r) { return r * NT < PIECES - NT ? r * NT : PIECES - NT; };
-    auto request_halo_rows = [&](int t, uint32_t (&hrow)[SHARE][N_HALO]) {
+    /* which halo row (of the tile's list) the lane's piece in halo round r of share v belongs to; negative: a main row */
+    auto halo_index = [&](int v, int r) { return (first_piece(N_MAIN + r) + (lw * SHARE + v) * 64 + lane) / RSP - VMHIP_TILE; };
+    /* the halo row numbers of tile t into registers (the prologue's way) */
+    auto load_halo_rows = [&](int t, uint32_t (&hrow)[SHARE][N_HALO]) {
 #pragma unroll
         for (int v = 0; v < SHARE; ++v)
 #pragma unroll
             for (int r = 0; r < N_HALO; ++r) {
-                const int h = (first_piece(N_MAIN + r) + (wave * SHARE + v) * 64 + lane) / RSP - VMHIP_TILE; /* negative: a main row, reads 0, unused */
+                const int h = halo_index(v, r);
                 hrow[v][r] = __builtin_amdgcn_raw_buffer_load_b32(halo_rsrc, h >= 0 ? (t * VMHIP_HALO_MAX + h) * 4 : 0xffffffffu, 0, 0);
             }
     };
-    /* tile t = {first row, .., halo rows, ..}; live = false moves nothing (zeros land in LDS) */
-    auto stage = [&](int t, int first, int halo, const uint32_t (&hrow)[SHARE][N_HALO], float* buf, bool live) {
-        const uint32_t base = lds_address(buf);
-        /* Name every halo row number before the first load below is issued: the compiler waits for a register a load
-         * fills by counting the vector memory instructions it knows were issued after that load, and the loads
-         * below are not among them, so a wait placed after some of them would drain those too. */
+    /* descriptor and halo row numbers of tile t into the loader's slot (the loop's way: N_AHEAD loads) */
+    auto request_ahead = [&](int t) {
+        const uint32_t base = lds_address(slot);
+        if (lane < 4) load_to_lds_b32(desc_lds_rsrc, base, t * 16 + lane * 4);
 #pragma unroll
         for (int v = 0; v < SHARE; ++v)
 #pragma unroll
-            for (int r = 0; r < N_HALO; ++r) asm volatile("" ::"v"(hrow[v][r]));
+            for (int r = 0; r < N_HALO; ++r) {
+                const int h = halo_index(v, r);
+                load_to_lds_b32(halo_lds_rsrc, base + (4 + (v * N_HALO + r) * 64) * 4, h >= 0 ? (uint32_t) ((t * VMHIP_HALO_MAX + h) * 4) : 0xffffffffu);
+            }
+    };
+    /* where in the input each piece this loader fetches for a tile lies: first = the tile's first row, halo = its halo
+     * rows, hrow(v, r) = the halo row number for the lane's piece; live = false moves nothing (zeros land in LDS) */
+    auto plan = [&](int first, int halo, bool live, auto hrow, uint32_t (&offs)[SHARE][N_DMA]) {
 #pragma unroll
         for (int v = 0; v < SHARE; ++v) {
-            const int vt = (wave * SHARE + v) * 64 + lane;
-            uint32_t offs[N_DMA];
+            const int vt = (lw * SHARE + v) * 64 + lane;
 #pragma unroll
             for (int r = 0; r < N_DMA; ++r) {
                 const int p = first_piece(r) + vt;
@@ -258,16 +288,23 @@ __global__ __launch_bounds__(FLOW_WAVES * 64) void vm_conv_flow_kernel(VmBatchDe
                 uint32_t off = (uint32_t) ((first + row_l) * Q4 + c) * 16u;
                 if (r >= N_MAIN) {
                     const int h = row_l - VMHIP_TILE;
-                    if (h >= 0) off = h < halo ? (hrow[v][r - N_MAIN] * Q4 + c) * 16u : 0xffffffffu;
+                    if (h >= 0) off = h < halo ? (hrow(v, r - N_MAIN) * Q4 + c) * 16u : 0xffffffffu;
                 }
                 if (RSP != Q4 && cp >= Q4) off = 0xffffffffu; /* padding piece */
-                if (!live) off = 0xffffffffu;
-                offs[r] = off;
+                offs[v][r] = live ? off : 0xffffffffu;
             }
+        }
+    };
+    /* the N_FILL loads of tile t */
+    auto fill = [&](int t, int first, bool live, const uint32_t (&offs)[SHARE][N_DMA], float* buf) {
+        const uint32_t base = lds_address(buf);
 #pragma unroll
-            for (int r = 0; r < N_DMA; ++r) load_to_lds_b128(in_rsrc, base + (first_piece(r) + (wave * SHARE + v) * 64) * 16, offs[r]);
+        for (int v = 0; v < SHARE; ++v) {
+#pragma unroll
+            for (int r = 0; r < N_DMA; ++r) load_to_lds_b128(in_rsrc, base + (first_piece(r) + (lw * SHARE + v) * 64) * 16, offs[v][r]);
             /* the tile's rows of the neighbour table, 4 bytes per lane */
-            load_to_lds_b32(nbl_rsrc, base + (NBL_AT + (wave * SHARE + v) * 64) * 4, live ? (uint32_t) (first * (VMHIP_NBL_STRIDE * 2) + vt * 4) : 0xffffffffu);
+            load_to_lds_b32(nbl_rsrc, base + (NBL_AT + (lw * SHARE + v) * 64) * 4,
+                            live ? (uint32_t) (first * (VMHIP_NBL_STRIDE * 2) + ((lw * SHARE + v) * 64 + lane) * 4) : 0xffffffffu);
         }
         /* and its descriptor (every loader writes the same four words) */
         if (lane < 4) load_to_lds_b32(desc_lds_rsrc, base + DESC_AT * 4, live ? (uint32_t) (t * 16 + lane * 4) : 0xffffffffu);
@@ -282,9 +319,6 @@ __global__ __launch_bounds__(FLOW_WAVES * 64) void vm_conv_flow_kernel(VmBatchDe
         return make_int4(__builtin_amdgcn_readfirstlane((int) d.x), __builtin_amdgcn_readfirstlane((int) d.y),
                          __builtin_amdgcn_readfirstlane((int) d.z), __builtin_amdgcn_readfirstlane((int) d.w));
     };
-    auto request_desc = [&](int t) {
-        if (lane < 4) load_to_lds_b32(desc_lds_rsrc, lds_address(desc_slot), t * 16 + lane * 4);
-    };
     auto read_desc = [&](const void* at) {
         const v4u d = *reinterpret_cast<const v4u*>(at);
         return make_int4(__builtin_amdgcn_readfirstlane((int) d.x), __builtin_amdgcn_readfirstlane((int) d.y),
@@ -296,20 +330,29 @@ __global__ __launch_bounds__(FLOW_WAVES * 64) void vm_conv_flow_kernel(VmBatchDe
     };
 
     /* ---- prologue: tiles 0 and 1 on their way into the two buffers, tile 2 described ---- */
-    const bool loader = wave < LOADERS;
-    uint32_t hrow_n2[SHARE][N_HALO];
+    const bool loader = lw < LOADERS;
+    uint32_t offs[SHARE][N_DMA]; /* a loader's plan for the tile it fills next */
+    int first_new = 0;
     if (loader) {
         uint32_t h0[SHARE][N_HALO], h1[SHARE][N_HALO];
-        request_halo_rows(tile_of(0), h0);
-        request_halo_rows(tile_of(1), h1);
+        load_halo_rows(tile_of(0), h0);
+        load_halo_rows(tile_of(1), h1);
         const int4 d0 = load_desc(tile_of(0)), d1 = load_desc(tile_of(1));
+        /* Name every register a load fills before the first load that the compiler does not know of: it waits for
+         * such a register by counting the vector memory instructions it knows were issued after the load, so a
+         * wait placed later would drain the unknown ones too. */
+#pragma unroll
+        for (int v = 0; v < SHARE; ++v)
+#pragma unroll
+            for (int r = 0; r < N_HALO; ++r) asm volatile("" ::"v"(h0[v][r]), "v"(h1[v][r]));
+        request_ahead(tile_of(2));
         __syncthreads(); /* weights, biases and the zeroed counters are in LDS */
-        stage(tile_of(0), d0.x, d0.z, h0, buf0, true);
-        stage(tile_of(1), d1.x, d1.z, h1, buf0 + BUF_FLOATS, 1 < count);
-        request_desc(tile_of(2));
-        request_halo_rows(tile_of(2), hrow_n2);
-        /* tile 0 has landed once only the requests made after it can still be in flight */
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N_FILL + N_AHEAD) : "memory");
+        plan(d0.x, d0.z, true, [&](int v, int r) { return h0[v][r]; }, offs);
+        fill(tile_of(0), d0.x, true, offs, buf0);
+        plan(d1.x, d1.z, 1 < count, [&](int v, int r) { return h1[v][r]; }, offs);
+        fill(tile_of(1), d1.x, 1 < count, offs, buf0 + BUF_FLOATS);
+        /* tile 0 has landed once only the loads of tile 1 can still be in flight */
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N_FILL) : "memory");
         if (lane == 0) atomicAdd(&counters[0], 1u);
     }
     else {
@@ -338,8 +381,8 @@ __global__ __launch_bounds__(FLOW_WAVES * 64) void vm_conv_flow_kernel(VmBatchDe
                 asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(before) : "v"(at) : "memory");
                 before = __builtin_amdgcn_readfirstlane(before);
             }
-            if (k == 0 || (int32_t) (before - NW * (uint32_t) (((k - 1) >> 1) + 1)) >= 0) __builtin_amdgcn_s_setprio(2);
-            else __builtin_amdgcn_s_setprio(0);
+            if (k == 0 || (int32_t) (before - NW * (uint32_t) (((k - 1) >> 1) + 1)) >= 0) __builtin_amdgcn_s_setprio(FLOW_PRIO_BEHIND);
+            else __builtin_amdgcn_s_setprio(FLOW_PRIO_AHEAD);
         }
 
         const bool in_use = d_cur.y > 0;
@@ -457,8 +500,19 @@ __global__ __launch_bounds__(FLOW_WAVES * 64) void vm_conv_flow_kernel(VmBatchDe
         /* every operand of the tile has been read (the matrix instructions above consumed them) */
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         if (lane == 0) atomicAdd(&counters[2 + b], 1u);
-        __builtin_amdgcn_s_setprio(3); /* what follows is short and keeps no matrix pipe busy: let it through */
+        __builtin_amdgcn_s_setprio(FLOW_PRIO_REST); /* what follows is short and keeps no matrix pipe busy: let it through */
         FLOW_T(1);
+        if (loader) {
+            /* The notes on tile k+2, requested a tile ago, are in the slot once nothing but what was requested after
+             * them can still be in flight: the loads of tile k+1 and the stores of tile k-1 (of tiles 0 and 1 at first). */
+            if (k == 0) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * N_FILL) : "memory");
+            else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N_STORE + N_FILL) : "memory");
+            const int4 d_new = read_desc(slot);
+            first_new = d_new.x;
+            plan(d_new.x, d_new.z, k + 2 < count, [&](int v, int r) { return slot[4 + (v * N_HALO + r) * 64 + lane]; }, offs);
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); /* the slot has been read: it may be written again */
+            request_ahead(tile_of(k + 3));
+        }
 
         /* activation: lane holds channels cb*16 + q*4 + {0..3} of row rb*16 + r16; one uniform branch */
         auto for_each_value = [&](auto fn) {
@@ -521,11 +575,7 @@ __global__ __launch_bounds__(FLOW_WAVES * 64) void vm_conv_flow_kernel(VmBatchDe
             /* tile k+2 goes where tile k was, once every wave has read the last of tile k */
             if (!wait_counter(&counters[2 + b], NW * round)) give_up();
             FLOW_T(4);
-            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N_STORE) : "memory"); /* tile k+2's descriptor and halo row numbers are here */
-            const int4 d_new = read_desc(desc_slot);
-            stage(tile_of(k + 2), d_new.x, d_new.z, hrow_n2, buf0 + b * BUF_FLOATS, k + 2 < count);
-            request_desc(tile_of(k + 3));
-            request_halo_rows(tile_of(k + 3), hrow_n2);
+            fill(tile_of(k + 2), first_new, k + 2 < count, offs, buf0 + b * BUF_FLOATS);
             FLOW_T(5);
         }
 #ifdef VM_FLOW_TIMING
