@@ -102,6 +102,7 @@ struct HostLayer {
     float* d_w = nullptr;
     float* d_b = nullptr;
     void* d_w_mfma = nullptr;
+    float* d_w_flow = nullptr; /* w_mfma in conv_flow.hip's LDS order */
     int32_t in_bf16 = 0, out_bf16 = 0, arith_bf16 = 0;
     bool use_lds = false, use_mfma = false, use_dma = false, use_flow = false, use_narrow = false; /* which matrix-core kernels may take the layer */
     std::vector<float> h_w; /* kept until the row types are planned */
@@ -416,7 +417,7 @@ int batch_enqueue(vmhip_batch* b) {
     int cur = 0;
     if (b->classify) {
         for (const HostLayer& L : E->layers) {
-            VmLayerDev ld{L.c_in, L.c_out, L.slots, L.activation, L.d_w, L.d_b, L.d_w_mfma, L.in_bf16, L.out_bf16, L.arith_bf16};
+            VmLayerDev ld{L.c_in, L.c_out, L.slots, L.activation, L.d_w, L.d_b, L.d_w_mfma, L.in_bf16, L.out_bf16, L.arith_bf16, L.d_w_flow};
             const char* name = "conv";
             HIP_TRY(P.begin());
             int rc = -1;
@@ -700,6 +701,13 @@ int vmhip_engine_create(const vmhip_network* net, int32_t n_neighbours, int32_t 
                 if (hipMalloc(&H.d_w_mfma, wp.size()) != hipSuccess) return bail(VMHIP_ERR_HIP, "engine_create: out of device memory");
                 if (hipMemcpy(H.d_w_mfma, wp.data(), wp.size(), hipMemcpyHostToDevice) != hipSuccess)
                     return bail(VMHIP_ERR_HIP, "engine_create: weight upload failed");
+                if (H.use_flow) {
+                    std::vector<float> wf(wp.size() / sizeof(float));
+                    vm_flow_order_weights(reinterpret_cast<const float*>(wp.data()), H.c_in, H.c_out, H.slots, wf.data());
+                    if (hipMalloc(&H.d_w_flow, wp.size()) != hipSuccess) return bail(VMHIP_ERR_HIP, "engine_create: out of device memory");
+                    if (hipMemcpy(H.d_w_flow, wf.data(), wp.size(), hipMemcpyHostToDevice) != hipSuccess)
+                        return bail(VMHIP_ERR_HIP, "engine_create: weight upload failed");
+                }
             }
             H.h_w.clear();
             H.h_w.shrink_to_fit();
@@ -717,6 +725,7 @@ void vmhip_engine_destroy(vmhip_engine* E) {
         if (L.d_w) (void) hipFree(L.d_w);
         if (L.d_b) (void) hipFree(L.d_b);
         if (L.d_w_mfma) (void) hipFree(L.d_w_mfma);
+        if (L.d_w_flow) (void) hipFree(L.d_w_flow);
     }
     if (E->stream) (void) hipStreamDestroy(E->stream);
     delete E;

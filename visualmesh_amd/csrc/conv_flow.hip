@@ -214,11 +214,17 @@ __global__ __launch_bounds__(FLOW_WAVES * 64) void vm_conv_flow_kernel(VmBatchDe
     float* const buf0 = b_lds + CB * 16;
     uint32_t* const counters = reinterpret_cast<uint32_t*>(buf0 + 2 * BUF_FLOATS); /* staged[2], consumed[2] */
     if (threadIdx.x < 4) counters[threadIdx.x] = 0;
-    for (int i = threadIdx.x; i < CB * 16; i += NT) b_lds[i] = i < C_OUT ? L.b[i] : 0.0f;
-    for (int i = threadIdx.x; i < W_FLOATS; i += NT) {
-        const int e = i % G, l = (i / G) % 64, jg = (i / (G * 64)) % (STEPS / G), cb = (i / (G * 64 * (STEPS / G))) % CB, sl = i / (STEPS * 64 * CB);
-        w_lds[i] = reinterpret_cast<const float*>(L.w_mfma)[((sl * STEPS + jg * G + e) * CB + cb) * 64 + l];
+    /* the weights lie in global memory in the order they have in LDS: whole waves of 16 bytes per lane, issued before
+     * anything else so that they travel together with the first descriptors */
+    static_assert(W_FLOATS % 256 == 0, "the weights are whole wave loads");
+    {
+        const v4u w_rsrc = raw_rsrc(L.w_flow, (uint64_t) W_FLOATS * 4);
+        const int wave_at = __builtin_amdgcn_readfirstlane((int) (threadIdx.x >> 6));
+        for (int i = wave_at * 256; i < W_FLOATS; i += NT * 4)
+            load_to_lds_b128(w_rsrc, lds_address(w_lds + i), (uint32_t) (i + (threadIdx.x & 63) * 4) * 4u);
     }
+    static_assert(CB * 16 <= NT, "one bias value per thread at most");
+    const float my_bias = threadIdx.x < C_OUT ? L.b[threadIdx.x] : 0.0f; /* requested now, written to LDS before the barrier */
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int) (threadIdx.x >> 6));
@@ -345,7 +351,9 @@ __global__ __launch_bounds__(FLOW_WAVES * 64) void vm_conv_flow_kernel(VmBatchDe
         for (int v = 0; v < SHARE; ++v)
 #pragma unroll
             for (int r = 0; r < N_HALO; ++r) asm volatile("" ::"v"(h0[v][r]), "v"(h1[v][r]));
+        if (threadIdx.x < CB * 16) b_lds[threadIdx.x] = my_bias;
         request_ahead(tile_of(2));
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N_AHEAD) : "memory"); /* my part of the weights (requested first of all) */
         __syncthreads(); /* weights, biases and the zeroed counters are in LDS */
         plan(d0.x, d0.z, true, [&](int v, int r) { return h0[v][r]; }, offs);
         fill(tile_of(0), d0.x, true, offs, buf0);
@@ -356,6 +364,8 @@ __global__ __launch_bounds__(FLOW_WAVES * 64) void vm_conv_flow_kernel(VmBatchDe
         if (lane == 0) atomicAdd(&counters[0], 1u);
     }
     else {
+        if (threadIdx.x < CB * 16) b_lds[threadIdx.x] = my_bias;
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); /* my part of the weights */
         __syncthreads();
     }
 
@@ -619,6 +629,16 @@ int launch_flow(const VmBatchDev& B, const VmLayerDev& L, const float* in, float
     X(32, 32, 7)                  \
     X(32, 16, 7)
 
+void vm_flow_order_weights(const float* w_mfma, int c_in, int c_out, int slots, float* out) {
+    const int STEPS = c_in / 4, CB = (c_out + 15) / 16;
+    const int G = STEPS % 4 == 0 ? 4 : STEPS % 2 == 0 ? 2 : 1;
+    const int n = slots * STEPS * CB * 64;
+    for (int i = 0; i < n; ++i) {
+        const int e = i % G, l = (i / G) % 64, jg = (i / (G * 64)) % (STEPS / G), cb = (i / (G * 64 * (STEPS / G))) % CB, sl = i / (STEPS * 64 * CB);
+        out[i] = w_mfma[((sl * STEPS + jg * G + e) * CB + cb) * 64 + l];
+    }
+}
+
 bool vm_flow_supported(int c_in, int c_out, int slots) {
 #define X(CI, CO, SL) \
     if (c_in == CI && c_out == CO && slots == SL) return true;
@@ -629,7 +649,7 @@ bool vm_flow_supported(int c_in, int c_out, int slots) {
 
 int vm_launch_conv_flow(const VmBatchDev& B, const VmLayerDev& L, const float* in, float* out, hipStream_t stream, const char** kernel_name) {
     if (B.n_row_tiles <= 0) return 0;
-    if (!B.row_nbl || !B.tile_halo || !B.tile_desc || !L.w_mfma || L.in_bf16 || L.out_bf16 || L.arith_bf16) return -1;
+    if (!B.row_nbl || !B.tile_halo || !B.tile_desc || !L.w_flow || L.in_bf16 || L.out_bf16 || L.arith_bf16) return -1;
 #define X(CI, CO, SL)                                                     \
     if (L.c_in == CI && L.c_out == CO && L.slots == SL) {                 \
         if (kernel_name) *kernel_name = "conv_flow_" #CI "x" #CO "s" #SL; \

@@ -113,6 +113,7 @@ struct VmLayerDev {
     int32_t in_bf16;    /* input rows are stored as bf16 */
     int32_t out_bf16;   /* output rows are stored as bf16 */
     int32_t arith_bf16; /* bf16 products with fp32 accumulation (weights in w_mfma are bf16 then) */
+    const float* w_flow; /* the fp32 w_mfma weights in the order conv_flow.hip keeps them in LDS, or null */
 };
 
 /* launchers, one per kernel; all asynchronous on `stream` */
@@ -170,6 +171,8 @@ int vm_launch_conv_dma(const VmBatchDev& B, const VmLayerDev& L, const float* in
 /* the same with LDS counters in place of the tile loop's barriers, so that the waves of a block run freely between
  * "my tile is staged" and "my buffer may be refilled" (conv_flow.hip) */
 bool vm_flow_supported(int c_in, int c_out, int slots);
+/* host side: w_mfma (fp32, vm_mfma_permute_weights' order) rearranged into that kernel's LDS order; same size */
+void vm_flow_order_weights(const float* w_mfma, int c_in, int c_out, int slots, float* out);
 int vm_launch_conv_flow(const VmBatchDev& B, const VmLayerDev& L, const float* in, float* out, hipStream_t stream,
                         const char** kernel_name);
 
