@@ -144,6 +144,33 @@ int vmhip_batch_run(vmhip_batch* batch);
 int vmhip_batch_counts(const vmhip_batch* batch, int32_t* n_visible);
 int vmhip_batch_fetch(vmhip_batch* batch, vmhip_result* results);
 
+/* What a consumer of the classified mesh does first, done on the device so that only detections cross PCIe. No
+ * counterpart inside the reference's engines: its consumers walk the whole ClassifiedMesh on the host
+ * (example/draw.hpp:41-59), over the neighbourhood table of engine/cpu/engine.hpp:113-129.
+ * A node of a frame is detected if its probability of class_index is at least threshold and, with arg_max_only != 0,
+ * no other class has a larger one (of equal ones the first wins, like std::max_element). Detections keep the order
+ * of the visible nodes. With clusters != 0 they are also grouped into the connected components of the neighbourhood
+ * graph restricted to the detections; clusters are numbered by their first detection.
+ * Per frame: capacity / cluster_capacity say how much the caller's arrays hold; n_detections / n_clusters are
+ * always written; if a capacity is too small the call returns VMHIP_ERR_CAPACITY and copies nothing.
+ * Any array pointer may be NULL to skip that output. */
+typedef struct vmhip_detections {
+    int32_t capacity;
+    int32_t cluster_capacity;
+    int32_t n_detections;
+    int32_t n_clusters;
+    int32_t* node;         /* [n_detections] index into the mesh */
+    float* pixel;          /* [n_detections][2] */
+    float* probability;    /* [n_detections] */
+    int32_t* cluster;      /* [n_detections] cluster number */
+    int32_t* cluster_size; /* [n_clusters] */
+    float* cluster_box;    /* [n_clusters][4] min x, min y, max x, max y */
+    float* cluster_centre; /* [n_clusters][2] mean pixel (summed in no fixed order: last bits may vary) */
+} vmhip_detections;
+/* works on the results of the last vmhip_batch_run of a batch staged with classify != 0; out has one entry per frame */
+int vmhip_batch_detect(vmhip_batch* batch, int32_t class_index, float threshold, int32_t arg_max_only, int32_t clusters,
+                       vmhip_detections* out);
+
 /* Per-kernel timing of vmhip_batch_run with HIP events on the stream the kernels run on.
  * enable = 1 brackets every kernel launch of later runs with events (an event pair between two
  * kernels costs a few microseconds of idle GPU); enable = 2, valid after a run made with enable = 1,

@@ -364,3 +364,77 @@ def test_mesh_cache_is_bounded_and_keeps_staged_meshes(oracle):
     assert_projection_parity(got, want[1], "staged mesh after other meshes went through a full cache")
     n, _ = engine.cache_info()
     assert n == 2, n  # the staged mesh and the last one used
+
+
+@pytest.mark.parametrize("arg_max_only", [False, True])
+def test_detections_and_clusters_on_the_device(oracle, arg_max_only):
+    """vmhip_batch_detect against the same selection and clustering done on the host from the full download of the same
+    run: the detected nodes (order, mesh indices, pixels, probabilities) must be identical, and the clusters must be
+    the connected components scipy finds in the neighbourhood graph restricted to the detections, numbered by their
+    first detection; sizes and bounding boxes exact, centres to rounding. (The probabilities themselves are checked
+    against the oracle by the tests above; here both sides start from the same device results.)"""
+    import scipy.sparse as sp
+    from scipy.sparse.csgraph import connected_components
+    cfg = wl.config(2, n_frames=3)
+    _, e_lens = lens_pair(cfg)
+    _, e_mesh = meshes_for(cfg, oracle)
+    engine = eng.Engine(cfg.network, cfg.model)
+    frames = [dict(mesh=e_mesh, Hoc=f["Hoc"], lens=e_lens, image=f["image"], fourcc=cfg.fourcc) for f in cfg.frames]
+    engine.stage(frames)
+    engine.run()
+    full = engine.fetch()
+    n_classes = full[0]["cls"].shape[1]
+    assert n_classes == 3
+    seen = dict(detections=0, clusters=0, largest=0)
+    for cls, thr in [(1, 0.34), (0, 0.5), (2, 0.9999)]:
+        got = engine.detect(cls, thr, arg_max_only=arg_max_only, clusters=True)
+        assert len(got) == len(full)
+        for f, (g, r) in enumerate(zip(got, full)):
+            V = len(r["gidx"])
+            p = r["cls"][:V]
+            hit = p[:, cls] >= np.float32(thr)
+            if arg_max_only:
+                hit &= np.argmax(p, axis=1) == cls  # numpy's argmax takes the first maximum too
+            rows = np.nonzero(hit)[0]
+            what = "class %d threshold %g frame %d" % (cls, thr, f)
+            assert len(g["node"]) == len(rows), what
+            np.testing.assert_array_equal(g["node"], r["gidx"][rows], what)
+            np.testing.assert_array_equal(g["pixel"], r["px"][rows], what)
+            np.testing.assert_array_equal(g["probability"], p[rows, cls], what)
+            # connected components of the detections under the (directed) neighbourhood table, taken as undirected
+            det_of_row = -np.ones(V + 1, np.int64)
+            det_of_row[rows] = np.arange(len(rows))
+            nb = r["nb"][rows]                      # [n_det, nn] local rows, V = not visible
+            src = np.repeat(np.arange(len(rows)), nb.shape[1])
+            dst = det_of_row[nb.reshape(-1)]
+            keep = dst >= 0
+            graph = sp.coo_matrix((np.ones(keep.sum()), (src[keep], dst[keep])), shape=(len(rows), len(rows)))
+            n_comp, label = connected_components(graph, directed=False)
+            assert len(g["cluster_size"]) == n_comp, what
+            if len(rows) == 0:
+                continue
+            # renumber scipy's labels by first appearance
+            first = np.full(n_comp, len(rows))
+            np.minimum.at(first, label, np.arange(len(rows)))
+            order = np.argsort(first)
+            renumber = np.empty(n_comp, np.int64)
+            renumber[order] = np.arange(n_comp)
+            want_cluster = renumber[label]
+            seen["detections"] += len(rows)
+            seen["clusters"] += n_comp
+            seen["largest"] = max(seen["largest"], int(np.bincount(want_cluster).max()))
+            np.testing.assert_array_equal(g["cluster"], want_cluster, what)
+            np.testing.assert_array_equal(g["cluster_size"], np.bincount(want_cluster, minlength=n_comp), what)
+            px = r["px"][rows]
+            for c in range(n_comp):
+                m = px[want_cluster == c]
+                np.testing.assert_array_equal(g["cluster_box"][c], [m[:, 0].min(), m[:, 1].min(), m[:, 0].max(), m[:, 1].max()], what)
+                np.testing.assert_allclose(g["cluster_centre"][c], m.astype(np.float64).mean(axis=0), rtol=1e-5, err_msg=what)
+    # the cases are not trivial: many detections, many clusters, clusters of more than a handful of nodes
+    assert seen["detections"] > 1000 and seen["clusters"] > 100 and seen["largest"] > 8, seen
+    # without clustering only the detections come back
+    got = engine.detect(1, 0.34, arg_max_only=arg_max_only, clusters=False)
+    assert all(len(g["cluster_size"]) == 0 and len(g["cluster"]) == 0 for g in got)
+    # a class the network does not have
+    with pytest.raises(RuntimeError):
+        engine.detect(3, 0.5)

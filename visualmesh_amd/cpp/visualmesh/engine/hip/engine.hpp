@@ -32,6 +32,7 @@
 
 #include <algorithm>
 #include <cstdint>
+#include <array>
 #include <cstring>
 #include <map>
 #include <stdexcept>
@@ -256,6 +257,54 @@ namespace engine {
                     r.classifications = out[i].classifications.data();
                 }
                 throw_on_error(vmhip_batch_fetch(batch_, results.data()));
+                return out;
+            }
+            /// The nodes of one class among the results of the last run, picked and clustered on the device so that
+            /// only they are downloaded (the reference's consumers walk the whole ClassifiedMesh on the host,
+            /// example/draw.hpp:41-59).
+            struct Detections {
+                std::vector<int32_t> node;                    ///< index into the mesh, in the order of the visible nodes
+                std::vector<std::array<Scalar, 2>> pixel;
+                std::vector<Scalar> probability;
+                std::vector<int32_t> cluster;                 ///< connected component (over the neighbourhood graph) of each
+                std::vector<int32_t> cluster_size;
+                std::vector<std::array<Scalar, 4>> cluster_box;     ///< min x, min y, max x, max y
+                std::vector<std::array<Scalar, 2>> cluster_centre;  ///< mean pixel
+            };
+            /// A node is detected if its probability of `class_index` is at least `threshold` and, with `arg_max_only`,
+            /// no other class has a larger one. One entry per staged frame.
+            std::vector<Detections> detect(int class_index, Scalar threshold, bool arg_max_only = false, bool clusters = true) const {
+                const size_t n = staged_.size();
+                std::vector<Detections> out(n);
+                if (n == 0) return out;
+                std::vector<vmhip_detections> raw(n);
+                for (auto& r : raw) std::memset(&r, 0, sizeof(r));
+                /* first call sizes (capacity 0 fits only empty frames), second call copies */
+                int rc = vmhip_batch_detect(batch_, class_index, float(threshold), arg_max_only, clusters, raw.data());
+                if (rc == VMHIP_ERR_CAPACITY) {
+                    for (size_t i = 0; i < n; ++i) {
+                        Detections& d = out[i];
+                        vmhip_detections& r = raw[i];
+                        d.node.resize(r.n_detections);
+                        d.pixel.resize(r.n_detections);
+                        d.probability.resize(r.n_detections);
+                        d.cluster.resize(clusters ? r.n_detections : 0);
+                        d.cluster_size.resize(r.n_clusters);
+                        d.cluster_box.resize(r.n_clusters);
+                        d.cluster_centre.resize(r.n_clusters);
+                        r.capacity = r.n_detections;
+                        r.cluster_capacity = r.n_clusters;
+                        r.node = d.node.data();
+                        r.pixel = reinterpret_cast<float*>(d.pixel.data());
+                        r.probability = d.probability.data();
+                        r.cluster = clusters ? d.cluster.data() : nullptr;
+                        r.cluster_size = d.cluster_size.data();
+                        r.cluster_box = reinterpret_cast<float*>(d.cluster_box.data());
+                        r.cluster_centre = reinterpret_cast<float*>(d.cluster_centre.data());
+                    }
+                    rc = vmhip_batch_detect(batch_, class_index, float(threshold), arg_max_only, clusters, raw.data());
+                }
+                throw_on_error(rc);
                 return out;
             }
             /// Visible nodes per staged frame after run().

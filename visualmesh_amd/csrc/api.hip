@@ -141,6 +141,10 @@ struct vmhip_batch {
     size_t h_pin_cap = 0;
     std::vector<uint64_t> h_force_valid, h_force_keep;
     bool have_run = false;
+    uint64_t run_serial = 0;    /* counts completed runs */
+    uint64_t detect_serial = 0; /* the run whose detections the workspace holds, with these parameters: */
+    int32_t detect_class = -1, detect_arg_max = 0, detect_clusters = 0;
+    float detect_threshold = 0.0f;
     uint32_t epoch = 0; /* host mirror of the device run stamp */
     /* the kernel sequence of a run, captured once per staged batch and replayed (no profiling, VMHIP_GRAPH != 0) */
     hipGraph_t graph = nullptr;
@@ -155,7 +159,9 @@ struct vmhip_batch {
 
     VmBatchDev dev{};
     DevBuf d_frames, d_ranges, d_images, d_cand_px, d_cand_keep, d_tile_count, d_force_valid, d_force_keep, d_frame_V,
-      d_amb_list, d_row_px, d_row_gidx, d_row_nb, d_row_nbl, d_tile_halo, d_tile_desc, d_act[2], d_lookup, d_epoch;
+      d_amb_list, d_row_px, d_row_gidx, d_row_nb, d_row_nbl, d_tile_halo, d_tile_desc, d_act[2], d_lookup, d_epoch, d_detect, d_detect_packed;
+    void* h_detect = nullptr; /* pinned landing area of vmhip_batch_detect */
+    size_t h_detect_cap = 0;
     float* final_act = nullptr;
 
     /* profiling */
@@ -170,11 +176,13 @@ struct vmhip_batch {
         DevBuf* all[] = {&d_frames, &d_ranges, &d_images, &d_cand_px, &d_cand_keep, &d_tile_count, &d_force_valid,
                          &d_force_keep, &d_frame_V, &d_amb_list, &d_row_px, &d_row_gidx, &d_row_nb,
                          &d_row_nbl, &d_tile_halo, &d_tile_desc, &d_epoch,
-                         &d_act[0], &d_act[1], &d_lookup};
+                         &d_act[0], &d_act[1], &d_lookup, &d_detect, &d_detect_packed};
         drop_graph();
         for (DevBuf* b : all) b->release();
         if (h_pin) (void) hipHostFree(h_pin);
         h_pin = nullptr, h_pin_cap = 0;
+        if (h_detect) (void) hipHostFree(h_detect);
+        h_detect = nullptr, h_detect_cap = 0;
         for (hipEvent_t e : events) (void) hipEventDestroy(e);
         events.clear();
     }
@@ -535,6 +543,7 @@ int batch_run(vmhip_batch* b) {
         if (rc < 0) return rc;
         if (rc == 0) {
             b->have_run = true;
+            ++b->run_serial;
             return VMHIP_OK;
         }
     }
@@ -793,6 +802,92 @@ int vmhip_batch_fetch(vmhip_batch* b, vmhip_result* results) {
     if (!b) return fail(VMHIP_ERR_ARGUMENT, "batch_fetch: null batch");
     return batch_fetch(b, results);
 }
+int vmhip_batch_detect(vmhip_batch* b, int32_t class_index, float threshold, int32_t arg_max_only, int32_t clusters,
+                       vmhip_detections* out) {
+    if (!b || !out) return fail(VMHIP_ERR_ARGUMENT, "batch_detect: null argument");
+    if (!b->have_run || !b->classify || !b->final_act) return fail(VMHIP_ERR_ARGUMENT, "batch_detect: no completed classifying run");
+    vmhip_engine* E = b->engine;
+    const int C = E->n_classes;
+    if (class_index < 0 || class_index >= C) return fail(VMHIP_ERR_ARGUMENT, "batch_detect: no such class");
+    const int n = int(b->frames.size());
+    hipStream_t s = E->stream;
+    HIP_TRY(b->d_detect.reserve(vm_detect_workspace_bytes(b->row_total, n)));
+    VmDetectDev D{};
+    vm_detect_carve(b->d_detect.p, b->row_total, n, &D);
+    D.probabilities = b->final_act;
+    D.n_classes = C, D.class_index = class_index, D.arg_max_only = arg_max_only != 0, D.threshold = threshold;
+    /* a caller that was told its arrays are too small asks again with the same arguments: nothing to recompute */
+    const bool held = !b->d_detect.grew && b->detect_serial == b->run_serial && b->detect_class == class_index
+                      && std::memcmp(&b->detect_threshold, &threshold, sizeof(float)) == 0 && b->detect_arg_max == (arg_max_only != 0)
+                      && b->detect_clusters == (clusters != 0);
+    if (!held) {
+        vm_launch_detect(b->dev, D, clusters != 0, s);
+        HIP_TRY(hipGetLastError());
+        b->detect_serial = b->run_serial, b->detect_class = class_index, b->detect_threshold = threshold;
+        b->detect_arg_max = arg_max_only != 0, b->detect_clusters = clusters != 0;
+    }
+    /* counts first (pinned, one wait), then one dense block with everything, then it is a matter of host copies */
+    auto pinned = [&](size_t bytes) -> hipError_t {
+        if (bytes <= b->h_detect_cap) return hipSuccess;
+        if (b->h_detect) (void) hipHostFree(b->h_detect);
+        b->h_detect = nullptr, b->h_detect_cap = 0;
+        hipError_t e = hipHostMalloc(&b->h_detect, bytes + bytes / 4 + 4096, hipHostMallocDefault);
+        if (e == hipSuccess) b->h_detect_cap = bytes + bytes / 4 + 4096;
+        return e;
+    };
+    HIP_TRY(pinned(size_t(n) * 8));
+    int32_t* counts = static_cast<int32_t*>(b->h_detect);
+    HIP_TRY(hipMemcpyAsync(counts, D.counts, size_t(n) * 8, hipMemcpyDeviceToHost, s));
+    HIP_TRY(hipStreamSynchronize(s));
+    bool fits = true;
+    size_t total_d = 0, total_c = 0;
+    std::vector<int32_t> nd(n), nc(n);
+    for (int f = 0; f < n; ++f) {
+        nd[f] = counts[2 * f], nc[f] = clusters ? counts[2 * f + 1] : 0;
+        out[f].n_detections = nd[f];
+        out[f].n_clusters = nc[f];
+        total_d += size_t(nd[f]), total_c += size_t(nc[f]);
+        fits = fits && out[f].capacity >= nd[f] && (!clusters || out[f].cluster_capacity >= nc[f]);
+    }
+    if (!fits) return fail(VMHIP_ERR_CAPACITY, "batch_detect: a frame has more detections or clusters than its arrays hold");
+    if (total_d == 0) return VMHIP_OK;
+    if (total_d > 0x7fffffffull) return fail(VMHIP_ERR_CAPACITY, "batch_detect: too many detections for one download");
+    const size_t words = 5 * total_d + 7 * total_c;
+    HIP_TRY(b->d_detect_packed.reserve(words * 4));
+    HIP_TRY(pinned(words * 4));
+    vm_launch_detect_pack(b->dev, D, static_cast<uint32_t*>(b->d_detect_packed.p), int(total_d), int(total_c), s);
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipMemcpyAsync(b->h_detect, b->d_detect_packed.p, words * 4, hipMemcpyDeviceToHost, s));
+    HIP_TRY(hipStreamSynchronize(s));
+    const uint32_t* node = static_cast<const uint32_t*>(b->h_detect);
+    const uint32_t* pixel = node + total_d;
+    const uint32_t* probability = pixel + 2 * total_d;
+    const uint32_t* cluster = probability + total_d;
+    const uint32_t* size = cluster + total_d;
+    const uint32_t* box = size + total_c;
+    const uint32_t* sum = box + 4 * total_c;
+    size_t d0 = 0, c0 = 0;
+    for (int f = 0; f < n; ++f) {
+        vmhip_detections& R = out[f];
+        const size_t d = size_t(nd[f]), c = size_t(nc[f]);
+        if (R.node) std::memcpy(R.node, node + d0, 4 * d);
+        if (R.pixel) std::memcpy(R.pixel, pixel + 2 * d0, 8 * d);
+        if (R.probability) std::memcpy(R.probability, probability + d0, 4 * d);
+        if (R.cluster && clusters) std::memcpy(R.cluster, cluster + d0, 4 * d);
+        if (R.cluster_size) std::memcpy(R.cluster_size, size + c0, 4 * c);
+        if (R.cluster_box) std::memcpy(R.cluster_box, box + 4 * c0, 16 * c);
+        if (R.cluster_centre) {
+            const float* sums = reinterpret_cast<const float*>(sum + 2 * c0);
+            for (size_t k = 0; k < c; ++k) {
+                R.cluster_centre[2 * k] = sums[2 * k] / float(int32_t(size[c0 + k]));
+                R.cluster_centre[2 * k + 1] = sums[2 * k + 1] / float(int32_t(size[c0 + k]));
+            }
+        }
+        d0 += d, c0 += c;
+    }
+    return VMHIP_OK;
+}
+
 int vmhip_batch_profile(vmhip_batch* b, int32_t enable) {
     if (!b) return fail(VMHIP_ERR_ARGUMENT, "batch_profile: null batch");
     if (enable < 0 || enable > 2) return fail(VMHIP_ERR_ARGUMENT, "batch_profile: mode must be 0, 1 or 2");

@@ -116,6 +116,31 @@ struct VmLayerDev {
     const float* w_flow; /* the fp32 w_mfma weights in the order conv_flow.hip keeps them in LDS, or null */
 };
 
+/* Device side of the detection step (detect.hip): every array is indexed like the row space, a frame's entries
+ * starting at its row_base, so the worst case (every node detected, every detection its own cluster) fits. */
+struct VmDetectDev {
+    const float* probabilities; /* the last run's final activations, [rows][n_classes] */
+    int32_t n_classes, class_index, arg_max_only;
+    float threshold;
+    int32_t* node;             /* mesh index of each detection */
+    float2* pixel;
+    float* probability;
+    int32_t* cluster;          /* cluster number of each detection */
+    int32_t* row_to_detection; /* per row: its detection number or -1 */
+    int32_t* parent;           /* union-find over a frame's detections */
+    int32_t* cluster_size;
+    int32_t* cluster_box;      /* [4] min x, min y, max x, max y as float bits */
+    float* cluster_sum;        /* [2] sum of pixels */
+    int32_t* counts;           /* [n_frames][2] detections, clusters */
+};
+#define VM_DETECT_BYTES_PER_ROW 64 /* 56 used, the rest covers the 16-byte alignment of each array */
+size_t vm_detect_workspace_bytes(size_t rows, int n_frames);
+/* points D's arrays into a workspace of that size (counts last, n_frames * 8 bytes) */
+void vm_detect_carve(void* workspace, size_t rows, int n_frames, VmDetectDev* D);
+void vm_launch_detect(const VmBatchDev& B, const VmDetectDev& D, int clusters, hipStream_t stream);
+/* packed: 5 * total_d + 7 * total_c words (detect.hip says in which order) */
+void vm_launch_detect_pack(const VmBatchDev& B, const VmDetectDev& D, uint32_t* packed, int total_d, int total_c, hipStream_t stream);
+
 /* launchers, one per kernel; all asynchronous on `stream` */
 void vm_launch_libm(int which, const float* x, float* y, int n, hipStream_t stream);
 void vm_launch_copy_probe(const void* src, void* dst, size_t bytes, hipStream_t stream);

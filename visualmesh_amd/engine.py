@@ -204,6 +204,37 @@ class Engine:
     def native_batch(self):
         return C.c_void_p(self._lib.vmh_engine_native_batch(self.ptr))
 
+    def detect(self, class_index, threshold, arg_max_only=False, clusters=True):
+        """The nodes of one class among the results of the last run, picked (probability >= threshold, optionally only
+        where the class is the arg max) and grouped into connected components of the neighbourhood graph on the
+        device; only they are downloaded. One dict per staged frame: node, pixel, probability, cluster,
+        cluster_size, cluster_box, cluster_centre."""
+        lib = native.hip()
+        n = len(self._staged)
+        raw = (native.Detections * n)()
+        rc = lib.vmhip_batch_detect(self.native_batch(), class_index, threshold, int(arg_max_only), int(clusters), raw)
+        out = []
+        if rc == native.ERR_CAPACITY:  # the first call only counted
+            for r in raw:
+                d = dict(node=np.empty(r.n_detections, np.int32), pixel=np.empty((r.n_detections, 2), np.float32),
+                         probability=np.empty(r.n_detections, np.float32),
+                         cluster=np.empty(r.n_detections if clusters else 0, np.int32),
+                         cluster_size=np.empty(r.n_clusters, np.int32), cluster_box=np.empty((r.n_clusters, 4), np.float32),
+                         cluster_centre=np.empty((r.n_clusters, 2), np.float32))
+                r.capacity, r.cluster_capacity = r.n_detections, r.n_clusters
+                r.node, r.pixel, r.probability = native._ip(d["node"]), native._fp(d["pixel"]), native._fp(d["probability"])
+                r.cluster = native._ip(d["cluster"]) if clusters else None
+                r.cluster_size, r.cluster_box = native._ip(d["cluster_size"]), native._fp(d["cluster_box"])
+                r.cluster_centre = native._fp(d["cluster_centre"])
+                out.append(d)
+            rc = lib.vmhip_batch_detect(self.native_batch(), class_index, threshold, int(arg_max_only), int(clusters), raw)
+        else:
+            out = [dict(node=np.empty(0, np.int32), pixel=np.empty((0, 2), np.float32), probability=np.empty(0, np.float32),
+                        cluster=np.empty(0, np.int32), cluster_size=np.empty(0, np.int32),
+                        cluster_box=np.empty((0, 4), np.float32), cluster_centre=np.empty((0, 2), np.float32)) for _ in range(n)]
+        native.hip_check(rc)
+        return out
+
     def profile(self, enable=True):
         """0/False off, 1/True every kernel, 2 only the kernel that took longest in the last fully profiled run"""
         if not self.native_batch():

@@ -23,7 +23,7 @@ FP32, BF16 = 0, 1
 HIP_SYMBOLS = [
     "vmhip_last_error", "vmhip_engine_create", "vmhip_engine_destroy", "vmhip_engine_n_classes", "vmhip_mesh_upload",
     "vmhip_mesh_release", "vmhip_project", "vmhip_classify", "vmhip_classify_batch", "vmhip_batch_create",
-    "vmhip_batch_destroy", "vmhip_batch_stage", "vmhip_batch_run", "vmhip_batch_counts", "vmhip_batch_fetch",
+    "vmhip_batch_destroy", "vmhip_batch_stage", "vmhip_batch_run", "vmhip_batch_counts", "vmhip_batch_fetch", "vmhip_batch_detect",
     "vmhip_batch_profile", "vmhip_batch_profile_read", "vmhip_selftest_libm", "vmhip_selftest_copy",
 ]
 
@@ -55,6 +55,13 @@ class NetworkC(C.Structure):
 class Frame(C.Structure):
     _fields_ = [("mesh", C.c_void_p), ("Rco", C.c_float * 9), ("lens", Lens), ("ranges", C.POINTER(C.c_int32)),
                 ("n_ranges", C.c_int32), ("image", C.c_void_p), ("fourcc", C.c_uint32)]
+
+
+class Detections(C.Structure):
+    _fields_ = [("capacity", C.c_int32), ("cluster_capacity", C.c_int32), ("n_detections", C.c_int32), ("n_clusters", C.c_int32),
+                ("node", C.POINTER(C.c_int32)), ("pixel", C.POINTER(C.c_float)), ("probability", C.POINTER(C.c_float)),
+                ("cluster", C.POINTER(C.c_int32)), ("cluster_size", C.POINTER(C.c_int32)), ("cluster_box", C.POINTER(C.c_float)),
+                ("cluster_centre", C.POINTER(C.c_float))]
 
 
 class Result(C.Structure):
@@ -121,6 +128,7 @@ def hip():
     L.vmhip_batch_run.argtypes = [vp]
     L.vmhip_batch_counts.argtypes = [vp, C.POINTER(C.c_int32)]
     L.vmhip_batch_fetch.argtypes = [vp, C.POINTER(Result)]
+    L.vmhip_batch_detect.argtypes = [vp, C.c_int32, C.c_float, C.c_int32, C.c_int32, C.POINTER(Detections)]
     L.vmhip_batch_profile.argtypes = [vp, C.c_int32]
     L.vmhip_batch_profile_read.argtypes = [vp, C.c_int32, C.POINTER(C.c_int32), C.POINTER(C.c_char_p), C.POINTER(C.c_float),
                                            C.POINTER(C.c_int64)]
