@@ -37,3 +37,6 @@ def test_struct_layouts_match_the_header():
     assert ctypes.sizeof(native.Layer) == 32
     assert ctypes.sizeof(native.Result) == 40
     assert native.Frame.Rco.offset == 8 and native.Frame.lens.offset == 44 and native.Frame.ranges.offset == 80
+    # vmhip_detections: four int32, then seven pointers
+    assert ctypes.sizeof(native.Detections) == 72
+    assert native.Detections.node.offset == 16 and native.Detections.cluster_centre.offset == 64
