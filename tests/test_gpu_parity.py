@@ -438,3 +438,29 @@ def test_detections_and_clusters_on_the_device(oracle, arg_max_only):
     # a class the network does not have
     with pytest.raises(RuntimeError):
         engine.detect(3, 0.5)
+
+
+def test_a_wait_that_runs_out_fails_the_run(oracle):
+    """The barrier-free convolution kernel bounds every wait by a poll count. With the count set to one poll (from the
+    host; the kernels still end normally: a wave whose wait runs out tells its block and leaves its tile loop, and so
+    does every wave that sees the flag) the run must be reported as failed, and with the count restored the same staged
+    batch must run and give the oracle's results."""
+    cfg = wl.config(2, n_frames=1)
+    o_lens, e_lens = lens_pair(cfg)
+    o_mesh, e_mesh = meshes_for(cfg, oracle)
+    engine = eng.Engine(cfg.network, cfg.model)
+    f = cfg.frames[0]
+    frames = [dict(mesh=e_mesh, Hoc=f["Hoc"], lens=e_lens, image=f["image"], fourcc=cfg.fourcc)]
+    engine.stage(frames)
+    lib = native.hip()
+    lib.vm_flow_set_poll_limit(1)
+    try:
+        with pytest.raises(RuntimeError, match="gave up waiting"):
+            engine.run()
+    finally:
+        lib.vm_flow_set_poll_limit(1 << 18)
+    assert lib.vm_flow_timeouts_read() == 0  # the failed run reset the count
+    engine.run()
+    got = engine.fetch()[0]
+    want = pick(o_mesh, f["Hoc"]).classify(f["Hoc"], o_lens, f["image"], cfg.fourcc, vmo.Network(cfg.network))
+    assert_classification_parity(got, want, PROB_TOL, "after a failed run")

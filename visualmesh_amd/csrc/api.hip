@@ -111,6 +111,7 @@ struct HostLayer {
 struct vmhip_engine {
     bool use_graph = true;               /* VMHIP_GRAPH=0: launch every run kernel by kernel */
     bool use_lds = false;                /* some layer gathers through the tile-local tables */
+    bool use_flow = false;               /* some layer runs the kernel that polls LDS counters instead of barriers */
     int32_t halo_cap = VMHIP_HALO_MAX;   /* VMHIP_HALO_CAP lowers it to exercise the not-staged path */
     int32_t nn = 0;
     int32_t precision = VMHIP_FP32;
@@ -277,7 +278,7 @@ int batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int
     HIP_TRY(b->d_force_keep.reserve(8 * std::max<size_t>(words, 1)));
     HIP_TRY(b->d_frame_V.reserve(8 * size_t(n_frames))); /* visible counts, then ambiguity counts */
     {
-        const size_t need = 8 * size_t(n_frames) + sizeof(int2) * size_t(n_frames) * vmhip_batch::AMB_HEAD;
+        const size_t need = 8 * size_t(n_frames) + sizeof(int2) * size_t(n_frames) * vmhip_batch::AMB_HEAD + 16;
         if (need > b->h_pin_cap) {
             if (b->h_pin) HIP_TRY(hipHostFree(b->h_pin));
             b->h_pin = nullptr, b->h_pin_cap = 0;
@@ -459,7 +460,17 @@ int batch_verify(vmhip_batch* b) {
     HIP_TRY(hipMemcpyAsync(pin_counts, b->d_frame_V.p, 8 * size_t(n), hipMemcpyDeviceToHost, E->stream));
     HIP_TRY(hipMemcpy2DAsync(pin_amb, sizeof(int2) * HEAD, b->d_amb_list.p, sizeof(int2) * VMHIP_AMB_CAP, sizeof(int2) * HEAD, n,
                              hipMemcpyDeviceToHost, E->stream));
+    /* the barrier-free convolution kernel bounds its waits; a wait that ran out (never in a correct run) means
+     * the results of this run cannot be trusted */
+    uint32_t* pin_timeouts = reinterpret_cast<uint32_t*>(pin_amb + size_t(n) * HEAD);
+    unsigned int* d_timeouts = (E->use_flow && b->classify) ? vm_flow_timeouts_address() : nullptr;
+    *pin_timeouts = 0;
+    if (d_timeouts) HIP_TRY(hipMemcpyAsync(pin_timeouts, d_timeouts, 4, hipMemcpyDeviceToHost, E->stream));
     HIP_TRY(hipStreamSynchronize(E->stream));
+    if (*pin_timeouts != 0) {
+        (void) hipMemset(d_timeouts, 0, 4);
+        return fail(VMHIP_ERR_HIP, "run: a convolution wave gave up waiting for its tile; the results of this run were discarded");
+    }
     std::copy(pin_counts, pin_counts + n, b->h_V.begin());
     std::copy(pin_counts + n, pin_counts + 2 * n, b->h_amb_count.begin());
     int changed = 0;
@@ -704,6 +715,7 @@ int vmhip_engine_create(const vmhip_network* net, int32_t n_neighbours, int32_t 
             H.use_narrow = allow_lds && !force_lds && !force_dma && plain && H.slots - 1 <= VMHIP_NBL_STRIDE
                            && vm_narrow_supported(H.c_in, H.c_out, H.slots);
             E->use_lds = E->use_lds || H.use_lds || H.use_dma || H.use_flow || H.use_narrow;
+            E->use_flow = E->use_flow || H.use_flow;
             if (H.use_mfma || H.use_lds || H.use_dma || H.use_flow) {
                 std::vector<unsigned char> wp(vm_mfma_weight_bytes(H.c_in, H.c_out, H.slots, H.arith_bf16));
                 vm_mfma_permute_weights(H.h_w.data(), H.c_in, H.c_out, H.slots, H.arith_bf16, wp.data());

@@ -20,8 +20,9 @@
  * issues those loads into buffer k & 1 once consumed[k & 1] says every wave is done with tile k, and reports its
  * loads of tile k+1 (issued a tile earlier) just before.
  * Everything a wave waits for at step k depends only on what all waves do at step k-1, so the waits cannot form a
- * cycle; each is nevertheless bounded by a poll count, after which the wave goes on (and counts the event in
- * vm_flow_timeouts) rather than hang.
+ * cycle; each is nevertheless bounded by a poll count, after which the wave tells its block, counts the event in
+ * vm_flow_timeouts and leaves the tile loop, as does every wave that then sees the block's flag: no wave hangs and
+ * none works on a tile that is not there. The host reads the count with every run and fails the run if it is not 0.
  * Loads are counted, not drained: a loader knows how many vector memory instructions it has issued after the ones
  * it needs (they complete in order) and waits with s_waitcnt vmcnt(that many), so the loads of the next tile, in
  * flight behind them, are not waited for. For that count to be a constant every load and store of the loop is
@@ -35,9 +36,21 @@
 
 #include "vmhip_internal.h"
 
-/* waits that ran out of polls (none in a correct run): the kernel then goes on with whatever its LDS holds, so that
- * every wave still ends */
+/* waits that ran out of polls (none in a correct run) */
 __device__ unsigned int vm_flow_timeouts;
+/* polls a wait may take; only a test of the give-up path sets it (to something tiny) */
+__device__ int vm_flow_poll_limit = 1 << 18;
+extern "C" void vm_flow_set_poll_limit(int polls) {
+    (void) hipMemcpyToSymbol(HIP_SYMBOL(vm_flow_poll_limit), &polls, sizeof(polls));
+}
+unsigned int* vm_flow_timeouts_address() {
+    static unsigned int* at = nullptr;
+    if (!at && hipGetSymbolAddress(reinterpret_cast<void**>(&at), HIP_SYMBOL(vm_flow_timeouts)) != hipSuccess) {
+        (void) hipGetLastError();
+        at = nullptr;
+    }
+    return at;
+}
 extern "C" unsigned int vm_flow_timeouts_read() {
     unsigned int v = 0;
     (void) hipMemcpyFromSymbol(&v, HIP_SYMBOL(vm_flow_timeouts), sizeof(v));
@@ -120,7 +133,6 @@ constexpr int FLOW_LOADERS = 4; /* measured: 8 loaders 2 % slower, every wave lo
 #define FLOW_PRIO_REST 3
 #define FLOW_SLEEP 1
 constexpr int FLOW_HALO = 192; /* halo rows staged per tile: two tiles, their neighbour tables and the loaders' slots fit beside the weights */
-constexpr int FLOW_POLLS = 1 << 18;
 /* rounds of NT loads that fill a buffer's rows, and how many of them reach into the halo rows */
 __host__ __device__ constexpr int flow_rounds(int c_in) { return ((VMHIP_TILE + FLOW_HALO) * (row_stride(c_in) / 4) + FLOW_WAVES * 64 - 1) / (FLOW_WAVES * 64); }
 __host__ __device__ constexpr int flow_halo_rounds(int c_in) { return flow_rounds(c_in) - VMHIP_TILE * (row_stride(c_in) / 4) / (FLOW_WAVES * 64); }
@@ -128,16 +140,20 @@ __host__ __device__ constexpr int flow_halo_rounds(int c_in) { return flow_round
 __host__ __device__ constexpr int flow_slot_words(int c_in) { return 4 + (FLOW_WAVES / FLOW_LOADERS) * flow_halo_rounds(c_in) * 64; }
 __host__ __device__ constexpr size_t flow_lds_bytes(int c_in, int c_out, int slots) {
     return (size_t(slots) * (c_in / 4) * ((c_out + 15) / 16) * 64 + size_t((c_out + 15) / 16) * 16
-            + 2 * (size_t(VMHIP_TILE + FLOW_HALO) * row_stride(c_in) + VMHIP_TILE * 4 + 4) + 4 + size_t(FLOW_LOADERS) * flow_slot_words(c_in)) * 4;
+            + 2 * (size_t(VMHIP_TILE + FLOW_HALO) * row_stride(c_in) + VMHIP_TILE * 4 + 4) + 8 + size_t(FLOW_LOADERS) * flow_slot_words(c_in)) * 4;
 }
 
-/* polls an LDS counter until it has reached target (wrap-safe); false when the polls ran out. The read is spelled
- * out: a volatile access would make the compiler wait for every vector memory instruction in flight as well. */
-__device__ __forceinline__ bool wait_counter(const uint32_t* counter, uint32_t target) {
+/* Polls an LDS counter until it has reached target (wrap-safe). False when the polls ran out or another wave of the
+ * block has given up (the word after the four counters says so): the caller then leaves the tile loop without
+ * touching the tile, whose descriptor and rows may not be there. The read is spelled out: a volatile access would
+ * make the compiler wait for every vector memory instruction in flight as well. */
+__device__ __forceinline__ bool wait_counter(const uint32_t* counter, const uint32_t* gave_up, uint32_t target, int polls) {
     const uint32_t at = (uint32_t) (uintptr_t) (const __attribute__((address_space(3))) uint32_t*) counter;
-    for (int spin = 0; spin < FLOW_POLLS; ++spin) {
-        uint32_t v;
-        asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(at) : "memory");
+    const uint32_t flag_at = (uint32_t) (uintptr_t) (const __attribute__((address_space(3))) uint32_t*) gave_up;
+    for (int spin = 0; spin < polls; ++spin) {
+        uint32_t v, flag;
+        asm volatile("ds_read_b32 %0, %2\n\tds_read_b32 %1, %3\n\ts_waitcnt lgkmcnt(0)" : "=&v"(v), "=&v"(flag) : "v"(at), "v"(flag_at) : "memory");
+        if (__builtin_amdgcn_readfirstlane(flag) != 0) return false;
         if ((int32_t) (__builtin_amdgcn_readfirstlane(v) - target) >= 0) return true;
         __builtin_amdgcn_s_sleep(FLOW_SLEEP);
     }
@@ -213,7 +229,7 @@ __global__ __launch_bounds__(FLOW_WAVES * 64) void vm_conv_flow_kernel(VmBatchDe
     float* const b_lds = w_lds + W_FLOATS;
     float* const buf0 = b_lds + CB * 16;
     uint32_t* const counters = reinterpret_cast<uint32_t*>(buf0 + 2 * BUF_FLOATS); /* staged[2], consumed[2] */
-    if (threadIdx.x < 4) counters[threadIdx.x] = 0;
+    if (threadIdx.x < 8) counters[threadIdx.x] = 0; /* staged[2], consumed[2], then the word that says a wave gave up */
     /* the weights lie in global memory in the order they have in LDS: whole waves of 16 bytes per lane, issued before
      * anything else so that they travel together with the first descriptors */
     static_assert(W_FLOATS % 256 == 0, "the weights are whole wave loads");
@@ -231,7 +247,7 @@ __global__ __launch_bounds__(FLOW_WAVES * 64) void vm_conv_flow_kernel(VmBatchDe
     const int q = lane >> 4, r16 = lane & 15;
     const int activation = L.activation;
     const int lw = wave; /* which loader this wave is, if it is one */
-    uint32_t* const slot = counters + 4 + SLOT_WORDS * (wave % LOADERS); /* a loader's notes on the tile it stages next */
+    uint32_t* const slot = counters + 8 + SLOT_WORDS * (wave % LOADERS); /* a loader's notes on the tile it stages next */
 
     const int n_tiles = B.n_row_tiles;
     const int xcd = blockIdx.x & 7, lb = blockIdx.x >> 3, gx = gridDim.x >> 3;
@@ -331,8 +347,14 @@ __global__ __launch_bounds__(FLOW_WAVES * 64) void vm_conv_flow_kernel(VmBatchDe
                          __builtin_amdgcn_readfirstlane((int) d.z), __builtin_amdgcn_readfirstlane((int) d.w));
     };
     auto tile_of = [&](int k) { return min(tile0 + k * gx, t_last); };
+    const int polls = vm_flow_poll_limit;
+    uint32_t* const gave_up = counters + 4;
+    /* a wait ran out: tell the block, count it for the host, and (the caller) leave the loop */
     auto give_up = [&] {
-        if (lane == 0) atomicAdd(&vm_flow_timeouts, 1u);
+        if (lane == 0) {
+            atomicOr(gave_up, 1u);
+            atomicAdd(&vm_flow_timeouts, 1u);
+        }
     };
 
     /* ---- prologue: tiles 0 and 1 on their way into the two buffers, tile 2 described ---- */
@@ -378,7 +400,10 @@ __global__ __launch_bounds__(FLOW_WAVES * 64) void vm_conv_flow_kernel(VmBatchDe
         const uint32_t round = (uint32_t) ((k >> 1) + 1); /* the round of buffer b that tile k is */
         const float* rows = buf0 + b * BUF_FLOATS;
 
-        if (!wait_counter(&counters[b], LOADERS * round)) give_up(); /* every loader's share of tile k has landed */
+        if (!wait_counter(&counters[b], gave_up, LOADERS * round, polls)) { /* every loader's share of tile k has landed */
+            give_up();
+            break;
+        }
         FLOW_T(0);
         const int4 d_cur = read_desc(rows + DESC_AT);
         /* The SIMDs serve their oldest wave first, so left alone the youngest falls a whole tile behind, and the
@@ -583,7 +608,10 @@ __global__ __launch_bounds__(FLOW_WAVES * 64) void vm_conv_flow_kernel(VmBatchDe
             if (lane == 0) atomicAdd(&counters[b ^ 1], 1u);
             FLOW_T(2);
             /* tile k+2 goes where tile k was, once every wave has read the last of tile k */
-            if (!wait_counter(&counters[2 + b], NW * round)) give_up();
+            if (!wait_counter(&counters[2 + b], gave_up, NW * round, polls)) {
+                give_up();
+                break;
+            }
             FLOW_T(4);
             fill(tile_of(k + 2), first_new, k + 2 < count, offs, buf0 + b * BUF_FLOATS);
             FLOW_T(5);

@@ -196,6 +196,8 @@ int vm_launch_conv_dma(const VmBatchDev& B, const VmLayerDev& L, const float* in
 /* the same with LDS counters in place of the tile loop's barriers, so that the waves of a block run freely between
  * "my tile is staged" and "my buffer may be refilled" (conv_flow.hip) */
 bool vm_flow_supported(int c_in, int c_out, int slots);
+/* device address of that kernel's count of waits that ran out of polls (0 in every correct run), or null */
+unsigned int* vm_flow_timeouts_address();
 /* host side: w_mfma (fp32, vm_mfma_permute_weights' order) rearranged into that kernel's LDS order; same size */
 void vm_flow_order_weights(const float* w_mfma, int c_in, int c_out, int slots, float* out);
 int vm_launch_conv_flow(const VmBatchDev& B, const VmLayerDev& L, const float* in, float* out, hipStream_t stream,
