@@ -23,6 +23,7 @@
 #ifndef VISUALMESH_HIP_H
 #define VISUALMESH_HIP_H
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -122,6 +123,13 @@ int32_t vmhip_engine_n_classes(const vmhip_engine* engine);
 int vmhip_mesh_upload(const float* rays, const int32_t* neighbours, int32_t n_nodes, int32_t n_neighbours,
                       vmhip_mesh** out);
 void vmhip_mesh_release(vmhip_mesh* mesh);
+
+/* Page-locked host memory for images (and result arrays): copies between it and the device run at the link's full
+ * rate and do not hold the caller up, copies from ordinary memory are staged through small buffers by the runtime.
+ * No counterpart in the reference, which leaves image memory to its caller (engine/opencl/engine.hpp:307-315 copies
+ * from whatever pointer it is given). NULL if the allocation fails. */
+void* vmhip_host_alloc(size_t bytes);
+void vmhip_host_free(void* memory);
 
 /* Replaces cpu::Engine::operator()(mesh, Hoc, lens) (reference engine/cpu/engine.hpp:84-147). */
 int vmhip_project(vmhip_engine* engine, const vmhip_frame* frame, vmhip_result* result);

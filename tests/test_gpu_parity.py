@@ -464,3 +464,18 @@ def test_a_wait_that_runs_out_fails_the_run(oracle):
     got = engine.fetch()[0]
     want = pick(o_mesh, f["Hoc"]).classify(f["Hoc"], o_lens, f["image"], cfg.fourcc, vmo.Network(cfg.network))
     assert_classification_parity(got, want, PROB_TOL, "after a failed run")
+
+
+def test_images_in_page_locked_memory(oracle):
+    """vmhip_host_alloc: an image that lies in page-locked memory is staged from there and gives the same results."""
+    cfg = wl.config(1)
+    o_lens, e_lens = lens_pair(cfg)
+    o_mesh, e_mesh = meshes_for(cfg, oracle)
+    engine = eng.Engine(cfg.network, cfg.model)
+    f = cfg.frames[0]
+    image = native.pinned_empty(f["image"].shape, f["image"].dtype)
+    image[...] = f["image"]
+    got = engine(e_mesh, f["Hoc"], e_lens, image, cfg.fourcc)
+    want = pick(o_mesh, f["Hoc"]).classify(f["Hoc"], o_lens, f["image"], cfg.fourcc, vmo.Network(cfg.network))
+    assert_classification_parity(got, want, PROB_TOL, "image in page-locked memory")
+    del image  # frees the allocation (the owner goes with the last view)

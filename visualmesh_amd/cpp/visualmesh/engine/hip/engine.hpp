@@ -33,6 +33,8 @@
 #include <algorithm>
 #include <cstdint>
 #include <array>
+#include <exception>
+#include <thread>
 #include <cstring>
 #include <map>
 #include <stdexcept>
@@ -146,6 +148,7 @@ namespace engine {
                                                                           const Lens<Scalar>& lens) const {
                 constexpr int N = Model<Scalar>::N_NEIGHBOURS;
                 FrameData fd;
+                find_ranges(mesh, Hoc, lens, fd);
                 describe(mesh, Hoc, lens, nullptr, 0, fd);
                 ProjectedMesh<Scalar, N> out;
                 if (fd.candidates == 0) return out;
@@ -212,7 +215,26 @@ namespace engine {
                 std::vector<vmhip_frame> flat(frames.size());
                 staging_ = true;  // meshes described from here on belong to the staged batch
                 try {
-                    for (size_t i = 0; i < frames.size(); ++i) {
+                    /* the lookups are independent of each other and of the device: a few threads share them (each takes
+                     * ~80 us for a 1.2e5-node mesh), then the frames are described one by one (the mesh cache is not
+                     * thread safe) */
+                    const size_t n = frames.size();
+                    const size_t workers = std::min<size_t>(std::min<size_t>(n, 8), std::max(1u, std::thread::hardware_concurrency()));
+                    std::vector<std::exception_ptr> failed(workers);
+                    auto look_up = [&](size_t w) {
+                        try {
+                            for (size_t i = w; i < n; i += workers) find_ranges(*frames[i].mesh, frames[i].Hoc, frames[i].lens, staged_[i]);
+                        } catch (...) {
+                            failed[w] = std::current_exception();
+                        }
+                    };
+                    std::vector<std::thread> pool;
+                    for (size_t w = 1; w < workers; ++w) pool.emplace_back(look_up, w);
+                    look_up(0);
+                    for (auto& t : pool) t.join();
+                    for (auto& e : failed)
+                        if (e) std::rethrow_exception(e);
+                    for (size_t i = 0; i < n; ++i) {
                         describe(*frames[i].mesh, frames[i].Hoc, frames[i].lens, frames[i].image, frames[i].format, staged_[i]);
                         flat[i] = staged_[i].frame;
                     }
@@ -421,10 +443,10 @@ namespace engine {
                 return dev;
             }
 
+            /// The host side of the path: the mesh's lookup, flattened for the C ABI. Touches nothing but `fd`.
             template <template <typename> class Model>
-            void describe(const Mesh<Scalar, Model>& mesh, const mat4<Scalar>& Hoc, const Lens<Scalar>& lens, const void* image,
-                          uint32_t format, FrameData& fd) const {
-                const auto ranges = mesh.lookup(Hoc, lens);  // host side of the path
+            static void find_ranges(const Mesh<Scalar, Model>& mesh, const mat4<Scalar>& Hoc, const Lens<Scalar>& lens, FrameData& fd) {
+                const auto ranges = mesh.lookup(Hoc, lens);
                 fd.ranges.resize(ranges.size() * 2);
                 fd.candidates = 0;
                 for (size_t i = 0; i < ranges.size(); ++i) {
@@ -432,6 +454,11 @@ namespace engine {
                     fd.ranges[2 * i + 1] = ranges[i].second;
                     fd.candidates += ranges[i].second - ranges[i].first;
                 }
+            }
+            /// Everything else about a frame whose ranges are known.
+            template <template <typename> class Model>
+            void describe(const Mesh<Scalar, Model>& mesh, const mat4<Scalar>& Hoc, const Lens<Scalar>& lens, const void* image,
+                          uint32_t format, FrameData& fd) const {
                 vmhip_frame& f = fd.frame;
                 std::memset(&f, 0, sizeof(f));
                 f.mesh = device_mesh(mesh);
@@ -447,7 +474,7 @@ namespace engine {
                 f.lens.k[1] = lens.k[1];
                 f.lens.fov = lens.fov;
                 f.ranges = fd.ranges.data();
-                f.n_ranges = int32_t(ranges.size());
+                f.n_ranges = int32_t(fd.ranges.size() / 2);
                 f.image = image;
                 f.fourcc = format;
             }

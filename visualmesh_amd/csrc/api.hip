@@ -814,6 +814,18 @@ int vmhip_batch_fetch(vmhip_batch* b, vmhip_result* results) {
     if (!b) return fail(VMHIP_ERR_ARGUMENT, "batch_fetch: null batch");
     return batch_fetch(b, results);
 }
+void* vmhip_host_alloc(size_t bytes) {
+    void* p = nullptr;
+    if (hipHostMalloc(&p, bytes ? bytes : 1, hipHostMallocDefault) != hipSuccess) {
+        (void) hipGetLastError();
+        return nullptr;
+    }
+    return p;
+}
+void vmhip_host_free(void* memory) {
+    if (memory) (void) hipHostFree(memory);
+}
+
 int vmhip_batch_detect(vmhip_batch* b, int32_t class_index, float threshold, int32_t arg_max_only, int32_t clusters,
                        vmhip_detections* out) {
     if (!b || !out) return fail(VMHIP_ERR_ARGUMENT, "batch_detect: null argument");

@@ -23,7 +23,7 @@ FP32, BF16 = 0, 1
 HIP_SYMBOLS = [
     "vmhip_last_error", "vmhip_engine_create", "vmhip_engine_destroy", "vmhip_engine_n_classes", "vmhip_mesh_upload",
     "vmhip_mesh_release", "vmhip_project", "vmhip_classify", "vmhip_classify_batch", "vmhip_batch_create",
-    "vmhip_batch_destroy", "vmhip_batch_stage", "vmhip_batch_run", "vmhip_batch_counts", "vmhip_batch_fetch", "vmhip_batch_detect",
+    "vmhip_batch_destroy", "vmhip_batch_stage", "vmhip_batch_run", "vmhip_batch_counts", "vmhip_batch_fetch", "vmhip_batch_detect", "vmhip_host_alloc", "vmhip_host_free",
     "vmhip_batch_profile", "vmhip_batch_profile_read", "vmhip_selftest_libm", "vmhip_selftest_copy",
 ]
 
@@ -129,6 +129,10 @@ def hip():
     L.vmhip_batch_counts.argtypes = [vp, C.POINTER(C.c_int32)]
     L.vmhip_batch_fetch.argtypes = [vp, C.POINTER(Result)]
     L.vmhip_batch_detect.argtypes = [vp, C.c_int32, C.c_float, C.c_int32, C.c_int32, C.POINTER(Detections)]
+    L.vmhip_host_alloc.restype = vp
+    L.vmhip_host_alloc.argtypes = [C.c_size_t]
+    L.vmhip_host_free.restype = None
+    L.vmhip_host_free.argtypes = [vp]
     L.vmhip_batch_profile.argtypes = [vp, C.c_int32]
     L.vmhip_batch_profile_read.argtypes = [vp, C.c_int32, C.POINTER(C.c_int32), C.POINTER(C.c_char_p), C.POINTER(C.c_float),
                                            C.POINTER(C.c_int64)]
@@ -234,3 +238,27 @@ def host_check(rc):
             raise ValueError(msg)
         raise VisualMeshError(rc, msg)
     return rc
+
+
+class _Pinned:
+    """owner of one page-locked allocation; freed when the last array viewing it goes away"""
+
+    def __init__(self, nbytes):
+        self.ptr = hip().vmhip_host_alloc(nbytes)
+        if not self.ptr:
+            raise MemoryError("vmhip_host_alloc(%d) failed" % nbytes)
+        self.buffer = (C.c_uint8 * max(nbytes, 1)).from_address(self.ptr)
+        self.buffer._owner = self  # numpy keeps the ctypes buffer alive; the buffer keeps this object alive
+
+    def __del__(self):
+        if getattr(self, "ptr", None):
+            hip().vmhip_host_free(self.ptr)
+            self.ptr = None
+
+
+def pinned_empty(shape, dtype=np.uint8):
+    """numpy array in page-locked host memory (vmhip_host_alloc): the place for camera images that go to the device"""
+    dtype = np.dtype(dtype)
+    n = int(np.prod(shape)) * dtype.itemsize
+    owner = _Pinned(n)
+    return np.frombuffer(owner.buffer, dtype=np.uint8, count=n).view(dtype).reshape(shape)
