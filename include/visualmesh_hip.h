@@ -148,6 +148,12 @@ int vmhip_batch_create(vmhip_engine* engine, vmhip_batch** out);
 void vmhip_batch_destroy(vmhip_batch* batch);
 int vmhip_batch_stage(vmhip_batch* batch, const vmhip_frame* frames, int32_t n_frames, int32_t classify);
 int vmhip_batch_run(vmhip_batch* batch);
+/* The two halves of vmhip_batch_run: run_async puts the pass on the engine's stream and returns, wait blocks until it
+ * is done (and settles the screen-edge decisions with the host, as run does). Between the two the caller is free,
+ * e.g. to stage the next frames into a batch of another engine, whose copies then overlap this pass. Counts, fetch
+ * and detect need the wait; the batch must not be staged or run again before it. */
+int vmhip_batch_run_async(vmhip_batch* batch);
+int vmhip_batch_wait(vmhip_batch* batch);
 /* n_visible[n_frames] of the last run */
 int vmhip_batch_counts(const vmhip_batch* batch, int32_t* n_visible);
 int vmhip_batch_fetch(vmhip_batch* batch, vmhip_result* results);

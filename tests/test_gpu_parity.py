@@ -479,3 +479,39 @@ def test_images_in_page_locked_memory(oracle):
     want = pick(o_mesh, f["Hoc"]).classify(f["Hoc"], o_lens, f["image"], cfg.fourcc, vmo.Network(cfg.network))
     assert_classification_parity(got, want, PROB_TOL, "image in page-locked memory")
     del image  # frees the allocation (the owner goes with the last view)
+
+
+def test_run_in_two_halves_and_two_engines_overlapping(oracle):
+    """vmhip_batch_run_async / vmhip_batch_wait: two engines take turns, each staging its frames while the other's pass is
+    in flight; results must equal the oracle's, and a batch in flight must refuse to be staged, run or read."""
+    cfg = wl.config(2, n_frames=4)
+    o_lens, e_lens = lens_pair(cfg)
+    o_mesh, e_mesh = meshes_for(cfg, oracle)
+    engines = [eng.Engine(cfg.network, cfg.model), eng.Engine(cfg.network, cfg.model)]
+    halves = [cfg.frames[:2], cfg.frames[2:]]
+    staged = [[dict(mesh=e_mesh, Hoc=f["Hoc"], lens=e_lens, image=f["image"], fourcc=cfg.fourcc) for f in h] for h in halves]
+    engines[0].stage(staged[0])
+    engines[0].run_async()
+    with pytest.raises(RuntimeError, match="in flight"):
+        engines[0].run_async()
+    with pytest.raises(RuntimeError, match="in flight"):
+        engines[0].stage(staged[0])
+    with pytest.raises(RuntimeError):
+        engines[0].fetch()            # no completed run yet
+    engines[1].stage(staged[1])       # overlaps the pass of engine 0
+    engines[1].run_async()
+    engines[0].wait()
+    got0 = engines[0].fetch()
+    engines[0].stage(staged[0])       # and again the other way round
+    engines[0].run_async()
+    engines[1].wait()
+    got1 = engines[1].fetch()
+    engines[0].wait()
+    again0 = engines[0].fetch()
+    with pytest.raises(RuntimeError, match="no run in flight"):
+        engines[0].wait()
+    net = vmo.Network(cfg.network)
+    for got, frames in ((got0, halves[0]), (got1, halves[1]), (again0, halves[0])):
+        for g, f in zip(got, frames):
+            want = pick(o_mesh, f["Hoc"]).classify(f["Hoc"], o_lens, f["image"], cfg.fourcc, net)
+            assert_classification_parity(g, want, PROB_TOL, "two engines taking turns")

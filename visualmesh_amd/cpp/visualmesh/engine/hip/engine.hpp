@@ -252,6 +252,15 @@ namespace engine {
             void run() const {
                 if (batch_ && !staged_.empty()) throw_on_error(vmhip_batch_run(batch_));
             }
+            /// The same in two halves: the pass runs while the caller does something else (staging the next frames on
+            /// a second engine, for one), and wait() blocks until it is done. fetch(), detect() and visible_counts()
+            /// need the wait.
+            void run_async() const {
+                if (batch_ && !staged_.empty()) throw_on_error(vmhip_batch_run_async(batch_));
+            }
+            void wait() const {
+                if (batch_ && !staged_.empty()) throw_on_error(vmhip_batch_wait(batch_));
+            }
             /// Download the results of the last run.
             template <template <typename> class Model>
             std::vector<ClassifiedMesh<Scalar, Model<Scalar>::N_NEIGHBOURS>> fetch() const {

@@ -142,6 +142,7 @@ struct vmhip_batch {
     size_t h_pin_cap = 0;
     std::vector<uint64_t> h_force_valid, h_force_keep;
     bool have_run = false;
+    bool in_flight = false;     /* vmhip_batch_run_async without its vmhip_batch_wait */
     uint64_t run_serial = 0;    /* counts completed runs */
     uint64_t detect_serial = 0; /* the run whose detections the workspace holds, with these parameters: */
     int32_t detect_class = -1, detect_arg_max = 0, detect_clusters = 0;
@@ -451,7 +452,9 @@ int batch_enqueue(vmhip_batch* b) {
 /* Re-decide, with the host's arithmetic, every candidate the device flagged as lying within the
  * ambiguity band of a screen edge. Returns the number of decisions that differ (those are written
  * into the force masks), or a negative status. */
-int batch_verify(vmhip_batch* b) {
+/* the run's one download (visible counts, ambiguity counts, heads of the ambiguity lists, the convolution kernel's
+ * count of waits that ran out) into the pinned landing area, behind the run's kernels */
+int batch_request_verdict(vmhip_batch* b) {
     vmhip_engine* E = b->engine;
     const int n = int(b->frames.size());
     constexpr int HEAD = vmhip_batch::AMB_HEAD;
@@ -466,6 +469,17 @@ int batch_verify(vmhip_batch* b) {
     unsigned int* d_timeouts = (E->use_flow && b->classify) ? vm_flow_timeouts_address() : nullptr;
     *pin_timeouts = 0;
     if (d_timeouts) HIP_TRY(hipMemcpyAsync(pin_timeouts, d_timeouts, 4, hipMemcpyDeviceToHost, E->stream));
+    return VMHIP_OK;
+}
+
+int batch_verify(vmhip_batch* b) {
+    vmhip_engine* E = b->engine;
+    const int n = int(b->frames.size());
+    constexpr int HEAD = vmhip_batch::AMB_HEAD;
+    int32_t* pin_counts = reinterpret_cast<int32_t*>(b->h_pin);
+    int2* pin_amb = reinterpret_cast<int2*>(pin_counts + 2 * n);
+    uint32_t* pin_timeouts = reinterpret_cast<uint32_t*>(pin_amb + size_t(n) * HEAD);
+    unsigned int* d_timeouts = (E->use_flow && b->classify) ? vm_flow_timeouts_address() : nullptr;
     HIP_TRY(hipStreamSynchronize(E->stream));
     if (*pin_timeouts != 0) {
         (void) hipMemset(d_timeouts, 0, 4);
@@ -521,44 +535,60 @@ int batch_verify(vmhip_batch* b) {
     return changed;
 }
 
-int batch_run(vmhip_batch* b) {
-    if (b->frames.empty()) return fail(VMHIP_ERR_ARGUMENT, "run: nothing staged");
+/* puts one pass over the staged frames, and the download of its verdict, on the engine's stream */
+int batch_launch(vmhip_batch* b) {
     vmhip_engine* E = b->engine;
-    for (int attempt = 0; attempt < 4; ++attempt) {
-        if (b->epoch == 0xffffffffu) { /* the device stamp is about to wrap: old stamps could look current again */
-            HIP_TRY(hipMemsetAsync(b->d_lookup.p, 0, b->d_lookup.cap, E->stream));
-            HIP_TRY(hipMemsetAsync(b->d_epoch.p, 0, 4, E->stream));
-            b->epoch = 0;
-        }
-        ++b->epoch; /* the reset kernel does the same on the device */
-        int rc = VMHIP_OK;
-        if (E->use_graph && !b->profile && b->eager_runs >= 1) {
-            if (!b->graph_exec) {
-                /* Capture the kernel sequence (kernels only: the clears are a kernel too, no memset nodes). The
-                 * first run after staging was eager, so every kernel's one-time attribute set-up is done. */
-                HIP_TRY(hipStreamBeginCapture(E->stream, hipStreamCaptureModeThreadLocal));
-                rc = batch_enqueue(b);
-                hipError_t e = hipStreamEndCapture(E->stream, &b->graph);
-                if (rc != VMHIP_OK) return rc;
-                HIP_TRY(e);
-                HIP_TRY(hipGraphInstantiate(&b->graph_exec, b->graph, nullptr, nullptr, 0));
-            }
-            HIP_TRY(hipGraphLaunch(b->graph_exec, E->stream));
-        }
-        else {
+    if (b->epoch == 0xffffffffu) { /* the device stamp is about to wrap: old stamps could look current again */
+        HIP_TRY(hipMemsetAsync(b->d_lookup.p, 0, b->d_lookup.cap, E->stream));
+        HIP_TRY(hipMemsetAsync(b->d_epoch.p, 0, 4, E->stream));
+        b->epoch = 0;
+    }
+    ++b->epoch; /* the reset kernel does the same on the device */
+    int rc = VMHIP_OK;
+    if (E->use_graph && !b->profile && b->eager_runs >= 1) {
+        if (!b->graph_exec) {
+            /* Capture the kernel sequence (kernels only: the clears are a kernel too, no memset nodes). The
+             * first run after staging was eager, so every kernel's one-time attribute set-up is done. */
+            HIP_TRY(hipStreamBeginCapture(E->stream, hipStreamCaptureModeThreadLocal));
             rc = batch_enqueue(b);
-            ++b->eager_runs;
+            hipError_t e = hipStreamEndCapture(E->stream, &b->graph);
+            if (rc != VMHIP_OK) return rc;
+            HIP_TRY(e);
+            HIP_TRY(hipGraphInstantiate(&b->graph_exec, b->graph, nullptr, nullptr, 0));
         }
-        if (rc != VMHIP_OK) return rc;
-        rc = batch_verify(b);
+        HIP_TRY(hipGraphLaunch(b->graph_exec, E->stream));
+    }
+    else {
+        rc = batch_enqueue(b);
+        ++b->eager_runs;
+    }
+    if (rc != VMHIP_OK) return rc;
+    return batch_request_verdict(b);
+}
+
+/* waits for a launched pass; repeats it (a few times at most) while the host overrules edge decisions of the device */
+int batch_complete(vmhip_batch* b) {
+    for (int attempt = 0; attempt < 4; ++attempt) {
+        int rc = batch_verify(b);
         if (rc < 0) return rc;
         if (rc == 0) {
             b->have_run = true;
             ++b->run_serial;
             return VMHIP_OK;
         }
+        if (attempt == 3) break;
+        rc = batch_launch(b);
+        if (rc != VMHIP_OK) return rc;
     }
     return fail(VMHIP_ERR_HIP, "run: edge decisions did not settle");
+}
+
+int batch_run(vmhip_batch* b) {
+    if (b->frames.empty()) return fail(VMHIP_ERR_ARGUMENT, "run: nothing staged");
+    if (b->in_flight) return fail(VMHIP_ERR_ARGUMENT, "run: a run of this batch is still in flight (vmhip_batch_wait first)");
+    const int rc = batch_launch(b);
+    if (rc != VMHIP_OK) return rc;
+    return batch_complete(b);
 }
 
 int batch_fetch(vmhip_batch* b, vmhip_result* results) {
@@ -797,6 +827,7 @@ void vmhip_batch_destroy(vmhip_batch* b) {
 }
 int vmhip_batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int32_t classify) {
     if (!b) return fail(VMHIP_ERR_ARGUMENT, "batch_stage: null batch");
+    if (b->in_flight) return fail(VMHIP_ERR_ARGUMENT, "batch_stage: a run of this batch is still in flight (vmhip_batch_wait first)");
     const int rc = batch_stage(b, frames, n_frames, classify);
     if (rc != VMHIP_OK) b->frames.clear();
     return rc;
@@ -804,6 +835,21 @@ int vmhip_batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frame
 int vmhip_batch_run(vmhip_batch* b) {
     if (!b) return fail(VMHIP_ERR_ARGUMENT, "batch_run: null batch");
     return batch_run(b);
+}
+int vmhip_batch_run_async(vmhip_batch* b) {
+    if (!b) return fail(VMHIP_ERR_ARGUMENT, "batch_run_async: null batch");
+    if (b->frames.empty()) return fail(VMHIP_ERR_ARGUMENT, "run: nothing staged");
+    if (b->in_flight) return fail(VMHIP_ERR_ARGUMENT, "run: a run of this batch is still in flight (vmhip_batch_wait first)");
+    b->have_run = false;
+    const int rc = batch_launch(b);
+    if (rc == VMHIP_OK) b->in_flight = true;
+    return rc;
+}
+int vmhip_batch_wait(vmhip_batch* b) {
+    if (!b) return fail(VMHIP_ERR_ARGUMENT, "batch_wait: null batch");
+    if (!b->in_flight) return fail(VMHIP_ERR_ARGUMENT, "batch_wait: no run in flight");
+    b->in_flight = false;
+    return batch_complete(b);
 }
 int vmhip_batch_counts(const vmhip_batch* b, int32_t* n_visible) {
     if (!b || !n_visible || !b->have_run) return fail(VMHIP_ERR_ARGUMENT, "batch_counts: no completed run");

@@ -161,6 +161,13 @@ class Engine:
     def run(self):
         native.host_check(self._lib.vmh_engine_run(self.ptr))
 
+    def run_async(self):
+        """launch the pass over the staged frames and return; wait() finishes it"""
+        native.hip_check(native.hip().vmhip_batch_run_async(self.native_batch()))
+
+    def wait(self):
+        native.hip_check(native.hip().vmhip_batch_wait(self.native_batch()))
+
     def counts(self):
         n = len(self._staged)
         v = np.zeros(n, np.int32)
