@@ -76,6 +76,21 @@ typedef struct vmhip_network {
 } vmhip_network;
 
 /* Inputs of one frame. */
+/* Lookup on the device instead of on the host (the reference walks its BSP on the host, mesh.hpp:499-595): the
+ * mesh carries its cone tree (vmhip_mesh_attach_tree), a frame names what the walk compares against, and
+ * vmhip_batch_stage works out the frame's ranges itself. The host side of the engine fills this in
+ * (cpp/visualmesh/detail/cone_tree.hpp: lookup_parameters). */
+typedef struct vmhip_tree_element {
+    int32_t first, last; /* node range [first, last) of the element */
+    int32_t child[2];    /* -1, -1 for a leaf */
+    float axis[3];       /* bounding cone of the element's nodes: axis, */
+    float c, s;          /* cosine and sine of its half angle */
+} vmhip_tree_element;
+typedef struct vmhip_lookup {
+    float cos_half_fov, sin_half_fov;
+    float edge[4][5];    /* cones hugging the four screen edges, in observation-plane space: axis, cosine, sine */
+} vmhip_lookup;
+
 typedef struct vmhip_frame {
     const struct vmhip_mesh* mesh;
     float Rco[9];          /* row major; Rco[i][j] = Hoc[j][i] (reference engine/cpu/engine.hpp:95) */
@@ -84,6 +99,7 @@ typedef struct vmhip_frame {
     int32_t n_ranges;
     const void* image;     /* tightly packed rows, width*height*bytes_per_pixel(fourcc) bytes; NULL when only projecting */
     uint32_t fourcc;       /* little-endian four character code (reference utility/fourcc.hpp:34-36) */
+    const vmhip_lookup* lookup; /* not NULL: ranges / n_ranges are ignored and the lookup runs on the device */
 } vmhip_frame;
 
 /* Outputs of one frame, in caller-owned buffers. capacity counts nodes: it must be at least the number
@@ -123,6 +139,8 @@ int32_t vmhip_engine_n_classes(const vmhip_engine* engine);
 int vmhip_mesh_upload(const float* rays, const int32_t* neighbours, int32_t n_nodes, int32_t n_neighbours,
                       vmhip_mesh** out);
 void vmhip_mesh_release(vmhip_mesh* mesh);
+/* copies the mesh's cone tree (element 0 is the root) to the device, for frames that ask for the lookup there */
+int vmhip_mesh_attach_tree(vmhip_mesh* mesh, const vmhip_tree_element* elements, int32_t n_elements);
 
 /* Page-locked host memory for images (and result arrays): copies between it and the device run at the link's full
  * rate and do not hold the caller up, copies from ordinary memory are staged through small buffers by the runtime.
@@ -147,6 +165,9 @@ int vmhip_classify_batch(vmhip_engine* engine, const vmhip_frame* frames, int32_
 int vmhip_batch_create(vmhip_engine* engine, vmhip_batch** out);
 void vmhip_batch_destroy(vmhip_batch* batch);
 int vmhip_batch_stage(vmhip_batch* batch, const vmhip_frame* frames, int32_t n_frames, int32_t classify);
+/* The lookup ranges of a staged frame, as pairs (first, one-past-last): the caller's own, or what the lookup on the
+ * device produced. Returns their number (ranges may be NULL to ask for it only) or a negative status. */
+int vmhip_batch_ranges(const vmhip_batch* batch, int32_t frame, int32_t* ranges, int32_t capacity);
 int vmhip_batch_run(vmhip_batch* batch);
 /* The two halves of vmhip_batch_run: run_async puts the pass on the engine's stream and returns, wait blocks until it
  * is done (and settles the screen-edge decisions with the host, as run does). Between the two the caller is free,

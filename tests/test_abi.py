@@ -27,7 +27,7 @@ def test_hip_library_exports_every_declared_symbol():
 def test_host_library_loads_and_links_the_hip_library():
     lib = native.host()
     for name in ("vmh_mesh_create", "vmh_mesh_lookup", "vmh_visualmesh_create", "vmh_engine_create", "vmh_engine_project",
-                 "vmh_engine_classify", "vmh_engine_stage", "vmh_engine_run", "vmh_engine_fetch", "vmh_engine_result"):
+                 "vmh_engine_classify", "vmh_engine_set_device_lookup", "vmh_engine_stage", "vmh_engine_run", "vmh_engine_fetch", "vmh_engine_result"):
         assert hasattr(lib, name)
 
 
@@ -37,6 +37,8 @@ def test_struct_layouts_match_the_header():
     assert ctypes.sizeof(native.Layer) == 32
     assert ctypes.sizeof(native.Result) == 40
     assert native.Frame.Rco.offset == 8 and native.Frame.lens.offset == 44 and native.Frame.ranges.offset == 80
+    # ranges 80, n_ranges 88 (+4 padding), image 96, fourcc 104 (+4 padding), lookup 112
+    assert native.Frame.lookup.offset == 112 and ctypes.sizeof(native.Frame) == 120
     # vmhip_detections: four int32, then seven pointers
     assert ctypes.sizeof(native.Detections) == 72
     assert native.Detections.node.offset == 16 and native.Detections.cluster_centre.offset == 64

@@ -515,3 +515,34 @@ def test_run_in_two_halves_and_two_engines_overlapping(oracle):
         for g, f in zip(got, frames):
             want = pick(o_mesh, f["Hoc"]).classify(f["Hoc"], o_lens, f["image"], cfg.fourcc, net)
             assert_classification_parity(g, want, PROB_TOL, "two engines taking turns")
+
+
+@pytest.mark.parametrize("index,n_frames", [(2, 6), (3, 2), (1, 2)])
+def test_lookup_on_the_device_gives_the_hosts_ranges(oracle, index, n_frames):
+    """The walk of the cone tree on the device (vmhip_frame.lookup) must cover exactly the nodes the host's walk covers:
+    the staged ranges are compared pair by pair with Mesh::lookup's, and the classification that follows with the
+    oracle's. Configuration 2 has frames at many pitches and several meshes, 3 a rectilinear lens (edge planes
+    instead of edge cones)."""
+    cfg = wl.config(index, n_frames=n_frames)
+    o_lens, e_lens = lens_pair(cfg)
+    o_mesh, e_mesh = meshes_for(cfg, oracle)
+    engine = eng.Engine(cfg.network, cfg.model)
+    engine.set_device_lookup(True)
+    frames = [dict(mesh=e_mesh, Hoc=f["Hoc"], lens=e_lens, image=f["image"], fourcc=cfg.fourcc) for f in cfg.frames]
+    engine.stage(frames)
+    for i, f in enumerate(cfg.frames):
+        want = engine._pick(e_mesh, f["Hoc"]).lookup(f["Hoc"], e_lens)
+        got = engine.staged_ranges(i)
+        print(cfg.name, "frame", i, "ranges", len(want), flush=True)
+        assert np.array_equal(got, want), "ranges of frame %d differ" % i
+    engine.run()
+    results = engine.fetch()
+    net = vmo.Network(cfg.network)
+    for i, f in enumerate(cfg.frames):
+        want = pick(o_mesh, f["Hoc"]).classify(f["Hoc"], o_lens, f["image"], cfg.fourcc, net)
+        assert_classification_parity(results[i], want, PROB_TOL, "%s frame %d, lookup on the device" % (cfg.name, i))
+    # and back: the same engine with the host's lookup stages the same ranges
+    engine.set_device_lookup(False)
+    engine.stage(frames)
+    for i, f in enumerate(cfg.frames):
+        assert np.array_equal(engine.staged_ranges(i), engine._pick(e_mesh, f["Hoc"]).lookup(f["Hoc"], e_lens))

@@ -314,6 +314,9 @@ int vmh_engine_result(vmh_engine* e, int i, int cap, float* px, int32_t* nb, int
 }
 void* vmh_engine_native_batch(vmh_engine* e) { return e->engine->native_batch(); }
 void vmh_engine_clear_cache(vmh_engine* e) { e->engine->clear_cache(); }
+void vmh_engine_set_device_lookup(vmh_engine* e, int on) {
+    if (e && e->engine) e->engine->set_device_lookup(on != 0);
+}
 void vmh_engine_set_cache_limit(vmh_engine* e, uint64_t bytes) { e->engine->set_cache_limit(size_t(bytes)); }
 int vmh_engine_cache_info(vmh_engine* e, uint64_t* bytes) {
     *bytes = e->engine->cache_bytes();

@@ -64,6 +64,21 @@ namespace detail {
 
         const std::vector<Element>& elements() const { return elements_; }
 
+        /// What a walk of the tree compares an element against, for one camera pose: the field-of-view cone and the
+        /// four cones (or planes) along the screen edges. visible_ranges() works these out for itself; a walk that
+        /// runs elsewhere (on the device) is handed them.
+        struct Parameters {
+            float cos_half_fov, sin_half_fov;
+            Cone edges[4];
+        };
+        static Parameters lookup_parameters(const mat4<float>& Hoc, const Lens<float>& lens) {
+            Parameters p;
+            p.cos_half_fov = std::cos(lens.fov * 0.5f);
+            p.sin_half_fov = std::sin(lens.fov * 0.5f);
+            screen_edges(Hoc, lens, p.edges);
+            return p;
+        }
+
         /// On-screen candidate ranges. ray_at(i) returns the unit vector of node i in sorted order.
         template <typename RayAt>
         std::vector<std::pair<int, int>> visible_ranges(const RayAt& ray_at, const mat4<float>& Hoc, const Lens<float>& lens) const {

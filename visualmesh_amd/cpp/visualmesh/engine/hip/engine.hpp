@@ -219,8 +219,9 @@ namespace engine {
                      * ~80 us for a 1.2e5-node mesh), then the frames are described one by one (the mesh cache is not
                      * thread safe) */
                     const size_t n = frames.size();
-                    const size_t workers = std::min<size_t>(std::min<size_t>(n, 8), std::max(1u, std::thread::hardware_concurrency()));
-                    std::vector<std::exception_ptr> failed(workers);
+                    for (size_t i = 0; i < n; ++i) staged_[i].lookup_on_device = device_lookup_;
+                    const size_t workers = device_lookup_ ? 0 : std::min<size_t>(std::min<size_t>(n, 8), std::max(1u, std::thread::hardware_concurrency()));
+                    std::vector<std::exception_ptr> failed(std::max<size_t>(workers, 1));
                     auto look_up = [&](size_t w) {
                         try {
                             for (size_t i = w; i < n; i += workers) find_ranges(*frames[i].mesh, frames[i].Hoc, frames[i].lens, staged_[i]);
@@ -230,7 +231,7 @@ namespace engine {
                     };
                     std::vector<std::thread> pool;
                     for (size_t w = 1; w < workers; ++w) pool.emplace_back(look_up, w);
-                    look_up(0);
+                    if (workers > 0) look_up(0);
                     for (auto& t : pool) t.join();
                     for (auto& e : failed)
                         if (e) std::rethrow_exception(e);
@@ -344,6 +345,11 @@ namespace engine {
                 if (!v.empty()) throw_on_error(vmhip_batch_counts(batch_, v.data()));
                 return v;
             }
+            /// Where stage() looks up the nodes that may be on screen: on the host (Mesh::lookup, shared by a few
+            /// threads; the default) or on the device, by a kernel that walks the same cone tree with the same
+            /// comparisons. The single-frame calls always use the host (they size their results by the lookup).
+            void set_device_lookup(bool on) { device_lookup_ = on; }
+            bool device_lookup() const { return device_lookup_; }
             /// The batch object behind stage/run/fetch, for profiling hooks.
             vmhip_batch* native_batch() const { return batch_; }
 
@@ -383,6 +389,8 @@ namespace engine {
                 vmhip_frame frame;
                 std::vector<int32_t> ranges;
                 int32_t candidates = 0;
+                bool lookup_on_device = false;  ///< the frame carries `lookup` instead of ranges
+                vmhip_lookup lookup;
             };
 
             vmhip_engine* handle(int n_neighbours) const {
@@ -444,6 +452,19 @@ namespace engine {
                 }
                 vmhip_mesh* dev = nullptr;
                 throw_on_error(vmhip_mesh_upload(rays.data(), nbr.data(), int32_t(n), N, &dev));
+                {  // the cone tree goes along, for lookups on the device
+                    const auto& elements = mesh.tree().elements();
+                    std::vector<vmhip_tree_element> tree(elements.size());
+                    for (size_t i = 0; i < elements.size(); ++i) {
+                        const auto& e = elements[i];
+                        tree[i] = vmhip_tree_element{e.first, e.last, {e.child[0], e.child[1]}, {e.cone.axis[0], e.cone.axis[1], e.cone.axis[2]}, e.cone.c, e.cone.s};
+                    }
+                    const int rc = tree.empty() ? VMHIP_OK : vmhip_mesh_attach_tree(dev, tree.data(), int32_t(tree.size()));
+                    if (rc != VMHIP_OK) {
+                        vmhip_mesh_release(dev);
+                        throw_on_error(rc);
+                    }
+                }
                 const size_t bytes = n * (3 * sizeof(float) + N * sizeof(int32_t));
                 const uint64_t now = ++clock_;
                 meshes_[&mesh] = MeshEntry{mesh.nodes.data(), n, fingerprint, dev, bytes, now, staging_ ? staged_since_ : 0};
@@ -484,6 +505,17 @@ namespace engine {
                 f.lens.fov = lens.fov;
                 f.ranges = fd.ranges.data();
                 f.n_ranges = int32_t(fd.ranges.size() / 2);
+                if (fd.lookup_on_device) {
+                    const auto p = detail::ConeTree::lookup_parameters(Hoc, lens);
+                    fd.lookup.cos_half_fov = p.cos_half_fov;
+                    fd.lookup.sin_half_fov = p.sin_half_fov;
+                    for (int i = 0; i < 4; ++i) {
+                        for (int c = 0; c < 3; ++c) fd.lookup.edge[i][c] = p.edges[i].axis[c];
+                        fd.lookup.edge[i][3] = p.edges[i].c;
+                        fd.lookup.edge[i][4] = p.edges[i].s;
+                    }
+                    f.lookup = &fd.lookup;
+                }
                 f.image = image;
                 f.fourcc = format;
             }
@@ -505,6 +537,7 @@ namespace engine {
             mutable std::map<const void*, MeshEntry> meshes_;
             mutable uint64_t clock_ = 0, staged_since_ = 0;
             mutable bool staging_ = false;
+            bool device_lookup_ = false;
             mutable size_t cache_bytes_ = 0, cache_limit_ = size_t(8) << 30;
             mutable std::vector<FrameData> staged_;
         };

@@ -58,6 +58,9 @@ public:
         return tree_.visible_ranges([this](int i) -> const detail::f3& { return nodes[i].ray; }, Hoc, lens);
     }
 
+    /// The cone tree behind lookup(), for engines that walk it themselves.
+    const detail::ConeTree& tree() const { return tree_; }
+
     Scalar h;                      ///< camera height this mesh was generated for
     Scalar max_distance;           ///< reach of the mesh
     std::vector<node_type> nodes;  ///< nodes in cone-tree order

@@ -95,6 +95,8 @@ struct vmhip_mesh {
     int32_t* d_nbr = nullptr;
     int32_t n_nodes = 0, nn = 0;
     std::vector<float> h_rays; /* host copy for the re-decision of ambiguous candidates */
+    VmTreeElement* d_tree = nullptr; /* the cone tree, for lookups on the device (vmhip_mesh_attach_tree) */
+    int32_t n_elements = 0;
 };
 
 struct HostLayer {
@@ -161,7 +163,8 @@ struct vmhip_batch {
 
     VmBatchDev dev{};
     DevBuf d_frames, d_ranges, d_images, d_cand_px, d_cand_keep, d_tile_count, d_force_valid, d_force_keep, d_frame_V,
-      d_amb_list, d_row_px, d_row_gidx, d_row_nb, d_row_nbl, d_tile_halo, d_tile_desc, d_act[2], d_lookup, d_epoch, d_detect, d_detect_packed;
+      d_amb_list, d_row_px, d_row_gidx, d_row_nb, d_row_nbl, d_tile_halo, d_tile_desc, d_act[2], d_lookup, d_epoch, d_detect, d_detect_packed, d_lookup_ws;
+    std::vector<std::vector<int32_t>> device_ranges; /* per frame: the ranges a lookup on the device produced */
     void* h_detect = nullptr; /* pinned landing area of vmhip_batch_detect */
     size_t h_detect_cap = 0;
     float* final_act = nullptr;
@@ -178,7 +181,7 @@ struct vmhip_batch {
         DevBuf* all[] = {&d_frames, &d_ranges, &d_images, &d_cand_px, &d_cand_keep, &d_tile_count, &d_force_valid,
                          &d_force_keep, &d_frame_V, &d_amb_list, &d_row_px, &d_row_gidx, &d_row_nb,
                          &d_row_nbl, &d_tile_halo, &d_tile_desc, &d_epoch,
-                         &d_act[0], &d_act[1], &d_lookup, &d_detect, &d_detect_packed};
+                         &d_act[0], &d_act[1], &d_lookup, &d_detect, &d_detect_packed, &d_lookup_ws};
         drop_graph();
         for (DevBuf* b : all) b->release();
         if (h_pin) (void) hipHostFree(h_pin);
@@ -810,7 +813,31 @@ void vmhip_mesh_release(vmhip_mesh* M) {
     if (!M) return;
     if (M->d_rays) (void) hipFree(M->d_rays);
     if (M->d_nbr) (void) hipFree(M->d_nbr);
+    if (M->d_tree) (void) hipFree(M->d_tree);
     delete M;
+}
+
+int vmhip_mesh_attach_tree(vmhip_mesh* M, const vmhip_tree_element* elements, int32_t n_elements) {
+    static_assert(sizeof(vmhip_tree_element) == sizeof(VmTreeElement), "the tree is uploaded as it comes");
+    if (!M || !elements || n_elements <= 0) return fail(VMHIP_ERR_ARGUMENT, "mesh_attach_tree: bad arguments");
+    for (int32_t i = 0; i < n_elements; ++i) {
+        const vmhip_tree_element& e = elements[i];
+        const bool leaf = e.child[0] < 0;
+        if (e.first < 0 || e.last < e.first || e.last > M->n_nodes || (leaf ? e.child[1] >= 0 : (e.child[0] >= n_elements || e.child[1] < 0 || e.child[1] >= n_elements)))
+            return fail(VMHIP_ERR_ARGUMENT, "mesh_attach_tree: an element points outside the mesh or the tree");
+        /* children come after their parent (the walk's lists hold every element at most once) */
+        if (!leaf && (e.child[0] <= i || e.child[1] <= i)) return fail(VMHIP_ERR_ARGUMENT, "mesh_attach_tree: children must follow their parent");
+    }
+    if (M->d_tree) (void) hipFree(M->d_tree);
+    M->d_tree = nullptr, M->n_elements = 0;
+    const size_t bytes = sizeof(VmTreeElement) * size_t(n_elements);
+    if (hipMalloc(&M->d_tree, bytes) != hipSuccess || hipMemcpy(M->d_tree, elements, bytes, hipMemcpyHostToDevice) != hipSuccess) {
+        if (M->d_tree) (void) hipFree(M->d_tree);
+        M->d_tree = nullptr;
+        return fail(VMHIP_ERR_HIP, "mesh_attach_tree: device allocation or copy failed");
+    }
+    M->n_elements = n_elements;
+    return VMHIP_OK;
 }
 
 int vmhip_batch_create(vmhip_engine* E, vmhip_batch** out) {
@@ -825,16 +852,127 @@ void vmhip_batch_destroy(vmhip_batch* b) {
     b->release();
     delete b;
 }
+/* Runs the lookup of every frame that asks for it on the device and returns the frames with their ranges filled in
+ * (in `patched`, whose range pointers point into b->device_ranges). */
+static int lookup_on_device(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, std::vector<vmhip_frame>& patched) {
+    vmhip_engine* E = b->engine;
+    hipStream_t s = E->stream;
+    patched.assign(frames, frames + n_frames);
+    std::vector<int> who;
+    for (int f = 0; f < n_frames; ++f)
+        if (frames[f].lookup) who.push_back(f);
+    b->device_ranges.assign(n_frames, std::vector<int32_t>());
+    if (who.empty()) return VMHIP_OK;
+    const int n = int(who.size());
+    /* workspace: the frame table, then per frame its bit map and two lists, then the cursor, the verdicts and the
+     * dense output */
+    size_t bytes = align_up(sizeof(VmLookupFrame) * n, 256);
+    std::vector<size_t> at_covered(n), at_list(n);
+    size_t dense_words = 0;
+    for (int i = 0; i < n; ++i) {
+        const vmhip_frame& in = frames[who[i]];
+        if (!in.mesh || !in.mesh->d_tree) return fail(VMHIP_ERR_ARGUMENT, "stage: a frame asks for the lookup on the device but its mesh has no tree");
+        if (in.lens.projection < VMHIP_RECTILINEAR || in.lens.projection > VMHIP_EQUIDISTANT)
+            return fail(VMHIP_ERR_LENS, "Cannot project: Unknown lens type");
+        at_covered[i] = bytes;
+        bytes += align_up(4 * ((size_t(in.mesh->n_nodes) + 31) / 32), 256);
+        at_list[i] = bytes;
+        bytes += 2 * align_up(4 * size_t(in.mesh->n_elements), 256);
+        dense_words += 2 * size_t(in.mesh->n_elements) + 1;
+    }
+    const size_t at_cursor = bytes;
+    bytes += 256;
+    const size_t at_verdict = bytes;
+    bytes += align_up(12 * size_t(n), 256);
+    const size_t at_dense = bytes;
+    bytes += 4 * dense_words;
+    HIP_TRY(b->d_lookup_ws.reserve(bytes));
+    char* const ws = static_cast<char*>(b->d_lookup_ws.p);
+    std::vector<VmLookupFrame> table(n);
+    for (int i = 0; i < n; ++i) {
+        const vmhip_frame& in = frames[who[i]];
+        VmLookupFrame& L = table[i];
+        std::memset(&L, 0, sizeof(L));
+        VmFrame& d = L.frame;
+        d.rays = in.mesh->d_rays;
+        d.n_nodes = in.mesh->n_nodes;
+        std::memcpy(d.Rco, in.Rco, sizeof(d.Rco));
+        d.focal = in.lens.focal_length;
+        d.centre_x = in.lens.centre[0];
+        d.centre_y = in.lens.centre[1];
+        vm_host_inverse_coefficients(in.lens.k, d.ik);
+        d.width = in.lens.width;
+        d.height = in.lens.height;
+        d.projection = in.lens.projection;
+        L.tree = in.mesh->d_tree;
+        L.n_elements = in.mesh->n_elements;
+        L.cos_half_fov = in.lookup->cos_half_fov;
+        L.sin_half_fov = in.lookup->sin_half_fov;
+        std::memcpy(L.edge, in.lookup->edge, sizeof(L.edge));
+        L.covered = reinterpret_cast<uint32_t*>(ws + at_covered[i]);
+        L.list[0] = reinterpret_cast<int32_t*>(ws + at_list[i]);
+        L.list[1] = reinterpret_cast<int32_t*>(ws + at_list[i] + align_up(4 * size_t(in.mesh->n_elements), 256));
+        L.capacity = in.mesh->n_elements;
+        L.cursor = reinterpret_cast<int32_t*>(ws + at_cursor);
+        L.dense = reinterpret_cast<int32_t*>(ws + at_dense);
+        L.verdict = reinterpret_cast<int32_t*>(ws + at_verdict) + 3 * i;
+    }
+    HIP_TRY(hipMemsetAsync(ws + at_cursor, 0, 4, s));
+    HIP_TRY(hipMemcpyAsync(ws, table.data(), sizeof(VmLookupFrame) * n, hipMemcpyHostToDevice, s));
+    vm_launch_lookup(reinterpret_cast<const VmLookupFrame*>(ws), n, s);
+    HIP_TRY(hipGetLastError());
+    std::vector<int32_t> verdict(3 * size_t(n));
+    HIP_TRY(hipMemcpyAsync(verdict.data(), ws + at_verdict, 12 * size_t(n), hipMemcpyDeviceToHost, s));
+    HIP_TRY(hipStreamSynchronize(s));
+    size_t used = 0;
+    for (int i = 0; i < n; ++i) {
+        if (verdict[3 * i] < 0) return fail(VMHIP_ERR_CAPACITY, "stage: a lookup on the device produced more ranges than it has room for");
+        used = std::max(used, size_t(verdict[3 * i + 2]) + 2 * size_t(verdict[3 * i]) + 1);
+    }
+    std::vector<int32_t> dense(std::max<size_t>(used, 1));
+    HIP_TRY(hipMemcpy(dense.data(), ws + at_dense, 4 * used, hipMemcpyDeviceToHost));
+    for (int i = 0; i < n; ++i) {
+        const int f = who[i], runs = verdict[3 * i];
+        const int32_t* first = dense.data() + verdict[3 * i + 2];
+        const int32_t* prefix = first + runs;
+        std::vector<int32_t>& r = b->device_ranges[f];
+        r.resize(2 * size_t(runs));
+        for (int k = 0; k < runs; ++k) {
+            r[2 * k] = first[k];
+            r[2 * k + 1] = first[k] + (prefix[k + 1] - prefix[k]);
+        }
+        patched[f].ranges = r.data();
+        patched[f].n_ranges = runs;
+    }
+    return VMHIP_OK;
+}
+
 int vmhip_batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int32_t classify) {
     if (!b) return fail(VMHIP_ERR_ARGUMENT, "batch_stage: null batch");
     if (b->in_flight) return fail(VMHIP_ERR_ARGUMENT, "batch_stage: a run of this batch is still in flight (vmhip_batch_wait first)");
-    const int rc = batch_stage(b, frames, n_frames, classify);
+    if (!frames || n_frames <= 0) return fail(VMHIP_ERR_ARGUMENT, "stage: no frames");
+    std::vector<vmhip_frame> patched;
+    int rc = lookup_on_device(b, frames, n_frames, patched);
+    if (rc == VMHIP_OK) rc = batch_stage(b, patched.data(), n_frames, classify);
     if (rc != VMHIP_OK) b->frames.clear();
     return rc;
 }
 int vmhip_batch_run(vmhip_batch* b) {
     if (!b) return fail(VMHIP_ERR_ARGUMENT, "batch_run: null batch");
     return batch_run(b);
+}
+int vmhip_batch_ranges(const vmhip_batch* b, int32_t frame, int32_t* ranges, int32_t capacity) {
+    if (!b || frame < 0 || frame >= int32_t(b->frames.size())) return fail(VMHIP_ERR_ARGUMENT, "batch_ranges: no such staged frame");
+    const HostFrame& hf = b->frames[frame];
+    const int32_t n = int32_t(hf.first.size());
+    if (ranges) {
+        if (capacity < n) return fail(VMHIP_ERR_CAPACITY, "batch_ranges: more ranges than the array holds");
+        for (int32_t r = 0; r < n; ++r) {
+            ranges[2 * r] = hf.first[r];
+            ranges[2 * r + 1] = hf.first[r] + (hf.prefix[r + 1] - hf.prefix[r]);
+        }
+    }
+    return n;
 }
 int vmhip_batch_run_async(vmhip_batch* b) {
     if (!b) return fail(VMHIP_ERR_ARGUMENT, "batch_run_async: null batch");

@@ -111,6 +111,212 @@ __global__ void vm_reset_kernel(VmBatchDev B) {
     if (i == 0) *B.epoch += 1; /* a new run: stamps of earlier runs stop matching */
 }
 
+/* ---- lookup on the device: the host's walk of the cone tree (cpp/visualmesh/detail/cone_tree.hpp, itself after the
+ * reference's mesh.hpp:499-595), one block per frame. Every test is the host's expression in the host's order, so
+ * the set of covered nodes is the same; the host merges what it covers into maximal runs, which is what the scan over
+ * the bit map at the end yields. ---- */
+constexpr int LOOKUP_THREADS = 1024;
+
+/* exclusive prefix of v over the block in thread order; total = the block's sum */
+__device__ __forceinline__ int lookup_block_scan(int v, int* wave_total, int& total) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int scan = v;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const int up = __shfl_up(scan, d);
+        if (lane >= d) scan += up;
+    }
+    __syncthreads(); /* wave_total may still be read from the call before */
+    if (lane == 63) wave_total[wave] = scan;
+    __syncthreads();
+    int before = scan - v, sum = 0;
+    for (int w = 0; w < LOOKUP_THREADS / 64; ++w) {
+        if (w < wave) before += wave_total[w];
+        sum += wave_total[w];
+    }
+    total = sum;
+    return before;
+}
+
+/* a load that does not trust the CU's L1: the words read this way were written by other threads of the block, some
+ * of them by atomics, which act on the L2 */
+template <typename T>
+__device__ __forceinline__ T lookup_read(const T* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+/* sets the bits [first, last): words that lie wholly inside belong to this range alone */
+__device__ __forceinline__ void cover(uint32_t* covered, int first, int last) {
+    if (last <= first) return;
+    const int w0 = first >> 5, w1 = (last - 1) >> 5;
+    const uint32_t head = 0xffffffffu << (first & 31), tail = 0xffffffffu >> (31 - ((last - 1) & 31));
+    if (w0 == w1) {
+        atomicOr(&covered[w0], head & tail);
+        return;
+    }
+    atomicOr(&covered[w0], head);
+    for (int w = w0 + 1; w < w1; ++w) covered[w] = 0xffffffffu;
+    atomicOr(&covered[w1], tail);
+}
+
+__global__ __launch_bounds__(LOOKUP_THREADS) void vm_lookup_kernel(const VmLookupFrame* frames) {
+    __shared__ int wave_total[LOOKUP_THREADS / 64];
+    __shared__ int n_now, n_next, n_wide;
+    __shared__ int2 wide[256]; /* ranges too long for one thread to cover by itself */
+    const VmLookupFrame& L = frames[blockIdx.x];
+    const VmFrame& F = L.frame;
+    const int tid = threadIdx.x;
+    const int words = (F.n_nodes + 31) >> 5;
+    for (int i = tid; i < words; i += LOOKUP_THREADS) L.covered[i] = 0;
+    if (tid == 0) {
+        L.list[0][0] = 0;
+        n_now = L.n_elements > 0 ? 1 : 0;
+        n_next = 0;
+        n_wide = 0;
+    }
+    __syncthreads();
+
+    const float ox = F.Rco[0], oy = F.Rco[1], oz = F.Rco[2]; /* the optical axis in observation-plane space */
+    const float W = (float) F.width, H = (float) F.height;
+    auto on_screen = [&](const float2 px) { return 0.0f <= px.x && px.x + 1.0f <= W && 0.0f <= px.y && px.y + 1.0f <= H; };
+    int cur = 0;
+    while (n_now > 0) {
+        const int n = n_now;
+        for (int i = tid; i < n; i += LOOKUP_THREADS) {
+            const VmTreeElement e = L.tree[lookup_read(&L.list[cur][i])];
+            /* field-of-view cone first: cos(a -/+ b) by the compound angle formula */
+            const float along = oz * e.axis[2] + (oy * e.axis[1] + ox * e.axis[0]);
+            bool outside = along < L.cos_half_fov * e.c - L.sin_half_fov * e.s;
+            bool inside = along > L.cos_half_fov * e.c + L.sin_half_fov * e.s;
+            if (!outside && inside) {
+                const bool axis_on_screen = on_screen(project_ray(F, e.axis[0], e.axis[1], e.axis[2]));
+                float edge_along[4];
+                bool beyond = false;
+                for (int k = 0; k < 4; ++k) {
+                    edge_along[k] = e.axis[2] * L.edge[k][2] + (e.axis[1] * L.edge[k][1] + e.axis[0] * L.edge[k][0]);
+                    beyond = beyond || edge_along[k] > L.edge[k][3] * e.c + L.edge[k][4] * e.s;
+                }
+                if (!axis_on_screen && beyond) {
+                    inside = false;
+                    outside = true;
+                }
+                else {
+                    bool clear = true;
+                    for (int k = 0; k < 4; ++k) clear = clear && edge_along[k] < L.edge[k][3] * e.c - L.edge[k][4] * e.s;
+                    inside = axis_on_screen && clear;
+                    outside = false;
+                }
+            }
+            if (inside) {
+                if (e.last - e.first > 2048) {
+                    const int at = atomicAdd(&n_wide, 1);
+                    if (at < 256) wide[at] = make_int2(e.first, e.last);
+                    else cover(L.covered, e.first, e.last);
+                }
+                else {
+                    cover(L.covered, e.first, e.last);
+                }
+            }
+            else if (outside) {
+            }
+            else if (e.child[0] < 0) {
+                for (int g = e.first; g < e.last; ++g) {
+                    const float* r = F.rays + (size_t) g * 3;
+                    const bool seen = oz * r[2] + (oy * r[1] + ox * r[0]) > L.cos_half_fov && on_screen(project_ray(F, r[0], r[1], r[2]));
+                    if (seen) atomicOr(&L.covered[g >> 5], 1u << (g & 31));
+                }
+            }
+            else {
+                const int at = atomicAdd(&n_next, 2);
+                L.list[cur ^ 1][at] = e.child[0];
+                L.list[cur ^ 1][at + 1] = e.child[1];
+            }
+        }
+        __syncthreads();
+        if (tid == 0) {
+            n_now = n_next;
+            n_next = 0;
+        }
+        cur ^= 1;
+        __syncthreads();
+    }
+    /* the long ranges, by everybody (whole words only; their ends as above) */
+    const int n_long = min(n_wide, 256);
+    for (int k = 0; k < n_long; ++k) {
+        const int first = wide[k].x, last = wide[k].y;
+        const int w0 = (first + 31) >> 5, w1 = last >> 5; /* whole words [w0, w1) */
+        for (int w = w0 + tid; w < w1; w += LOOKUP_THREADS) L.covered[w] = 0xffffffffu;
+        if (tid == 0) { /* such a range spans many words, so w0 < w1 */
+            cover(L.covered, first, w0 << 5);
+            cover(L.covered, w1 << 5, last);
+        }
+    }
+    __syncthreads();
+
+    /* maximal runs of covered nodes, in order: their starts into list[0], their ends into list[1] */
+    int runs = 0, run_ends = 0;
+    for (int base = 0; base < words; base += LOOKUP_THREADS) {
+        const int w = base + tid;
+        uint32_t v = 0, starts = 0, ends = 0;
+        if (w < words) {
+            v = lookup_read(&L.covered[w]);
+            const uint32_t below = w > 0 ? lookup_read(&L.covered[w - 1]) >> 31 : 0u;
+            const uint32_t above = w + 1 < words ? lookup_read(&L.covered[w + 1]) & 1u : 0u;
+            starts = v & ~((v << 1) | below);
+            ends = v & ~((v >> 1) | (above << 31));
+        }
+        int total_starts, total_ends;
+        int at = runs + lookup_block_scan(__popc(starts), wave_total, total_starts);
+        int at_end = run_ends + lookup_block_scan(__popc(ends), wave_total, total_ends);
+        while (starts) {
+            const int bit = __ffs((int) starts) - 1;
+            if (at < L.capacity) L.list[0][at] = (w << 5) + bit;
+            ++at;
+            starts &= starts - 1;
+        }
+        while (ends) {
+            const int bit = __ffs((int) ends) - 1;
+            if (at_end < L.capacity) L.list[1][at_end] = (w << 5) + bit + 1;
+            ++at_end;
+            ends &= ends - 1;
+        }
+        runs += total_starts;
+        run_ends += total_ends;
+    }
+    __syncthreads();
+    __shared__ int dense_at;
+    if (runs > L.capacity) { /* cannot happen with capacity = n_elements, but nothing is written past it either */
+        if (tid == 0) L.verdict[0] = -1, L.verdict[1] = 0, L.verdict[2] = 0;
+        return;
+    }
+    if (tid == 0) dense_at = atomicAdd(L.cursor, 2 * runs + 1);
+    __syncthreads();
+    int32_t* const first_out = L.dense + dense_at;
+    int32_t* const prefix_out = first_out + runs;
+    int candidates = 0;
+    for (int base = 0; base < runs; base += LOOKUP_THREADS) {
+        const int k = base + tid;
+        int length = 0, first = 0;
+        if (k < runs) {
+            first = lookup_read(&L.list[0][k]);
+            length = lookup_read(&L.list[1][k]) - first;
+        }
+        int total;
+        const int before = candidates + lookup_block_scan(length, wave_total, total);
+        if (k < runs) {
+            first_out[k] = first;
+            prefix_out[k] = before;
+        }
+        candidates += total;
+    }
+    if (tid == 0) {
+        prefix_out[runs] = candidates;
+        L.verdict[0] = runs;
+        L.verdict[1] = candidates;
+        L.verdict[2] = dense_at;
+    }
+}
+
 __global__ __launch_bounds__(VMHIP_TILE) void vm_project_kernel(VmBatchDev B) {
     __shared__ int wave_count[VMHIP_TILE / 64];
     const int tile = blockIdx.x;
@@ -489,6 +695,10 @@ void vm_launch_compact(const VmBatchDev& B, float* feat, int classify, hipStream
         hipLaunchKernelGGL(vm_compact_kernel, dim3(B.n_cand_tiles), dim3(VMHIP_TILE), 0, stream, B,
                            reinterpret_cast<float4*>(feat), classify);
 }
+void vm_launch_lookup(const VmLookupFrame* frames, int n_frames, hipStream_t stream) {
+    if (n_frames > 0) hipLaunchKernelGGL(vm_lookup_kernel, dim3(n_frames), dim3(LOOKUP_THREADS), 0, stream, frames);
+}
+
 void vm_launch_neighbourhood(const VmBatchDev& B, hipStream_t stream) {
     if (B.n_row_tiles > 0) hipLaunchKernelGGL(vm_neighbourhood_kernel, dim3(B.n_row_tiles), dim3(VMHIP_TILE), 0, stream, B);
 }

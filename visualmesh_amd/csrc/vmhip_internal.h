@@ -101,6 +101,29 @@ struct VmBatchDev {
     int32_t halo_cap;     /* halo slots handed out per tile, <= VMHIP_HALO_MAX (smaller only to test the far path) */
 };
 
+/* Lookup on the device (project.hip: vm_lookup_kernel): the cone tree over a mesh's nodes and what a frame's walk of it
+ * needs. The tree, the walk and every comparison in it are those of the host's lookup (cpp/visualmesh/detail/
+ * cone_tree.hpp), so the ranges are the same. */
+struct VmTreeElement {
+    int32_t first, last; /* node range [first, last) */
+    int32_t child[2];    /* -1, -1 for a leaf */
+    float axis[3], c, s; /* bounding cone: axis, cosine and sine of its half angle */
+};
+struct VmLookupFrame {
+    VmFrame frame;              /* rays, n_nodes, pose, lens: what project_ray reads */
+    const VmTreeElement* tree;
+    int32_t n_elements;
+    float cos_half_fov, sin_half_fov;
+    float edge[4][5];           /* the four screen-edge cones: axis, cosine, sine */
+    uint32_t* covered;          /* [ceil(n_nodes / 32)] one bit per node */
+    int32_t* list[2];           /* [n_elements] each: the walk's frontiers, then the runs' starts and ends */
+    int32_t capacity;           /* ranges a frame may produce: n_elements */
+    int32_t* cursor;            /* one word for the whole launch: next free word of `dense` */
+    int32_t* dense;             /* every frame's first[n] and prefix[n + 1], one frame after the other */
+    int32_t* verdict;           /* [3] ranges (-1: more than capacity), candidates, offset into dense */
+};
+void vm_launch_lookup(const VmLookupFrame* frames, int n_frames, hipStream_t stream);
+
 /* Layer descriptor on the device side (host struct, passed by value to launchers). */
 struct VmLayerDev {
     int32_t c_in;    /* width of one gathered row */

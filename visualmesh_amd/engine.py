@@ -161,6 +161,19 @@ class Engine:
     def run(self):
         native.host_check(self._lib.vmh_engine_run(self.ptr))
 
+    def set_device_lookup(self, on=True):
+        """stage() looks up the nodes that may be on screen on the device (same cone tree, same comparisons) instead of
+        on the host"""
+        self._lib.vmh_engine_set_device_lookup(self.ptr, int(bool(on)))
+
+    def staged_ranges(self, index):
+        """the lookup ranges of staged frame `index` as an [n, 2] array"""
+        lib = native.hip()
+        n = native.hip_check(lib.vmhip_batch_ranges(self.native_batch(), index, None, 0))
+        out = np.zeros((max(n, 1), 2), np.int32)
+        native.hip_check(lib.vmhip_batch_ranges(self.native_batch(), index, native._ip(out), n))
+        return out[:n]
+
     def run_async(self):
         """launch the pass over the staged frames and return; wait() finishes it"""
         native.hip_check(native.hip().vmhip_batch_run_async(self.native_batch()))
