@@ -348,7 +348,12 @@ namespace engine {
             /// Where stage() looks up the nodes that may be on screen: on the host (Mesh::lookup, shared by a few
             /// threads; the default) or on the device, by a kernel that walks the same cone tree with the same
             /// comparisons. The single-frame calls always use the host (they size their results by the lookup).
+            /// Needs a Mesh that exposes its cone tree (VISUALMESH_MESH_HAS_CONE_TREE); otherwise the host's lookup stays
+#if defined(VISUALMESH_MESH_HAS_CONE_TREE)
             void set_device_lookup(bool on) { device_lookup_ = on; }
+#else
+            void set_device_lookup(bool) {}
+#endif
             bool device_lookup() const { return device_lookup_; }
             /// The batch object behind stage/run/fetch, for profiling hooks.
             vmhip_batch* native_batch() const { return batch_; }
@@ -452,6 +457,7 @@ namespace engine {
                 }
                 vmhip_mesh* dev = nullptr;
                 throw_on_error(vmhip_mesh_upload(rays.data(), nbr.data(), int32_t(n), N, &dev));
+#if defined(VISUALMESH_MESH_HAS_CONE_TREE)
                 {  // the cone tree goes along, for lookups on the device
                     const auto& elements = mesh.tree().elements();
                     std::vector<vmhip_tree_element> tree(elements.size());
@@ -465,6 +471,7 @@ namespace engine {
                         throw_on_error(rc);
                     }
                 }
+#endif
                 const size_t bytes = n * (3 * sizeof(float) + N * sizeof(int32_t));
                 const uint64_t now = ++clock_;
                 meshes_[&mesh] = MeshEntry{mesh.nodes.data(), n, fingerprint, dev, bytes, now, staging_ ? staged_since_ : 0};
@@ -505,6 +512,7 @@ namespace engine {
                 f.lens.fov = lens.fov;
                 f.ranges = fd.ranges.data();
                 f.n_ranges = int32_t(fd.ranges.size() / 2);
+#if defined(VISUALMESH_MESH_HAS_CONE_TREE)
                 if (fd.lookup_on_device) {
                     const auto p = detail::ConeTree::lookup_parameters(Hoc, lens);
                     fd.lookup.cos_half_fov = p.cos_half_fov;
@@ -516,6 +524,7 @@ namespace engine {
                     }
                     f.lookup = &fd.lookup;
                 }
+#endif
                 f.image = image;
                 f.fourcc = format;
             }

@@ -59,6 +59,8 @@ public:
     }
 
     /// The cone tree behind lookup(), for engines that walk it themselves.
+    /// The cone tree, for walks that run elsewhere (the HIP engine's lookup on the device)
+#define VISUALMESH_MESH_HAS_CONE_TREE 1
     const detail::ConeTree& tree() const { return tree_; }
 
     Scalar h;                      ///< camera height this mesh was generated for
