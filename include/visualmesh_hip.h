@@ -168,6 +168,25 @@ int vmhip_batch_stage(vmhip_batch* batch, const vmhip_frame* frames, int32_t n_f
 /* The lookup ranges of a staged frame, as pairs (first, one-past-last): the caller's own, or what the lookup on the
  * device produced. Returns their number (ranges may be NULL to ask for it only) or a negative status. */
 int vmhip_batch_ranges(const vmhip_batch* batch, int32_t frame, int32_t* ranges, int32_t capacity);
+
+/* Replaces the LookupVisualMesh op of the training pipeline (reference tensorflow/lookup.cpp:186-249) for the frames of
+ * a staged batch (no run needed): per frame, for every node of its lookup ranges in order,
+ *   vectors [capacity][3]               the node's unit vector (the op's output "vectors")
+ *   graph   [capacity][n_neighbours+1]  its own position, then its neighbours' positions along the ranges (the op's
+ *                                       output "neighbours"); a neighbour outside the ranges is INT32_MIN with
+ *                                       VMHIP_EDGE_HARD and the node's own position with VMHIP_EDGE_SAME
+ *                                       (training/dataset/projection/visual_mesh.py:82-89)
+ *   pixels  [capacity][2]               (x, y) as vmhip_project computes them, on screen or not; may be NULL
+ * n_points is written by the library; capacity must be at least the sum of the frame's range lengths. */
+enum { VMHIP_EDGE_HARD = 0, VMHIP_EDGE_SAME = 1 };
+typedef struct vmhip_lookup_export {
+    int32_t capacity;
+    int32_t n_points;
+    float* vectors;
+    int32_t* graph;
+    float* pixels;
+} vmhip_lookup_export;
+int vmhip_batch_export(vmhip_batch* batch, int32_t edge_type, vmhip_lookup_export* per_frame);
 int vmhip_batch_run(vmhip_batch* batch);
 /* The two halves of vmhip_batch_run: run_async puts the pass on the engine's stream and returns, wait blocks until it
  * is done (and settles the screen-edge decisions with the host, as run does). Between the two the caller is free,

@@ -213,6 +213,24 @@ class Mesh:
                 return r[:n].copy()
             cap = n
 
+    def lookup_graph(self, Hoc, lens, same_edges=False):
+        """What the training pipeline's LookupVisualMesh op returns, restated from the reference's
+        tensorflow/lookup.cpp:186-249 (that file needs TensorFlow's headers and cannot be compiled here; the reference
+        holds no test or fixture of the op, so tests pin this restatement by the graph's own invariants instead):
+        vectors[n,3] = the unit vectors of the nodes in the lookup ranges, in order; graph[n,nn+1] = own position, then
+        the neighbours' positions along the ranges through a reverse table that starts out as the most negative int32
+        (lookup.cpp:207-216, 231-235). same_edges applies training/dataset/projection/visual_mesh.py:86-87:
+        negative entries become the row's first column. -> dict(vectors, graph, gidx)"""
+        rays, nbr = self.arrays()
+        ranges = self.lookup(Hoc, lens)
+        gidx = np.concatenate([np.arange(a, b, dtype=np.int64) for a, b in ranges]) if len(ranges) else np.zeros(0, np.int64)
+        r_lookup = np.full(self.n_nodes + 1, np.iinfo(np.int32).min, np.int32)
+        r_lookup[gidx] = np.arange(len(gidx), dtype=np.int32)
+        graph = np.concatenate([np.arange(len(gidx), dtype=np.int32)[:, None], r_lookup[nbr[gidx]]], axis=1)
+        if same_edges:
+            graph = np.where(graph < 0, graph[:, :1], graph)
+        return dict(vectors=rays[gidx].copy(), graph=graph.astype(np.int32), gidx=gidx.astype(np.int32))
+
     def project(self, Hoc, lens):
         """-> dict(px[V,2], nb[V+1,nn], gidx[V])"""
         H = np.ascontiguousarray(Hoc, dtype=np.float32)

@@ -39,6 +39,7 @@ def test_struct_layouts_match_the_header():
     assert native.Frame.Rco.offset == 8 and native.Frame.lens.offset == 44 and native.Frame.ranges.offset == 80
     # ranges 80, n_ranges 88 (+4 padding), image 96, fourcc 104 (+4 padding), lookup 112
     assert native.Frame.lookup.offset == 112 and ctypes.sizeof(native.Frame) == 120
+    assert ctypes.sizeof(native.LookupExport) == 32 and native.LookupExport.vectors.offset == 8
     # vmhip_detections: four int32, then seven pointers
     assert ctypes.sizeof(native.Detections) == 72
     assert native.Detections.node.offset == 16 and native.Detections.cluster_centre.offset == 64

@@ -546,3 +546,32 @@ def test_lookup_on_the_device_gives_the_hosts_ranges(oracle, index, n_frames):
     engine.stage(frames)
     for i, f in enumerate(cfg.frames):
         assert np.array_equal(engine.staged_ranges(i), engine._pick(e_mesh, f["Hoc"]).lookup(f["Hoc"], e_lens))
+
+
+@pytest.mark.parametrize("index,n_frames", [(2, 3), (3, 1)])
+def test_lookup_graph_export(oracle, index, n_frames):
+    """vmhip_batch_export against the oracle's restatement of the LookupVisualMesh op: vectors and graph bit-exact for
+    HARD and SAME edges; the pixel of every exported node within 1e-3 px of the oracle's projection of its vector
+    (all visible ones through the projected mesh, a sample of the others one by one)."""
+    cfg = wl.config(index, n_frames=n_frames)
+    o_lens, e_lens = lens_pair(cfg)
+    o_mesh, e_mesh = meshes_for(cfg, oracle)
+    engine = eng.Engine(cfg.network, cfg.model)
+    engine.stage([dict(mesh=e_mesh, Hoc=f["Hoc"], lens=e_lens, image=f["image"], fourcc=cfg.fourcc) for f in cfg.frames])
+    for i, f in enumerate(cfg.frames):
+        mesh = pick(o_mesh, f["Hoc"])
+        want = mesh.lookup_graph(f["Hoc"], o_lens)
+        got = engine.lookup_graph(i)
+        print(cfg.name, "frame", i, "points", len(want["gidx"]), flush=True)
+        assert np.array_equal(got["vectors"], want["vectors"])
+        assert np.array_equal(got["graph"], want["graph"])
+        assert (want["graph"] < 0).any(), "the frame must cut the mesh for the edges to matter"
+        assert np.array_equal(engine.lookup_graph(i, same_edges=True)["graph"], mesh.lookup_graph(f["Hoc"], o_lens, same_edges=True)["graph"])
+        projected = mesh.project(f["Hoc"], o_lens)
+        rows = np.searchsorted(want["gidx"], projected["gidx"])
+        assert np.abs(got["px"][rows] - projected["px"]).max() <= 1e-3
+        Rco = np.asarray(f["Hoc"], np.float32)[:3, :3].T
+        for r in np.linspace(0, len(want["gidx"]) - 1, 200).astype(int):
+            v = want["vectors"][r]
+            cam = np.array([Rco[k, 2] * v[2] + (Rco[k, 1] * v[1] + Rco[k, 0] * v[0]) for k in range(3)], np.float32)
+            assert np.abs(oracle.fn_project(cam, o_lens) - got["px"][r]).max() <= 1e-3

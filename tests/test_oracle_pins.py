@@ -273,6 +273,41 @@ def test_projected_mesh_invariants_and_brute_force_neighbourhood(oracle, model):
         assert np.array_equal(p["nb"], want)
 
 
+@pytest.mark.parametrize("model", [wl.RING6, wl.NMGRID8])
+def test_lookup_graph_by_brute_force(oracle, model):
+    """The LookupVisualMesh restatement against a dictionary walk in the other direction: every row starts with its own
+    position; an entry >= 0 points at the row that holds exactly that neighbour; an entry < 0 is the most negative int32
+    and its neighbour lies in no range (or is the null node); SAME edges differ from HARD edges only there, by the row's
+    own position; the vectors are the rays of the range nodes in ascending order."""
+    args = (model, wl.SPHERE, 0.0949, 1.0, 3.0, 8.0) if model == wl.RING6 else (model, wl.CIRCLE, 0.05, 1.0, 4.0, 2.0)
+    mesh = oracle.mesh(*args)
+    rays, nbr = mesh.arrays()
+    W, H, proj, f, fov = LENSES["equisolid"]
+    lens = vmo.make_lens(W // 4, H // 4, proj, f / 4, fov)
+    Hoc = wl.make_hoc(1.0, math.radians(50), 0.1, 0.7)
+    ranges = mesh.lookup(Hoc, lens)
+    hard = mesh.lookup_graph(Hoc, lens)
+    same = mesh.lookup_graph(Hoc, lens, same_edges=True)
+    members = [g for a, b in ranges for g in range(a, b)]
+    n = len(members)
+    assert 0 < n < mesh.n_nodes, "the pose must cut the mesh for the edges to matter"
+    assert hard["gidx"].tolist() == members and np.array_equal(hard["vectors"], rays[members])
+    assert hard["graph"].shape == (n, mesh.n_neighbours + 1) and hard["graph"].dtype == np.int32
+    position = {g: i for i, g in enumerate(members)}
+    lowest = np.iinfo(np.int32).min
+    missing = 0
+    for i, g in enumerate(members):
+        assert hard["graph"][i, 0] == i and same["graph"][i, 0] == i
+        for j in range(mesh.n_neighbours):
+            entry, neighbour = int(hard["graph"][i, j + 1]), int(nbr[g, j])
+            if neighbour in position:
+                assert entry == position[neighbour] and same["graph"][i, j + 1] == entry
+            else:
+                assert entry == lowest and same["graph"][i, j + 1] == i
+                missing += 1
+    assert missing > 0
+
+
 def test_camera_looking_up_sees_nothing(oracle):
     mesh = oracle.mesh(wl.RING6, wl.SPHERE, 0.0949, 1.0, 3.0, 8.0)
     lens = vmo.make_lens(320, 256, wl.RECTILINEAR, 175.0, math.pi / 2)

@@ -312,6 +312,33 @@ int vmh_engine_result(vmh_engine* e, int i, int cap, float* px, int32_t* nb, int
         return V;
     })
 }
+/* lookup_graph() of staged frame i: returns its number of points; copies when the arrays hold that many rows */
+int vmh_engine_lookup_graph(vmh_engine* e, int i, int same_edges, int cap, float* vectors, int32_t* graph, float* pixels) {
+    GUARD({
+        typedef HipEngine E;
+        const E::EdgeType edges = same_edges ? E::SAME : E::HARD;
+        if (e->model == VMH_RING6) {
+            const auto all = e->engine->lookup_graph<Ring6>(edges);
+            const auto& g = all.at(i);
+            const int n = int(g.vectors.size());
+            if (n <= cap && n > 0) {
+                std::memcpy(vectors, g.vectors.data(), sizeof(float) * 3 * n);
+                std::memcpy(graph, g.graph.data(), sizeof(int32_t) * 7 * n);
+                if (pixels) std::memcpy(pixels, g.pixel_coordinates.data(), sizeof(float) * 2 * n);
+            }
+            return n;
+        }
+        const auto all = e->engine->lookup_graph<NMGrid8>(edges);
+        const auto& g = all.at(i);
+        const int n = int(g.vectors.size());
+        if (n <= cap && n > 0) {
+            std::memcpy(vectors, g.vectors.data(), sizeof(float) * 3 * n);
+            std::memcpy(graph, g.graph.data(), sizeof(int32_t) * 9 * n);
+            if (pixels) std::memcpy(pixels, g.pixel_coordinates.data(), sizeof(float) * 2 * n);
+        }
+        return n;
+    })
+}
 void* vmh_engine_native_batch(vmh_engine* e) { return e->engine->native_batch(); }
 void vmh_engine_clear_cache(vmh_engine* e) { e->engine->clear_cache(); }
 void vmh_engine_set_device_lookup(vmh_engine* e, int on) {

@@ -339,6 +339,43 @@ namespace engine {
                 throw_on_error(rc);
                 return out;
             }
+            /// What the training pipeline's LookupVisualMesh op returns (reference tensorflow/lookup.cpp:186-249), for
+            /// every staged frame (no run needed): per node of the frame's lookup ranges its unit vector and a row
+            /// [own position, positions of its neighbours along the ranges]. A neighbour outside the ranges is
+            /// std::numeric_limits<int>::lowest() with HARD edges, the node's own position with SAME edges
+            /// (training/dataset/projection/visual_mesh.py:82-89). Pixel coordinates (x, y) go along, on screen or not.
+            enum EdgeType { HARD = VMHIP_EDGE_HARD, SAME = VMHIP_EDGE_SAME };
+            template <int N>
+            struct LookupGraph {
+                std::vector<std::array<Scalar, 3>> vectors;
+                std::vector<std::array<int32_t, N + 1>> graph;
+                std::vector<std::array<Scalar, 2>> pixel_coordinates;
+            };
+            template <template <typename> class Model>
+            std::vector<LookupGraph<Model<Scalar>::N_NEIGHBOURS>> lookup_graph(EdgeType edges = HARD) const {
+                constexpr int N = Model<Scalar>::N_NEIGHBOURS;
+                const size_t n = staged_.size();
+                std::vector<LookupGraph<N>> out(n);
+                if (n == 0) return out;
+                std::vector<vmhip_lookup_export> raw(n);
+                for (auto& r : raw) std::memset(&r, 0, sizeof(r));
+                /* first call sizes (capacity 0 fits only empty frames), second call copies */
+                int rc = vmhip_batch_export(batch_, int32_t(edges), raw.data());
+                if (rc == VMHIP_ERR_CAPACITY) {
+                    for (size_t i = 0; i < n; ++i) {
+                        out[i].vectors.resize(raw[i].n_points);
+                        out[i].graph.resize(raw[i].n_points);
+                        out[i].pixel_coordinates.resize(raw[i].n_points);
+                        raw[i].capacity = raw[i].n_points;
+                        raw[i].vectors = reinterpret_cast<float*>(out[i].vectors.data());
+                        raw[i].graph = reinterpret_cast<int32_t*>(out[i].graph.data());
+                        raw[i].pixels = reinterpret_cast<float*>(out[i].pixel_coordinates.data());
+                    }
+                    rc = vmhip_batch_export(batch_, int32_t(edges), raw.data());
+                }
+                throw_on_error(rc);
+                return out;
+            }
             /// Visible nodes per staged frame after run().
             std::vector<int32_t> visible_counts() const {
                 std::vector<int32_t> v(staged_.size());

@@ -163,7 +163,7 @@ struct vmhip_batch {
 
     VmBatchDev dev{};
     DevBuf d_frames, d_ranges, d_images, d_cand_px, d_cand_keep, d_tile_count, d_force_valid, d_force_keep, d_frame_V,
-      d_amb_list, d_row_px, d_row_gidx, d_row_nb, d_row_nbl, d_tile_halo, d_tile_desc, d_act[2], d_lookup, d_epoch, d_detect, d_detect_packed, d_lookup_ws;
+      d_amb_list, d_row_px, d_row_gidx, d_row_nb, d_row_nbl, d_tile_halo, d_tile_desc, d_act[2], d_lookup, d_epoch, d_detect, d_detect_packed, d_lookup_ws, d_export;
     std::vector<std::vector<int32_t>> device_ranges; /* per frame: the ranges a lookup on the device produced */
     void* h_detect = nullptr; /* pinned landing area of vmhip_batch_detect */
     size_t h_detect_cap = 0;
@@ -181,7 +181,7 @@ struct vmhip_batch {
         DevBuf* all[] = {&d_frames, &d_ranges, &d_images, &d_cand_px, &d_cand_keep, &d_tile_count, &d_force_valid,
                          &d_force_keep, &d_frame_V, &d_amb_list, &d_row_px, &d_row_gidx, &d_row_nb,
                          &d_row_nbl, &d_tile_halo, &d_tile_desc, &d_epoch,
-                         &d_act[0], &d_act[1], &d_lookup, &d_detect, &d_detect_packed, &d_lookup_ws};
+                         &d_act[0], &d_act[1], &d_lookup, &d_detect, &d_detect_packed, &d_lookup_ws, &d_export};
         drop_graph();
         for (DevBuf* b : all) b->release();
         if (h_pin) (void) hipHostFree(h_pin);
@@ -973,6 +973,38 @@ int vmhip_batch_ranges(const vmhip_batch* b, int32_t frame, int32_t* ranges, int
         }
     }
     return n;
+}
+int vmhip_batch_export(vmhip_batch* b, int32_t edge_type, vmhip_lookup_export* per_frame) {
+    if (!b || !per_frame) return fail(VMHIP_ERR_ARGUMENT, "batch_export: null argument");
+    if (b->frames.empty()) return fail(VMHIP_ERR_ARGUMENT, "batch_export: nothing staged");
+    if (b->in_flight) return fail(VMHIP_ERR_ARGUMENT, "batch_export: a run of this batch is still in flight (vmhip_batch_wait first)");
+    if (edge_type != VMHIP_EDGE_HARD && edge_type != VMHIP_EDGE_SAME) return fail(VMHIP_ERR_ARGUMENT, "batch_export: unknown edge type");
+    const int n = int(b->frames.size());
+    for (int f = 0; f < n; ++f) per_frame[f].n_points = b->frames[f].dev.n_cand; /* all of them, so that a caller can size */
+    for (int f = 0; f < n; ++f) {
+        if (per_frame[f].capacity < per_frame[f].n_points) return fail(VMHIP_ERR_CAPACITY, "batch_export: capacity is smaller than the number of nodes in the frame's ranges");
+        if (per_frame[f].n_points > 0 && (!per_frame[f].vectors || !per_frame[f].graph)) return fail(VMHIP_ERR_ARGUMENT, "batch_export: null output array");
+    }
+    hipStream_t s = b->engine->stream;
+    const size_t slots = std::max<size_t>(b->cand_total, 1), width = size_t(b->dev.nb_stride) + 1;
+    const size_t at_graph = align_up(12 * slots, 256), at_pixels = at_graph + align_up(4 * slots * width, 256);
+    HIP_TRY(b->d_export.reserve(at_pixels + 8 * slots));
+    char* const ws = static_cast<char*>(b->d_export.p);
+    float* const vectors = reinterpret_cast<float*>(ws);
+    int32_t* const graph = reinterpret_cast<int32_t*>(ws + at_graph);
+    float* const pixels = reinterpret_cast<float*>(ws + at_pixels);
+    vm_launch_lookup_export(b->dev, edge_type == VMHIP_EDGE_SAME, vectors, graph, pixels, s);
+    HIP_TRY(hipGetLastError());
+    for (int f = 0; f < n; ++f) {
+        const VmFrame& d = b->frames[f].dev;
+        const size_t base = size_t(d.cand_base), count = size_t(d.n_cand);
+        if (count == 0) continue;
+        HIP_TRY(hipMemcpyAsync(per_frame[f].vectors, vectors + base * 3, 12 * count, hipMemcpyDeviceToHost, s));
+        HIP_TRY(hipMemcpyAsync(per_frame[f].graph, graph + base * width, 4 * count * size_t(d.nn + 1), hipMemcpyDeviceToHost, s));
+        if (per_frame[f].pixels) HIP_TRY(hipMemcpyAsync(per_frame[f].pixels, pixels + base * 2, 8 * count, hipMemcpyDeviceToHost, s));
+    }
+    HIP_TRY(hipStreamSynchronize(s));
+    return VMHIP_OK;
 }
 int vmhip_batch_run_async(vmhip_batch* b) {
     if (!b) return fail(VMHIP_ERR_ARGUMENT, "batch_run_async: null batch");

@@ -317,6 +317,41 @@ __global__ __launch_bounds__(LOOKUP_THREADS) void vm_lookup_kernel(const VmLooku
     }
 }
 
+/* ---- the lookup as a training pipeline wants it (reference tensorflow/lookup.cpp:186-249): for every node of the
+ * frame's ranges its unit vector and a row [own position, positions of its neighbours], positions counted along the
+ * ranges; a neighbour outside the ranges is the most negative int32 (HARD edges) or the node itself (SAME edges,
+ * training/dataset/projection/visual_mesh.py:82-89). Pixel coordinates go along, as project() gives them. ---- */
+__global__ __launch_bounds__(VMHIP_TILE) void vm_lookup_export_kernel(VmBatchDev B, int same_edges, float* __restrict__ vectors,
+                                                                       int32_t* __restrict__ graph, float2* __restrict__ pixels) {
+    const int tile = blockIdx.x;
+    const int f = find_frame_by_cand_tile(B.frames, B.n_frames, tile);
+    const VmFrame& F = B.frames[f];
+    const int p = (tile - F.cand_tile0) * VMHIP_TILE + threadIdx.x;
+    if (p >= F.n_cand) return;
+    const int g = cand_to_global(F, p);
+    const size_t slot = (size_t) F.cand_base + p;
+    const float* r = F.rays + (size_t) g * 3;
+    vectors[slot * 3 + 0] = r[0];
+    vectors[slot * 3 + 1] = r[1];
+    vectors[slot * 3 + 2] = r[2];
+    pixels[slot] = project_ray(F, r[0], r[1], r[2]);
+    int32_t* row = graph + (size_t) F.cand_base * (B.nb_stride + 1) + (size_t) p * (F.nn + 1);
+    row[0] = p;
+    for (int j = 0; j < F.nn; ++j) {
+        const int n = F.nbr[(size_t) g * F.nn + j];
+        /* the last range that starts at or before n, if any, and whether n lies inside it */
+        int lo = 0, hi = F.n_ranges - 1;
+        while (lo < hi) {
+            const int mid = (lo + hi + 1) >> 1;
+            if (F.range_first[mid] <= n) lo = mid;
+            else hi = mid - 1;
+        }
+        const int first = F.range_first[lo], length = F.range_prefix[lo + 1] - F.range_prefix[lo];
+        const bool found = n >= first && n - first < length;
+        row[j + 1] = found ? F.range_prefix[lo] + (n - first) : same_edges ? p : (int32_t) 0x80000000;
+    }
+}
+
 __global__ __launch_bounds__(VMHIP_TILE) void vm_project_kernel(VmBatchDev B) {
     __shared__ int wave_count[VMHIP_TILE / 64];
     const int tile = blockIdx.x;
@@ -695,6 +730,12 @@ void vm_launch_compact(const VmBatchDev& B, float* feat, int classify, hipStream
         hipLaunchKernelGGL(vm_compact_kernel, dim3(B.n_cand_tiles), dim3(VMHIP_TILE), 0, stream, B,
                            reinterpret_cast<float4*>(feat), classify);
 }
+void vm_launch_lookup_export(const VmBatchDev& B, int same_edges, float* vectors, int32_t* graph, float* pixels, hipStream_t stream) {
+    if (B.n_cand_tiles > 0)
+        hipLaunchKernelGGL(vm_lookup_export_kernel, dim3(B.n_cand_tiles), dim3(VMHIP_TILE), 0, stream, B, same_edges, vectors, graph,
+                           reinterpret_cast<float2*>(pixels));
+}
+
 void vm_launch_lookup(const VmLookupFrame* frames, int n_frames, hipStream_t stream) {
     if (n_frames > 0) hipLaunchKernelGGL(vm_lookup_kernel, dim3(n_frames), dim3(LOOKUP_THREADS), 0, stream, frames);
 }

@@ -123,6 +123,9 @@ struct VmLookupFrame {
     int32_t* verdict;           /* [3] ranges (-1: more than capacity), candidates, offset into dense */
 };
 void vm_launch_lookup(const VmLookupFrame* frames, int n_frames, hipStream_t stream);
+/* vectors [cand][3], pixels [cand][2] at the frames' candidate bases; graph rows of nn+1 words, a frame's block at
+ * cand_base * (nb_stride + 1) */
+void vm_launch_lookup_export(const VmBatchDev& B, int same_edges, float* vectors, int32_t* graph, float* pixels, hipStream_t stream);
 
 /* Layer descriptor on the device side (host struct, passed by value to launchers). */
 struct VmLayerDev {

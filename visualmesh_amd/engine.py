@@ -174,6 +174,16 @@ class Engine:
         native.hip_check(lib.vmhip_batch_ranges(self.native_batch(), index, native._ip(out), n))
         return out[:n]
 
+    def lookup_graph(self, index, same_edges=False):
+        """Engine::lookup_graph of staged frame `index` (the training pipeline's LookupVisualMesh output): dict(vectors[n,3],
+        graph[n,nn+1], px[n,2])"""
+        nn = self._staged[index].n_neighbours
+        n = native.host_check(self._lib.vmh_engine_lookup_graph(self.ptr, index, int(same_edges), 0, None, None, None))
+        vectors, graph, px = np.zeros((n, 3), np.float32), np.zeros((n, nn + 1), np.int32), np.zeros((n, 2), np.float32)
+        if n:
+            native.host_check(self._lib.vmh_engine_lookup_graph(self.ptr, index, int(same_edges), n, _fp(vectors), _ip(graph), _fp(px)))
+        return dict(vectors=vectors, graph=graph, px=px)
+
     def run_async(self):
         """launch the pass over the staged frames and return; wait() finishes it"""
         native.hip_check(native.hip().vmhip_batch_run_async(self.native_batch()))

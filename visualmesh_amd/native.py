@@ -23,7 +23,7 @@ FP32, BF16 = 0, 1
 HIP_SYMBOLS = [
     "vmhip_last_error", "vmhip_engine_create", "vmhip_engine_destroy", "vmhip_engine_n_classes", "vmhip_mesh_upload",
     "vmhip_mesh_release", "vmhip_project", "vmhip_classify", "vmhip_classify_batch", "vmhip_batch_create",
-    "vmhip_batch_destroy", "vmhip_mesh_attach_tree", "vmhip_batch_stage", "vmhip_batch_ranges", "vmhip_batch_run", "vmhip_batch_run_async", "vmhip_batch_wait", "vmhip_batch_counts", "vmhip_batch_fetch", "vmhip_batch_detect", "vmhip_host_alloc", "vmhip_host_free",
+    "vmhip_batch_destroy", "vmhip_mesh_attach_tree", "vmhip_batch_stage", "vmhip_batch_ranges", "vmhip_batch_export", "vmhip_batch_run", "vmhip_batch_run_async", "vmhip_batch_wait", "vmhip_batch_counts", "vmhip_batch_fetch", "vmhip_batch_detect", "vmhip_host_alloc", "vmhip_host_free",
     "vmhip_batch_profile", "vmhip_batch_profile_read", "vmhip_selftest_libm", "vmhip_selftest_copy",
 ]
 
@@ -55,6 +55,11 @@ class NetworkC(C.Structure):
 class Frame(C.Structure):
     _fields_ = [("mesh", C.c_void_p), ("Rco", C.c_float * 9), ("lens", Lens), ("ranges", C.POINTER(C.c_int32)),
                 ("n_ranges", C.c_int32), ("image", C.c_void_p), ("fourcc", C.c_uint32), ("lookup", C.c_void_p)]
+
+
+class LookupExport(C.Structure):
+    _fields_ = [("capacity", C.c_int32), ("n_points", C.c_int32), ("vectors", C.POINTER(C.c_float)),
+                ("graph", C.POINTER(C.c_int32)), ("pixels", C.POINTER(C.c_float))]
 
 
 class Detections(C.Structure):
@@ -129,6 +134,7 @@ def hip():
     L.vmhip_batch_counts.argtypes = [vp, C.POINTER(C.c_int32)]
     L.vmhip_batch_fetch.argtypes = [vp, C.POINTER(Result)]
     L.vmhip_batch_run_async.argtypes = [vp]
+    L.vmhip_batch_export.argtypes = [vp, C.c_int32, C.POINTER(LookupExport)]
     L.vmhip_batch_ranges.argtypes = [vp, C.c_int32, C.POINTER(C.c_int32), C.c_int32]
     L.vmhip_mesh_attach_tree.argtypes = [vp, vp, C.c_int32]
     L.vmhip_batch_wait.argtypes = [vp]
@@ -215,6 +221,7 @@ def host():
     L.vmh_engine_fetch.argtypes = [vp]
     L.vmh_engine_result.argtypes = [vp, C.c_int, C.c_int, C.POINTER(C.c_float), C.POINTER(C.c_int32), C.POINTER(C.c_int32),
                                     C.POINTER(C.c_float)]
+    L.vmh_engine_lookup_graph.argtypes = [vp, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_float), C.POINTER(C.c_int32), C.POINTER(C.c_float)]
     L.vmh_engine_native_batch.restype = vp
     L.vmh_engine_native_batch.argtypes = [vp]
     L.vmh_engine_clear_cache.argtypes = [vp]
