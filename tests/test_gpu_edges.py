@@ -1,0 +1,193 @@
+"""Edge cases of the HIP engine against the CPU oracle, through the C++ engine and the C ABI: every pixel format the
+reference's CPU engine reads, lens centre offsets and distortion, groups of several dense layers with every activation,
+frames that see nothing (alone and inside a batch), batches whose frames differ in mesh, lens, image size and format,
+and the error paths. Gates as in test_gpu_parity.py; sampled inputs and pixels are compared bit for bit."""
+import math
+
+import numpy as np
+import pytest
+
+from helpers import PROB_TOL, assert_classification_parity, assert_projection_parity
+from oracle import vmo
+from visualmesh_amd import engine as eng
+from visualmesh_amd import native
+from visualmesh_amd import workloads as wl
+
+pytestmark = pytest.mark.gpu
+
+RING = (wl.RING6, wl.SPHERE, 0.0949, 1.0, 4.0, 8.0)
+GRID = (wl.NMGRID8, wl.CIRCLE, 0.05, 1.0, 4.0, 2.0)
+BYTES = {"RGBA": 4, "BGRA": 4, "RGB3": 3, "RGB8": 3, "BGR3": 3, "BGR8": 3}
+
+
+def lenses(W, H, projection, focal, fov, **kw):
+    return vmo.make_lens(W, H, projection, focal, fov, **kw), native.make_lens(W, H, projection, focal, fov, **kw)
+
+
+def bits(a):
+    return np.ascontiguousarray(a).view(np.uint32)
+
+
+@pytest.mark.parametrize("code", ["RGBA", "BGRA", "RGB3", "RGB8", "BGR3", "BGR8", "GRAY", "GREY", "Y8  ", "GRBG", "RGGB", "GBRG", "BGGR"])
+def test_every_pixel_format(oracle, code):
+    """engine/cpu/pixel.hpp:43-102 and bayer.hpp:95-158 on the device: with an empty network the classifications are the
+    sampled inputs, which must carry the CPU engine's bits (channel order, alpha, integer demosaic without clamping)."""
+    rng = np.random.default_rng(31)
+    W, H = 322, 254  # not multiples of the tile sizes, odd Bayer phase at the right and bottom borders
+    o_lens, e_lens = lenses(W, H, wl.EQUISOLID, 105.0, math.pi)
+    image = wl.random_image(rng, W, H, BYTES.get(code, 1))
+    Hoc = wl.make_hoc(1.0, math.radians(40), 0.05, -0.4)
+    o_mesh, e_mesh = oracle.mesh(*RING), eng.Mesh(*RING)
+    got = eng.Engine([], wl.RING6)(e_mesh, Hoc, e_lens, image, wl.fourcc(code))
+    want = o_mesh.classify(Hoc, o_lens, image, wl.fourcc(code), vmo.Network([]))
+    assert len(want["gidx"]) > 1000
+    assert np.array_equal(got["gidx"], want["gidx"]) and np.array_equal(got["nb"], want["nb"])
+    assert np.array_equal(bits(got["px"]), bits(want["px"]))
+    assert np.array_equal(bits(got["cls"]), bits(want["cls"])), code + ": sampled inputs differ"
+
+
+@pytest.mark.parametrize("projection,focal,fov", [(wl.EQUISOLID, 420.0, math.pi), (wl.EQUIDISTANT, 420.0, math.pi), (wl.RECTILINEAR, 700.0, math.pi / 2)])
+def test_lens_centre_and_distortion(oracle, projection, focal, fov):
+    """utility/projection.hpp:104-120,162-187 with a centre offset and both distortion coefficients: pixels bit for bit,
+    then a small network on top."""
+    rng = np.random.default_rng(32)
+    o_mesh, e_mesh = oracle.mesh(*RING), eng.Mesh(*RING)
+    network = wl.glorot_network(rng, [3, 8, 3], 6, wl.SELU)
+    engine = eng.Engine(network, wl.RING6)
+    image = wl.random_image(rng, 1280, 1024, 4)
+    for centre, k in (((7.5, -3.25), (0.0, 0.0)), ((0.0, 0.0), (-1.0e-7, 2.0e-14)), ((-12.0, 9.0), (2.0e-8, -1.0e-14))):
+        o_lens, e_lens = lenses(1280, 1024, projection, focal, fov, centre=centre, k=k)
+        Hoc = wl.make_hoc(1.0, math.radians(rng.uniform(15, 60)), math.radians(rng.uniform(-8, 8)), math.radians(rng.uniform(-180, 180)))
+        got = engine(e_mesh, Hoc, e_lens, image, wl.fourcc("RGBA"))
+        want = o_mesh.classify(Hoc, o_lens, image, wl.fourcc("RGBA"), vmo.Network(network))
+        label = "projection %d centre %r k %r" % (projection, centre, k)
+        assert len(want["gidx"]) > 1000, label
+        assert_classification_parity(got, want, PROB_TOL, label)
+        assert np.array_equal(bits(got["px"]), bits(want["px"])), label + ": pixel bits"
+
+
+def test_multi_layer_groups_and_all_activations(oracle):
+    """network_structure.hpp:25-52: a group is one gather followed by one or more dense layers; selu, relu, tanh and
+    softmax (apply_activation.hpp:34-84) in the middle of the network as well as at its end."""
+    rng = np.random.default_rng(21)
+
+    def layer(k, c, act):
+        return (rng.normal(0, 0.3, (k, c)).astype(np.float32), rng.normal(0, 0.1, c).astype(np.float32), act)
+
+    networks = {
+        "two groups of two": [[layer(28, 8, wl.TANH), layer(8, 6, wl.RELU)], [layer(42, 5, wl.SELU), layer(5, 3, wl.SOFTMAX)]],
+        "softmax inside": [[layer(28, 16, wl.SOFTMAX)], [layer(112, 16, wl.TANH), layer(16, 16, wl.RELU), layer(16, 4, wl.SELU)]],
+        "one group of three": [[layer(28, 32, wl.RELU), layer(32, 32, wl.SELU), layer(32, 2, wl.SOFTMAX)]],
+    }
+    o_lens, e_lens = lenses(320, 256, wl.EQUISOLID, 105.0, math.pi)
+    Hoc = wl.make_hoc(1.0, math.radians(35), 0.03, -0.02)
+    image = wl.random_image(rng, 320, 256, 4)
+    o_mesh, e_mesh = oracle.mesh(*RING), eng.Mesh(*RING)
+    for name, groups in networks.items():
+        got = eng.Engine(groups, wl.RING6)(e_mesh, Hoc, e_lens, image, wl.fourcc("RGBA"))
+        want = o_mesh.classify(Hoc, o_lens, image, wl.fourcc("RGBA"), vmo.Network(groups))
+        assert_classification_parity(got, want, PROB_TOL, name)
+
+
+def test_frames_that_see_nothing(oracle):
+    """engine/cpu/engine.hpp:193: nothing visible is not an error, the result is empty - for the single calls, and for
+    such a frame at the start, in the middle and at the end of a batch whose other frames are ordinary."""
+    rng = np.random.default_rng(33)
+    o_lens, e_lens = lenses(320, 256, wl.RECTILINEAR, 175.0, math.pi / 2)
+    o_mesh, e_mesh = oracle.mesh(*RING), eng.Mesh(*RING)
+    network = wl.glorot_network(rng, [3, 8, 2], 6, wl.SELU)
+    engine = eng.Engine(network, wl.RING6)
+    up = wl.make_hoc(1.0, math.radians(-80), 0.0, 0.0)
+    down = wl.make_hoc(1.0, math.radians(50), 0.02, 0.3)
+    image = wl.random_image(rng, 320, 256, 4)
+    assert len(o_mesh.project(up, o_lens)["gidx"]) == 0
+    got = engine(e_mesh, up, e_lens)
+    assert len(got["gidx"]) == 0 and len(got["px"]) == 0
+    got = engine(e_mesh, up, e_lens, image, wl.fourcc("RGBA"))
+    assert len(got["gidx"]) == 0 and got["cls"].shape[0] == 0
+    poses = [up, down, up, up, down, up]
+    results = engine.classify_batch([dict(mesh=e_mesh, Hoc=H, lens=e_lens, image=image, fourcc=wl.fourcc("RGBA")) for H in poses])
+    want = o_mesh.classify(down, o_lens, image, wl.fourcc("RGBA"), vmo.Network(network))
+    assert len(want["gidx"]) > 500
+    for H, r in zip(poses, results):
+        if H is up:
+            assert len(r["gidx"]) == 0 and r["cls"].shape[0] == 0
+        else:
+            assert_classification_parity(r, want, PROB_TOL, "the frame beside the empty ones")
+    # a batch of nothing but empty frames
+    results = engine.classify_batch([dict(mesh=e_mesh, Hoc=up, lens=e_lens, image=image, fourcc=wl.fourcc("RGBA"))] * 2)
+    assert all(len(r["gidx"]) == 0 for r in results)
+
+
+def test_ragged_batch(oracle):
+    """One batch whose frames differ in everything a frame can differ in: mesh (and with it the node count), lens
+    projection, image size and pixel format."""
+    rng = np.random.default_rng(34)
+    o_a, e_a = oracle.mesh(*RING), eng.Mesh(*RING)
+    other = (wl.RING6, wl.CIRCLE, 0.05, 0.9, 5.0, 4.0)
+    o_b, e_b = oracle.mesh(*other), eng.Mesh(*other)
+    network = wl.glorot_network(rng, [3, 16, 32, 3], 6, wl.SELU)
+    engine = eng.Engine(network, wl.RING6)
+    specs = [
+        (o_a, e_a, lenses(1280, 1024, wl.EQUISOLID, 420.0, math.pi), "RGBA", wl.make_hoc(1.0, math.radians(30), 0.0, 0.1)),
+        (o_b, e_b, lenses(640, 480, wl.RECTILINEAR, 350.0, math.pi / 2), "GRBG", wl.make_hoc(0.9, math.radians(45), 0.05, -2.0)),
+        (o_a, e_a, lenses(322, 254, wl.EQUIDISTANT, 100.0, math.pi), "BGR3", wl.make_hoc(1.0, math.radians(60), -0.05, 1.0)),
+        (o_b, e_b, lenses(1280, 1024, wl.EQUISOLID, 420.0, math.pi), "GRAY", wl.make_hoc(0.9, math.radians(20), 0.0, 3.0)),
+        (o_a, e_a, lenses(64, 48, wl.EQUISOLID, 21.0, math.pi), "BGRA", wl.make_hoc(1.0, math.radians(35), 0.0, 0.0)),
+    ]
+    frames, wants = [], []
+    for o_mesh, e_mesh, (o_lens, e_lens), code, Hoc in specs:
+        image = wl.random_image(rng, o_lens.width, o_lens.height, BYTES.get(code, 1))
+        frames.append(dict(mesh=e_mesh, Hoc=Hoc, lens=e_lens, image=image, fourcc=wl.fourcc(code)))
+        wants.append(o_mesh.classify(Hoc, o_lens, image, wl.fourcc(code), vmo.Network(network)))
+    results = engine.classify_batch(frames)
+    for i, (r, want) in enumerate(zip(results, wants)):
+        print("ragged frame", i, "V =", len(want["gidx"]), flush=True)
+        assert len(want["gidx"]) > 50
+        assert_classification_parity(r, want, PROB_TOL, "ragged frame %d" % i)
+    # the same engine, projection only
+    for i, ((o_mesh, e_mesh, (o_lens, e_lens), code, Hoc), want) in enumerate(zip(specs, wants)):
+        assert_projection_parity(engine(e_mesh, Hoc, e_lens), want, "ragged frame %d, projection" % i)
+
+
+def test_error_paths(oracle):
+    """The reference throws for an image format it cannot read (engine/cpu/pixel.hpp:100) and for a lens projection it
+    does not know (utility/projection.hpp:174); so does this engine, and it stays usable afterwards."""
+    rng = np.random.default_rng(35)
+    o_lens, e_lens = lenses(320, 256, wl.EQUISOLID, 105.0, math.pi)
+    o_mesh, e_mesh = oracle.mesh(*RING), eng.Mesh(*RING)
+    network = wl.glorot_network(rng, [3, 8, 2], 6, wl.SELU)
+    engine = eng.Engine(network, wl.RING6)
+    Hoc = wl.make_hoc(1.0, math.radians(40), 0.0, 0.0)
+    image = wl.random_image(rng, 320, 256, 4)
+    with pytest.raises((RuntimeError, ValueError), match="Unsupported image format"):
+        engine(e_mesh, Hoc, e_lens, image, wl.fourcc("YUYV"))
+    bad = native.make_lens(320, 256, 7, 105.0, math.pi)
+    with pytest.raises((RuntimeError, ValueError), match="[Uu]nknown lens"):
+        engine(e_mesh, Hoc, bad, image, wl.fourcc("RGBA"))
+    with pytest.raises((RuntimeError, ValueError)):
+        engine.classify_batch([dict(mesh=e_mesh, Hoc=Hoc, lens=e_lens, image=image, fourcc=wl.fourcc("RGBA")),
+                               dict(mesh=e_mesh, Hoc=Hoc, lens=e_lens, image=image, fourcc=wl.fourcc("YUYV"))])
+    # a network whose first layer does not fit the mesh model's neighbourhood: known at the first call, when the
+    # engine meets the mesh model (like the reference's engines, the constructor only takes the network)
+    misfit = eng.Engine(wl.glorot_network(rng, [3, 8, 2], 8, wl.SELU), wl.RING6)
+    with pytest.raises((RuntimeError, ValueError), match="expects"):
+        misfit(e_mesh, Hoc, e_lens, image, wl.fourcc("RGBA"))
+    want = o_mesh.classify(Hoc, o_lens, image, wl.fourcc("RGBA"), vmo.Network(network))
+    assert_classification_parity(engine(e_mesh, Hoc, e_lens, image, wl.fourcc("RGBA")), want, PROB_TOL, "after the errors")
+
+
+def test_nmgrid8_with_every_bayer_phase(oracle):
+    """Eight neighbours per node and a one-byte mosaic, for the four Bayer orders, with a network on top."""
+    rng = np.random.default_rng(36)
+    o_lens, e_lens = lenses(640, 480, wl.RECTILINEAR, 350.0, math.pi / 2)
+    o_mesh, e_mesh = oracle.mesh(*GRID), eng.Mesh(*GRID)
+    network = wl.glorot_network(rng, [3, 24, 24, 4], 8, wl.RELU)
+    engine = eng.Engine(network, wl.NMGRID8)
+    image = wl.random_image(rng, 640, 480, 1)
+    Hoc = wl.make_hoc(1.0, math.radians(40), 0.03, 0.5)
+    frames = [dict(mesh=e_mesh, Hoc=Hoc, lens=e_lens, image=image, fourcc=wl.fourcc(code)) for code in ("GRBG", "RGGB", "GBRG", "BGGR")]
+    for frame, r in zip(frames, engine.classify_batch(frames)):
+        want = o_mesh.classify(Hoc, o_lens, image, frame["fourcc"], vmo.Network(network))
+        assert len(want["gidx"]) > 1000
+        assert_classification_parity(r, want, PROB_TOL, "bayer order %08x" % frame["fourcc"])
