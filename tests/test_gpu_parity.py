@@ -232,7 +232,6 @@ def test_every_convolution_kernel_agrees_with_the_oracle(oracle, kernel, monkeyp
     for i, f in enumerate(cfg.frames):
         want = pick(o_mesh, f["Hoc"]).classify(f["Hoc"], o_lens, f["image"], cfg.fourcc, vmo.Network(cfg.network))
         assert_classification_parity(results[i], want, PROB_TOL, "%s frame %d" % (kernel, i))
-    assert native.hip().vm_flow_timeouts_read() == 0  # no wave of the barrier-free kernel ever ran out of polls
 
 
 @pytest.mark.parametrize("kernel", ["lds", "dma", "flow"])
@@ -256,7 +255,6 @@ def test_rows_beyond_the_halo_capacity(oracle, index, kernel, monkeypatch):
         assert any(n.startswith("conv_%s_" % kernel) for n in names), names
     want = pick(o_mesh, f["Hoc"]).classify(f["Hoc"], o_lens, f["image"], cfg.fourcc, vmo.Network(cfg.network))
     assert_classification_parity(got, want, PROB_TOL, "halo cap 8, cfg%d, %s" % (index, kernel))
-    assert native.hip().vm_flow_timeouts_read() == 0
 
 
 def test_graph_replays_match_eager_runs(oracle, monkeypatch):
@@ -459,8 +457,7 @@ def test_a_wait_that_runs_out_fails_the_run(oracle):
             engine.run()
     finally:
         lib.vm_flow_set_poll_limit(1 << 18)
-    assert lib.vm_flow_timeouts_read() == 0  # the failed run reset the count
-    engine.run()
+    engine.run()  # the failed run reset the batch's count of such waits, or this one would fail too
     got = engine.fetch()[0]
     want = pick(o_mesh, f["Hoc"]).classify(f["Hoc"], o_lens, f["image"], cfg.fourcc, vmo.Network(cfg.network))
     assert_classification_parity(got, want, PROB_TOL, "after a failed run")

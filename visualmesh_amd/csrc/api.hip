@@ -373,6 +373,7 @@ int batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int
     D.tile_desc = local_tables ? b->d_tile_desc.as<int4>() : nullptr;
     D.halo_cap = E->halo_cap;
     D.epoch = b->d_epoch.as<uint32_t>();
+    D.flow_timeouts = b->d_epoch.as<unsigned int>() + 16; /* same zeroed block, a cache line of its own */
     b->h_V.assign(n_frames, 0);
     b->h_amb_count.assign(n_frames, 0);
     return VMHIP_OK;
@@ -469,7 +470,7 @@ int batch_request_verdict(vmhip_batch* b) {
     /* the barrier-free convolution kernel bounds its waits; a wait that ran out (never in a correct run) means
      * the results of this run cannot be trusted */
     uint32_t* pin_timeouts = reinterpret_cast<uint32_t*>(pin_amb + size_t(n) * HEAD);
-    unsigned int* d_timeouts = (E->use_flow && b->classify) ? vm_flow_timeouts_address() : nullptr;
+    unsigned int* d_timeouts = (E->use_flow && b->classify) ? b->dev.flow_timeouts : nullptr;
     *pin_timeouts = 0;
     if (d_timeouts) HIP_TRY(hipMemcpyAsync(pin_timeouts, d_timeouts, 4, hipMemcpyDeviceToHost, E->stream));
     return VMHIP_OK;
@@ -482,7 +483,7 @@ int batch_verify(vmhip_batch* b) {
     int32_t* pin_counts = reinterpret_cast<int32_t*>(b->h_pin);
     int2* pin_amb = reinterpret_cast<int2*>(pin_counts + 2 * n);
     uint32_t* pin_timeouts = reinterpret_cast<uint32_t*>(pin_amb + size_t(n) * HEAD);
-    unsigned int* d_timeouts = (E->use_flow && b->classify) ? vm_flow_timeouts_address() : nullptr;
+    unsigned int* d_timeouts = (E->use_flow && b->classify) ? b->dev.flow_timeouts : nullptr;
     HIP_TRY(hipStreamSynchronize(E->stream));
     if (*pin_timeouts != 0) {
         (void) hipMemset(d_timeouts, 0, 4);

@@ -21,7 +21,7 @@
  * loads of tile k+1 (issued a tile earlier) just before.
  * Everything a wave waits for at step k depends only on what all waves do at step k-1, so the waits cannot form a
  * cycle; each is nevertheless bounded by a poll count, after which the wave tells its block, counts the event in
- * vm_flow_timeouts and leaves the tile loop, as does every wave that then sees the block's flag: no wave hangs and
+ * the batch's flow_timeouts word and leaves the tile loop, as does every wave that then sees the block's flag: no wave hangs and
  * none works on a tile that is not there. The host reads the count with every run and fails the run if it is not 0.
  * Loads are counted, not drained: a loader knows how many vector memory instructions it has issued after the ones
  * it needs (they complete in order) and waits with s_waitcnt vmcnt(that many), so the loads of the next tile, in
@@ -36,25 +36,10 @@
 
 #include "vmhip_internal.h"
 
-/* waits that ran out of polls (none in a correct run) */
-__device__ unsigned int vm_flow_timeouts;
 /* polls a wait may take; only a test of the give-up path sets it (to something tiny) */
 __device__ int vm_flow_poll_limit = 1 << 18;
 extern "C" void vm_flow_set_poll_limit(int polls) {
     (void) hipMemcpyToSymbol(HIP_SYMBOL(vm_flow_poll_limit), &polls, sizeof(polls));
-}
-unsigned int* vm_flow_timeouts_address() {
-    static unsigned int* at = nullptr;
-    if (!at && hipGetSymbolAddress(reinterpret_cast<void**>(&at), HIP_SYMBOL(vm_flow_timeouts)) != hipSuccess) {
-        (void) hipGetLastError();
-        at = nullptr;
-    }
-    return at;
-}
-extern "C" unsigned int vm_flow_timeouts_read() {
-    unsigned int v = 0;
-    (void) hipMemcpyFromSymbol(&v, HIP_SYMBOL(vm_flow_timeouts), sizeof(v));
-    return v;
 }
 
 #ifdef VM_FLOW_TIMING
@@ -353,7 +338,7 @@ __global__ __launch_bounds__(FLOW_WAVES * 64) void vm_conv_flow_kernel(VmBatchDe
     auto give_up = [&] {
         if (lane == 0) {
             atomicOr(gave_up, 1u);
-            atomicAdd(&vm_flow_timeouts, 1u);
+            atomicAdd(B.flow_timeouts, 1u);
         }
     };
 

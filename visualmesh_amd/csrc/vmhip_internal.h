@@ -98,7 +98,7 @@ struct VmBatchDev {
     uint16_t* row_nbl;    /* [rows][VMHIP_NBL_STRIDE]: 0..255 own tile, 256+h halo slot h, VMHIP_NBL_FAR not staged */
     uint32_t* tile_halo;  /* [n_row_tiles][VMHIP_HALO_MAX] batch-global row of each halo slot */
     int4* tile_desc;      /* [n_row_tiles] {first batch-global row, rows in use (0..256), halo rows, frame's row_base} */
-    int32_t halo_cap;     /* halo slots handed out per tile, <= VMHIP_HALO_MAX (smaller only to test the far path) */
+    int32_t halo_cap;     /* halo slots handed out per tile, <= VMHIP_HALO_MAX (smaller only to test the far path) */    unsigned int* flow_timeouts; /* the batch's count of waits of the barrier-free kernel that ran out of polls (0 in a correct run) */
 };
 
 /* Lookup on the device (project.hip: vm_lookup_kernel): the cone tree over a mesh's nodes and what a frame's walk of it
@@ -222,8 +222,6 @@ int vm_launch_conv_dma(const VmBatchDev& B, const VmLayerDev& L, const float* in
 /* the same with LDS counters in place of the tile loop's barriers, so that the waves of a block run freely between
  * "my tile is staged" and "my buffer may be refilled" (conv_flow.hip) */
 bool vm_flow_supported(int c_in, int c_out, int slots);
-/* device address of that kernel's count of waits that ran out of polls (0 in every correct run), or null */
-unsigned int* vm_flow_timeouts_address();
 /* host side: w_mfma (fp32, vm_mfma_permute_weights' order) rearranged into that kernel's LDS order; same size */
 void vm_flow_order_weights(const float* w_mfma, int c_in, int c_out, int slots, float* out);
 int vm_launch_conv_flow(const VmBatchDev& B, const VmLayerDev& L, const float* in, float* out, hipStream_t stream,
