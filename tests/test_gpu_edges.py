@@ -191,3 +191,39 @@ def test_nmgrid8_with_every_bayer_phase(oracle):
         want = o_mesh.classify(Hoc, o_lens, image, frame["fourcc"], vmo.Network(network))
         assert len(want["gidx"]) > 1000
         assert_classification_parity(r, want, PROB_TOL, "bayer order %08x" % frame["fourcc"])
+
+
+def test_one_engine_per_host_thread_sharing_a_mesh(oracle):
+    """The reference's concurrency pattern (example/benchmark.cpp:86-100): several host threads, each with an engine
+    of its own, all reading one immutable mesh. Every thread classifies its own frames several times over while the
+    others do the same; each result must be the oracle's."""
+    import threading
+    cfg = wl.config(2, n_frames=4)
+    o_lens, e_lens = vmo.make_lens(*cfg.lens_tuple()), native.make_lens(*cfg.lens_tuple())
+    v = cfg.visualmesh
+    args = (cfg.model, cfg.shape, cfg.radius, v["min_h"], v["max_h"], cfg.k, v["max_error"], cfg.max_distance)
+    o_mesh, e_mesh = oracle.visualmesh(*args), eng.VisualMesh(*args)
+    net = vmo.Network(cfg.network)
+    wants = [o_mesh.height(float(f["Hoc"][2][3])).classify(f["Hoc"], o_lens, f["image"], cfg.fourcc, net) for f in cfg.frames]
+    failures = []
+
+    def work(t):
+        try:
+            engine = eng.Engine(cfg.network, cfg.model)
+            for repeat in range(3):
+                f = cfg.frames[t]
+                got = engine(e_mesh, f["Hoc"], e_lens, f["image"], cfg.fourcc)
+                assert_classification_parity(got, wants[t], PROB_TOL, "thread %d repeat %d" % (t, repeat))
+                batch = engine.classify_batch([dict(mesh=e_mesh, Hoc=g["Hoc"], lens=e_lens, image=g["image"], fourcc=cfg.fourcc)
+                                               for g in (cfg.frames[t], cfg.frames[(t + 1) % 4])])
+                assert_classification_parity(batch[1], wants[(t + 1) % 4], PROB_TOL, "thread %d repeat %d, batch" % (t, repeat))
+        except BaseException as e:  # reported by the main thread
+            failures.append((t, repr(e)))
+
+    threads = [threading.Thread(target=work, args=(t,)) for t in range(4)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join(timeout=100)
+    assert not any(th.is_alive() for th in threads), "a thread did not finish"
+    assert not failures, failures

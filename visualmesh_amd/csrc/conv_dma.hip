@@ -20,6 +20,8 @@
 #include <cstdlib>
 #include <type_traits>
 
+#include <atomic>
+
 #include "vmhip_internal.h"
 
 namespace {
@@ -405,7 +407,7 @@ int launch_dma(const VmBatchDev& B, const VmLayerDev& L, const float* in, float*
     constexpr bool single = 2 * lds > 160 * 1024; /* one block of 16 waves, else two (or more) of 8 */
     constexpr int NW = single ? 16 : 8;
     auto kernel = vm_conv_dma_kernel<C_IN, C_OUT, SLOTS, NW>;
-    static bool configured = false;
+    static std::atomic<bool> configured{false}; /* engines on several host threads may get here together */
     if (!configured) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, int(lds)) != hipSuccess) {
             (void) hipGetLastError();

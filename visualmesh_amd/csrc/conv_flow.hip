@@ -34,6 +34,8 @@
 #include <cstdlib>
 #include <type_traits>
 
+#include <atomic>
+
 #include "vmhip_internal.h"
 
 /* polls a wait may take; only a test of the give-up path sets it (to something tiny) */
@@ -619,7 +621,7 @@ int launch_flow(const VmBatchDev& B, const VmLayerDev& L, const float* in, float
     /* the kernel addresses its input rows with 32-bit byte offsets */
     if ((uint64_t) B.n_row_tiles * VMHIP_TILE * C_IN * 4 > 0xffffffffull) return -1;
     auto kernel = vm_conv_flow_kernel<C_IN, C_OUT, SLOTS>;
-    static bool configured = false;
+    static std::atomic<bool> configured{false}; /* engines on several host threads may get here together */
     if (!configured) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, int(lds)) != hipSuccess) {
             (void) hipGetLastError();

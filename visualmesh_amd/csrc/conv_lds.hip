@@ -26,6 +26,8 @@
 #include <cstdlib>
 #include <type_traits>
 
+#include <atomic>
+
 #include "vmhip_internal.h"
 
 /* Build with -DVM_LDS_TIMING to count, per phase of the tile loop, the shader clock cycles every wave spends in
@@ -461,7 +463,7 @@ int launch_lds(const VmBatchDev& B, const VmLayerDev& L, const float* in, float*
     constexpr bool single = 2 * lds > 160 * 1024;
     constexpr int NW = single ? 16 : 8;
     auto kernel = vm_conv_lds_kernel<C_IN, C_OUT, SLOTS, NW, HALO>;
-    static bool configured = false;
+    static std::atomic<bool> configured{false}; /* engines on several host threads may get here together */
     if (!configured) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, int(lds)) != hipSuccess) {
             (void) hipGetLastError();

@@ -41,6 +41,8 @@
 #include <cstring>
 #include <type_traits>
 
+#include <atomic>
+
 #include "vmhip_internal.h"
 
 namespace {
@@ -438,7 +440,7 @@ int launch_mfma(const VmBatchDev& B, const VmLayerDev& L, const void* in, void* 
     constexpr bool one_big_block = OP::PARTS > 1 && lds > 80 * 1024;
     constexpr int NW = one_big_block ? 16 : 8, RB = VMHIP_TILE / (16 * NW);
     auto kernel = vm_conv_mfma_kernel<OP, C_OUT, SLOTS, OUT_T, NW, RB>;
-    static bool configured = false;
+    static std::atomic<bool> configured{false}; /* engines on several host threads may get here together */
     if (!configured) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, int(lds)) != hipSuccess) {
             (void) hipGetLastError();

@@ -16,6 +16,8 @@
 #include <cstdlib>
 #include <type_traits>
 
+#include <atomic>
+
 #include "vmhip_internal.h"
 
 namespace {
@@ -341,7 +343,7 @@ int launch_narrow(const VmBatchDev& B, const VmLayerDev& L, const float* in, flo
     static_assert(lds <= 160 * 1024, "weights and two row buffers must fit the CU's LDS");
     if ((uint64_t) B.n_row_tiles * VMHIP_TILE * C_IN * 4 > 0xffffffffull) return -1; /* 32-bit byte offsets */
     auto kernel = vm_conv_narrow_kernel<C_IN, C_OUT, SLOTS>;
-    static bool configured = false;
+    static std::atomic<bool> configured{false}; /* engines on several host threads may get here together */
     if (!configured) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, int(lds)) != hipSuccess) {
             (void) hipGetLastError();
