@@ -49,11 +49,15 @@ def layer_table(cfg, n_neighbours):
 
 
 def cpu_baseline(cfg, threads, passes):
-    """The CPU oracle (a port of the reference CPU engine) on `threads` host threads, one frame per task, a
-    fresh engine state per frame, the mesh shared - the reference benchmark's own pattern. The batch is worked
-    through `passes` times so that the sample is several seconds of CPU work."""
+    """The reference's CPU engine, compiled from its own headers behind the oracle's interface, where that library was
+    built (kind "reference"); otherwise the CPU oracle, a port of it (kind "port"). `threads` host threads, one frame
+    per task, a fresh engine per frame, the mesh shared - the reference benchmark's own pattern. The batch is
+    worked through `passes` times so that the sample is several seconds of CPU work."""
     from oracle import vmo
-    O = vmo.load("oracle")
+    O = vmo.load("reference")
+    kind = "reference"
+    if O is None:
+        O, kind = vmo.load("oracle"), "port"
     lens = vmo.make_lens(*cfg.lens_tuple())
     if cfg.visualmesh is None:
         mesh = O.mesh(cfg.model, cfg.shape, cfg.radius, cfg.mesh_h, cfg.k, cfg.max_distance)
@@ -85,7 +89,7 @@ def cpu_baseline(cfg, threads, passes):
     for t in pool:
         t.join()
     dt = time.perf_counter() - t0
-    return sum(visible) * passes / dt, len(frames) * passes / dt, dt
+    return sum(visible) * passes / dt, len(frames) * passes / dt, dt, kind
 
 
 def main():
@@ -203,8 +207,8 @@ def main():
         elif args.config != 2:
             passes = 1
             note = "all %d frames of the batch once, one frame per task" % len(cfg.frames)
-        nps, fps, dt = cpu_baseline(sample, threads, passes)
-        cpu = dict(value=nps, unit="nodes/s", cores=threads, kind="port", frames_per_s=fps, seconds=dt, sample=note)
+        nps, fps, dt, kind = cpu_baseline(sample, threads, passes)
+        cpu = dict(value=nps, unit="nodes/s", cores=threads, kind=kind, frames_per_s=fps, seconds=dt, sample=note)
 
     out = {
         "metric": "mesh nodes classified/sec",
