@@ -572,3 +572,23 @@ def test_lookup_graph_export(oracle, index, n_frames):
             v = want["vectors"][r]
             cam = np.array([Rco[k, 2] * v[2] + (Rco[k, 1] * v[1] + Rco[k, 0] * v[0]) for k in range(3)], np.float32)
             assert np.abs(oracle.fn_project(cam, o_lens) - got["px"][r]).max() <= 1e-3
+
+
+def test_results_into_page_locked_memory(oracle):
+    """vmhip_batch_fetch into arrays from vmhip_host_alloc gives the results of the ordinary fetch, also when the arrays
+    are reused by a second, smaller batch."""
+    cfg = wl.config(2, n_frames=3)
+    o_lens, e_lens = lens_pair(cfg)
+    o_mesh, e_mesh = meshes_for(cfg, oracle)
+    engine = eng.Engine(cfg.network, cfg.model)
+    frames = [dict(mesh=e_mesh, Hoc=f["Hoc"], lens=e_lens, image=f["image"], fourcc=cfg.fourcc) for f in cfg.frames]
+    for chosen in (frames, frames[1:2]):
+        engine.stage(chosen)
+        engine.run()
+        plain = engine.fetch()
+        pinned = engine.fetch_pinned()
+        assert len(plain) == len(pinned) == len(chosen)
+        for a, b in zip(plain, pinned):
+            assert len(a["gidx"]) > 1000
+            for key in ("px", "nb", "gidx", "cls"):
+                assert np.array_equal(a[key], b[key]), key
