@@ -103,7 +103,9 @@ def main():
     ap.add_argument("--no-events", action="store_true",
                     help="no HIP events in the timed passes (they then replay the captured HIP graph); no roofline is reported")
     ap.add_argument("--copy-probe", action="store_true",
-                    help="also run a 1 GiB plain copy kernel (the dispatch of known size that memory counters are scaled by)")
+                    help="accepted for older command lines: the 1 GiB plain copy kernel (the practical ceiling of the memory "
+                         "system and the dispatch of known size that memory counters are scaled by) runs unless --no-copy-probe")
+    ap.add_argument("--no-copy-probe", action="store_true", help="skip the plain copy kernel")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (frames would shard across GPUs "
@@ -190,7 +192,7 @@ def main():
                         traffic=MEASURED_TRAFFIC.get((cfg.name, dominant)))
 
     copy_gbs = None
-    if args.copy_probe:
+    if not args.no_copy_probe:
         nbytes = 1 << 30
         copy_gbs = 2 * nbytes / (native.copy_probe(nbytes, 5) * 1e-3) / 1e9
 
