@@ -17,18 +17,20 @@
  * contracting their rows like everyone else they bring in all data: a tile's rows, its rows of the neighbour table
  * and its descriptor go into the buffer; the descriptor and the halo row numbers of the tile after go into a slot
  * of the loader's own, from which it works out, right after a contraction, where each piece of that tile lies. It
- * issues those loads into buffer k & 1 once consumed[k & 1] says every wave is done with tile k, and reports its
- * loads of tile k+1 (issued a tile earlier) just before.
+ * issues those loads into buffer k & 1 once consumed[k & 1] says every wave is done with tile k; its loads of tile
+ * k+1, issued a tile earlier, it reports right after its contraction of tile k.
  * Everything a wave waits for at step k depends only on what all waves do at step k-1, so the waits cannot form a
  * cycle; each is nevertheless bounded by a poll count, after which the wave tells its block, counts the event in
  * the batch's flow_timeouts word and leaves the tile loop, as does every wave that then sees the block's flag: no wave hangs and
  * none works on a tile that is not there. The host reads the count with every run and fails the run if it is not 0.
- * Loads are counted, not drained: a loader knows how many vector memory instructions it has issued after the ones
- * it needs (they complete in order) and waits with s_waitcnt vmcnt(that many), so the loads of the next tile, in
- * flight behind them, are not waited for. For that count to be a constant every load and store of the loop is
- * issued unconditionally, with an out-of-range offset where there is nothing to move, and no load of the loop
- * returns into a register: the compiler would wait for such a register by its own count, which misses the loads
- * written as assembly below.
+ * In the prologue loads are counted, not drained: a loader knows how many vector memory instructions it has issued
+ * after the ones it needs (they complete in order) and waits with s_waitcnt vmcnt(that many), so the loads of the
+ * second tile, in flight behind those of the first, are not waited for; every load is therefore issued
+ * unconditionally, with an out-of-range offset where there is nothing to move. In the loop a loader waits once per
+ * tile, right after its contraction, for everything it has in flight - all of it requested a contraction or more
+ * ago. No load of the loop returns into a register: the compiler would wait for such a register by its own count,
+ * which misses the loads written as assembly below, and a register carried round the loop while a load still fills
+ * it forces a full drain at the copy.
  * A wave never ends with LDS loads in flight (the LDS could already belong to another block).
  */
 #include <cstdlib>
@@ -46,14 +48,26 @@ extern "C" void vm_flow_set_poll_limit(int polls) {
 
 #ifdef VM_FLOW_TIMING
 /* Build with -DVM_FLOW_TIMING to sum, per wave of a block and per phase of the tile loop, the shader clock cycles spent
- * (32 -> 32 layers only): 0 wait for the tile, 1 contraction, 2 wait for my share of the next tile, 3 activation +
+ * (layers of one shape, 32 -> 32 unless -DVM_FLOW_TIMING_CIN= / -DVM_FLOW_TIMING_COUT= say otherwise): 0 wait for the tile, 1 contraction, 2 wait for my share of the next tile, 3 activation +
  * stores, 4 wait for the buffer, 5 requests, 6 tiles. */
 __device__ unsigned long long vm_flow_timing[16 * 8];
+__device__ unsigned long long vm_flow_timing_clocks[2];
+extern "C" void vm_flow_timing_clocks_read(unsigned long long* out) {
+    (void) hipMemcpyFromSymbol(out, HIP_SYMBOL(vm_flow_timing_clocks), sizeof(vm_flow_timing_clocks));
+    unsigned long long zero[2] = {};
+    (void) hipMemcpyToSymbol(HIP_SYMBOL(vm_flow_timing_clocks), zero, sizeof(zero));
+}
 extern "C" void vm_flow_timing_read(unsigned long long* out) {
     (void) hipMemcpyFromSymbol(out, HIP_SYMBOL(vm_flow_timing), sizeof(vm_flow_timing));
     unsigned long long zero[16 * 8] = {};
     (void) hipMemcpyToSymbol(HIP_SYMBOL(vm_flow_timing), zero, sizeof(zero));
 }
+#ifndef VM_FLOW_TIMING_CIN
+#define VM_FLOW_TIMING_CIN 32
+#endif
+#ifndef VM_FLOW_TIMING_COUT
+#define VM_FLOW_TIMING_COUT 32
+#endif
 #define FLOW_T(i) do { const unsigned long long now_ = clock64(); tsum[i] += now_ - tprev; tprev = now_; } while (0)
 #else
 #define FLOW_T(i) do { } while (0)
@@ -203,13 +217,12 @@ __global__ __launch_bounds__(FLOW_WAVES * 64) void vm_conv_flow_kernel(VmBatchDe
     constexpr int LOADERS = FLOW_LOADERS, SHARE = NW / LOADERS;
     constexpr int N_FILL = SHARE * (N_DMA + 1) + 1;
     constexpr int N_AHEAD = 1 + SHARE * N_HALO;
-    constexpr int N_STORE = RB * CB;
-    static_assert(N_STORE + 2 * N_FILL + N_AHEAD < 64, "the counts must fit s_waitcnt vmcnt");
+    static_assert(RB * CB + 2 * N_FILL + N_AHEAD < 64, "a loader's loads and stores in flight must fit the vmcnt counter");
     static_assert(N_DMA == flow_rounds(C_IN) && N_HALO == flow_halo_rounds(C_IN), "the LDS size is computed from the same rounds");
     constexpr int SLOT_WORDS = flow_slot_words(C_IN);
 
 #ifdef VM_FLOW_TIMING
-    const unsigned long long t_kernel = clock64();
+    const unsigned long long t_kernel = clock64(), w_kernel = wall_clock64();
 #endif
     extern __shared__ float4 lds4[];
     float* const w_lds = reinterpret_cast<float*>(lds4);
@@ -527,8 +540,12 @@ __global__ __launch_bounds__(FLOW_WAVES * 64) void vm_conv_flow_kernel(VmBatchDe
         if (loader) {
             /* The notes on tile k+2, requested a tile ago, are in the slot once nothing but what was requested after
              * them can still be in flight: the loads of tile k+1 and the stores of tile k-1 (of tiles 0 and 1 at first). */
-            if (k == 0) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * N_FILL) : "memory");
-            else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N_STORE + N_FILL) : "memory");
+            /* Everything in flight was requested at least a contraction ago - the notes on tile k+2, the stores of
+             * tile k-1, my share of tile k+1 - so it has landed or is about to: tile k+1 is reported here, before the
+             * activation, and a wave that is done with tile k early can go on (reporting it only after the stores,
+             * with a wait by count that let them stay in flight, was 3 % slower on the 32 -> 32 layer). */
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            if (lane == 0) atomicAdd(&counters[b ^ 1], 1u);
             const int4 d_new = read_desc(slot);
             first_new = d_new.x;
             plan(d_new.x, d_new.z, k + 2 < count, [&](int v, int r) { return slot[4 + (v * N_HALO + r) * 64 + lane]; }, offs);
@@ -591,8 +608,6 @@ __global__ __launch_bounds__(FLOW_WAVES * 64) void vm_conv_flow_kernel(VmBatchDe
         if (loader) {
             /* my share of tile k+1, requested a tile ago, has landed once nothing but what was requested after it and
              * the stores above can still be in flight */
-            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N_AHEAD + N_STORE) : "memory");
-            if (lane == 0) atomicAdd(&counters[b ^ 1], 1u);
             FLOW_T(2);
             /* tile k+2 goes where tile k was, once every wave has read the last of tile k */
             if (!wait_counter(&counters[2 + b], gave_up, NW * round, polls)) {
@@ -608,8 +623,13 @@ __global__ __launch_bounds__(FLOW_WAVES * 64) void vm_conv_flow_kernel(VmBatchDe
 #endif
     }
 #ifdef VM_FLOW_TIMING
-    if (lane == 0 && C_IN == 32 && C_OUT == 32)
+    if (lane == 0 && C_IN == VM_FLOW_TIMING_CIN && C_OUT == VM_FLOW_TIMING_COUT)
         for (int i = 0; i < 8; ++i) atomicAdd(&vm_flow_timing[wave * 8 + i], tsum[i]);
+    if (lane == 0 && wave == 0 && blockIdx.x == 0 && C_IN == VM_FLOW_TIMING_CIN && C_OUT == VM_FLOW_TIMING_COUT) {
+        /* shader clock against the constant 100 MHz clock over this block's life */
+        atomicAdd(&vm_flow_timing_clocks[0], clock64() - t_kernel);
+        atomicAdd(&vm_flow_timing_clocks[1], wall_clock64() - w_kernel);
+    }
 #endif
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); /* no LDS load may outlive the wave */
 }
