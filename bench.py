@@ -48,6 +48,32 @@ def layer_table(cfg, n_neighbours):
     return out
 
 
+def conv_roofline(name, avg_ms, rows):
+    """Roofline entry of one launch of a graph-convolution kernel over `rows` rows: the layer shape is in the kernel
+    name, conv_<kind>_<cin>x<cout>s<slots>, and so are storage and arithmetic (conv_bf16x2*: bf16 rows in,
+    conv_*_tobf16: bf16 rows out, conv_bf16*: bf16 matrix instructions). Flops are the layer's algorithmic ones, not
+    the hi/lo extras. -> (dict, algorithmic bytes per row, flops per row)"""
+    shape = name.split("_")[-1]
+    c_in, rest = shape.split("x")
+    c_out, slots = rest.split("s")
+    c_in, c_out, slots = int(c_in), int(c_out), int(slots)
+    bf16_arith = name.startswith("conv_bf16")
+    s_in = 2 if name.startswith("conv_bf16x2") else 4
+    s_out = 2 if "_tobf16_" in name else (4 if not name.startswith("conv_bf16x2") or "_tof32_" in name else 2)
+    bytes_per_row = c_in * s_in + 4 * (slots - 1) + c_out * s_out
+    flops_per_row = 2 * slots * c_in * c_out
+    intensity = flops_per_row / bytes_per_row
+    matrix_peak = BF16_PEAK_TFLOPS if bf16_arith else FP32_PEAK_TFLOPS
+    ridge = matrix_peak * 1e12 / (HBM_PEAK_GBS * 1e9)
+    if intensity > ridge:
+        achieved = flops_per_row * rows / (avg_ms * 1e-3) / 1e12
+        entry = dict(bound="mfma", achieved=achieved, peak=matrix_peak, unit="TFLOP/s", frac=achieved / matrix_peak)
+    else:
+        achieved = bytes_per_row * rows / (avg_ms * 1e-3) / 1e9
+        entry = dict(bound="hbm", achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s", frac=achieved / HBM_PEAK_GBS)
+    return entry, bytes_per_row, flops_per_row
+
+
 def cpu_baseline(cfg, threads, passes):
     """The reference's CPU engine, compiled from its own headers behind the oracle's interface, where that library was
     built (kind "reference"); otherwise the CPU oracle, a port of it (kind "port"). `threads` host threads, one frame
@@ -141,8 +167,10 @@ def main():
     engine.profile(1)
     engine.run()
     kernel_ms_per_step = {}
+    launches_per_step = {}
     for name, ms, units in engine.profile_read():
         kernel_ms_per_step[name] = kernel_ms_per_step.get(name, 0.0) + ms
+        launches_per_step[name] = launches_per_step.get(name, 0) + 1
     engine.profile(0 if args.no_events else 2)   # --no-events: the timed passes replay the captured HIP graph
     kernel_ms = {}
     kernel_launches = {}
@@ -166,30 +194,17 @@ def main():
     roofline = None
     if dominant:
         avg_ms = kernel_ms[dominant] / kernel_launches[dominant]
-        # the layer shape is in the kernel name: conv_<kind>_<cin>x<cout>s<slots>
-        shape = dominant.split("_")[-1]
-        c_in, rest = shape.split("x")
-        c_out, slots = rest.split("s")
-        c_in, c_out, slots = int(c_in), int(c_out), int(slots)
-        # storage and arithmetic are in the kernel name too (conv_bf16x2*: bf16 rows in, conv_*_tobf16: bf16 rows
-        # out, conv_bf16*: bf16 matrix instructions); flops are the layer's algorithmic ones, not the hi/lo extras
-        bf16_arith = dominant.startswith("conv_bf16")
-        s_in = 2 if dominant.startswith("conv_bf16x2") else 4
-        s_out = 2 if "_tobf16_" in dominant else (4 if not dominant.startswith("conv_bf16x2") or "_tof32_" in dominant else 2)
-        bytes_per_row = c_in * s_in + 4 * (slots - 1) + c_out * s_out
-        flops_per_row = 2 * slots * c_in * c_out
-        intensity = flops_per_row / bytes_per_row
-        matrix_peak = BF16_PEAK_TFLOPS if bf16_arith else FP32_PEAK_TFLOPS
-        ridge = matrix_peak * 1e12 / (HBM_PEAK_GBS * 1e9)
-        if intensity > ridge:
-            achieved = flops_per_row * rows / (avg_ms * 1e-3) / 1e12
-            roofline = dict(bound="mfma", achieved=achieved, peak=matrix_peak, unit="TFLOP/s", frac=achieved / matrix_peak)
-        else:
-            achieved = bytes_per_row * rows / (avg_ms * 1e-3) / 1e9
-            roofline = dict(bound="hbm", achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s", frac=achieved / HBM_PEAK_GBS)
+        roofline, bytes_per_row, flops_per_row = conv_roofline(dominant, avg_ms, rows)
         roofline.update(kernel=dominant, avg_launch_ms=avg_ms, launches_per_step=kernel_launches[dominant] // args.steps,
                         rows_per_launch=rows, algorithmic_bytes_per_row=bytes_per_row, flops_per_row=flops_per_row,
                         traffic=MEASURED_TRAFFIC.get((cfg.name, dominant)))
+
+    # every graph-convolution kernel against its own roofline, from the one fully bracketed (untimed) pass
+    conv_rooflines = {}
+    for name, ms in sorted(kernel_ms_per_step.items()):
+        if name.startswith("conv"):
+            entry = conv_roofline(name, ms / launches_per_step[name], nodes + len(frames))[0]
+            conv_rooflines[name] = dict(bound=entry["bound"], achieved=entry["achieved"], unit=entry["unit"], frac=entry["frac"])
 
     copy_gbs = None
     if not args.no_copy_probe:
@@ -239,6 +254,7 @@ def main():
         "cpu_baseline": cpu,
         "copy_kernel_GBps": copy_gbs,
         "kernel_ms_per_step": dict(sorted(kernel_ms_per_step.items())),   # from the one fully profiled, untimed pass
+        "conv_rooflines": conv_rooflines,
     }
     print(json.dumps(out))
 
