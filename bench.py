@@ -186,13 +186,26 @@ def main():
     ms_per_step = elapsed * 1e3 / args.steps
     value = nodes * args.steps / elapsed
 
-    # roofline of the dominant graph-convolution kernel
+    # roofline of the dominant kernel: a graph-convolution kernel, or (small single-frame workloads) one of the
+    # kernels before the network, which move bytes only
     rows = nodes + len(frames)    # visible nodes + one null row per frame
     table = layer_table(cfg, nn)
     conv = {k: v for k, v in kernel_ms.items() if k.startswith("conv")}
     dominant = max(conv, key=conv.get) if conv else None
     roofline = None
-    if dominant:
+    if not dominant and kernel_ms:
+        dominant = max(kernel_ms, key=kernel_ms.get)
+        avg_ms = kernel_ms[dominant] / kernel_launches[dominant]
+        candidates = sum(int((r[:, 1] - r[:, 0]).sum()) for r in (engine.staged_ranges(i) for i in range(len(frames))))
+        texel_bytes = 16 if cfg.fourcc == wl.fourcc("RGBA") else 36   # four RGBA8 texels / the 6x6 union of four Bayer patches
+        algorithmic = {"project": 12 * candidates + 12 * nodes,            # rays read; pixel and index written per visible node
+                       "compact_sample": (texel_bytes + 16) * nodes,       # texels read, four floats written
+                       "neighbourhood": 12 * nn * nodes}[dominant]         # table read, reverse-lookup gathers, table written
+        achieved = algorithmic / (avg_ms * 1e-3) / 1e9
+        roofline = dict(bound="hbm", achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s", frac=achieved / HBM_PEAK_GBS, kernel=dominant,
+                        avg_launch_ms=avg_ms, launches_per_step=kernel_launches[dominant] // args.steps, algorithmic_bytes_per_launch=algorithmic,
+                        traffic=MEASURED_TRAFFIC.get((cfg.name, dominant)))
+    elif dominant:
         avg_ms = kernel_ms[dominant] / kernel_launches[dominant]
         roofline, bytes_per_row, flops_per_row = conv_roofline(dominant, avg_ms, rows)
         roofline.update(kernel=dominant, avg_launch_ms=avg_ms, launches_per_step=kernel_launches[dominant] // args.steps,
