@@ -227,3 +227,54 @@ def test_one_engine_per_host_thread_sharing_a_mesh(oracle):
         th.join(timeout=100)
     assert not any(th.is_alive() for th in threads), "a thread did not finish"
     assert not failures, failures
+
+
+@pytest.mark.parametrize("index", [2, 4])
+def test_full_size_batch_properties(oracle, index):
+    """Configurations 2 and 4 at their full batch size (16 and 64 frames; the oracle would need ~45 s per frame for 4),
+    checked through what holds at any size: a frame's result does not depend on its place in the batch nor on the
+    batch around it (bit for bit against single-frame calls and against the reversed batch), runs repeat bit for bit,
+    indices ascend, the neighbour table stays in range with the null row pointing at itself, and the probabilities of
+    every row sum to one."""
+    cfg = wl.config(index)
+    lens = native.make_lens(*cfg.lens_tuple())
+    if cfg.visualmesh is None:
+        mesh = eng.Mesh(cfg.model, cfg.shape, cfg.radius, cfg.mesh_h, cfg.k, cfg.max_distance)
+    else:
+        v = cfg.visualmesh
+        mesh = eng.VisualMesh(cfg.model, cfg.shape, cfg.radius, v["min_h"], v["max_h"], cfg.k, v["max_error"], cfg.max_distance)
+    engine = eng.Engine(cfg.network, cfg.model)
+    frames = [dict(mesh=mesh, Hoc=f["Hoc"], lens=lens, image=f["image"], fourcc=cfg.fourcc) for f in cfg.frames]
+    n = len(frames)
+    print(cfg.name, n, "frames", flush=True)
+    engine.stage(frames)
+    engine.run()
+    first = engine.fetch_pinned()
+    first = [{k: a[k].copy() for k in a} for a in first]
+    engine.run()
+    again = engine.fetch_pinned()
+    nn = wl.N_NEIGHBOURS[cfg.model]
+    for i, (a, b) in enumerate(zip(first, again)):
+        V = len(a["gidx"])
+        assert V > 10000, "frame %d sees too little to matter" % i
+        for key in ("px", "nb", "gidx", "cls"):
+            assert np.array_equal(bits(a[key]) if a[key].dtype == np.float32 else a[key], bits(b[key]) if b[key].dtype == np.float32 else b[key]), "frame %d: %s differs between runs" % (i, key)
+        assert np.all(np.diff(a["gidx"]) > 0)
+        assert a["nb"].shape == (V + 1, nn) and a["nb"].min() >= 0 and a["nb"].max() <= V and np.all(a["nb"][V] == V)
+        assert np.abs(a["cls"].sum(axis=1) - 1.0).max() < 1e-5
+        assert np.all((a["px"][:, 0] >= 0) & (a["px"][:, 0] + 1 < cfg.width) & (a["px"][:, 1] >= 0) & (a["px"][:, 1] + 1 < cfg.height))
+    # the reversed batch
+    engine.stage(frames[::-1])
+    engine.run()
+    reversed_results = engine.fetch_pinned()
+    for i in range(n):
+        a, b = first[i], reversed_results[n - 1 - i]
+        for key in ("px", "nb", "gidx", "cls"):
+            assert np.array_equal(a[key], b[key]), "frame %d: %s depends on the frame's place in the batch" % (i, key)
+    # single-frame calls
+    for i in sorted({0, n // 3, n - 1}):
+        f = cfg.frames[i]
+        alone = engine(mesh, f["Hoc"], lens, f["image"], cfg.fourcc)
+        for key in ("px", "nb", "gidx"):
+            assert np.array_equal(alone[key], first[i][key]), "frame %d: %s depends on the batch" % (i, key)
+        assert np.abs(alone["cls"] - first[i]["cls"]).max() <= 1e-6, "frame %d: probabilities depend on the batch" % i
