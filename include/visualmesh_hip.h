@@ -197,6 +197,13 @@ int vmhip_batch_wait(vmhip_batch* batch);
 /* n_visible[n_frames] of the last run */
 int vmhip_batch_counts(const vmhip_batch* batch, int32_t* n_visible);
 int vmhip_batch_fetch(vmhip_batch* batch, vmhip_result* results);
+/* The two halves of vmhip_batch_fetch: fetch_async queues the copies on the engine's stream and returns (n_visible is
+ * already written), fetch_wait blocks until they are done. With result arrays from vmhip_host_alloc the copies run
+ * while the caller stages the next frames into another engine's batch, on the bus's other direction; into ordinary
+ * memory they are not asynchronous. Between the two the batch must not be staged, run, read or exported, and the
+ * arrays must not be touched. */
+int vmhip_batch_fetch_async(vmhip_batch* batch, vmhip_result* results);
+int vmhip_batch_fetch_wait(vmhip_batch* batch);
 
 /* What a consumer of the classified mesh does first, done on the device so that only detections cross PCIe. No
  * counterpart inside the reference's engines: its consumers walk the whole ClassifiedMesh on the host

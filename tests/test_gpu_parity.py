@@ -592,3 +592,44 @@ def test_results_into_page_locked_memory(oracle):
             assert len(a["gidx"]) > 1000
             for key in ("px", "nb", "gidx", "cls"):
                 assert np.array_equal(a[key], b[key]), key
+
+
+def test_fetch_in_two_halves_and_three_engines_in_rotation(oracle):
+    """vmhip_batch_fetch_async / vmhip_batch_fetch_wait: three engines in rotation, one staging, one running and one
+    copying its results out at any time; every batch must give the oracle's results, and a batch whose fetch is in
+    flight must refuse to be staged, run or fetched again."""
+    cfg = wl.config(2, n_frames=6)
+    o_lens, e_lens = lens_pair(cfg)
+    o_mesh, e_mesh = meshes_for(cfg, oracle)
+    engines = [eng.Engine(cfg.network, cfg.model) for _ in range(3)]
+    groups = [cfg.frames[0:2], cfg.frames[2:4], cfg.frames[4:6]]
+    staged = [[dict(mesh=e_mesh, Hoc=f["Hoc"], lens=e_lens, image=f["image"], fourcc=cfg.fourcc) for f in g] for g in groups]
+    net = vmo.Network(cfg.network)
+    wants = [[pick(o_mesh, f["Hoc"]).classify(f["Hoc"], o_lens, f["image"], cfg.fourcc, net) for f in g] for g in groups]
+    results = {}
+    pending = {}
+    for step in range(3 + 2):          # every engine's group once, then the pipeline drains
+        if step < 3:
+            e = engines[step]
+            e.stage(staged[step])
+            e.run_async()
+        if 1 <= step <= 3:
+            e = engines[step - 1]
+            e.wait()
+            pending[step - 1] = e.fetch_pinned(wait=False)
+            if step == 1:
+                with pytest.raises(RuntimeError, match="fetch of this batch is still in flight"):
+                    e.run()
+                with pytest.raises(RuntimeError, match="fetch of this batch is still in flight"):
+                    e.stage(staged[0])
+                with pytest.raises(RuntimeError, match="fetch of this batch is still in flight"):
+                    e.fetch()
+        if step >= 2:
+            e = engines[step - 2]
+            e.fetch_wait()
+            results[step - 2] = pending.pop(step - 2)
+    with pytest.raises(RuntimeError, match="no fetch in flight"):
+        engines[0].fetch_wait()
+    for g in range(3):
+        for got, want in zip(results[g], wants[g]):
+            assert_classification_parity(got, want, PROB_TOL, "group %d of the rotation" % g)

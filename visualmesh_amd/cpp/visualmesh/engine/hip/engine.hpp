@@ -298,6 +298,15 @@ namespace engine {
                 if (results.size() != staged_.size()) throw std::invalid_argument("fetch_into: one result per staged frame");
                 if (!results.empty()) throw_on_error(vmhip_batch_fetch(batch_, results.data()));
             }
+            /// fetch_into in two halves: the copies are queued and run while the caller does something else (with
+            /// page-locked arrays; e.g. staging the next frames into another engine), fetch_wait() finishes them.
+            void fetch_into_async(std::vector<vmhip_result>& results) const {
+                if (results.size() != staged_.size()) throw std::invalid_argument("fetch_into_async: one result per staged frame");
+                if (!results.empty()) throw_on_error(vmhip_batch_fetch_async(batch_, results.data()));
+            }
+            void fetch_wait() const {
+                if (batch_ && !staged_.empty()) throw_on_error(vmhip_batch_fetch_wait(batch_));
+            }
             /// The nodes of one class among the results of the last run, picked and clustered on the device so that
             /// only they are downloaded (the reference's consumers walk the whole ClassifiedMesh on the host,
             /// example/draw.hpp:41-59).

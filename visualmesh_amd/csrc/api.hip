@@ -145,6 +145,7 @@ struct vmhip_batch {
     std::vector<uint64_t> h_force_valid, h_force_keep;
     bool have_run = false;
     bool in_flight = false;     /* vmhip_batch_run_async without its vmhip_batch_wait */
+    bool fetching = false;      /* vmhip_batch_fetch_async without its vmhip_batch_fetch_wait */
     uint64_t run_serial = 0;    /* counts completed runs */
     uint64_t detect_serial = 0; /* the run whose detections the workspace holds, with these parameters: */
     int32_t detect_class = -1, detect_arg_max = 0, detect_clusters = 0;
@@ -590,14 +591,17 @@ int batch_complete(vmhip_batch* b) {
 int batch_run(vmhip_batch* b) {
     if (b->frames.empty()) return fail(VMHIP_ERR_ARGUMENT, "run: nothing staged");
     if (b->in_flight) return fail(VMHIP_ERR_ARGUMENT, "run: a run of this batch is still in flight (vmhip_batch_wait first)");
+    if (b->fetching) return fail(VMHIP_ERR_ARGUMENT, "run: a fetch of this batch is still in flight (vmhip_batch_fetch_wait first)");
     const int rc = batch_launch(b);
     if (rc != VMHIP_OK) return rc;
     return batch_complete(b);
 }
 
-int batch_fetch(vmhip_batch* b, vmhip_result* results) {
+/* the copies of a fetch, on the engine's stream; the caller waits for the stream */
+int batch_fetch_enqueue(vmhip_batch* b, vmhip_result* results) {
     if (!b->have_run) return fail(VMHIP_ERR_ARGUMENT, "fetch: no completed run");
     if (!results) return fail(VMHIP_ERR_ARGUMENT, "fetch: null results");
+    if (b->fetching) return fail(VMHIP_ERR_ARGUMENT, "fetch: a fetch of this batch is still in flight (vmhip_batch_fetch_wait first)");
     vmhip_engine* E = b->engine;
     hipStream_t s = E->stream;
     const int n = int(b->frames.size());
@@ -625,7 +629,15 @@ int batch_fetch(vmhip_batch* b, vmhip_result* results) {
         if (R.classifications && b->classify)
             HIP_TRY(hipMemcpyAsync(R.classifications, b->final_act + base * C, 4 * size_t(V + 1) * C, hipMemcpyDeviceToHost, s));
     }
-    HIP_TRY(hipStreamSynchronize(s));
+    return VMHIP_OK;
+}
+
+int batch_fetch(vmhip_batch* b, vmhip_result* results) {
+    const int rc = batch_fetch_enqueue(b, results);
+    /* wait also when a copy could not be queued: the ones before it write into the caller's arrays */
+    const hipError_t e = hipStreamSynchronize(b->engine->stream);
+    if (rc != VMHIP_OK) return rc;
+    HIP_TRY(e);
     return VMHIP_OK;
 }
 
@@ -951,6 +963,7 @@ static int lookup_on_device(vmhip_batch* b, const vmhip_frame* frames, int32_t n
 int vmhip_batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int32_t classify) {
     if (!b) return fail(VMHIP_ERR_ARGUMENT, "batch_stage: null batch");
     if (b->in_flight) return fail(VMHIP_ERR_ARGUMENT, "batch_stage: a run of this batch is still in flight (vmhip_batch_wait first)");
+    if (b->fetching) return fail(VMHIP_ERR_ARGUMENT, "batch_stage: a fetch of this batch is still in flight (vmhip_batch_fetch_wait first)");
     if (!frames || n_frames <= 0) return fail(VMHIP_ERR_ARGUMENT, "stage: no frames");
     std::vector<vmhip_frame> patched;
     int rc = lookup_on_device(b, frames, n_frames, patched);
@@ -979,6 +992,7 @@ int vmhip_batch_export(vmhip_batch* b, int32_t edge_type, vmhip_lookup_export* p
     if (!b || !per_frame) return fail(VMHIP_ERR_ARGUMENT, "batch_export: null argument");
     if (b->frames.empty()) return fail(VMHIP_ERR_ARGUMENT, "batch_export: nothing staged");
     if (b->in_flight) return fail(VMHIP_ERR_ARGUMENT, "batch_export: a run of this batch is still in flight (vmhip_batch_wait first)");
+    if (b->fetching) return fail(VMHIP_ERR_ARGUMENT, "batch_export: a fetch of this batch is still in flight (vmhip_batch_fetch_wait first)");
     if (edge_type != VMHIP_EDGE_HARD && edge_type != VMHIP_EDGE_SAME) return fail(VMHIP_ERR_ARGUMENT, "batch_export: unknown edge type");
     const int n = int(b->frames.size());
     for (int f = 0; f < n; ++f) per_frame[f].n_points = b->frames[f].dev.n_cand; /* all of them, so that a caller can size */
@@ -1011,6 +1025,7 @@ int vmhip_batch_run_async(vmhip_batch* b) {
     if (!b) return fail(VMHIP_ERR_ARGUMENT, "batch_run_async: null batch");
     if (b->frames.empty()) return fail(VMHIP_ERR_ARGUMENT, "run: nothing staged");
     if (b->in_flight) return fail(VMHIP_ERR_ARGUMENT, "run: a run of this batch is still in flight (vmhip_batch_wait first)");
+    if (b->fetching) return fail(VMHIP_ERR_ARGUMENT, "run: a fetch of this batch is still in flight (vmhip_batch_fetch_wait first)");
     b->have_run = false;
     const int rc = batch_launch(b);
     if (rc == VMHIP_OK) b->in_flight = true;
@@ -1031,6 +1046,23 @@ int vmhip_batch_fetch(vmhip_batch* b, vmhip_result* results) {
     if (!b) return fail(VMHIP_ERR_ARGUMENT, "batch_fetch: null batch");
     return batch_fetch(b, results);
 }
+int vmhip_batch_fetch_async(vmhip_batch* b, vmhip_result* results) {
+    if (!b) return fail(VMHIP_ERR_ARGUMENT, "batch_fetch_async: null batch");
+    const int rc = batch_fetch_enqueue(b, results);
+    if (rc != VMHIP_OK) {
+        (void) hipStreamSynchronize(b->engine->stream); /* copies queued before the failure write into the caller's arrays */
+        return rc;
+    }
+    b->fetching = true;
+    return VMHIP_OK;
+}
+int vmhip_batch_fetch_wait(vmhip_batch* b) {
+    if (!b) return fail(VMHIP_ERR_ARGUMENT, "batch_fetch_wait: null batch");
+    if (!b->fetching) return fail(VMHIP_ERR_ARGUMENT, "batch_fetch_wait: no fetch in flight");
+    b->fetching = false;
+    HIP_TRY(hipStreamSynchronize(b->engine->stream));
+    return VMHIP_OK;
+}
 void* vmhip_host_alloc(size_t bytes) {
     void* p = nullptr;
     if (hipHostMalloc(&p, bytes ? bytes : 1, hipHostMallocDefault) != hipSuccess) {
@@ -1047,6 +1079,7 @@ int vmhip_batch_detect(vmhip_batch* b, int32_t class_index, float threshold, int
                        vmhip_detections* out) {
     if (!b || !out) return fail(VMHIP_ERR_ARGUMENT, "batch_detect: null argument");
     if (!b->have_run || !b->classify || !b->final_act) return fail(VMHIP_ERR_ARGUMENT, "batch_detect: no completed classifying run");
+    if (b->fetching) return fail(VMHIP_ERR_ARGUMENT, "batch_detect: a fetch of this batch is still in flight (vmhip_batch_fetch_wait first)");
     vmhip_engine* E = b->engine;
     const int C = E->n_classes;
     if (class_index < 0 || class_index >= C) return fail(VMHIP_ERR_ARGUMENT, "batch_detect: no such class");

@@ -217,10 +217,11 @@ class Engine:
                 out.append(dict(px=px, nb=nb, gidx=gidx, cls=cls))
         return out
 
-    def fetch_pinned(self):
+    def fetch_pinned(self, wait=True):
         """fetch() straight through the C ABI into page-locked arrays (vmhip_host_alloc), which the copies from the
         device reach at full PCIe speed and without a second copy on the host. The arrays belong to the engine and are
-        reused by the next call."""
+        reused by the next call. wait=False queues the copies and returns (vmhip_batch_fetch_async); fetch_wait() finishes
+        them."""
         lib = native.hip()
         counts = self.counts()
         n = len(counts)
@@ -240,8 +241,16 @@ class Engine:
                 self._pinned_results[i] = held
             raw[i] = native.Result(held["cap"], 0, _fp(held["px"]), _ip(held["gidx"]), _ip(held["nb"]), _fp(held["cls"]))
             out.append(dict(px=held["px"][:V], nb=held["nb"][:V + 1 if V else 0], gidx=held["gidx"][:V], cls=held["cls"][:V + 1 if V else 0]))
-        native.hip_check(lib.vmhip_batch_fetch(self.native_batch(), raw))
+        if wait:
+            native.hip_check(lib.vmhip_batch_fetch(self.native_batch(), raw))
+        else:
+            native.hip_check(lib.vmhip_batch_fetch_async(self.native_batch(), raw))
+            self._raw_results = raw  # the copies read this table's pointers only at the call, but keep it with the arrays
         return out
+
+    def fetch_wait(self):
+        """finishes fetch_pinned(wait=False): the arrays it returned are valid from here on"""
+        native.hip_check(native.hip().vmhip_batch_fetch_wait(self.native_batch()))
 
     def classify_batch(self, frames):
         self.stage(frames)

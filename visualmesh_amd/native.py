@@ -23,7 +23,7 @@ FP32, BF16 = 0, 1
 HIP_SYMBOLS = [
     "vmhip_last_error", "vmhip_engine_create", "vmhip_engine_destroy", "vmhip_engine_n_classes", "vmhip_mesh_upload",
     "vmhip_mesh_release", "vmhip_project", "vmhip_classify", "vmhip_classify_batch", "vmhip_batch_create",
-    "vmhip_batch_destroy", "vmhip_mesh_attach_tree", "vmhip_batch_stage", "vmhip_batch_ranges", "vmhip_batch_export", "vmhip_batch_run", "vmhip_batch_run_async", "vmhip_batch_wait", "vmhip_batch_counts", "vmhip_batch_fetch", "vmhip_batch_detect", "vmhip_host_alloc", "vmhip_host_free",
+    "vmhip_batch_destroy", "vmhip_mesh_attach_tree", "vmhip_batch_stage", "vmhip_batch_ranges", "vmhip_batch_export", "vmhip_batch_run", "vmhip_batch_run_async", "vmhip_batch_wait", "vmhip_batch_counts", "vmhip_batch_fetch", "vmhip_batch_fetch_async", "vmhip_batch_fetch_wait", "vmhip_batch_detect", "vmhip_host_alloc", "vmhip_host_free",
     "vmhip_batch_profile", "vmhip_batch_profile_read", "vmhip_selftest_libm", "vmhip_selftest_copy",
 ]
 
@@ -133,6 +133,8 @@ def hip():
     L.vmhip_batch_run.argtypes = [vp]
     L.vmhip_batch_counts.argtypes = [vp, C.POINTER(C.c_int32)]
     L.vmhip_batch_fetch.argtypes = [vp, C.POINTER(Result)]
+    L.vmhip_batch_fetch_async.argtypes = [vp, C.POINTER(Result)]
+    L.vmhip_batch_fetch_wait.argtypes = [vp]
     L.vmhip_batch_run_async.argtypes = [vp]
     L.vmhip_batch_export.argtypes = [vp, C.c_int32, C.POINTER(LookupExport)]
     L.vmhip_batch_ranges.argtypes = [vp, C.c_int32, C.POINTER(C.c_int32), C.c_int32]
