@@ -132,6 +132,7 @@ def main():
                     help="accepted for older command lines: the 1 GiB plain copy kernel (the practical ceiling of the memory "
                          "system and the dispatch of known size that memory counters are scaled by) runs unless --no-copy-probe")
     ap.add_argument("--no-copy-probe", action="store_true", help="skip the plain copy kernel")
+    ap.add_argument("--no-pcie", action="store_true", help="skip the PCIe-inclusive passes (stage + run + fetch through page-locked host memory)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (frames would shard across GPUs "
@@ -224,6 +225,27 @@ def main():
         nbytes = 1 << 30
         copy_gbs = 2 * nbytes / (native.copy_probe(nbytes, 5) * 1e-3) / 1e9
 
+    # PCIe-inclusive figure (never `value`): images in page-locked host memory -> stage + run + fetch of the whole
+    # classified mesh into page-locked host arrays, one engine, the three steps one after the other
+    pcie = None
+    if not args.no_pcie:
+        engine.profile(0)
+        held = []
+        for f in cfg.frames:
+            a = native.pinned_empty(f["image"].shape, f["image"].dtype)
+            a[...] = f["image"]
+            held.append(a)
+        pinned_frames = [dict(mesh=mesh, Hoc=f["Hoc"], lens=lens, image=a, fourcc=cfg.fourcc) for f, a in zip(cfg.frames, held)]
+        for _ in range(2):
+            engine.stage(pinned_frames), engine.run(), engine.fetch_pinned()
+        passes = 5
+        t0 = time.perf_counter()
+        for _ in range(passes):
+            engine.stage(pinned_frames), engine.run(), engine.fetch_pinned()
+        dt = (time.perf_counter() - t0) / passes
+        pcie = dict(ms_per_batch=dt * 1e3, nodes_per_s=nodes / dt, frames_per_s=len(frames) / dt,
+                    what="stage from page-locked images + run + fetch into page-locked arrays, one engine, serial")
+
     cpu = None
     if not args.no_cpu:
         threads = min(16, os.cpu_count() or 1, len(cfg.frames))
@@ -266,6 +288,7 @@ def main():
         "roofline": roofline,
         "cpu_baseline": cpu,
         "copy_kernel_GBps": copy_gbs,
+        "pcie_inclusive": pcie,
         "kernel_ms_per_step": dict(sorted(kernel_ms_per_step.items())),   # from the one fully profiled, untimed pass
         "conv_rooflines": conv_rooflines,
     }
