@@ -260,7 +260,19 @@ def main():
             passes = 1
             note = "all %d frames of the batch once, one frame per task" % len(cfg.frames)
         nps, fps, dt, kind = cpu_baseline(sample, threads, passes)
-        cpu = dict(value=nps, unit="nodes/s", cores=threads, kind=kind, frames_per_s=fps, seconds=dt, sample=note)
+        # the reference engine is single-threaded by design: the same engine on one thread, on a few frames
+        one = None
+        if args.config in (1, 2, 3):
+            few = wl.config(args.config, n_frames=min(3, len(cfg.frames)))
+            nps1, fps1, dt1, _ = cpu_baseline(few, 1, 1)
+            one = dict(value=nps1, frames_per_s=fps1, seconds=dt1, sample="the first %d frames of the batch once" % len(few.frames))
+        model = ""
+        try:
+            with open("/proc/cpuinfo") as f:
+                model = next((line.split(":", 1)[1].strip() for line in f if line.startswith("model name")), "")
+        except OSError:
+            pass
+        cpu = dict(value=nps, unit="nodes/s", cores=threads, kind=kind, cpu_model=model, one_thread=one, frames_per_s=fps, seconds=dt, sample=note)
 
     out = {
         "metric": "mesh nodes classified/sec",
