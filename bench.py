@@ -121,8 +121,10 @@ def cpu_baseline(cfg, threads, passes):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    # a pass takes about a millisecond and the GPU's clocks need some tens of them to settle: the defaults time one
+    # second of steady state (20 timed passes after 3 read 4-8 % slower)
+    ap.add_argument("--steps", type=int, default=None, help="timed passes (default 1000; 100 for configurations 4 and 5, whose pass takes 40-80 ms)")
+    ap.add_argument("--warmup", type=int, default=None, help="untimed passes before them (default 100; 10 for configurations 4 and 5)")
     ap.add_argument("--config", type=int, default=2, help="workload configuration 1..5 (default 2: batched 1280x1024)")
     ap.add_argument("--frames", type=int, default=None, help="frames per batch (default: the configuration's own)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
@@ -134,6 +136,9 @@ def main():
     ap.add_argument("--no-copy-probe", action="store_true", help="skip the plain copy kernel")
     ap.add_argument("--no-pcie", action="store_true", help="skip the PCIe-inclusive passes (stage + run + fetch through page-locked host memory)")
     args = ap.parse_args()
+    big = args.config in (4, 5)
+    args.steps = (100 if big else 1000) if args.steps is None else args.steps
+    args.warmup = (10 if big else 100) if args.warmup is None else args.warmup
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (frames would shard across GPUs "
               "without any exchange); run with --gpus 1", file=sys.stderr)
