@@ -163,7 +163,7 @@ struct vmhip_batch {
     size_t cand_total = 0, row_total = 0, lookup_total = 0;
 
     VmBatchDev dev{};
-    DevBuf d_frames, d_ranges, d_images, d_cand_px, d_cand_keep, d_tile_count, d_force_valid, d_force_keep, d_frame_V,
+    DevBuf d_frames, d_ranges, d_images, d_cand_px, d_cand_g, d_cand_keep, d_tile_count, d_force_valid, d_force_keep, d_frame_V,
       d_amb_list, d_row_px, d_row_gidx, d_row_nb, d_row_nbl, d_tile_halo, d_tile_desc, d_act[2], d_lookup, d_epoch, d_detect, d_detect_packed, d_lookup_ws, d_export;
     std::vector<std::vector<int32_t>> device_ranges; /* per frame: the ranges a lookup on the device produced */
     void* h_detect = nullptr; /* pinned landing area of vmhip_batch_detect */
@@ -179,7 +179,7 @@ struct vmhip_batch {
     int n_slots = 0;
 
     void release() {
-        DevBuf* all[] = {&d_frames, &d_ranges, &d_images, &d_cand_px, &d_cand_keep, &d_tile_count, &d_force_valid,
+        DevBuf* all[] = {&d_frames, &d_ranges, &d_images, &d_cand_px, &d_cand_g, &d_cand_keep, &d_tile_count, &d_force_valid,
                          &d_force_keep, &d_frame_V, &d_amb_list, &d_row_px, &d_row_gidx, &d_row_nb,
                          &d_row_nbl, &d_tile_halo, &d_tile_desc, &d_epoch,
                          &d_act[0], &d_act[1], &d_lookup, &d_detect, &d_detect_packed, &d_lookup_ws, &d_export};
@@ -277,6 +277,7 @@ int batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int
     HIP_TRY(b->d_ranges.reserve(sizeof(int32_t) * std::max<size_t>(range_ints, 1)));
     HIP_TRY(b->d_images.reserve(std::max<size_t>(image_bytes, 256)));
     HIP_TRY(b->d_cand_px.reserve(sizeof(float2) * std::max<size_t>(b->cand_total, 1)));
+    HIP_TRY(b->d_cand_g.reserve(4 * std::max<size_t>(b->cand_total, 1)));
     HIP_TRY(b->d_cand_keep.reserve(8 * std::max<size_t>(words, 1)));
     HIP_TRY(b->d_tile_count.reserve(4 * std::max<size_t>(cand_tiles, 1)));
     HIP_TRY(b->d_force_valid.reserve(8 * std::max<size_t>(words, 1)));
@@ -360,6 +361,7 @@ int batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int
     D.n_cand_tiles = int32_t(cand_tiles);
     D.n_row_tiles = int32_t(row_tiles);
     D.cand_px = b->d_cand_px.as<float2>();
+    D.cand_g = b->d_cand_g.as<int32_t>();
     D.cand_keep = b->d_cand_keep.as<uint64_t>();
     D.tile_count = b->d_tile_count.as<int32_t>();
     D.frame_V = b->d_frame_V.as<int32_t>();

@@ -383,6 +383,7 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_project_kernel(VmBatchDev B) {
             if (slot < VMHIP_AMB_CAP) B.amb_list[(size_t) f * VMHIP_AMB_CAP + slot] = make_int2(p, keep ? 1 : 0);
         }
         B.cand_px[(size_t) F.cand_base + p] = px;
+        B.cand_g[(size_t) F.cand_base + p] = g;
     }
 
     const uint64_t mask = __ballot(keep);
@@ -556,7 +557,7 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_compact_kernel(VmBatchDev B, fl
     if ((mask >> lane) & 1ull) {
         const int local = base + before + __popcll(mask & ((1ull << lane) - 1ull));
         const size_t row = (size_t) F.row_base + local;
-        const int g = cand_to_global(F, p);
+        const int g = B.cand_g[(size_t) F.cand_base + p];
         const float2 px = B.cand_px[(size_t) F.cand_base + p];
         B.row_px[row] = px;
         B.row_gidx[row] = g;

@@ -83,6 +83,7 @@ struct VmBatchDev {
     uint32_t* epoch;      /* device word: the run's stamp for the reverse lookup; the reset kernel increments it */
     /* candidate space */
     float2* cand_px;
+    int32_t* cand_g;      /* the candidate's node (global index), worked out once by the projection */
     uint64_t* cand_keep;  /* one 64-bit mask per wave of candidates */
     int32_t* tile_count;  /* [n_cand_tiles] kept candidates per tile */
     /* per frame */
