@@ -628,12 +628,29 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_neighbourhood_kernel(VmBatchDev
         for (int it = threadIdx.x; it < n_items; it += VMHIP_TILE) resolve(it);
         return;
     }
+    /* the three dependent reads of an item (row -> node, node -> neighbour node, neighbour node -> its row), level by
+     * level over all of the thread's items, so that the items' reads are in flight together and no store stands
+     * between them */
+    int item_row[MAX_ITEMS], item_slot[MAX_ITEMS], node[MAX_ITEMS];
+#pragma unroll
+    for (int k = 0; k < MAX_ITEMS; ++k) {
+        const int it = threadIdx.x + k * VMHIP_TILE;
+        item_row[k] = row0 + it / nn;
+        item_slot[k] = it - (it / nn) * nn;
+        node[k] = (it < n_items && item_row[k] < V) ? B.row_gidx[(size_t) F.row_base + item_row[k]] : -1;
+    }
+#pragma unroll
+    for (int k = 0; k < MAX_ITEMS; ++k) node[k] = node[k] >= 0 ? min(F.nbr[(size_t) node[k] * nn + item_slot[k]], F.n_nodes) : -1;
+    uint2 stamp[MAX_ITEMS];
+#pragma unroll
+    for (int k = 0; k < MAX_ITEMS; ++k) stamp[k] = node[k] >= 0 ? F.r_lookup[node[k]] : make_uint2(epoch + 1u, 0u);
 #pragma unroll
     for (int k = 0; k < MAX_ITEMS; ++k) {
         const int it = threadIdx.x + k * VMHIP_TILE;
         outs[k] = -1;
         if (it < n_items) {
-            const int out = resolve(it);
+            const int out = stamp[k].x == epoch ? (int) stamp[k].y : V;
+            B.row_nb[((size_t) F.row_base + item_row[k]) * B.nb_stride + item_slot[k]] = out;
             outs[k] = out;
             if (out < row0 || out >= row0 + VMHIP_TILE) {
                 uint32_t slot = hash((uint32_t) out);
