@@ -28,8 +28,8 @@ BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix
 # HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, keyed by
 # (workload, kernel); filled in from the summaries under profiles/ (None = not measured).
 MEASURED_TRAFFIC = {
-    # profiles/conv_flow_32x32_config2.md: (2.0 * 76486.7 + 131194.1) KiB per launch
-    ("cfg2", "conv_flow_32x32s7"): int((2.0 * 76486.7 + 131194.1) * 1024),
+    # profiles/conv_flow_32x32_config2.md: (2.0 * 76506.2 + 131194.2) KiB per launch
+    ("cfg2", "conv_flow_32x32s7"): int((2.0 * 76506.2 + 131194.2) * 1024),
 }
 
 
