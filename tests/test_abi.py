@@ -43,3 +43,19 @@ def test_struct_layouts_match_the_header():
     # vmhip_detections: four int32, then seven pointers
     assert ctypes.sizeof(native.Detections) == 72
     assert native.Detections.node.offset == 16 and native.Detections.cluster_centre.offset == 64
+
+
+def build_integration_snippet(directory):
+    """the reference's call sites with the engine type changed, compiled as C++14 against the host headers and linked
+    with the HIP library; returns the executable"""
+    import subprocess
+    exe = os.path.join(str(directory), "integration_snippet")
+    lib_dir = os.path.dirname(native.HIP_LIB)
+    subprocess.run(["g++", "-std=c++14", "-O1", "-Wall", "-Wextra", "-Werror", "-I" + os.path.join(ROOT, "visualmesh_amd", "cpp"),
+                    "-I" + os.path.join(ROOT, "include"), os.path.join(ROOT, "tests", "native", "integration_snippet.cpp"),
+                    "-L" + lib_dir, "-lvisualmesh_hip", "-Wl,-rpath," + lib_dir, "-o", exe], check=True)
+    return exe
+
+
+def test_reference_call_sites_compile_against_the_host_headers(tmp_path):
+    assert os.path.exists(build_integration_snippet(tmp_path))

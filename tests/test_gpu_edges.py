@@ -278,3 +278,13 @@ def test_full_size_batch_properties(oracle, index):
         for key in ("px", "nb", "gidx"):
             assert np.array_equal(alone[key], first[i][key]), "frame %d: %s depends on the batch" % (i, key)
         assert np.abs(alone["cls"] - first[i]["cls"]).max() <= 1e-6, "frame %d: probabilities depend on the batch" % i
+
+
+def test_cpp_call_sites_run(tmp_path):
+    """tests/native/integration_snippet.cpp: the reference's call sites (and the batch calls this engine adds) in C++,
+    without Python in between; the program checks that its calls agree with each other."""
+    import subprocess
+    from test_abi import build_integration_snippet
+    out = subprocess.run([build_integration_snippet(tmp_path)], capture_output=True, text=True, timeout=120)
+    print(out.stdout, out.stderr, flush=True)
+    assert out.returncode == 0 and out.stdout.strip().endswith("ok"), out.stdout + out.stderr
