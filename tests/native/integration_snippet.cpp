@@ -48,13 +48,34 @@ int main() {
     engine.run_async();
     engine.wait();
     auto fetched = engine.fetch<visualmesh::model::Ring6>();
+    // results into arrays of the caller's (page-locked ones make the copies asynchronous), in one call or in two halves
+    const std::vector<int32_t> visible = engine.visible_counts();
+    const int classes = 4;  // an empty network returns the four sampled channels
+    std::vector<std::vector<float>> px(frames.size()), cls(frames.size());
+    std::vector<std::vector<int32_t>> gidx(frames.size()), nb(frames.size());
+    std::vector<vmhip_result> into(frames.size());
+    for (size_t i = 0; i < frames.size(); ++i) {
+        px[i].resize(size_t(visible[i]) * 2), gidx[i].resize(visible[i]), nb[i].resize((size_t(visible[i]) + 1) * 6),
+          cls[i].resize((size_t(visible[i]) + 1) * classes);
+        into[i] = vmhip_result{visible[i], 0, px[i].data(), gidx[i].data(), nb[i].data(), cls[i].data()};
+    }
+    engine.fetch_into(into);
+    const bool into_same = gidx[1] == fetched[1].global_indices;
+    engine.fetch_into_async(into);
+    engine.fetch_wait();
+    engine.set_device_lookup(true);
+    engine.stage(frames);
+    engine.run();
+    const bool device_lookup_same = engine.visible_counts() == visible;
+    engine.set_device_lookup(false);
     std::printf("projected %zu %zu classified %zu by_height %zu batch %zu %zu detections %zu graph %zu fetched %zu\n",
                 projected.global_indices.size(), projected_too.global_indices.size(), classified.global_indices.size(),
                 by_height.global_indices.size(), results.size(), results[1].global_indices.size(), detections.size(),
                 graph[0].vectors.size(), fetched[0].global_indices.size());
     const bool same = projected.global_indices == projected_too.global_indices && projected.global_indices == classified.global_indices
                       && classified.global_indices == results[1].global_indices && classified.global_indices == fetched[0].global_indices
-                      && graph[0].vectors.size() >= projected.global_indices.size() && !projected.global_indices.empty();
+                      && graph[0].vectors.size() >= projected.global_indices.size() && !projected.global_indices.empty() && into_same
+                      && device_lookup_same;
     std::printf(same ? "ok\n" : "MISMATCH\n");
     return same ? 0 : 1;
 }
