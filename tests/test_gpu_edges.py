@@ -288,3 +288,28 @@ def test_cpp_call_sites_run(tmp_path):
     out = subprocess.run([build_integration_snippet(tmp_path)], capture_output=True, text=True, timeout=120)
     print(out.stdout, out.stderr, flush=True)
     assert out.returncode == 0 and out.stdout.strip().endswith("ok"), out.stdout + out.stderr
+
+
+@pytest.mark.parametrize("seed", [7, 99, 2024])
+def test_other_seeds(oracle, seed):
+    """The configurations' own seeds fix images, poses and weights; configuration 2 (batched, all kernel families) and
+    configuration 3 (NMGrid8, Bayer, rectilinear) drawn from other seeds must agree with the oracle just the same."""
+    for index, n_frames in ((2, 3), (3, 1)):
+        cfg = wl.config(index, n_frames=n_frames, seed=seed)
+        o_lens, e_lens = vmo.make_lens(*cfg.lens_tuple()), native.make_lens(*cfg.lens_tuple())
+        if cfg.visualmesh is None:
+            args = (cfg.model, cfg.shape, cfg.radius, cfg.mesh_h, cfg.k, min(cfg.max_distance, 3.0))
+            o_mesh, e_mesh = oracle.mesh(*args), eng.Mesh(*args)
+            pick = lambda m, H: m
+        else:
+            v = cfg.visualmesh
+            args = (cfg.model, cfg.shape, cfg.radius, v["min_h"], v["max_h"], cfg.k, v["max_error"], cfg.max_distance)
+            o_mesh, e_mesh = oracle.visualmesh(*args), eng.VisualMesh(*args)
+            pick = lambda m, H: m.height(float(H[2][3]))
+        engine = eng.Engine(cfg.network, cfg.model)
+        results = engine.classify_batch([dict(mesh=e_mesh, Hoc=f["Hoc"], lens=e_lens, image=f["image"], fourcc=cfg.fourcc) for f in cfg.frames])
+        net = vmo.Network(cfg.network)
+        for i, f in enumerate(cfg.frames):
+            want = pick(o_mesh, f["Hoc"]).classify(f["Hoc"], o_lens, f["image"], cfg.fourcc, net)
+            assert len(want["gidx"]) > 1000
+            assert_classification_parity(results[i], want, PROB_TOL, "cfg%d seed %d frame %d" % (index, seed, i))
