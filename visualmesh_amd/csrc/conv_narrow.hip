@@ -62,16 +62,20 @@ __device__ __forceinline__ uint32_t nbl_entry(const v4u& t, int k) {
     return (k & 1) ? (w >> 16) : (w & 0xffffu);
 }
 
-/* LDS rows: 64-byte rows (C_IN = 16) have their 16-byte pieces XORed with the low two bits of the row number, so
- * that 64 lanes reading piece c of 64 different rows spread over all banks; other widths get one piece of padding,
- * which rotates consecutive rows through the banks by itself */
+/* LDS rows: a lane reads piece c of its own source row, all lanes of an instruction the same c. A 64-byte row
+ * (C_IN = 16) spans 16 of the 64 banks, so row r, piece c lies in the four banks 16 (r % 4) + 4 c: with the pieces
+ * left where they are, sixteen lanes would meet in four groups of banks. The pieces are therefore XORed with bits
+ * 2 and 3 of the row number: sixteen consecutive rows then reach sixteen different groups (XORing with bits 0 and
+ * 1, which already choose the quarter of the banks, leaves the four-way conflict: 35 us against 31 us on 16 -> 3).
+ * Other widths get one piece of padding, which rotates consecutive rows through the banks by itself. */
 __host__ __device__ constexpr bool row_swizzled(int c_in) { return c_in == 16; }
 __host__ __device__ constexpr int row_stride(int c_in) { return c_in == 16 ? c_in : c_in + 4; }
 constexpr int HALO = VMHIP_HALO_MAX;
 constexpr int NW = 4; /* 64 rows per wave */
-/* Row buffers per block. Two (tile t+1 lands while t is worked on, two blocks of four waves per CU) measured
- * faster than one (four blocks per CU, each waiting for its own next tile): 39 us against 43 us on 16 -> 3. */
-constexpr int NBUFS = 2;
+/* Row buffers per block. One, with up to four blocks of four waves sharing a CU (each meets its next tile at the top
+ * of its loop while the others work), measured faster than two buffers and two blocks per CU: 28 us against 31 us
+ * on 16 -> 3. */
+constexpr int NBUFS = 1;
 __host__ __device__ constexpr size_t narrow_lds_bytes(int c_in, int slots) {
     return (size_t(slots) * c_in * 4 + 4 + NBUFS * size_t(VMHIP_TILE + HALO) * row_stride(c_in)) * 4;
 }
@@ -146,7 +150,7 @@ __global__ __launch_bounds__(NW * 64) void vm_conv_narrow_kernel(VmBatchDev B, V
             if (k * NT + wave * 64 >= PIECES) continue; /* wave-uniform; only in a last, partial round */
             const int p = threadIdx.x + k * NT;
             const int row_l = p / RSP, cp = p - row_l * RSP;
-            const int c = SWZ ? (cp ^ (row_l & 3)) : cp;
+            const int c = SWZ ? (cp ^ ((row_l >> 2) & 3)) : cp;
             uint32_t off;
             if ((k + 1) * NT <= MAIN_PIECES) {
                 off = (uint32_t) ((d.x + row_l) * Q4 + c) * 16u;
@@ -227,7 +231,7 @@ __global__ __launch_bounds__(NW * 64) void vm_conv_narrow_kernel(VmBatchDev B, V
 #pragma unroll
                 for (int k4 = 0; k4 < Q4; ++k4) {
                     float t[4];
-                    load_floats<4>(rows + at * RS + ((SWZ ? (k4 ^ (int) (at & 3)) : k4) << 2), t);
+                    load_floats<4>(rows + at * RS + ((SWZ ? (k4 ^ (int) ((at >> 2) & 3)) : k4) << 2), t);
 #pragma unroll
                     for (int e = 0; e < 4; ++e) x[k4 * 4 + e] = t[e];
                 }
