@@ -205,6 +205,36 @@ int vmhip_batch_fetch(vmhip_batch* batch, vmhip_result* results);
 int vmhip_batch_fetch_async(vmhip_batch* batch, vmhip_result* results);
 int vmhip_batch_fetch_wait(vmhip_batch* batch);
 
+/* vmhip_project for callers that cannot allocate: code under HIP graph capture, serving loops that must not call
+ * hipMalloc, harnesses that forbid it. No counterpart in the reference. The call only launches kernels on hip_stream
+ * (a hipStream_t, NULL = the default stream) and returns without waiting: no allocation, no copy, no wait.
+ * Every pointer below is read or written by the device, so it must be device memory or memory from vmhip_host_alloc.
+ *   ranges        n_ranges pairs (first, one-past-last) as Mesh::lookup returns them
+ *   n_candidates  the sum of the range lengths (the launch grids are sized from it); capacity >= n_candidates
+ *   n_visible     one word: the visible count, or -1 if the device found the pairs not ascending, not disjoint, outside
+ *                 the mesh or not summing to n_candidates (then nothing else is written)
+ *   pixel_coordinates [capacity][2], global_indices [capacity], neighbourhood [capacity+1][n_neighbours]
+ *                 as in vmhip_result; all four are required. With visible nodes the null row follows them.
+ * The workspace is one array of fixed size inside the library (15.5 MB per device, held until the process ends), so
+ * sizes are limited as below and VMHIP_ERR_CAPACITY says which limit a call exceeds; calls that overlap on one
+ * device race on that array, calls on one stream do not. The on-screen decisions are the device's own: they equal the
+ * host's bit for bit where the host's C library is the one the device arithmetic reproduces (glibc's), and the
+ * re-decision of near-edge nodes on the host that vmhip_project adds for other C libraries is not made here. */
+enum {
+    VMHIP_NOALLOC_MAX_CANDIDATES = 524288,
+    VMHIP_NOALLOC_MAX_NODES = 1048576,
+    VMHIP_NOALLOC_MAX_RANGES = 65536
+};
+typedef struct vmhip_projection_device {
+    int32_t capacity;
+    int32_t* n_visible;
+    float* pixel_coordinates;
+    int32_t* global_indices;
+    int32_t* neighbourhood;
+} vmhip_projection_device;
+int vmhip_project_noalloc(const vmhip_mesh* mesh, const float* Rco, const vmhip_lens* lens, const int32_t* ranges,
+                          int32_t n_ranges, int32_t n_candidates, const vmhip_projection_device* out, void* hip_stream);
+
 /* What a consumer of the classified mesh does first, done on the device so that only detections cross PCIe. No
  * counterpart inside the reference's engines: its consumers walk the whole ClassifiedMesh on the host
  * (example/draw.hpp:41-59), over the neighbourhood table of engine/cpu/engine.hpp:113-129.

@@ -66,6 +66,7 @@ def build_hip(force=False):
         ("conv_flow.hip", HIP_FLAGS),
         ("conv_narrow.hip", HIP_FLAGS),
         ("detect.hip", HIP_FLAGS),
+        ("noalloc.hip", HIP_FLAGS),
         ("api.hip", HIP_FLAGS),
     ]
     for name, flags in units:

@@ -90,15 +90,6 @@ inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 }  // namespace
 
-struct vmhip_mesh {
-    float* d_rays = nullptr;
-    int32_t* d_nbr = nullptr;
-    int32_t n_nodes = 0, nn = 0;
-    std::vector<float> h_rays; /* host copy for the re-decision of ambiguous candidates */
-    VmTreeElement* d_tree = nullptr; /* the cone tree, for lookups on the device (vmhip_mesh_attach_tree) */
-    int32_t n_elements = 0;
-};
-
 struct HostLayer {
     int32_t c_in, c_out, slots, activation;
     float* d_w = nullptr;
@@ -653,6 +644,8 @@ int ensure_scratch(vmhip_engine* E) {
 
 }  // namespace
 
+int vm_set_error(int code, const char* message) { return fail(code, message); }
+
 extern "C" {
 
 const char* vmhip_last_error(void) { return g_error.c_str(); }
@@ -812,6 +805,12 @@ int vmhip_mesh_upload(const float* rays, const int32_t* neighbours, int32_t n_no
     vmhip_mesh* M = new vmhip_mesh();
     M->n_nodes = n_nodes;
     M->nn = n_neighbours;
+    /* the one place every caller of vmhip_project_noalloc has passed through on its device: resolve that entry
+     * point's workspace here, so that the entry point itself has nothing left to set up */
+    if (hipGetDevice(&M->device) != hipSuccess || vm_noalloc_setup() != hipSuccess) {
+        delete M;
+        return fail(VMHIP_ERR_HIP, "mesh_upload: no usable device");
+    }
     M->h_rays.assign(rays, rays + size_t(n_nodes) * 3);
     const size_t rb = sizeof(float) * 3 * size_t(n_nodes), nb = sizeof(int32_t) * size_t(n_nodes) * n_neighbours;
     if (hipMalloc(&M->d_rays, rb) != hipSuccess || hipMalloc(&M->d_nbr, nb) != hipSuccess

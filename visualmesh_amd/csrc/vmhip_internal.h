@@ -236,4 +236,23 @@ int vm_launch_conv_narrow(const VmBatchDev& B, const VmLayerDev& L, const float*
 
 #include "host_project.h"
 
+#include <vector>
+
+/* a mesh on the device (api.hip: vmhip_mesh_upload) */
+struct vmhip_mesh {
+    float* d_rays = nullptr;
+    int32_t* d_nbr = nullptr;
+    int32_t n_nodes = 0, nn = 0;
+    int device = 0;            /* the device that holds it */
+    std::vector<float> h_rays; /* host copy for the re-decision of ambiguous candidates */
+    VmTreeElement* d_tree = nullptr; /* the cone tree, for lookups on the device (vmhip_mesh_attach_tree) */
+    int32_t n_elements = 0;
+};
+
+/* noalloc.hip: the entry point that allocates nothing. vm_noalloc_setup finds the current device's copy of that file's
+ * scratch array (once per device; mesh uploads call it, so the entry point itself finds it done); vm_set_error records
+ * the calling thread's message for vmhip_last_error and returns code. */
+hipError_t vm_noalloc_setup(void);
+int vm_set_error(int code, const char* message);
+
 #endif

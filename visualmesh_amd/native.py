@@ -24,7 +24,7 @@ HIP_SYMBOLS = [
     "vmhip_last_error", "vmhip_engine_create", "vmhip_engine_destroy", "vmhip_engine_n_classes", "vmhip_mesh_upload",
     "vmhip_mesh_release", "vmhip_project", "vmhip_classify", "vmhip_classify_batch", "vmhip_batch_create",
     "vmhip_batch_destroy", "vmhip_mesh_attach_tree", "vmhip_batch_stage", "vmhip_batch_ranges", "vmhip_batch_export", "vmhip_batch_run", "vmhip_batch_run_async", "vmhip_batch_wait", "vmhip_batch_counts", "vmhip_batch_fetch", "vmhip_batch_fetch_async", "vmhip_batch_fetch_wait", "vmhip_batch_detect", "vmhip_host_alloc", "vmhip_host_free",
-    "vmhip_batch_profile", "vmhip_batch_profile_read", "vmhip_selftest_libm", "vmhip_selftest_copy",
+    "vmhip_batch_profile", "vmhip_batch_profile_read", "vmhip_selftest_libm", "vmhip_selftest_copy", "vmhip_project_noalloc",
 ]
 
 
@@ -67,6 +67,12 @@ class Detections(C.Structure):
                 ("node", C.POINTER(C.c_int32)), ("pixel", C.POINTER(C.c_float)), ("probability", C.POINTER(C.c_float)),
                 ("cluster", C.POINTER(C.c_int32)), ("cluster_size", C.POINTER(C.c_int32)), ("cluster_box", C.POINTER(C.c_float)),
                 ("cluster_centre", C.POINTER(C.c_float))]
+
+
+class ProjectionDevice(C.Structure):
+    """vmhip_projection_device: where vmhip_project_noalloc writes; every pointer must be addressable by the device"""
+    _fields_ = [("capacity", C.c_int32), ("n_visible", C.POINTER(C.c_int32)), ("pixel_coordinates", C.POINTER(C.c_float)),
+                ("global_indices", C.POINTER(C.c_int32)), ("neighbourhood", C.POINTER(C.c_int32))]
 
 
 class Result(C.Structure):
@@ -150,6 +156,8 @@ def hip():
                                            C.POINTER(C.c_int64)]
     L.vmhip_selftest_libm.argtypes = [C.c_int32, C.POINTER(C.c_float), C.POINTER(C.c_float), C.c_int32]
     L.vmhip_selftest_copy.argtypes = [C.c_int64, C.c_int32, C.POINTER(C.c_float)]
+    L.vmhip_project_noalloc.argtypes = [vp, C.POINTER(C.c_float), C.POINTER(Lens), C.POINTER(C.c_int32), C.c_int32, C.c_int32,
+                                        C.POINTER(ProjectionDevice), vp]
     _hip = L
     return L
 
