@@ -273,6 +273,23 @@ int vmhip_batch_profile(vmhip_batch* batch, int32_t enable);
 int vmhip_batch_profile_read(vmhip_batch* batch, int32_t max_slots, int32_t* n_slots, const char** names,
                              float* milliseconds, int64_t* units);
 
+/* Test knobs, process wide, with no counterpart in the reference. They exist so that tests can drive paths that never
+ * run on a healthy system, with every kernel still ending normally; production code has no use for them.
+ *   VMHIP_DEBUG_FLOW_POLL_LIMIT   polls a wave of the barrier-free convolution kernel waits for a tile before it gives
+ *                                 up and the run fails (takes effect at once; <= 0 restores the default)
+ *   VMHIP_DEBUG_PROJECTION_ERROR  pixels added to both coordinates of every projected node on the device, as if the
+ *                                 device's lens arithmetic differed from the host's: the host's re-decision of near-edge
+ *                                 nodes must then overrule the device (read when a batch is staged; 0 = off)
+ *   VMHIP_DEBUG_EDGE_BAND         width in pixels of the band along the screen edges inside which nodes are re-decided
+ *                                 on the host (read when a batch is staged; <= 0 restores the default, 1/64) */
+enum { VMHIP_DEBUG_FLOW_POLL_LIMIT = 0, VMHIP_DEBUG_PROJECTION_ERROR = 1, VMHIP_DEBUG_EDGE_BAND = 2 };
+int vmhip_debug_set(int32_t what, double value);
+/* What the edge guard did in the runs of a batch since it was staged: near-edge nodes the device listed (summed over
+ * frames and passes), the most it listed for one frame in one pass, device decisions the host overruled, passes
+ * repeated because of that. The last two are zero on a host whose C library is the one the device arithmetic
+ * reproduces. Any pointer may be NULL. */
+int vmhip_batch_guard_stats(const vmhip_batch* batch, int64_t* listed, int64_t* most_listed, int64_t* overruled, int64_t* reruns);
+
 /* Diagnostic with no counterpart in the reference: evaluates on the device, for n floats, the library's
  * own acosf (which = 0), sinf (1), tanf (2) or sqrtf (3) - the functions the lens projection is built from
  * and which must return the host C library's bits. x and y are host buffers. */

@@ -68,6 +68,18 @@ int main() {
     engine.run();
     const bool device_lookup_same = engine.visible_counts() == visible;
     engine.set_device_lookup(false);
+    // an engine moved while a batch is staged: the staged frames' mesh stays pinned in the moved-to engine's cache (the
+    // limit below is smaller than any mesh, so everything that is not pinned goes when another mesh comes in), and the
+    // cache's accounting travels along
+    engine.set_cache_limit(1);
+    engine.stage(frames);
+    const size_t bytes_before = engine.cache_bytes();
+    visualmesh::engine::hip::Engine<Scalar> moved(std::move(engine));
+    const bool accounting_moved = moved.cache_bytes() == bytes_before && bytes_before > 0 && engine.cache_bytes() == 0;
+    auto other_mesh = moved(heights, Hoc, lens);  // uploads the height's mesh and trims the cache
+    moved.run();                                  // runs on the staged mesh, which must still be on the device
+    const bool moved_same = moved.visible_counts() == visible && moved.cached_meshes() >= 1 && accounting_moved
+                            && other_mesh.global_indices == by_height.global_indices;
     std::printf("projected %zu %zu classified %zu by_height %zu batch %zu %zu detections %zu graph %zu fetched %zu\n",
                 projected.global_indices.size(), projected_too.global_indices.size(), classified.global_indices.size(),
                 by_height.global_indices.size(), results.size(), results[1].global_indices.size(), detections.size(),
@@ -75,7 +87,7 @@ int main() {
     const bool same = projected.global_indices == projected_too.global_indices && projected.global_indices == classified.global_indices
                       && classified.global_indices == results[1].global_indices && classified.global_indices == fetched[0].global_indices
                       && graph[0].vectors.size() >= projected.global_indices.size() && !projected.global_indices.empty() && into_same
-                      && device_lookup_same;
+                      && device_lookup_same && moved_same;
     std::printf(same ? "ok\n" : "MISMATCH\n");
     return same ? 0 : 1;
 }

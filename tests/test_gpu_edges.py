@@ -7,7 +7,7 @@ import math
 import numpy as np
 import pytest
 
-from helpers import PROB_TOL, assert_classification_parity, assert_projection_parity
+from helpers import PROB_TOL, assert_classification_parity, assert_projection_parity, lens_pair, meshes_for, pick
 from oracle import vmo
 from visualmesh_amd import engine as eng
 from visualmesh_amd import native
@@ -103,6 +103,8 @@ def test_frames_that_see_nothing(oracle):
     assert len(o_mesh.project(up, o_lens)["gidx"]) == 0
     got = engine(e_mesh, up, e_lens)
     assert len(got["gidx"]) == 0 and len(got["px"]) == 0
+    # an empty projection keeps its null row, pointing at itself (engine/cpu/engine.hpp:127-143 with no points)
+    assert np.array_equal(got["nb"], o_mesh.project(up, o_lens)["nb"]) and got["nb"].shape == (1, 6)
     got = engine(e_mesh, up, e_lens, image, wl.fourcc("RGBA"))
     assert len(got["gidx"]) == 0 and got["cls"].shape[0] == 0
     poses = [up, down, up, up, down, up]
@@ -114,9 +116,24 @@ def test_frames_that_see_nothing(oracle):
             assert len(r["gidx"]) == 0 and r["cls"].shape[0] == 0
         else:
             assert_classification_parity(r, want, PROB_TOL, "the frame beside the empty ones")
+    # detections on the device for that batch: the frames that see nothing have none, whatever an earlier batch left in
+    # the workspace where their counts live (staged after an ordinary batch, so those words hold old counts)
+    ordinary = [dict(mesh=e_mesh, Hoc=down, lens=e_lens, image=image, fourcc=wl.fourcc("RGBA"))] * len(poses)
+    engine.classify_batch(ordinary)
+    results = engine.classify_batch([dict(mesh=e_mesh, Hoc=H, lens=e_lens, image=image, fourcc=wl.fourcc("RGBA")) for H in poses])
+    found = engine.detect(1, 0.0, arg_max_only=False, clusters=True)
+    for H, r, d in zip(poses, results, found):
+        if H is up:
+            assert len(d["node"]) == 0 and len(d["cluster_size"]) == 0
+        else:
+            # threshold 0: every visible node is a detection, in order
+            assert np.array_equal(d["node"], r["gidx"]) and np.array_equal(d["pixel"], r["px"])
+            assert np.array_equal(d["probability"], r["cls"][:len(r["gidx"]), 1])
+            assert d["cluster_size"].sum() == len(r["gidx"])
     # a batch of nothing but empty frames
     results = engine.classify_batch([dict(mesh=e_mesh, Hoc=up, lens=e_lens, image=image, fourcc=wl.fourcc("RGBA"))] * 2)
     assert all(len(r["gidx"]) == 0 for r in results)
+    assert all(len(d["node"]) == 0 for d in engine.detect(0, 0.0))
 
 
 def test_ragged_batch(oracle):
@@ -313,3 +330,60 @@ def test_other_seeds(oracle, seed):
             want = pick(o_mesh, f["Hoc"]).classify(f["Hoc"], o_lens, f["image"], cfg.fourcc, net)
             assert len(want["gidx"]) > 1000
             assert_classification_parity(results[i], want, PROB_TOL, "cfg%d seed %d frame %d" % (index, seed, i))
+
+
+@pytest.mark.parametrize("band,path", [(0.25, "head"), (6.0, "list"), (100.0, "frame")])
+def test_edge_guard_overrules_a_device_whose_arithmetic_differs(oracle, band, path):
+    """The guard for hosts whose C library is not the one the device arithmetic reproduces: nodes within a band along
+    the screen edges are listed by the device and re-decided by the host; where the host disagrees its decision is
+    forced and the pass repeated. With the engine's own libm both sides agree to the bit, so the test makes the device
+    differ: 0.2 px added to every projected coordinate on the device (a test knob of the library; the band, 1/64 px by
+    default, is widened to more than that by a second knob). The visible set and
+    the neighbourhood table must still be the oracle's bit for bit, at least one decision must have been overruled and
+    the pass repeated. The band's width drives the three ways the list reaches the host: with the per-run download
+    (at most 64 entries per frame), by a second download (more than 64), and - the list overflowing at 2048 - the
+    whole frame decided on the host. Every kernel ends normally in all of them."""
+    cfg = wl.config(2, n_frames=2)
+    o_lens, e_lens = lens_pair(cfg)
+    o_mesh, e_mesh = meshes_for(cfg, oracle)
+    engine = eng.Engine(cfg.network, cfg.model)
+    frames = [dict(mesh=e_mesh, Hoc=f["Hoc"], lens=e_lens, image=f["image"], fourcc=cfg.fourcc) for f in cfg.frames]
+    lib = native.hip()
+    error = 0.2
+    native.hip_check(lib.vmhip_debug_set(native.DEBUG_PROJECTION_ERROR, error))
+    native.hip_check(lib.vmhip_debug_set(native.DEBUG_EDGE_BAND, band))
+    try:
+        engine.stage(frames)
+        engine.run()
+        results = engine.fetch()
+        stats = native.guard_stats(engine.native_batch())
+        engine.run()  # the forced decisions stay in place: a further run has nothing left to overrule
+        again = engine.fetch()
+        stats_again = native.guard_stats(engine.native_batch())
+    finally:
+        native.hip_check(lib.vmhip_debug_set(native.DEBUG_PROJECTION_ERROR, 0.0))
+        native.hip_check(lib.vmhip_debug_set(native.DEBUG_EDGE_BAND, 0.0))
+    print(path, stats, flush=True)
+    assert stats["overruled"] >= 1 and stats["reruns"] >= 1
+    assert stats_again["overruled"] == stats["overruled"] and stats_again["reruns"] == stats["reruns"]
+    if path == "head":
+        assert 0 < stats["most_listed"] <= 64
+    elif path == "list":
+        assert 64 < stats["most_listed"] <= 2048
+    else:
+        assert stats["most_listed"] > 2048
+    for i, f in enumerate(cfg.frames):
+        want = pick(o_mesh, f["Hoc"]).project(f["Hoc"], o_lens)
+        for got in (results[i], again[i]):
+            assert np.array_equal(got["gidx"], want["gidx"]), "frame %d: visible set differs" % i
+            assert np.array_equal(got["nb"], want["nb"]), "frame %d: neighbourhood differs" % i
+            assert np.abs(got["px"] - (want["px"] + np.float32(error))).max() <= 1e-3
+    # and without the knob the same engine agrees with the oracle again, nothing listed is overruled
+    engine.stage(frames)
+    engine.run()
+    clean = engine.fetch()
+    stats = native.guard_stats(engine.native_batch())
+    assert stats["overruled"] == 0 and stats["reruns"] == 0
+    for i, f in enumerate(cfg.frames):
+        want = pick(o_mesh, f["Hoc"]).project(f["Hoc"], o_lens)
+        assert_projection_parity(clean[i], want, "frame %d without the knob" % i)

@@ -451,12 +451,15 @@ def test_a_wait_that_runs_out_fails_the_run(oracle):
     frames = [dict(mesh=e_mesh, Hoc=f["Hoc"], lens=e_lens, image=f["image"], fourcc=cfg.fourcc)]
     engine.stage(frames)
     lib = native.hip()
-    lib.vm_flow_set_poll_limit(1)
+    native.hip_check(lib.vmhip_debug_set(native.DEBUG_FLOW_POLL_LIMIT, 1))
     try:
         with pytest.raises(RuntimeError, match="gave up waiting"):
             engine.run()
+        # a failed run leaves nothing to fetch
+        with pytest.raises(RuntimeError):
+            engine.fetch()
     finally:
-        lib.vm_flow_set_poll_limit(1 << 18)
+        native.hip_check(lib.vmhip_debug_set(native.DEBUG_FLOW_POLL_LIMIT, 0))
     engine.run()  # the failed run reset the batch's count of such waits, or this one would fail too
     got = engine.fetch()[0]
     want = pick(o_mesh, f["Hoc"]).classify(f["Hoc"], o_lens, f["image"], cfg.fourcc, vmo.Network(cfg.network))

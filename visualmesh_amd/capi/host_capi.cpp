@@ -123,10 +123,11 @@ int export_result(const R& r, int cap, float* px, int32_t* nb, int32_t* gidx) {
         g_error = "result capacity too small";
         return VMHIP_ERR_CAPACITY;
     }
+    /* an empty projection still has its null row (the caller's table holds cap + 1 rows); an empty classification has none */
+    if (nb && !r.neighbourhood.empty()) std::memcpy(nb, r.neighbourhood.data(), sizeof(r.neighbourhood[0]) * r.neighbourhood.size());
     if (V == 0) return 0;
     if (px) std::memcpy(px, r.pixel_coordinates.data(), sizeof(float) * 2 * V);
     if (gidx) std::memcpy(gidx, r.global_indices.data(), sizeof(int32_t) * V);
-    if (nb) std::memcpy(nb, r.neighbourhood.data(), sizeof(r.neighbourhood[0]) * r.neighbourhood.size());
     return V;
 }
 }  // namespace

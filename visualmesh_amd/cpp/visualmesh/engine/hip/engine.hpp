@@ -134,9 +134,21 @@ namespace engine {
                     batch_ = o.batch_;
                     meshes_ = std::move(o.meshes_);
                     staged_ = std::move(o.staged_);
+                    /* the cache's book-keeping travels with the meshes: the staged frames' meshes are pinned by
+                     * staged_since_, entries age against clock_, the byte count decides what is released */
+                    clock_ = o.clock_;
+                    staged_since_ = o.staged_since_;
+                    staging_ = o.staging_;
+                    device_lookup_ = o.device_lookup_;
+                    cache_bytes_ = o.cache_bytes_;
+                    cache_limit_ = o.cache_limit_;
                     o.engine_ = nullptr;
+                    o.engine_nn_ = -1;
                     o.batch_ = nullptr;
                     o.meshes_.clear();
+                    o.staged_.clear();
+                    o.clock_ = 0, o.staged_since_ = 0, o.staging_ = false;
+                    o.cache_bytes_ = 0;
                 }
                 return *this;
             }
@@ -151,7 +163,14 @@ namespace engine {
                 find_ranges(mesh, Hoc, lens, fd);
                 describe(mesh, Hoc, lens, nullptr, 0, fd);
                 ProjectedMesh<Scalar, N> out;
-                if (fd.candidates == 0) return out;
+                /* nothing visible: no pixels, no indices, and the neighbourhood table is its null row alone, pointing
+                 * at itself (reference engine/cpu/engine.hpp:127-143 with n_points = 0) */
+                std::array<int, N> null_row;
+                null_row.fill(0);
+                if (fd.candidates == 0) {
+                    out.neighbourhood.assign(1, null_row);
+                    return out;
+                }
                 out.pixel_coordinates.resize(fd.candidates);
                 out.global_indices.resize(fd.candidates);
                 out.neighbourhood.resize(size_t(fd.candidates) + 1);
@@ -161,7 +180,11 @@ namespace engine {
                 r.global_indices = out.global_indices.data();
                 r.neighbourhood = reinterpret_cast<int32_t*>(out.neighbourhood.data());
                 throw_on_error(vmhip_project(handle(N), &fd.frame, &r));
-                if (r.n_visible == 0) return ProjectedMesh<Scalar, N>();
+                if (r.n_visible == 0) {
+                    ProjectedMesh<Scalar, N> none;
+                    none.neighbourhood.assign(1, null_row);
+                    return none;
+                }
                 out.pixel_coordinates.resize(r.n_visible);
                 out.global_indices.resize(r.n_visible);
                 out.neighbourhood.resize(size_t(r.n_visible) + 1);

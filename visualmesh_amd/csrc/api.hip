@@ -3,6 +3,7 @@
  * staging, the launch sequence, the host re-decision of edge-ambiguous candidates, result download.
  */
 #include <algorithm>
+#include <atomic>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -16,6 +17,10 @@
 namespace {
 
 thread_local std::string g_error;
+
+/* test knobs (vmhip_debug_set); read when a batch is staged */
+std::atomic<float> g_debug_px_error{0.0f};
+std::atomic<float> g_debug_edge_band{VMHIP_AMB_EPS_DEFAULT};
 
 int fail(int code, const std::string& msg) {
     g_error = msg;
@@ -142,6 +147,8 @@ struct vmhip_batch {
     int32_t detect_class = -1, detect_arg_max = 0, detect_clusters = 0;
     float detect_threshold = 0.0f;
     uint32_t epoch = 0; /* host mirror of the device run stamp */
+    /* what the edge guard did since the batch was staged (vmhip_batch_guard_stats) */
+    int64_t reruns = 0, overruled = 0, amb_seen = 0, amb_most = 0;
     /* the kernel sequence of a run, captured once per staged batch and replayed (no profiling, VMHIP_GRAPH != 0) */
     hipGraph_t graph = nullptr;
     hipGraphExec_t graph_exec = nullptr;
@@ -368,6 +375,9 @@ int batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int
     D.halo_cap = E->halo_cap;
     D.epoch = b->d_epoch.as<uint32_t>();
     D.flow_timeouts = b->d_epoch.as<unsigned int>() + 16; /* same zeroed block, a cache line of its own */
+    D.amb_eps = g_debug_edge_band.load();
+    D.px_error = g_debug_px_error.load();
+    b->reruns = 0, b->overruled = 0, b->amb_seen = 0, b->amb_most = 0;
     b->h_V.assign(n_frames, 0);
     b->h_amb_count.assign(n_frames, 0);
     return VMHIP_OK;
@@ -495,6 +505,8 @@ int batch_verify(vmhip_batch* b) {
         }
         const int count = b->h_amb_count[f];
         if (count == 0) continue;
+        b->amb_seen += count;
+        b->amb_most = std::max<int64_t>(b->amb_most, count);
         const float* rays = hf.mesh->h_rays.data();
         auto redecide = [&](int p, int gpu_keep, bool force_all) {
             /* candidate slot -> global index */
@@ -525,6 +537,8 @@ int batch_verify(vmhip_batch* b) {
         }
     }
     if (changed > 0) {
+        b->overruled += changed;
+        ++b->reruns;
         const size_t words = std::max<size_t>(b->cand_total / 64, 1);
         HIP_TRY(hipMemcpyAsync(b->d_force_valid.p, b->h_force_valid.data(), 8 * words, hipMemcpyHostToDevice, E->stream));
         HIP_TRY(hipMemcpyAsync(b->d_force_keep.p, b->h_force_keep.data(), 8 * words, hipMemcpyHostToDevice, E->stream));
@@ -585,6 +599,7 @@ int batch_run(vmhip_batch* b) {
     if (b->frames.empty()) return fail(VMHIP_ERR_ARGUMENT, "run: nothing staged");
     if (b->in_flight) return fail(VMHIP_ERR_ARGUMENT, "run: a run of this batch is still in flight (vmhip_batch_wait first)");
     if (b->fetching) return fail(VMHIP_ERR_ARGUMENT, "run: a fetch of this batch is still in flight (vmhip_batch_fetch_wait first)");
+    b->have_run = false; /* a run that fails leaves nothing to fetch */
     const int rc = batch_launch(b);
     if (rc != VMHIP_OK) return rc;
     return batch_complete(b);
@@ -1199,6 +1214,27 @@ int vmhip_batch_profile_read(vmhip_batch* b, int32_t max_slots, int32_t* n_slots
         ++n;
     }
     *n_slots = n;
+    return VMHIP_OK;
+}
+
+int vmhip_debug_set(int32_t what, double value) {
+    switch (what) {
+        case VMHIP_DEBUG_FLOW_POLL_LIMIT: {
+            const int polls = value <= 0.0 ? VM_FLOW_POLL_LIMIT_DEFAULT : int(value);
+            HIP_TRY(vm_flow_set_poll_limit(polls));
+            return VMHIP_OK;
+        }
+        case VMHIP_DEBUG_PROJECTION_ERROR: g_debug_px_error.store(float(value)); return VMHIP_OK;
+        case VMHIP_DEBUG_EDGE_BAND: g_debug_edge_band.store(value <= 0.0 ? VMHIP_AMB_EPS_DEFAULT : float(value)); return VMHIP_OK;
+        default: return fail(VMHIP_ERR_ARGUMENT, "debug_set: unknown knob");
+    }
+}
+int vmhip_batch_guard_stats(const vmhip_batch* b, int64_t* listed, int64_t* most_listed, int64_t* overruled, int64_t* reruns) {
+    if (!b) return fail(VMHIP_ERR_ARGUMENT, "batch_guard_stats: null batch");
+    if (listed) *listed = b->amb_seen;
+    if (most_listed) *most_listed = b->amb_most;
+    if (overruled) *overruled = b->overruled;
+    if (reruns) *reruns = b->reruns;
     return VMHIP_OK;
 }
 

@@ -40,38 +40,13 @@
 
 #include "vmhip_internal.h"
 
-/* polls a wait may take; only a test of the give-up path sets it (to something tiny) */
-__device__ int vm_flow_poll_limit = 1 << 18;
-extern "C" void vm_flow_set_poll_limit(int polls) {
-    (void) hipMemcpyToSymbol(HIP_SYMBOL(vm_flow_poll_limit), &polls, sizeof(polls));
+/* polls a wait may take (a poll is ~100 cycles, a tile ~20 000: the default is hundreds of tile periods, a fifth of a
+ * second); only a test of the give-up path sets it, to something tiny (vmhip_debug_set) */
+__device__ int vm_flow_poll_limit = VM_FLOW_POLL_LIMIT_DEFAULT;
+hipError_t vm_flow_set_poll_limit(int polls) {
+    return hipMemcpyToSymbol(HIP_SYMBOL(vm_flow_poll_limit), &polls, sizeof(polls));
 }
 
-#ifdef VM_FLOW_TIMING
-/* Build with -DVM_FLOW_TIMING to sum, per wave of a block and per phase of the tile loop, the shader clock cycles spent
- * (layers of one shape, 32 -> 32 unless -DVM_FLOW_TIMING_CIN= / -DVM_FLOW_TIMING_COUT= say otherwise): 0 wait for the tile, 1 contraction, 2 wait for my share of the next tile, 3 activation +
- * stores, 4 wait for the buffer, 5 requests, 6 tiles. */
-__device__ unsigned long long vm_flow_timing[16 * 8];
-__device__ unsigned long long vm_flow_timing_clocks[2];
-extern "C" void vm_flow_timing_clocks_read(unsigned long long* out) {
-    (void) hipMemcpyFromSymbol(out, HIP_SYMBOL(vm_flow_timing_clocks), sizeof(vm_flow_timing_clocks));
-    unsigned long long zero[2] = {};
-    (void) hipMemcpyToSymbol(HIP_SYMBOL(vm_flow_timing_clocks), zero, sizeof(zero));
-}
-extern "C" void vm_flow_timing_read(unsigned long long* out) {
-    (void) hipMemcpyFromSymbol(out, HIP_SYMBOL(vm_flow_timing), sizeof(vm_flow_timing));
-    unsigned long long zero[16 * 8] = {};
-    (void) hipMemcpyToSymbol(HIP_SYMBOL(vm_flow_timing), zero, sizeof(zero));
-}
-#ifndef VM_FLOW_TIMING_CIN
-#define VM_FLOW_TIMING_CIN 32
-#endif
-#ifndef VM_FLOW_TIMING_COUT
-#define VM_FLOW_TIMING_COUT 32
-#endif
-#define FLOW_T(i) do { const unsigned long long now_ = clock64(); tsum[i] += now_ - tprev; tprev = now_; } while (0)
-#else
-#define FLOW_T(i) do { } while (0)
-#endif
 
 namespace {
 
@@ -175,10 +150,10 @@ __device__ __forceinline__ uint32_t lds_address(const void* p) {
     return (uint32_t) (uintptr_t) (const __attribute__((address_space(3))) void*) p;
 }
 __device__ __forceinline__ void load_to_lds_b128(const v4u& rsrc, uint32_t lds_base, uint32_t offset) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(lds_base), "v"(offset), "s"(rsrc) : "memory");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(lds_base), "v"(offset), "s"(rsrc) : "memory", "m0");
 }
 __device__ __forceinline__ void load_to_lds_b32(const v4u& rsrc, uint32_t lds_base, uint32_t offset) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, 0 offen lds" ::"s"(lds_base), "v"(offset), "s"(rsrc) : "memory");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, 0 offen lds" ::"s"(lds_base), "v"(offset), "s"(rsrc) : "memory", "m0");
 }
 
 template <int C_IN, int C_OUT, int SLOTS>
@@ -221,9 +196,6 @@ __global__ __launch_bounds__(FLOW_WAVES * 64) void vm_conv_flow_kernel(VmBatchDe
     static_assert(N_DMA == flow_rounds(C_IN) && N_HALO == flow_halo_rounds(C_IN), "the LDS size is computed from the same rounds");
     constexpr int SLOT_WORDS = flow_slot_words(C_IN);
 
-#ifdef VM_FLOW_TIMING
-    const unsigned long long t_kernel = clock64(), w_kernel = wall_clock64();
-#endif
     extern __shared__ float4 lds4[];
     float* const w_lds = reinterpret_cast<float*>(lds4);
     float* const b_lds = w_lds + W_FLOATS;
@@ -391,10 +363,6 @@ __global__ __launch_bounds__(FLOW_WAVES * 64) void vm_conv_flow_kernel(VmBatchDe
         __syncthreads();
     }
 
-#ifdef VM_FLOW_TIMING
-    unsigned long long tsum[8] = {}, tprev = clock64();
-    tsum[7] = tprev - t_kernel; /* the prologue */
-#endif
     for (int k = 0; k < count; ++k) {
         const int b = k & 1;
         const uint32_t round = (uint32_t) ((k >> 1) + 1); /* the round of buffer b that tile k is */
@@ -404,7 +372,6 @@ __global__ __launch_bounds__(FLOW_WAVES * 64) void vm_conv_flow_kernel(VmBatchDe
             give_up();
             break;
         }
-        FLOW_T(0);
         const int4 d_cur = read_desc(rows + DESC_AT);
         /* The SIMDs serve their oldest wave first, so left alone the youngest falls a whole tile behind, and the
          * buffer it still reads cannot be refilled. A wave that starts a tile while the tile before is not yet
@@ -536,7 +503,6 @@ __global__ __launch_bounds__(FLOW_WAVES * 64) void vm_conv_flow_kernel(VmBatchDe
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         if (lane == 0) atomicAdd(&counters[2 + b], 1u);
         __builtin_amdgcn_s_setprio(FLOW_PRIO_REST); /* what follows is short and keeps no matrix pipe busy: let it through */
-        FLOW_T(1);
         if (loader) {
             /* The notes on tile k+2, requested a tile ago, are in the slot once nothing but what was requested after
              * them can still be in flight: the loads of tile k+1 and the stores of tile k-1 (of tiles 0 and 1 at first). */
@@ -604,33 +570,17 @@ __global__ __launch_bounds__(FLOW_WAVES * 64) void vm_conv_flow_kernel(VmBatchDe
             }
         }
 
-        FLOW_T(3);
         if (loader) {
             /* my share of tile k+1, requested a tile ago, has landed once nothing but what was requested after it and
              * the stores above can still be in flight */
-            FLOW_T(2);
             /* tile k+2 goes where tile k was, once every wave has read the last of tile k */
             if (!wait_counter(&counters[2 + b], gave_up, NW * round, polls)) {
                 give_up();
                 break;
             }
-            FLOW_T(4);
             fill(tile_of(k + 2), first_new, k + 2 < count, offs, buf0 + b * BUF_FLOATS);
-            FLOW_T(5);
         }
-#ifdef VM_FLOW_TIMING
-        tsum[6] += 1;
-#endif
     }
-#ifdef VM_FLOW_TIMING
-    if (lane == 0 && C_IN == VM_FLOW_TIMING_CIN && C_OUT == VM_FLOW_TIMING_COUT)
-        for (int i = 0; i < 8; ++i) atomicAdd(&vm_flow_timing[wave * 8 + i], tsum[i]);
-    if (lane == 0 && wave == 0 && blockIdx.x == 0 && C_IN == VM_FLOW_TIMING_CIN && C_OUT == VM_FLOW_TIMING_COUT) {
-        /* shader clock against the constant 100 MHz clock over this block's life */
-        atomicAdd(&vm_flow_timing_clocks[0], clock64() - t_kernel);
-        atomicAdd(&vm_flow_timing_clocks[1], wall_clock64() - w_kernel);
-    }
-#endif
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); /* no LDS load may outlive the wave */
 }
 

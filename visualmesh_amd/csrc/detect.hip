@@ -55,7 +55,7 @@ __global__ __launch_bounds__(DETECT_THREADS) void vm_detect_kernel(VmBatchDev B,
     __shared__ int scratch[DETECT_THREADS / 64];
     const int f = blockIdx.x;
     const VmFrame& F = B.frames[f];
-    const int V = B.frame_V[f];
+    const int V = F.n_cand > 0 ? B.frame_V[f] : 0; /* a frame without candidates has no rows */
     const size_t base = (size_t) F.row_base;
     const int C = D.n_classes, cls = D.class_index;
     int running = 0;
@@ -84,7 +84,7 @@ __global__ __launch_bounds__(DETECT_THREADS) void vm_detect_kernel(VmBatchDev B,
         running += total;
     }
     if (threadIdx.x == 0) {
-        D.row_to_detection[base + V] = -1; /* the null row */
+        if (F.n_cand > 0) D.row_to_detection[base + V] = -1; /* the null row (a frame without candidates owns no row at all) */
         D.counts[2 * f] = running;
         D.counts[2 * f + 1] = 0;
     }
@@ -116,7 +116,7 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_cluster_union_kernel(VmBatchDev
     const int tile = blockIdx.x;
     const int f = frame_of_row_tile(B.frames, B.n_frames, tile);
     const VmFrame& F = B.frames[f];
-    const int V = B.frame_V[f];
+    const int V = F.n_cand > 0 ? B.frame_V[f] : 0; /* a frame without candidates has no rows */
     const int r = (tile - F.row_tile0) * VMHIP_TILE + (int) threadIdx.x;
     if (r >= V) return;
     const size_t base = (size_t) F.row_base;

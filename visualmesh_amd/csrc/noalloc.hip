@@ -221,6 +221,8 @@ extern "C" int vmhip_project_noalloc(const vmhip_mesh* mesh, const float* Rco, c
     B.row_nbl = nullptr, B.tile_halo = nullptr, B.tile_desc = nullptr;
     B.halo_cap = 0;
     B.flow_timeouts = nullptr;
+    B.amb_eps = VMHIP_AMB_EPS_DEFAULT;
+    B.px_error = 0.0f;
 
     hipLaunchKernelGGL(vm_noalloc_prepare_kernel, dim3(1), dim3(PREPARE_THREADS), 0, s, F, ranges, n_candidates, header, d_frame, range_first,
                        range_prefix, out->n_visible);

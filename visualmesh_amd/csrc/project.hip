@@ -23,8 +23,6 @@
 
 #include "libm_exact.h"
 
-#define AMB_EPS 0.015625f /* 1/64 px: far above any device/host libm difference, far below node spacing */
-
 namespace {
 
 __device__ __forceinline__ int find_frame_by_cand_tile(const VmFrame* frames, int n, int tile) {
@@ -107,7 +105,10 @@ __global__ __launch_bounds__(256) void vm_copy_probe_kernel(const float4* __rest
 
 __global__ void vm_reset_kernel(VmBatchDev B) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < B.n_frames) B.amb_count[i] = 0;
+    if (i < B.n_frames) {
+        B.amb_count[i] = 0;
+        B.frame_V[i] = 0; /* a frame without candidates has no tile that would write its count */
+    }
     if (i == 0) *B.epoch += 1; /* a new run: stamps of earlier runs stop matching */
 }
 
@@ -366,13 +367,14 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_project_kernel(VmBatchDev B) {
         const int g = cand_to_global(F, p);
         const float* r = F.rays + (size_t) g * 3;
         px = project_ray(F, r[0], r[1], r[2]);
+        px.x += B.px_error, px.y += B.px_error; /* zero outside tests of the edge guard */
         const float W = (float) F.width, H = (float) F.height;
         /* strict test of the CPU engine, engine/cpu/engine.hpp:116-117 */
         keep = 0.0f <= px.x && px.x + 1.0f < W && 0.0f <= px.y && px.y + 1.0f < H;
 
         /* distance to the nearest decision boundary; NaN counts as ambiguous */
         const float d = fminf(fminf(fabsf(px.x), fabsf(px.x + 1.0f - W)), fminf(fabsf(px.y), fabsf(px.y + 1.0f - H)));
-        const bool ambiguous = !(d >= AMB_EPS);
+        const bool ambiguous = !(d >= B.amb_eps);
 
         const size_t word = (size_t) (F.cand_base + p) >> 6;
         const uint64_t bit = 1ull << (threadIdx.x & 63);

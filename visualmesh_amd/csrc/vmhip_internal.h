@@ -99,8 +99,14 @@ struct VmBatchDev {
     uint16_t* row_nbl;    /* [rows][VMHIP_NBL_STRIDE]: 0..255 own tile, 256+h halo slot h, VMHIP_NBL_FAR not staged */
     uint32_t* tile_halo;  /* [n_row_tiles][VMHIP_HALO_MAX] batch-global row of each halo slot */
     int4* tile_desc;      /* [n_row_tiles] {first batch-global row, rows in use (0..256), halo rows, frame's row_base} */
-    int32_t halo_cap;     /* halo slots handed out per tile, <= VMHIP_HALO_MAX (smaller only to test the far path) */    unsigned int* flow_timeouts; /* the batch's count of waits of the barrier-free kernel that ran out of polls (0 in a correct run) */
+    int32_t halo_cap;     /* halo slots handed out per tile, <= VMHIP_HALO_MAX (smaller only to test the far path) */
+    unsigned int* flow_timeouts; /* the batch's count of waits of the barrier-free kernel that ran out of polls (0 in a correct run) */
+    /* edge guard: a candidate closer than amb_eps pixels to a screen edge is listed for the host's re-decision.
+     * px_error is 0 outside tests: added to both pixel coordinates, it stands for a device whose lens arithmetic
+     * differs from the host's (vmhip_debug_set) */
+    float amb_eps, px_error;
 };
+#define VMHIP_AMB_EPS_DEFAULT 0.015625f /* 1/64 px: far above any device/host libm difference, far below node spacing */
 
 /* Lookup on the device (project.hip: vm_lookup_kernel): the cone tree over a mesh's nodes and what a frame's walk of it
  * needs. The tree, the walk and every comparison in it are those of the host's lookup (cpp/visualmesh/detail/
@@ -227,6 +233,8 @@ bool vm_flow_supported(int c_in, int c_out, int slots);
 void vm_flow_order_weights(const float* w_mfma, int c_in, int c_out, int slots, float* out);
 int vm_launch_conv_flow(const VmBatchDev& B, const VmLayerDev& L, const float* in, float* out, hipStream_t stream,
                         const char** kernel_name);
+#define VM_FLOW_POLL_LIMIT_DEFAULT (1 << 22)
+hipError_t vm_flow_set_poll_limit(int polls); /* process wide; tests of the give-up path only */
 
 /* layers with at most four output channels on v_mfma_f32_4x4x1 (64 rows x 4 channels per instruction), staged like
  * conv_dma.hip (conv_narrow.hip); reads the plain row-major weights */

@@ -119,8 +119,7 @@ class Engine:
         nb = np.zeros((cap + 1, m.n_neighbours), np.int32)
         gidx = np.zeros(max(cap, 1), np.int32)
         V = native.host_check(self._lib.vmh_engine_project(self.ptr, m.ptr, _fp(H), C.byref(lens), cap, _fp(px), _ip(nb), _ip(gidx)))
-        if V == 0:
-            return dict(px=px[:0], nb=nb[:0], gidx=gidx[:0])
+        # nothing visible: the neighbourhood table is its null row alone, as the reference's projection returns it
         return dict(px=px[:V].copy(), nb=nb[:V + 1].copy(), gidx=gidx[:V].copy())
 
     def classify(self, mesh, Hoc, lens, image, fcc):

@@ -18,13 +18,14 @@ HOST_LIB = os.path.join(PKG, "lib", "libvisualmesh_host.so")
 
 OK, ERR_HIP, ERR_FORMAT, ERR_LENS, ERR_ARGUMENT, ERR_CAPACITY = 0, -1, -2, -3, -4, -5
 FP32, BF16 = 0, 1
+DEBUG_FLOW_POLL_LIMIT, DEBUG_PROJECTION_ERROR, DEBUG_EDGE_BAND = 0, 1, 2
 
 # every symbol include/visualmesh_hip.h declares
 HIP_SYMBOLS = [
     "vmhip_last_error", "vmhip_engine_create", "vmhip_engine_destroy", "vmhip_engine_n_classes", "vmhip_mesh_upload",
     "vmhip_mesh_release", "vmhip_project", "vmhip_classify", "vmhip_classify_batch", "vmhip_batch_create",
     "vmhip_batch_destroy", "vmhip_mesh_attach_tree", "vmhip_batch_stage", "vmhip_batch_ranges", "vmhip_batch_export", "vmhip_batch_run", "vmhip_batch_run_async", "vmhip_batch_wait", "vmhip_batch_counts", "vmhip_batch_fetch", "vmhip_batch_fetch_async", "vmhip_batch_fetch_wait", "vmhip_batch_detect", "vmhip_host_alloc", "vmhip_host_free",
-    "vmhip_batch_profile", "vmhip_batch_profile_read", "vmhip_selftest_libm", "vmhip_selftest_copy", "vmhip_project_noalloc",
+    "vmhip_batch_profile", "vmhip_batch_profile_read", "vmhip_selftest_libm", "vmhip_selftest_copy", "vmhip_project_noalloc", "vmhip_debug_set", "vmhip_batch_guard_stats",
 ]
 
 
@@ -156,6 +157,8 @@ def hip():
                                            C.POINTER(C.c_int64)]
     L.vmhip_selftest_libm.argtypes = [C.c_int32, C.POINTER(C.c_float), C.POINTER(C.c_float), C.c_int32]
     L.vmhip_selftest_copy.argtypes = [C.c_int64, C.c_int32, C.POINTER(C.c_float)]
+    L.vmhip_debug_set.argtypes = [C.c_int32, C.c_double]
+    L.vmhip_batch_guard_stats.argtypes = [vp, C.POINTER(C.c_int64), C.POINTER(C.c_int64), C.POINTER(C.c_int64), C.POINTER(C.c_int64)]
     L.vmhip_project_noalloc.argtypes = [vp, C.POINTER(C.c_float), C.POINTER(Lens), C.POINTER(C.c_int32), C.c_int32, C.c_int32,
                                         C.POINTER(ProjectionDevice), vp]
     _hip = L
@@ -166,6 +169,13 @@ def hip_check(rc):
     if rc < 0:
         raise VisualMeshError(rc, hip().vmhip_last_error().decode())
     return rc
+
+
+def guard_stats(batch_ptr):
+    """dict(listed, most_listed, overruled, reruns): what the edge guard did in the runs of a vmhip_batch since it was staged"""
+    v = [C.c_int64(0) for _ in range(4)]
+    hip_check(hip().vmhip_batch_guard_stats(batch_ptr, *[C.byref(x) for x in v]))
+    return dict(listed=v[0].value, most_listed=v[1].value, overruled=v[2].value, reruns=v[3].value)
 
 
 def copy_probe(nbytes=1 << 30, repeats=5):
