@@ -50,16 +50,17 @@ def layer_table(cfg, n_neighbours):
 
 def conv_roofline(name, avg_ms, rows):
     """Roofline entry of one launch of a graph-convolution kernel over `rows` rows: the layer shape is in the kernel
-    name, conv_<kind>_<cin>x<cout>s<slots>, and so are storage and arithmetic (conv_bf16x2*: bf16 rows in,
-    conv_*_tobf16: bf16 rows out, conv_bf16*: bf16 matrix instructions). Flops are the layer's algorithmic ones, not
-    the hi/lo extras. -> (dict, algorithmic bytes per row, flops per row)"""
+    name, conv_<kind>_<cin>x<cout>s<slots>, and so are storage and arithmetic: conv_bf16_<in>_to<out>_* runs on the
+    bf16 matrix instructions and reads / writes rows as bf16 (2 bytes per channel), x2 (hi + lo pairs of bf16, 4 bytes)
+    or f32; conv_lds_tox2_* writes x2 rows. Flops are the layer's algorithmic ones, not the hi/lo extras.
+    -> (dict, algorithmic bytes per row, flops per row)"""
     shape = name.split("_")[-1]
     c_in, rest = shape.split("x")
     c_out, slots = rest.split("s")
     c_in, c_out, slots = int(c_in), int(c_out), int(slots)
     bf16_arith = name.startswith("conv_bf16")
-    s_in = 2 if name.startswith("conv_bf16x2") else 4
-    s_out = 2 if "_tobf16_" in name else (4 if not name.startswith("conv_bf16x2") or "_tof32_" in name else 2)
+    s_in = 2 if name.startswith("conv_bf16_bf16_") else 4
+    s_out = 2 if "_tobf16_" in name else 4
     bytes_per_row = c_in * s_in + 4 * (slots - 1) + c_out * s_out
     flops_per_row = 2 * slots * c_in * c_out
     intensity = flops_per_row / bytes_per_row

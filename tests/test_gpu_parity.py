@@ -180,8 +180,8 @@ def test_bf16_engine(oracle):
     engine.profile(True)
     engine.run()
     names = [n for n, _, _ in engine.profile_read() if n.startswith("conv")]
-    assert names == ["conv_lds_4x64s7", "conv_bf16x3_tobf16_64x64s7", "conv_bf16x2_tof32_64x64s7", "conv_bf16x3_tobf16_64x64s7",
-                     "conv_bf16x2_tof32_64x64s7", "conv_bf16x3_64x64s7"], names
+    assert names == ["conv_lds_tox2_4x64s7", "conv_bf16_x2_tobf16_64x64s7", "conv_bf16_bf16_tox2_64x64s7", "conv_bf16_x2_tobf16_64x64s7",
+                     "conv_bf16_bf16_tox2_64x64s7", "conv_bf16_x2_tof32_64x64s7"], names
     worst = 0.0
     for i, f in enumerate(cfg.frames):
         want = o_mesh.classify(f["Hoc"], o_lens, f["image"], cfg.fourcc, vmo.Network(net))

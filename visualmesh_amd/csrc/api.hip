@@ -110,6 +110,7 @@ struct vmhip_engine {
     bool use_graph = true;               /* VMHIP_GRAPH=0: launch every run kernel by kernel */
     bool use_lds = false;                /* some layer gathers through the tile-local tables */
     bool use_flow = false;               /* some layer runs the kernel that polls LDS counters instead of barriers */
+    bool use_bf16 = false;               /* some layer runs on the bf16 matrix instructions (half-tile tables) */
     int32_t halo_cap = VMHIP_HALO_MAX;   /* VMHIP_HALO_CAP lowers it to exercise the not-staged path */
     int32_t nn = 0;
     int32_t precision = VMHIP_FP32;
@@ -162,7 +163,7 @@ struct vmhip_batch {
 
     VmBatchDev dev{};
     DevBuf d_frames, d_ranges, d_images, d_cand_px, d_cand_g, d_cand_keep, d_tile_count, d_force_valid, d_force_keep, d_frame_V,
-      d_amb_list, d_row_px, d_row_gidx, d_row_nb, d_row_nbl, d_tile_halo, d_tile_desc, d_act[2], d_lookup, d_epoch, d_detect, d_detect_packed, d_lookup_ws, d_export;
+      d_amb_list, d_row_px, d_row_gidx, d_row_nb, d_row_nbl, d_tile_halo, d_tile_desc, d_row_nbl_h, d_tile_note_h, d_active_h, d_act[2], d_lookup, d_epoch, d_detect, d_detect_packed, d_lookup_ws, d_export;
     std::vector<std::vector<int32_t>> device_ranges; /* per frame: the ranges a lookup on the device produced */
     void* h_detect = nullptr; /* pinned landing area of vmhip_batch_detect */
     size_t h_detect_cap = 0;
@@ -179,7 +180,7 @@ struct vmhip_batch {
     void release() {
         DevBuf* all[] = {&d_frames, &d_ranges, &d_images, &d_cand_px, &d_cand_g, &d_cand_keep, &d_tile_count, &d_force_valid,
                          &d_force_keep, &d_frame_V, &d_amb_list, &d_row_px, &d_row_gidx, &d_row_nb,
-                         &d_row_nbl, &d_tile_halo, &d_tile_desc, &d_epoch,
+                         &d_row_nbl, &d_tile_halo, &d_tile_desc, &d_row_nbl_h, &d_tile_note_h, &d_active_h, &d_epoch,
                          &d_act[0], &d_act[1], &d_lookup, &d_detect, &d_detect_packed, &d_lookup_ws, &d_export};
         drop_graph();
         for (DevBuf* b : all) b->release();
@@ -304,6 +305,13 @@ int batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int
         HIP_TRY(b->d_tile_halo.reserve(4 * row_tiles * VMHIP_HALO_MAX));
         HIP_TRY(b->d_tile_desc.reserve(sizeof(int4) * row_tiles));
     }
+    const bool half_tables = classify && E->use_bf16 && nb_stride <= VMHIP_NBL_STRIDE;
+    if (half_tables) {
+        const size_t row_tiles = std::max<size_t>(b->row_total / VMHIP_TILE, 1);
+        HIP_TRY(b->d_row_nbl_h.reserve(2 * std::max<size_t>(b->row_total, 1) * VMHIP_NBL_STRIDE));
+        HIP_TRY(b->d_tile_note_h.reserve(4 * 2 * row_tiles * VMHIP_NOTE_WORDS));
+        HIP_TRY(b->d_active_h.reserve(4 * (size_t(n_frames) + 1)));
+    }
     HIP_TRY(b->d_lookup.reserve(sizeof(uint2) * lookup_entries));
     if (b->d_lookup.grew) {
         /* a fresh reverse-lookup table holds no valid stamp; epochs start above zero */
@@ -373,6 +381,9 @@ int batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int
     D.tile_halo = local_tables ? b->d_tile_halo.as<uint32_t>() : nullptr;
     D.tile_desc = local_tables ? b->d_tile_desc.as<int4>() : nullptr;
     D.halo_cap = E->halo_cap;
+    D.active_h = half_tables ? b->d_active_h.as<int32_t>() : nullptr;
+    D.row_nbl_h = half_tables ? b->d_row_nbl_h.as<uint16_t>() : nullptr;
+    D.tile_note_h = half_tables ? b->d_tile_note_h.as<uint32_t>() : nullptr;
     D.epoch = b->d_epoch.as<uint32_t>();
     D.flow_timeouts = b->d_epoch.as<unsigned int>() + 16; /* same zeroed block, a cache line of its own */
     D.amb_eps = g_debug_edge_band.load();
@@ -431,6 +442,11 @@ int batch_enqueue(vmhip_batch* b) {
     HIP_TRY(P.begin());
     vm_launch_neighbourhood(D, s);
     HIP_TRY(P.end("neighbourhood", rows));
+    if (b->classify && D.row_nbl_h) {
+        HIP_TRY(P.begin());
+        vm_launch_half_tables(D, s);
+        HIP_TRY(P.end("half_tables", rows));
+    }
 
     int cur = 0;
     if (b->classify) {
@@ -439,13 +455,14 @@ int batch_enqueue(vmhip_batch* b) {
             const char* name = "conv";
             HIP_TRY(P.begin());
             int rc = -1;
-            if (L.use_narrow && D.row_nbl) rc = vm_launch_conv_narrow(D, ld, b->d_act[cur].as<float>(), b->d_act[cur ^ 1].as<float>(), s, &name);
+            if (L.arith_bf16) rc = vm_launch_conv_bf16(D, ld, b->d_act[cur].p, b->d_act[cur ^ 1].p, s, &name);
+            if (rc != 0 && !L.arith_bf16 && L.use_narrow && D.row_nbl) rc = vm_launch_conv_narrow(D, ld, b->d_act[cur].as<float>(), b->d_act[cur ^ 1].as<float>(), s, &name);
             if (rc != 0 && L.use_flow && D.row_nbl) rc = vm_launch_conv_flow(D, ld, b->d_act[cur].as<float>(), b->d_act[cur ^ 1].as<float>(), s, &name);
             if (rc != 0 && L.use_dma && D.row_nbl) rc = vm_launch_conv_dma(D, ld, b->d_act[cur].as<float>(), b->d_act[cur ^ 1].as<float>(), s, &name);
             if (rc != 0 && L.use_lds && D.row_nbl) rc = vm_launch_conv_lds(D, ld, b->d_act[cur].as<float>(), b->d_act[cur ^ 1].as<float>(), s, &name);
-            if (rc != 0 && L.d_w_mfma && L.use_mfma) rc = vm_launch_conv_mfma(D, ld, b->d_act[cur].p, b->d_act[cur ^ 1].p, s, &name);
+            if (rc != 0 && L.d_w_mfma && L.use_mfma) rc = vm_launch_conv_mfma(D, ld, b->d_act[cur].as<float>(), b->d_act[cur ^ 1].as<float>(), s, &name);
             /* the one-row-per-lane kernels only know fp32 rows */
-            if (rc != 0 && !L.in_bf16 && !L.out_bf16) rc = vm_launch_conv(D, ld, b->d_act[cur].as<float>(), b->d_act[cur ^ 1].as<float>(), s, &name);
+            if (rc != 0 && !L.in_bf16 && !L.out_bf16 && !L.arith_bf16) rc = vm_launch_conv(D, ld, b->d_act[cur].as<float>(), b->d_act[cur ^ 1].as<float>(), s, &name);
             if (rc != 0) return fail(VMHIP_ERR_HIP, "no kernel could be launched for a layer");
             HIP_TRY(P.end(name, rows));
             cur ^= 1;
@@ -707,13 +724,15 @@ int vmhip_engine_create(const vmhip_network* net, int32_t n_neighbours, int32_t 
     }
     E->n_classes = width;
 
-    /* Row types and arithmetic per layer. fp32 engine: everything fp32. bf16 engine: layers reading rows at
-     * least 64 wide run on the bf16 matrix instructions (fp32 accumulation, weights as hi + lo pairs of bf16).
-     * Such a layer reads either bf16 rows, which costs one bf16 rounding of its inputs against the fp32 result,
-     * or fp32 rows split into hi + lo in registers, which costs nothing measurable. Each rounding moves the
-     * final probabilities of a 6 x 64 network by up to ~4.6e-3, so to stay inside the 1e-2 gate with margin
-     * only every second eligible boundary is stored as bf16 (the 2nd, 4th, ...); the others stay fp32. A choice
-     * is only made where the kernels on both sides of the boundary exist for it. */
+    /* Row formats and arithmetic per layer. fp32 engine: everything fp32. bf16 engine: the layers that conv_bf16.hip
+     * has a kernel for (64 -> 64) run on the bf16 matrix instructions with fp32 accumulation and weights as hi + lo
+     * pairs of bf16. The rows such a layer reads are stored either as bf16 (half the bytes, one bf16 rounding of
+     * that layer's inputs against the fp32 result) or as hi + lo pairs of bf16 (the bytes of an fp32 row, no
+     * bf16-sized error). One rounded boundary moves the final probabilities of a 6 x 64 network by up to ~4.6e-3,
+     * n of them by about sqrt(n) times that (two: 7.2e-3, all five: 1.03e-2, measured on full-size frames), so to stay
+     * inside the 1e-2 gate with margin every second boundary between bf16 layers is rounded and never more than two
+     * in a network, however deep. A bf16 layer behind a kernel that cannot write hi + lo rows reads fp32 rows and
+     * splits them in registers. */
     {
         /* VMHIP_CONV_KERNEL selects the kernel family for A/B runs: "rows" = one row per lane, "mfma" = matrix
          * cores gathering into registers, "lds" = matrix cores gathering from LDS (rows staged through registers),
@@ -728,27 +747,20 @@ int vmhip_engine_create(const vmhip_network* net, int32_t n_neighbours, int32_t 
         if (const char* g = getenv("VMHIP_GRAPH")) E->use_graph = atoi(g) != 0;
         if (const char* cap = getenv("VMHIP_HALO_CAP")) E->halo_cap = std::min(std::max(atoi(cap), 0), VMHIP_HALO_MAX);
         const int n = int(E->layers.size());
-        std::vector<int> bf(n + 1, 0); /* bf[l] = rows entering layer l are bf16; bf[n] = final output (never) */
-        std::vector<int> ar(n, 0);     /* ar[l] = layer l uses the bf16 matrix instructions */
+        std::vector<int> bf(n + 1, VM_ROWS_F32); /* bf[l] = format of the rows entering layer l; bf[n] = final output (fp32) */
+        std::vector<int> ar(n, 0);               /* ar[l] = layer l uses the bf16 matrix instructions */
         if (precision == VMHIP_BF16 && !rows_only) {
-            int eligible = 0;
-            for (int l = 0; l < n; ++l) ar[l] = (E->layers[l].c_in >= 64 && E->layers[l].c_in % 32 == 0) ? 1 : 0;
-            for (int l = 1; l < n; ++l)
-                if (ar[l] && (++eligible % 2) == 0) bf[l] = 1;
-        }
-        auto ok = [&](int l) {
-            const HostLayer& H = E->layers[l];
-            return vm_mfma_supported(H.c_in, H.c_out, H.slots, bf[l], bf[l + 1], ar[l]);
-        };
-        for (bool changed = true; changed;) {
-            changed = false;
-            for (int l = 0; l < n; ++l) {
-                if (ok(l) || (!bf[l] && !bf[l + 1] && !ar[l])) continue;
-                /* give up bf16 storage around the layer first, then its bf16 arithmetic */
-                if (bf[l] || bf[l + 1]) bf[l] = 0, bf[l + 1] = 0;
-                else ar[l] = 0;
-                bf[n] = 0;
-                changed = true;
+            for (int l = 0; l < n; ++l)
+                ar[l] = (E->layers[l].slots - 1 <= VMHIP_NBL_STRIDE && vm_bf16_supported(E->layers[l].c_in, E->layers[l].c_out, E->layers[l].slots)) ? 1 : 0;
+            int eligible = 0, rounded = 0;
+            for (int l = 1; l < n; ++l) {
+                if (!ar[l]) continue;
+                ++eligible;
+                const HostLayer& P = E->layers[l - 1];
+                const bool splits = ar[l - 1] || (allow_lds && P.slots - 1 <= VMHIP_NBL_STRIDE && vm_lds_supported(P.c_in, P.c_out, P.slots, VM_ROWS_BF16X2));
+                if (!splits) continue; /* the layer before writes fp32 rows */
+                if (ar[l - 1] && eligible % 2 == 0 && rounded < 2) bf[l] = VM_ROWS_BF16, ++rounded;
+                else bf[l] = VM_ROWS_BF16X2;
             }
         }
         auto arith = [&](int l) { return ar[l]; };
@@ -756,12 +768,14 @@ int vmhip_engine_create(const vmhip_network* net, int32_t n_neighbours, int32_t 
             HostLayer& H = E->layers[l];
             H.in_bf16 = bf[l], H.out_bf16 = bf[l + 1], H.arith_bf16 = arith(l);
             const bool plain = !H.in_bf16 && !H.out_bf16 && !H.arith_bf16;
-            H.use_mfma = !rows_only && vm_mfma_supported(H.c_in, H.c_out, H.slots, H.in_bf16, H.out_bf16, H.arith_bf16);
-            H.use_lds = allow_lds && plain && H.slots - 1 <= VMHIP_NBL_STRIDE && vm_lds_supported(H.c_in, H.c_out, H.slots);
+            H.use_mfma = !rows_only && plain && vm_mfma_supported(H.c_in, H.c_out, H.slots, 0, 0, 0);
+            H.use_lds = allow_lds && !H.in_bf16 && !H.arith_bf16 && H.slots - 1 <= VMHIP_NBL_STRIDE && vm_lds_supported(H.c_in, H.c_out, H.slots, H.out_bf16);
+            E->use_bf16 = E->use_bf16 || H.arith_bf16;
             /* Measured on the 16-frame 1280x1024 workload: the LDS gather is the faster matrix-core kernel on every
              * shape it has (32->32: 157 us against 166 us, 32->16: 89 against 122, 4->16: 29 against 44); only the
              * 2- and 3-class output layers are quicker with one row per lane (46 us against 56 us). */
             if (H.use_lds && !force_lds && H.c_out < 4) H.use_lds = false;
+            if (H.out_bf16 && !H.arith_bf16 && !H.use_lds) return bail(VMHIP_ERR_ARGUMENT, "engine_create: no kernel writes the rows the next layer was planned to read");
             H.use_dma = force_dma && plain && H.slots - 1 <= VMHIP_NBL_STRIDE && vm_dma_supported(H.c_in, H.c_out, H.slots);
             /* the barrier-free variant of the LDS gather is the faster one where the matrix pipe is the limit
              * (32 -> 32: 147 us against 158 us, 32 -> 16: 93 against 99) and makes no difference for 16-wide input */
@@ -772,9 +786,16 @@ int vmhip_engine_create(const vmhip_network* net, int32_t n_neighbours, int32_t 
                            && vm_narrow_supported(H.c_in, H.c_out, H.slots);
             E->use_lds = E->use_lds || H.use_lds || H.use_dma || H.use_flow || H.use_narrow;
             E->use_flow = E->use_flow || H.use_flow;
-            if (H.use_mfma || H.use_lds || H.use_dma || H.use_flow) {
-                std::vector<unsigned char> wp(vm_mfma_weight_bytes(H.c_in, H.c_out, H.slots, H.arith_bf16));
-                vm_mfma_permute_weights(H.h_w.data(), H.c_in, H.c_out, H.slots, H.arith_bf16, wp.data());
+            if (H.arith_bf16) {
+                std::vector<unsigned char> wp(vm_bf16_weight_bytes(H.c_in, H.c_out, H.slots));
+                vm_bf16_permute_weights(H.h_w.data(), H.c_in, H.c_out, H.slots, wp.data());
+                if (hipMalloc(&H.d_w_mfma, wp.size()) != hipSuccess) return bail(VMHIP_ERR_HIP, "engine_create: out of device memory");
+                if (hipMemcpy(H.d_w_mfma, wp.data(), wp.size(), hipMemcpyHostToDevice) != hipSuccess)
+                    return bail(VMHIP_ERR_HIP, "engine_create: weight upload failed");
+            }
+            else if (H.use_mfma || H.use_lds || H.use_dma || H.use_flow) {
+                std::vector<unsigned char> wp(vm_mfma_weight_bytes(H.c_in, H.c_out, H.slots, 0));
+                vm_mfma_permute_weights(H.h_w.data(), H.c_in, H.c_out, H.slots, 0, wp.data());
                 if (hipMalloc(&H.d_w_mfma, wp.size()) != hipSuccess) return bail(VMHIP_ERR_HIP, "engine_create: out of device memory");
                 if (hipMemcpy(H.d_w_mfma, wp.data(), wp.size(), hipMemcpyHostToDevice) != hipSuccess)
                     return bail(VMHIP_ERR_HIP, "engine_create: weight upload failed");

@@ -120,8 +120,9 @@ __host__ __device__ constexpr int halo_rows(int c_in, int c_out, int slots) {
 }
 
 /* NW waves per block, RB row blocks of 16 rows per wave: NW * RB * 16 == VMHIP_TILE. */
-template <int C_IN, int C_OUT, int SLOTS, int NW, int HALO>
+template <int C_IN, int C_OUT, int SLOTS, int NW, int HALO, int OUT_FMT>
 __global__ __launch_bounds__(NW * 64, 4) void vm_conv_lds_kernel(VmBatchDev B, VmLayerDev L, const float* __restrict__ in, float* __restrict__ out) {
+    static_assert(OUT_FMT == VM_ROWS_F32 || (OUT_FMT == VM_ROWS_BF16X2 && C_OUT % 16 == 0), "rows go out as fp32, or as hi + lo pairs of bf16 for a bf16 layer to read");
     constexpr int RB = VMHIP_TILE / (16 * NW);
     static_assert(NW * RB * 16 == VMHIP_TILE, "a block covers one tile");
     static_assert(C_IN % 4 == 0, "rows are staged in 16-byte pieces");
@@ -420,7 +421,24 @@ __global__ __launch_bounds__(NW * 64, 4) void vm_conv_lds_kernel(VmBatchDev B, V
                 for (int cb = 0; cb < CB; ++cb) {
                     const int o = cb * 16 + q * 4;
                     const uint32_t at = (li[rb][0] * C_OUT + o) * 4;
-                    if constexpr (C_OUT % 4 == 0) {
+                    if constexpr (OUT_FMT == VM_ROWS_BF16X2) {
+                        /* hi = bf16(x), lo = bf16(x - hi), the difference being exact; C_OUT hi values, then C_OUT lo values */
+                        typedef uint32_t v2u __attribute__((ext_vector_type(2)));
+                        typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+                        auto pack = [](float a, float b) {
+                            v2bf t;
+                            t[0] = (__bf16) a, t[1] = (__bf16) b;
+                            return __builtin_bit_cast(uint32_t, t);
+                        };
+                        const v4f x = acc[rb][cb];
+                        const v2u hi = {pack(x[0], x[1]), pack(x[2], x[3])};
+                        const v2u lo = {pack(x[0] - __uint_as_float(hi.x << 16), x[1] - __uint_as_float(hi.x & 0xffff0000u)),
+                                        pack(x[2] - __uint_as_float(hi.y << 16), x[3] - __uint_as_float(hi.y & 0xffff0000u))};
+                        const uint32_t at2 = li[rb][0] * (C_OUT * 4) + o * 2;
+                        __builtin_amdgcn_raw_buffer_store_b64(hi, out_rsrc, valid[rb] ? at2 : 0xffffffffu, 0, 0);
+                        __builtin_amdgcn_raw_buffer_store_b64(lo, out_rsrc, valid[rb] ? at2 + C_OUT * 2 : 0xffffffffu, 0, 0);
+                    }
+                    else if constexpr (C_OUT % 4 == 0) {
                         __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, acc[rb][cb]), out_rsrc, (valid[rb] && o < C_OUT) ? at : 0xffffffffu, 0, 0);
                     }
                     else {
@@ -451,7 +469,7 @@ __global__ __launch_bounds__(NW * 64, 4) void vm_conv_lds_kernel(VmBatchDev B, V
     VM_T_FLUSH
 }
 
-template <int C_IN, int C_OUT, int SLOTS>
+template <int C_IN, int C_OUT, int SLOTS, int OUT_FMT = VM_ROWS_F32>
 int launch_lds(const VmBatchDev& B, const VmLayerDev& L, const float* in, float* out, hipStream_t stream) {
     constexpr int HALO = halo_rows(C_IN, C_OUT, SLOTS);
     constexpr size_t lds = lds_bytes(C_IN, C_OUT, SLOTS, HALO);
@@ -462,7 +480,7 @@ int launch_lds(const VmBatchDev& B, const VmLayerDev& L, const float* in, float*
      * per SIMD); otherwise one block of 16 waves. */
     constexpr bool single = 2 * lds > 160 * 1024;
     constexpr int NW = single ? 16 : 8;
-    auto kernel = vm_conv_lds_kernel<C_IN, C_OUT, SLOTS, NW, HALO>;
+    auto kernel = vm_conv_lds_kernel<C_IN, C_OUT, SLOTS, NW, HALO, OUT_FMT>;
     static std::atomic<bool> configured{false}; /* engines on several host threads may get here together */
     if (!configured) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, int(lds)) != hipSuccess) {
@@ -499,17 +517,37 @@ int launch_lds(const VmBatchDev& B, const VmLayerDev& L, const float* in, float*
     X(8, 8, 7)                   \
     X(8, 5, 7)
 
-bool vm_lds_supported(int c_in, int c_out, int slots) {
+/* ... and the shapes that can also write their rows as hi + lo pairs of bf16 */
+#define VM_FOR_EACH_LDS_SPLIT_SHAPE(X) \
+    X(4, 64, 7)
+
+bool vm_lds_supported(int c_in, int c_out, int slots, int out_fmt) {
 #define X(CI, CO, SL) \
     if (c_in == CI && c_out == CO && slots == SL) return true;
-    VM_FOR_EACH_LDS_SHAPE(X)
+    if (out_fmt == VM_ROWS_F32) {
+        VM_FOR_EACH_LDS_SHAPE(X)
+    }
+    else if (out_fmt == VM_ROWS_BF16X2) {
+        VM_FOR_EACH_LDS_SPLIT_SHAPE(X)
+    }
 #undef X
     return false;
 }
 
 int vm_launch_conv_lds(const VmBatchDev& B, const VmLayerDev& L, const float* in, float* out, hipStream_t stream, const char** kernel_name) {
     if (B.n_row_tiles <= 0) return 0;
-    if (!B.row_nbl || !B.tile_halo || !B.tile_desc || !L.w_mfma || L.in_bf16 || L.out_bf16 || L.arith_bf16) return -1;
+    if (!B.row_nbl || !B.tile_halo || !B.tile_desc || !L.w_mfma || L.in_bf16 || L.arith_bf16) return -1;
+    if (L.out_bf16 == VM_ROWS_BF16X2) {
+#define X(CI, CO, SL)                                                          \
+    if (L.c_in == CI && L.c_out == CO && L.slots == SL) {                      \
+        if (kernel_name) *kernel_name = "conv_lds_tox2_" #CI "x" #CO "s" #SL;  \
+        return launch_lds<CI, CO, SL, VM_ROWS_BF16X2>(B, L, in, out, stream);  \
+    }
+        VM_FOR_EACH_LDS_SPLIT_SHAPE(X)
+#undef X
+        return -1;
+    }
+    if (L.out_bf16) return -1;
 #define X(CI, CO, SL)                                                       \
     if (L.c_in == CI && L.c_out == CO && L.slots == SL) {                   \
         if (kernel_name) *kernel_name = "conv_lds_" #CI "x" #CO "s" #SL;    \

@@ -33,6 +33,18 @@
 #define VMHIP_HALO_MAX 256 /* rows of other tiles that a row tile can stage next to its own 256 rows */
 #define VMHIP_NBL_STRIDE 8 /* tile-local neighbour table: 8 x uint16 per row */
 #define VMHIP_NBL_FAR 0xffffu /* tile-local neighbour entry: not staged, read the row from global memory */
+/* the bf16 layers (conv_bf16.hip) work on half tiles: 128 rows and up to 128 rows of other half tiles, so that two
+ * buffers of 256-byte rows fit the LDS beside each other */
+#define VMHIP_HTILE 128
+#define VMHIP_HHALO 128
+#define VMHIP_NOTE_WORDS (4 + VMHIP_HHALO) /* a half tile's note: {first row, rows in use, halo rows, frame's first row}, then its halo rows */
+
+/* how the rows of an activation matrix are stored (VmLayerDev::in_bf16 / out_bf16) */
+enum {
+    VM_ROWS_F32 = 0,    /* C floats */
+    VM_ROWS_BF16 = 1,   /* C bf16: the value rounded once */
+    VM_ROWS_BF16X2 = 2  /* C bf16 "hi" then C bf16 "lo", hi = bf16(x), lo = bf16(x - hi): 16 significant bits, ready as matrix operands */
+};
 
 /* image sampling kinds (derived from the fourcc on the host) */
 enum {
@@ -100,6 +112,11 @@ struct VmBatchDev {
     uint32_t* tile_halo;  /* [n_row_tiles][VMHIP_HALO_MAX] batch-global row of each halo slot */
     int4* tile_desc;      /* [n_row_tiles] {first batch-global row, rows in use (0..256), halo rows, frame's row_base} */
     int32_t halo_cap;     /* halo slots handed out per tile, <= VMHIP_HALO_MAX (smaller only to test the far path) */
+    /* the same for half tiles (null unless the engine has bf16 layers). Only half tiles with rows in use are numbered:
+     * half tile t of frame f is number active_h[f] + t */
+    int32_t* active_h;    /* [n_frames + 1] half tiles in use before each frame; the last entry is their total */
+    uint16_t* row_nbl_h;  /* [rows][VMHIP_NBL_STRIDE]: 0..127 own half tile, 128+h halo slot h, VMHIP_NBL_FAR not staged */
+    uint32_t* tile_note_h; /* [half tiles in use][VMHIP_NOTE_WORDS] */
     unsigned int* flow_timeouts; /* the batch's count of waits of the barrier-free kernel that ran out of polls (0 in a correct run) */
     /* edge guard: a candidate closer than amb_eps pixels to a screen edge is listed for the host's re-decision.
      * px_error is 0 outside tests: added to both pixel coordinates, it stands for a device whose lens arithmetic
@@ -143,8 +160,8 @@ struct VmLayerDev {
     const float* w;  /* [slots*c_in][c_out] fp32 row major */
     const float* b;  /* [c_out] */
     const void* w_mfma; /* the same weights in the matrix-core kernel's consumption order, or null */
-    int32_t in_bf16;    /* input rows are stored as bf16 */
-    int32_t out_bf16;   /* output rows are stored as bf16 */
+    int32_t in_bf16;    /* how the input rows are stored: VM_ROWS_* */
+    int32_t out_bf16;   /* how the output rows are stored: VM_ROWS_* */
     int32_t arith_bf16; /* bf16 products with fp32 accumulation (weights in w_mfma are bf16 then) */
     const float* w_flow; /* the fp32 w_mfma weights in the order conv_flow.hip keeps them in LDS, or null */
 };
@@ -192,9 +209,18 @@ void vm_mfma_permute_weights(const float* w, int c_in, int c_out, int slots, int
 int vm_launch_conv_mfma(const VmBatchDev& B, const VmLayerDev& L, const void* in, void* out, hipStream_t stream,
                         const char** kernel_name);
 
+/* the bf16 engine's layers (conv_bf16.hip): bf16 matrix instructions with fp32 accumulation, weights in registers, rows
+ * of half tiles staged in LDS. vm_launch_half_tables builds the half-tile tables from the neighbour table of the run. */
+bool vm_bf16_supported(int c_in, int c_out, int slots);
+size_t vm_bf16_weight_bytes(int c_in, int c_out, int slots);
+void vm_bf16_permute_weights(const float* w, int c_in, int c_out, int slots, void* wp);
+void vm_launch_half_tables(const VmBatchDev& B, hipStream_t stream);
+int vm_launch_conv_bf16(const VmBatchDev& B, const VmLayerDev& L, const void* in, void* out, hipStream_t stream,
+                        const char** kernel_name);
+
 /* matrix-core variant gathering from LDS through the tile-local tables (conv_lds.hip); fp32 rows and arithmetic,
- * weights in vm_mfma_permute_weights' fp32 order */
-bool vm_lds_supported(int c_in, int c_out, int slots);
+ * weights in vm_mfma_permute_weights' fp32 order; writes fp32 rows, or hi + lo rows for a bf16 layer to read */
+bool vm_lds_supported(int c_in, int c_out, int slots, int out_fmt = VM_ROWS_F32);
 int vm_launch_conv_lds(const VmBatchDev& B, const VmLayerDev& L, const float* in, float* out, hipStream_t stream,
                        const char** kernel_name);
 
