@@ -191,6 +191,46 @@ def test_bf16_engine(oracle):
     assert worst > PROB_TOL  # two boundaries are stored as bf16: an error this small would mean they were not
 
 
+@pytest.mark.parametrize("variant", ["halo8", "fp32_rows_in", "relu_tanh", "selu_last"])
+def test_bf16_layer_variants(oracle, variant, monkeypatch):
+    """The bf16 layers' less travelled paths on configuration 1's geometry, each within 1e-2 of the fp32 oracle:
+    halo8          only 8 halo slots per (half) tile: most neighbours outside a half tile are fetched from global memory;
+    fp32_rows_in   the layer before the first bf16 layer writes fp32 rows (the register-gather kernel cannot write hi + lo
+                   rows): the bf16 layer splits them at every use;
+    relu_tanh      relu and tanh between the layers instead of selu;
+    selu_last      a last layer that is not a softmax."""
+    if variant == "halo8":
+        monkeypatch.setenv("VMHIP_HALO_CAP", "8")
+    if variant == "fp32_rows_in":
+        monkeypatch.setenv("VMHIP_CONV_KERNEL", "mfma")
+    cfg = wl.config(1, n_frames=1)
+    rng = np.random.default_rng(77)
+    net = wl.glorot_network(rng, [3, 64, 64, 64, 64], 6, wl.SELU)
+    if variant == "relu_tanh":
+        net = [[(w, b, a if a == wl.SOFTMAX else (wl.RELU if i % 2 == 0 else wl.TANH)) for (w, b, a) in g] for i, g in enumerate(net)]
+    if variant == "selu_last":
+        net = [[(w, b, wl.SELU) for (w, b, a) in g] for g in net]
+    o_lens, e_lens = lens_pair(cfg)
+    o_mesh, e_mesh = meshes_for(cfg, oracle)
+    engine = eng.Engine(net, cfg.model, precision=native.BF16)
+    f = cfg.frames[0]
+    got = engine(e_mesh, f["Hoc"], e_lens, f["image"], cfg.fourcc)
+    engine.profile(True)
+    engine.run()
+    names = [n for n, _, _ in engine.profile_read() if n.startswith("conv")]
+    first = "conv_mfma_4x64s7" if variant == "fp32_rows_in" else "conv_lds_tox2_4x64s7"
+    second = "conv_bf16_f32_tobf16_64x64s7" if variant == "fp32_rows_in" else "conv_bf16_x2_tobf16_64x64s7"
+    assert names == [first, second, "conv_bf16_bf16_tox2_64x64s7", "conv_bf16_x2_tof32_64x64s7"], names
+    want = o_mesh.classify(f["Hoc"], o_lens, f["image"], cfg.fourcc, vmo.Network(net))
+    worst = float(np.abs(got["cls"] - want["cls"]).max())
+    print("bf16 %s worst absolute error: %.3e" % (variant, worst), flush=True)
+    if variant == "selu_last":  # the outputs are not probabilities: the gate scales with their size
+        assert np.array_equal(got["gidx"], want["gidx"]) and np.array_equal(got["nb"], want["nb"])
+        assert worst <= BF16_TOL * max(1.0, float(np.abs(want["cls"]).max())), worst
+    else:
+        assert_classification_parity(got, want, BF16_TOL, "bf16 " + variant)
+
+
 def test_bf16_engine_keeps_narrow_networks_in_fp32(oracle):
     """Rows narrower than 64 channels are not worth bf16 storage (one rounding already costs ~1e-2 on a 3-class
     softmax): a bf16 engine built on configuration 2's network meets the fp32 gate."""

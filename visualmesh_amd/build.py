@@ -22,7 +22,7 @@ CXX = os.environ.get("CXX", "g++")
 ARCH = "gfx950"
 
 # Packed-fp32 instructions are switched off for all device code.
-HIP_FLAGS = ["--offload-arch=" + ARCH] + os.environ.get("VM_EXTRA_HIP_FLAGS", "").split() + [ "-O3", "-std=c++17", "-fPIC", "-I" + INCLUDE, "-I" + CSRC,
+HIP_FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC", "-I" + INCLUDE, "-I" + CSRC,
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument", "-Wno-inline-asm"]
 # Host code that must reproduce the reference's fp32 arithmetic: one IEEE operation per step.
 HOST_EXACT_FLAGS = ["-std=c++14", "-O2", "-ffp-contract=off", "-fPIC", "-Wall", "-Wextra"]

@@ -42,24 +42,12 @@
 #include <cstdlib>
 #include <cstring>
 #include <type_traits>
+#include <utility>
 
 #include <atomic>
 
 #include "vmhip_internal.h"
 
-#ifdef VM_BF16_TIMING
-__device__ unsigned long long vm_bf16_times[2][13];
-extern "C" void vm_bf16_read_times(unsigned long long* out, int clear) {
-    (void) hipMemcpyFromSymbol(out, HIP_SYMBOL(vm_bf16_times), 208);
-    if (clear) {
-        unsigned long long z[26] = {};
-        (void) hipMemcpyToSymbol(HIP_SYMBOL(vm_bf16_times), z, 208);
-    }
-}
-#define VM_T(i) { const unsigned long long now = __builtin_readcyclecounter(); t_acc[i] += now - t_last; t_last = now; }
-#else
-#define VM_T(i)
-#endif
 
 namespace {
 
@@ -84,6 +72,18 @@ __device__ __forceinline__ int find_frame_by_row_tile(const VmFrame* frames, int
         else hi = mid - 1;
     }
     return lo;
+}
+
+/* body(integral_constant<int, 0>) ... body(integral_constant<int, N - 1>): a loop whose index is a constant in every
+ * round, whatever the optimiser thinks of the size of what it unrolls (an index that stayed a variable would put the
+ * weights, an array in registers, into scratch memory) */
+template <class F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& body, std::integer_sequence<int, I...>) {
+    (body(std::integral_constant<int, I>()), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& body) {
+    static_for_impl(body, std::make_integer_sequence<int, N>());
 }
 
 /* selu with the hardware exponential: the branch that needs it has s < 0, where alpha * e^s - alpha is off by at most
@@ -149,6 +149,20 @@ __host__ __device__ constexpr int row_bytes(int fmt) { return fmt == VM_ROWS_BF1
 __host__ __device__ constexpr int bf16_buf_bytes(int in_fmt) { return BROWS * row_bytes(in_fmt) + BT * 16; }
 /* two row buffers (rows, then the half tile's neighbour table), a note per wave, the biases, the softmax's exchange */
 __host__ __device__ constexpr size_t bf16_lds_bytes(int in_fmt) { return 2 * size_t(bf16_buf_bytes(in_fmt)) + 4 * NOTE * 4 + CH * 4 + BT * 2 * 4; }
+
+/* the side work of a half tile in the order it is issued: every FILL_EVERY-th item is a load of the half tile after, the
+ * others are the pieces of the half tile before */
+constexpr int FILL_EVERY = 3;
+constexpr int slice_of_item(int item, int n_fill) { return item - (item / FILL_EVERY + 1 < n_fill ? item / FILL_EVERY + 1 : n_fill); }
+/* stores (pieces 32.., of which with fp32 or bf16 rows out only the even ones store) issued after the last load */
+constexpr int stores_after_fills(int n_fill, int n_slices, bool two_stores) {
+    int n = 0;
+    for (int item = FILL_EVERY * (n_fill - 1) + 1; slice_of_item(item, n_fill) < n_slices; ++item) {
+        const int sl = slice_of_item(item, n_fill);
+        if (sl >= 32 && (two_stores || (sl - 32) % 2 == 0)) ++n;
+    }
+    return n;
+}
 
 /* what a wave remembers of a half tile until its results are stored */
 struct Done {
@@ -367,27 +381,20 @@ __global__ __launch_bounds__(256) void vm_conv_bf16_kernel(VmBatchDev B, VmLayer
         return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<char*>(out) + (size_t) t.first * OUTB, 0, BT * OUTB, 0x00020000);
     };
 
-#ifdef VM_BF16_TIMING
-    unsigned long long t_acc[12] = {}, t_last = __builtin_readcyclecounter();
-#endif
     for (int k = 0; k < count; ++k) {
         const int b = k & 1;
         const char* const rows = lds + b * BUF;
-        VM_T(0)
         /* my loads of half tile k and the note of k+1 have landed once nothing but the stores issued after them can
          * be in flight (vector memory operations complete in order); before the first stores: once nothing is */
         if (k == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N_STORES) : "memory");
-        VM_T(1)
+        else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(stores_after_fills(N_FILL, 48, OUT_FMT == VM_ROWS_BF16X2)) : "memory");
         __syncthreads(); /* everyone's have landed; everyone has read the last of half tile k-1 */
-        VM_T(2)
         const int4 d_cur = d_next;
         d_next = read_note();
         Plan plan; /* the loads of half tile k+1 into the other buffer: issued between the matrix instructions below */
         plan_fill(d_next, k + 1 < count, b ^ 1, plan);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); /* the slot has been read: it may be written again */
         request_note(tile_of(k + 2), k + 2 < count);
-        VM_T(3)
 
         /* the lane's rows and where their gather slots lie in the buffer */
         Done cur;
@@ -413,11 +420,6 @@ __global__ __launch_bounds__(256) void vm_conv_bf16_kernel(VmBatchDev B, VmLayer
             }
         }
         const bool any_far = __any(far);
-        VM_T(4)
-#ifdef VM_BF16_TIMING
-        t_acc[7] += any_far ? 1 : 0;
-        const unsigned long long t_before = t_acc[5];
-#endif
 
         v16f acc[2];
 #pragma unroll
@@ -480,7 +482,7 @@ __global__ __launch_bounds__(256) void vm_conv_bf16_kernel(VmBatchDev B, VmLayer
             constexpr int CHUNKS = SLOTS * 4;
             constexpr int PER = WIDE ? 6 : 4;       /* matrix instructions per chunk */
             constexpr int ITEMS = WIDE ? 4 : 3;     /* ... of which so many are followed by an item of the side work */
-            static_assert(CHUNKS * ITEMS >= N_FILL + N_SLICES, "every item of the side work finds its place");
+            static_assert(CHUNKS * ITEMS >= FILL_EVERY * N_FILL + N_SLICES, "every item of the side work finds its place");
             /* The operands of a chunk are requested AHEAD chunks ahead: the four waves ask in step, and an LDS that serves
              * sixteen requests at once (more where lanes collide in a bank) and the loads landing in the other buffer takes
              * some hundred cycles to answer - more than the 128 cycles that a chunk of four matrix instructions lasts. */
@@ -491,47 +493,35 @@ __global__ __launch_bounds__(256) void vm_conv_bf16_kernel(VmBatchDev B, VmLayer
                 gather(c, 0, xh[c][0], xl[c][0]);
                 gather(c, 1, xh[c][1], xl[c][1]);
             }
-#pragma unroll
-            for (int c = 0; c < CHUNKS; ++c) {
-                const int s = c >> 2, j = c & 3, u = c % NB, u2 = (c + AHEAD) % NB;
-#ifdef VM_BF16_TIMING
-                if (!FAR && (c == 0 || c == 5 || c == 17)) { const unsigned long long now = __builtin_readcyclecounter(); t_acc[c == 0 ? 8 : c == 5 ? 9 : 10] -= now; t_acc[c == 0 ? 11 : c == 5 ? 8 : 9] += (c == 0 ? 0 : now); }
-#endif
+            static_for<CHUNKS>([&](auto chunk) {
+                constexpr int c = decltype(chunk)::value;
+                constexpr int s = c >> 2, j = c & 3, u = c % NB, u2 = (c + AHEAD) % NB;
                 const v8bf a_hi = __builtin_bit_cast(v8bf, w[s][j][0]), a_lo = __builtin_bit_cast(v8bf, w[s][j][1]);
                 /* A wave issues in order and a matrix instruction keeps the pipe busy for 32 cycles: whatever else is
                  * to be done goes between the matrix instructions, a little after each (the scheduling barriers keep
                  * it there). After the first two: the operands of the chunk after, one row block each. After some:
                  * an item of the side work - first the loads of half tile k+1, then the activation and stores of
                  * half tile k-1. */
-#pragma unroll
-                for (int m = 0; m < PER; ++m) {
-                    const int rb = m & 1;
-                    const int kind = m >> 1; /* x_hi * w_hi, then (hi + lo rows) x_lo * w_hi, then x_hi * w_lo */
+                static_for<PER>([&](auto mm) {
+                    constexpr int m = decltype(mm)::value;
+                    constexpr int rb = m & 1;
+                    constexpr int kind = m >> 1; /* x_hi * w_hi, then (hi + lo rows) x_lo * w_hi, then x_hi * w_lo */
                     const v8bf a_op = kind == PER / 2 - 1 ? a_lo : a_hi;
                     const v8bf b_op = __builtin_bit_cast(v8bf, (WIDE && kind == 1) ? xl[u][rb] : xh[u][rb]);
-#ifndef VM_EXP_NOMFMA
                     acc[rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_op, b_op, acc[rb], 0, 0, 0);
-#else
-                    asm volatile("" : "+v"(acc[rb]) : "v"(a_op), "v"(b_op));
-#endif
                     __builtin_amdgcn_sched_barrier(0);
-#ifndef VM_EXP_NOGATHER
-                    if (m < 2 && c + AHEAD < CHUNKS) gather(c + AHEAD, m, xh[u2][m], xl[u2][m]);
-#endif
-#ifndef VM_EXP_NOSIDE
-                    if (m >= PER - ITEMS) {
-                        const int item = c * ITEMS + (m - (PER - ITEMS));
-                        if (item < N_FILL) fill_item(item, plan);
-                        else if (item < N_FILL + N_SLICES) finish_slice(item - N_FILL, acc_done, done, rs);
+                    if constexpr (m < 2 && c + AHEAD < CHUNKS) gather(c + AHEAD, m, xh[u2][m], xl[u2][m]);
+                    if constexpr (m >= PER - ITEMS) {
+                        /* every third item is a load until there are no more: issued in a row they fill the memory
+                         * pipeline, and the wave stands at the issue of the next */
+                        constexpr int item = c * ITEMS + (m - (PER - ITEMS));
+                        if constexpr (item % FILL_EVERY == 0 && item / FILL_EVERY < N_FILL) fill_item(item / FILL_EVERY, plan);
+                        else if constexpr (slice_of_item(item, N_FILL) < N_SLICES) finish_slice(slice_of_item(item, N_FILL), acc_done, done, rs);
                     }
-#endif
                     __builtin_amdgcn_sched_barrier(0);
-                }
-            }
+                });
+            });
         };
-#ifdef VM_BF16_TIMING
-        if (!any_far) t_acc[11] += 1;
-#endif
         if (any_far) {
             contract(std::true_type());
             /* the side path's loads are not part of the count above: none may be in flight when the next wait counts */
@@ -541,23 +531,10 @@ __global__ __launch_bounds__(256) void vm_conv_bf16_kernel(VmBatchDev B, VmLayer
             contract(std::false_type());
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); /* every operand of the half tile has been read */
-#ifdef VM_BF16_TIMING
-        if (!any_far) t_acc[10] += __builtin_readcyclecounter();
-#endif
-        VM_T(5)
-#ifdef VM_BF16_TIMING
-        if (any_far) t_acc[6] += t_acc[5] - t_before; /* the part of phase 5 spent in half tiles with the side path */
-#endif
 #pragma unroll
         for (int rb = 0; rb < 2; ++rb) acc_done[rb] = acc[rb];
         done = cur;
     }
-#ifdef VM_BF16_TIMING
-    if (lane == 0) {
-        for (int i = 0; i < 12; ++i) atomicAdd(&vm_bf16_times[WIDE ? 1 : 0][i], t_acc[i]);
-        atomicAdd(&vm_bf16_times[WIDE ? 1 : 0][12], (unsigned long long) count);
-    }
-#endif
     /* the last half tile's results; and no LDS load may outlive the wave */
     __syncthreads(); /* the exchange area of the softmax is free again */
     if constexpr (ACT == VMHIP_SOFTMAX) prepare_softmax(acc_done);
