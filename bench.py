@@ -1,12 +1,14 @@
 """Benchmark of the Visual Mesh inference hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2] [--frames F] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2] [--frames F] [--no-cpu] [--no-pcie] [--no-configs]
 
 A step is one pass of the whole device path (projection, filter/compaction, sampling, neighbourhood, all
 graph-convolution layers) over one staged batch of synthetic frames whose inputs are already resident in
-device memory. Prints one JSON line: nodes classified per second, plus frames per second, the roofline
-position of the dominant kernel (timed live with HIP events on the engine's stream) and the CPU oracle
-timed on the host's cores as a baseline.
+device memory. Prints one JSON line: nodes classified per second (`value`, configuration 2 unless --config says
+otherwise), frames per second, the roofline position of the dominant kernel (timed live with HIP events on the
+engine's stream), the reference's CPU engine timed on the host's cores as a baseline, the end-to-end figure (host
+images to classified mesh in host arrays, pipelined over three engines) next to the serial one, and a short run of
+each of the other configurations (`configs`).
 """
 import argparse
 import json
@@ -25,12 +27,30 @@ HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 FP32_PEAK_TFLOPS = 157.3   # MI355X dense fp32 matrix
 BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix
 
-# HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, keyed by
-# (workload, kernel); filled in from the summaries under profiles/ (None = not measured).
-MEASURED_TRAFFIC = {
-    # profiles/conv_flow_32x32_config2.md: (2.0 * 76506.2 + 131194.2) KiB per launch
-    ("cfg2", "conv_flow_32x32s7"): int((2.0 * 76506.2 + 131194.2) * 1024),
-}
+def measured_traffic(workload, kernel):
+    """HBM bytes per launch of `kernel` on `workload` from the rocprofv3 FETCH_SIZE / WRITE_SIZE summaries under
+    profiles/: each summary carries lines
+        <!-- traffic: workload=cfg2 kernel=conv_flow_32x32s7 bytes_per_launch=N source=<kernel source file> sha256=<of that file> -->
+    written when the counters were read. A figure counts only while the kernel's source is still the file that was
+    measured; otherwise (or without a summary) -> (None, why)."""
+    import glob
+    import hashlib
+    import re
+    found = None
+    for path in sorted(glob.glob(os.path.join(ROOT, "profiles", "*.md"))):
+        for m in re.finditer(r"<!-- traffic: workload=(\S+) kernel=(\S+) bytes_per_launch=(\d+) source=(\S+) sha256=([0-9a-f]+) -->", open(path).read()):
+            if m.group(1) == workload and m.group(2) == kernel:
+                found = (int(m.group(3)), m.group(4), m.group(5), os.path.basename(path))
+    if found is None:
+        return None, "no counter summary under profiles/ for this kernel and workload"
+    nbytes, source, sha, where = found
+    try:
+        now = hashlib.sha256(open(os.path.join(ROOT, source), "rb").read()).hexdigest()
+    except OSError:
+        return None, "the measured source file %s is gone" % source
+    if now != sha:
+        return None, "profiles/%s was measured on another version of %s" % (where, source)
+    return nbytes, "profiles/" + where
 
 
 def layer_table(cfg, n_neighbours):
@@ -119,38 +139,12 @@ def cpu_baseline(cfg, threads, passes):
     return sum(visible) * passes / dt, len(frames) * passes / dt, dt, kind
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    # a pass takes about a millisecond and the GPU's clocks need some tens of them to settle: the defaults time one
-    # second of steady state (20 timed passes after 3 read 4-8 % slower)
-    ap.add_argument("--steps", type=int, default=None, help="timed passes (default 1000; 100 for configurations 4 and 5, whose pass takes 40-80 ms)")
-    ap.add_argument("--warmup", type=int, default=None, help="untimed passes before them (default 100; 10 for configurations 4 and 5)")
-    ap.add_argument("--config", type=int, default=2, help="workload configuration 1..5 (default 2: batched 1280x1024)")
-    ap.add_argument("--frames", type=int, default=None, help="frames per batch (default: the configuration's own)")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    ap.add_argument("--no-events", action="store_true",
-                    help="no HIP events in the timed passes (they then replay the captured HIP graph); no roofline is reported")
-    ap.add_argument("--copy-probe", action="store_true",
-                    help="accepted for older command lines: the 1 GiB plain copy kernel (the practical ceiling of the memory "
-                         "system and the dispatch of known size that memory counters are scaled by) runs unless --no-copy-probe")
-    ap.add_argument("--no-copy-probe", action="store_true", help="skip the plain copy kernel")
-    ap.add_argument("--no-pcie", action="store_true", help="skip the PCIe-inclusive passes (stage + run + fetch through page-locked host memory)")
-    args = ap.parse_args()
-    big = args.config in (4, 5)
-    args.steps = (100 if big else 1000) if args.steps is None else args.steps
-    args.warmup = (10 if big else 100) if args.warmup is None else args.warmup
-    if args.gpus != 1:
-        print("bench.py measures one GPU: this build has no multi-GPU path (frames would shard across GPUs "
-              "without any exchange); run with --gpus 1", file=sys.stderr)
-        sys.exit(2)
-
+def build_workload(index, n_frames=None):
+    """configuration `index` staged on a fresh engine -> (cfg, engine, mesh, lens, frames)"""
     from visualmesh_amd import engine as eng
     from visualmesh_amd import native
     from visualmesh_amd import workloads as wl
-
-    cfg = wl.config(args.config, n_frames=args.frames)
-    nn = wl.N_NEIGHBOURS[cfg.model]
+    cfg = wl.config(index, n_frames=n_frames)
     lens = native.make_lens(*cfg.lens_tuple())
     if cfg.visualmesh is None:
         mesh = eng.Mesh(cfg.model, cfg.shape, cfg.radius, cfg.mesh_h, cfg.k, cfg.max_distance)
@@ -160,9 +154,32 @@ def main():
     precision = native.BF16 if cfg.precision == "bf16" else native.FP32
     engine = eng.Engine(cfg.network, cfg.model, precision)
     frames = [dict(mesh=mesh, Hoc=f["Hoc"], lens=lens, image=f["image"], fourcc=cfg.fourcc) for f in cfg.frames]
+    return cfg, engine, mesh, lens, frames
 
-    engine.stage(frames)          # inputs become resident in HBM here, outside the timed region
-    for _ in range(args.warmup):
+
+def workload_name(cfg, n_frames, table):
+    from visualmesh_amd import workloads as wl
+    return "%s: %d frames of %dx%d %s, %s lens, %s mesh, network %s" % (
+        cfg.name, n_frames, cfg.width, cfg.height, "RGBA8" if cfg.fourcc == wl.fourcc("RGBA") else "GRBG8",
+        {0: "rectilinear", 1: "equisolid", 2: "equidistant"}[cfg.projection],
+        {0: "Ring6", 1: "NMGrid8"}[cfg.model], "->".join(["4"] + [str(t[1]) for t in table]))
+
+
+def measure(cfg, engine, frames, steps, warmup, settle_s, events=True):
+    """Stages `frames` (inputs resident in HBM from then on), lets the clocks settle, then W untimed and K timed passes.
+    -> dict with the throughput, the dominant kernel's roofline (timed live with HIP events on the engine's stream in the
+    timed passes) and every graph-convolution kernel's (from one fully bracketed, untimed pass)."""
+    from visualmesh_amd import workloads as wl
+    nn = wl.N_NEIGHBOURS[cfg.model]
+    engine.stage(frames)
+    # The GPU's clocks need some tens of milliseconds of work to settle (20 timed passes right after staging read 4-8 %
+    # slower): an untimed pre-roll of the same pass, stated in the result, comes before the warm-up passes.
+    settle_passes, t0 = 0, time.perf_counter()
+    while settle_s > 0 and (time.perf_counter() - t0 < settle_s or settle_passes < 3):
+        engine.run()
+        settle_passes += 1
+    settle_ms = (time.perf_counter() - t0) * 1e3
+    for _ in range(warmup):
         engine.run()
     visible = engine.counts()
     nodes = int(visible.sum())
@@ -173,30 +190,26 @@ def main():
     # the gap it causes) between every two kernels.
     engine.profile(1)
     engine.run()
-    kernel_ms_per_step = {}
-    launches_per_step = {}
+    kernel_ms_per_step, launches_per_step = {}, {}
     for name, ms, units in engine.profile_read():
         kernel_ms_per_step[name] = kernel_ms_per_step.get(name, 0.0) + ms
         launches_per_step[name] = launches_per_step.get(name, 0) + 1
-    engine.profile(0 if args.no_events else 2)   # --no-events: the timed passes replay the captured HIP graph
-    kernel_ms = {}
-    kernel_launches = {}
+    engine.profile(2 if events else 0)   # without events the timed passes replay the captured HIP graph
+    kernel_ms, kernel_launches = {}, {}
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         engine.run()              # launches the whole path and waits for it
-        if args.no_events:
+        if not events:
             continue
         for name, ms, units in engine.profile_read():
             kernel_ms[name] = kernel_ms.get(name, 0.0) + ms
             kernel_launches[name] = kernel_launches.get(name, 0) + 1
     elapsed = time.perf_counter() - t0
-    ms_per_step = elapsed * 1e3 / args.steps
-    value = nodes * args.steps / elapsed
+    engine.profile(0)
 
     # roofline of the dominant kernel: a graph-convolution kernel, or (small single-frame workloads) one of the
     # kernels before the network, which move bytes only
     rows = nodes + len(frames)    # visible nodes + one null row per frame
-    table = layer_table(cfg, nn)
     conv = {k: v for k, v in kernel_ms.items() if k.startswith("conv")}
     dominant = max(conv, key=conv.get) if conv else None
     roofline = None
@@ -207,41 +220,127 @@ def main():
         texel_bytes = 16 if cfg.fourcc == wl.fourcc("RGBA") else 36   # four RGBA8 texels / the 6x6 union of four Bayer patches
         algorithmic = {"project": 12 * candidates + 12 * nodes,            # rays read; pixel and index written per visible node
                        "compact_sample": (texel_bytes + 16) * nodes,       # texels read, four floats written
-                       "neighbourhood": 12 * nn * nodes}[dominant]         # table read, reverse-lookup gathers, table written
+                       "neighbourhood": 12 * nn * nodes,                   # table read, reverse-lookup gathers, table written
+                       "half_tables": (4 * nn + 16) * nodes}[dominant]     # table read, half-tile positions written
         achieved = algorithmic / (avg_ms * 1e-3) / 1e9
         roofline = dict(bound="hbm", achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s", frac=achieved / HBM_PEAK_GBS, kernel=dominant,
-                        avg_launch_ms=avg_ms, launches_per_step=kernel_launches[dominant] // args.steps, algorithmic_bytes_per_launch=algorithmic,
-                        traffic=MEASURED_TRAFFIC.get((cfg.name, dominant)))
+                        avg_launch_ms=avg_ms, launches_per_step=kernel_launches[dominant] // steps, algorithmic_bytes_per_launch=algorithmic)
     elif dominant:
         avg_ms = kernel_ms[dominant] / kernel_launches[dominant]
         roofline, bytes_per_row, flops_per_row = conv_roofline(dominant, avg_ms, rows)
-        roofline.update(kernel=dominant, avg_launch_ms=avg_ms, launches_per_step=kernel_launches[dominant] // args.steps,
-                        rows_per_launch=rows, algorithmic_bytes_per_row=bytes_per_row, flops_per_row=flops_per_row,
-                        traffic=MEASURED_TRAFFIC.get((cfg.name, dominant)))
+        roofline.update(kernel=dominant, avg_launch_ms=avg_ms, launches_per_step=kernel_launches[dominant] // steps,
+                        rows_per_launch=rows, algorithmic_bytes_per_row=bytes_per_row, flops_per_row=flops_per_row)
+    if roofline is not None:
+        roofline["traffic"], roofline["traffic_source"] = measured_traffic(cfg.name, dominant)
 
     # every graph-convolution kernel against its own roofline, from the one fully bracketed (untimed) pass
     conv_rooflines = {}
     for name, ms in sorted(kernel_ms_per_step.items()):
         if name.startswith("conv"):
-            entry = conv_roofline(name, ms / launches_per_step[name], nodes + len(frames))[0]
-            conv_rooflines[name] = dict(bound=entry["bound"], achieved=entry["achieved"], unit=entry["unit"], frac=entry["frac"])
+            entry = conv_roofline(name, ms / launches_per_step[name], rows)[0]
+            conv_rooflines[name] = dict(bound=entry["bound"], achieved=entry["achieved"], unit=entry["unit"], frac=entry["frac"],
+                                        avg_launch_ms=ms / launches_per_step[name])
+    return dict(value=nodes * steps / elapsed, frames_per_s=len(frames) * steps / elapsed, ms_per_step=elapsed * 1e3 / steps, nodes=nodes,
+                settle_passes=settle_passes, settle_ms=settle_ms, roofline=roofline, kernel_ms_per_step=dict(sorted(kernel_ms_per_step.items())),
+                conv_rooflines=conv_rooflines)
+
+
+def pinned_copies(cfg, mesh, lens):
+    from visualmesh_amd import native
+    held = []
+    for f in cfg.frames:
+        a = native.pinned_empty(f["image"].shape, f["image"].dtype)
+        a[...] = f["image"]
+        held.append(a)
+    return held, [dict(mesh=mesh, Hoc=f["Hoc"], lens=lens, image=a, fourcc=cfg.fourcc) for f, a in zip(cfg.frames, held)]
+
+
+def end_to_end(cfg, mesh, lens, nodes, batches):
+    """What a caller pays per batch from host images to the whole classified mesh in host arrays (the reference
+    benchmark's frame: example/benchmark.cpp:50-58 runs the whole operator() per frame): the host's lookups, the upload of
+    images, poses and ranges, every kernel, and the download of pixels, indices, neighbourhoods and probabilities. Three
+    engines in rotation, one staging, one running and one copying its results out at any time, all buffers page-locked;
+    the timed region covers `batches` batches in steady state."""
+    from visualmesh_amd import engine as eng
+    from visualmesh_amd import native
+    from visualmesh_amd import workloads as wl
+    precision = native.BF16 if cfg.precision == "bf16" else native.FP32
+    engines = [eng.Engine(cfg.network, cfg.model, precision) for _ in range(3)]
+    held, frames = pinned_copies(cfg, mesh, lens)
+
+    def rotate(n):
+        for step in range(n + 2):
+            if step < n:
+                e = engines[step % 3]
+                e.stage(frames)
+                e.run_async()
+            if 1 <= step <= n:
+                e = engines[(step - 1) % 3]
+                e.wait()
+                e.fetch_pinned(wait=False)
+            if step >= 2:
+                engines[(step - 2) % 3].fetch_wait()
+
+    rotate(6)  # buffers allocated, graphs captured
+    t0 = time.perf_counter()
+    rotate(batches)
+    dt = (time.perf_counter() - t0) / batches
+    nn = wl.N_NEIGHBOURS[cfg.model]
+    classes = cfg.network[-1][-1][0].shape[1]
+    h2d = sum(int(f["image"].nbytes) for f in cfg.frames)
+    d2h = nodes * (8 + 4) + (nodes + len(cfg.frames)) * 4 * (nn + classes)
+    return dict(ms_per_batch=dt * 1e3, nodes_per_s=nodes / dt, frames_per_s=len(cfg.frames) / dt, engines=3, batches=batches,
+                h2d_bytes_per_batch=h2d, d2h_bytes_per_batch=d2h, pcie_GBps_each_way=[h2d / dt / 1e9, d2h / dt / 1e9],
+                what="host lookup + upload from page-locked images + all kernels + download of the whole classified mesh into "
+                     "page-locked arrays; three engines in rotation (one staging, one running, one copying out)")
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=None, help="timed passes (default 1000; 50 for configurations 4 and 5, whose pass takes 20-80 ms)")
+    ap.add_argument("--warmup", type=int, default=None, help="untimed passes before them (default 100; 5 for configurations 4 and 5)")
+    ap.add_argument("--settle", type=float, default=0.25, help="seconds of untimed passes before the warm-up, for the clocks to settle (0: none)")
+    ap.add_argument("--config", type=int, default=2, help="workload configuration 1..5 (default 2: batched 1280x1024)")
+    ap.add_argument("--frames", type=int, default=None, help="frames per batch (default: the configuration's own)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--no-events", action="store_true",
+                    help="no HIP events in the timed passes (they then replay the captured HIP graph); no roofline is reported")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="accepted for older command lines: the 1 GiB plain copy kernel (the practical ceiling of the memory "
+                         "system and the dispatch of known size that memory counters are scaled by) runs unless --no-copy-probe")
+    ap.add_argument("--no-copy-probe", action="store_true", help="skip the plain copy kernel")
+    ap.add_argument("--no-pcie", action="store_true", help="skip the PCIe-inclusive figures (serial stage + run + fetch, and the pipelined end-to-end loop)")
+    ap.add_argument("--no-configs", action="store_true", help="skip the short runs of the other configurations")
+    args = ap.parse_args()
+    big = args.config in (4, 5)
+    args.steps = (50 if big else 1000) if args.steps is None else args.steps
+    args.warmup = (5 if big else 100) if args.warmup is None else args.warmup
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (frames would shard across GPUs "
+              "without any exchange); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    from visualmesh_amd import native
+    from visualmesh_amd import workloads as wl
+
+    cfg, engine, mesh, lens, frames = build_workload(args.config, args.frames)
+    nn = wl.N_NEIGHBOURS[cfg.model]
+    m = measure(cfg, engine, frames, args.steps, args.warmup, args.settle, events=not args.no_events)
+    nodes = m["nodes"]
+    table = layer_table(cfg, nn)
 
     copy_gbs = None
     if not args.no_copy_probe:
         nbytes = 1 << 30
         copy_gbs = 2 * nbytes / (native.copy_probe(nbytes, 5) * 1e-3) / 1e9
 
-    # PCIe-inclusive figure (never `value`): images in page-locked host memory -> stage + run + fetch of the whole
-    # classified mesh into page-locked host arrays, one engine, the three steps one after the other
-    pcie = None
+    # PCIe-inclusive figures (never `value`). Serial: images in page-locked host memory -> stage + run + fetch of the
+    # whole classified mesh into page-locked host arrays, one engine, the three steps one after the other. Pipelined:
+    # end_to_end() above.
+    pcie, e2e = None, None
     if not args.no_pcie:
-        engine.profile(0)
-        held = []
-        for f in cfg.frames:
-            a = native.pinned_empty(f["image"].shape, f["image"].dtype)
-            a[...] = f["image"]
-            held.append(a)
-        pinned_frames = [dict(mesh=mesh, Hoc=f["Hoc"], lens=lens, image=a, fourcc=cfg.fourcc) for f, a in zip(cfg.frames, held)]
+        held, pinned_frames = pinned_copies(cfg, mesh, lens)
         for _ in range(2):
             engine.stage(pinned_frames), engine.run(), engine.fetch_pinned()
         passes = 5
@@ -251,6 +350,8 @@ def main():
         dt = (time.perf_counter() - t0) / passes
         pcie = dict(ms_per_batch=dt * 1e3, nodes_per_s=nodes / dt, frames_per_s=len(frames) / dt,
                     what="stage from page-locked images + run + fetch into page-locked arrays, one engine, serial")
+        del held, pinned_frames
+        e2e = end_to_end(cfg, mesh, lens, nodes, 12 if big else 60)
 
     cpu = None
     if not args.no_cpu:
@@ -280,35 +381,52 @@ def main():
             pass
         cpu = dict(value=nps, unit="nodes/s", cores=threads, kind=kind, cpu_model=model, one_thread=one, frames_per_s=fps, seconds=dt, sample=note)
 
+    # the other configurations, briefly (device-resident like `value`; each one's dominant kernel against its roofline)
+    others = None
+    if not args.no_configs:
+        others = {}
+        del engine, frames
+        for index in (1, 2, 3, 4, 5):
+            if index == args.config:
+                continue
+            heavy = index in (4, 5)
+            c, e, _, _, fr = build_workload(index)
+            r = measure(c, e, fr, 10 if heavy else 300, 2 if heavy else 30, 0.1 if heavy else args.settle, events=True)
+            others[c.name] = dict(workload=workload_name(c, len(fr), layer_table(c, wl.N_NEIGHBOURS[c.model])), dtype="bf16" if c.precision == "bf16" else "f32",
+                                  nodes_per_s=r["value"], frames_per_s=r["frames_per_s"], ms_per_step=r["ms_per_step"], steps=10 if heavy else 300,
+                                  visible_nodes_per_batch=r["nodes"], roofline=r["roofline"], conv_rooflines=r["conv_rooflines"])
+            del e, fr, c
+
     out = {
         "metric": "mesh nodes classified/sec",
-        "value": value,
+        "value": m["value"],
         "unit": "nodes/s",
-        "frames_per_s": len(frames) * args.steps / elapsed,
+        "frames_per_s": m["frames_per_s"],
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": ms_per_step,
+        "ms_per_step": m["ms_per_step"],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "bf16" if cfg.precision == "bf16" else "f32",
         "data": "synthetic",
         "config": {
-            "workload": "%s: %d frames of %dx%d %s, %s lens, %s mesh, network %s" % (
-                cfg.name, len(frames), cfg.width, cfg.height, "RGBA8" if cfg.fourcc == wl.fourcc("RGBA") else "GRBG8",
-                {0: "rectilinear", 1: "equisolid", 2: "equidistant"}[cfg.projection],
-                {0: "Ring6", 1: "NMGrid8"}[cfg.model], "->".join(["4"] + [str(t[1]) for t in table])),
-            "frames": len(frames),
+            "workload": workload_name(cfg, len(cfg.frames), table),
+            "frames": len(cfg.frames),
             "visible_nodes_per_batch": nodes,
             "inputs": "resident in HBM before the timed region",
+            "settle_passes": m["settle_passes"],   # untimed, before the warm-up passes: the clocks settle
+            "settle_ms": m["settle_ms"],
         },
-        "roofline": roofline,
+        "roofline": m["roofline"],
         "cpu_baseline": cpu,
         "copy_kernel_GBps": copy_gbs,
+        "end_to_end": e2e,
         "pcie_inclusive": pcie,
-        "kernel_ms_per_step": dict(sorted(kernel_ms_per_step.items())),   # from the one fully profiled, untimed pass
-        "conv_rooflines": conv_rooflines,
+        "kernel_ms_per_step": m["kernel_ms_per_step"],   # from the one fully profiled, untimed pass
+        "conv_rooflines": m["conv_rooflines"],
+        "configs": others,
     }
     print(json.dumps(out))
 

@@ -3,6 +3,8 @@ import ctypes
 import os
 import re
 
+import pytest
+
 from visualmesh_amd import native
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -59,3 +61,31 @@ def build_integration_snippet(directory):
 
 def test_reference_call_sites_compile_against_the_host_headers(tmp_path):
     assert os.path.exists(build_integration_snippet(tmp_path))
+
+
+REFERENCE_CPP = "/root/reference/cpp"
+
+
+@pytest.mark.skipif(not os.path.isdir(os.path.join(REFERENCE_CPP, "visualmesh")), reason="the reference tree is not mounted here")
+def test_engine_header_compiles_against_the_references_own_headers():
+    """engine/hip/engine.hpp dropped into the reference tree: its Mesh, VisualMesh, Lens, NetworkStructure, ProjectedMesh and
+    ClassifiedMesh are then the reference's (their include directory comes first); syntax and templates only."""
+    import subprocess
+    cmd = ["g++", "-std=c++14", "-fsyntax-only", "-Wall", "-Wextra", "-I" + REFERENCE_CPP, "-I" + os.path.join(ROOT, "visualmesh_amd", "cpp"),
+           "-I" + os.path.join(ROOT, "include"), os.path.join(ROOT, "tests", "native", "reference_interface.cpp")]
+    done = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, universal_newlines=True)
+    assert done.returncode == 0, done.stdout[-4000:]
+    # the reference's headers were really the ones found: a dependency list names them
+    deps = subprocess.run(cmd[:2] + ["-MM"] + cmd[3:], stdout=subprocess.PIPE, universal_newlines=True, check=True).stdout
+    assert REFERENCE_CPP + "/visualmesh/mesh.hpp" in deps and "visualmesh_amd/cpp/visualmesh/engine/hip/engine.hpp" in deps, deps
+    assert "visualmesh_amd/cpp/visualmesh/mesh.hpp" not in deps, deps
+
+
+def test_engine_can_be_compiled_out():
+    """VISUALMESH_DISABLE_HIP (what cmake/HipEngine.cmake defines when BUILD_HIP_ENGINE is off, as the reference does for
+    its OpenCL and Vulkan engines) leaves an empty header: nothing of the HIP library is needed then."""
+    import subprocess
+    src = '#include "visualmesh/engine/hip/engine.hpp"\n#ifdef VISUALMESH_HIP_H\n#error the C ABI header was included\n#endif\nint main() { return 0; }\n'
+    done = subprocess.run(["g++", "-std=c++14", "-fsyntax-only", "-DVISUALMESH_DISABLE_HIP", "-I" + os.path.join(ROOT, "visualmesh_amd", "cpp"), "-x", "c++", "-"],
+                          input=src, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, universal_newlines=True)
+    assert done.returncode == 0, done.stdout[-2000:]

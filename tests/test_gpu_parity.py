@@ -52,7 +52,8 @@ def test_config1_projection_only(oracle):
 
 
 def test_config2_batch(oracle):
-    _run_config(oracle, 2, 4, batch=True)
+    """all 16 frames of the batch against the oracle"""
+    _run_config(oracle, 2, 16, batch=True)
 
 
 def test_config3_bayer(oracle):
@@ -244,7 +245,7 @@ def test_bf16_engine_keeps_narrow_networks_in_fp32(oracle):
     assert_classification_parity(got, want, PROB_TOL, "bf16 engine, narrow network")
 
 
-@pytest.mark.parametrize("kernel", ["rows", "mfma", "lds", "dma", "flow"])
+@pytest.mark.parametrize("kernel", ["rows", "mfma", "lds", "flow"])
 def test_every_convolution_kernel_agrees_with_the_oracle(oracle, kernel, monkeypatch):
     """Every layer shape of configuration 2 through the one-row-per-lane kernel, the matrix-core kernel that
     gathers into registers and the matrix-core kernels that gather from LDS (rows staged through registers /
@@ -274,7 +275,7 @@ def test_every_convolution_kernel_agrees_with_the_oracle(oracle, kernel, monkeyp
         assert_classification_parity(results[i], want, PROB_TOL, "%s frame %d" % (kernel, i))
 
 
-@pytest.mark.parametrize("kernel", ["lds", "dma", "flow"])
+@pytest.mark.parametrize("kernel", ["lds", "flow"])
 @pytest.mark.parametrize("index", [2, 3])
 def test_rows_beyond_the_halo_capacity(oracle, index, kernel, monkeypatch):
     """With only 8 halo slots per tile most out-of-tile neighbours are marked as not staged and the LDS kernel
@@ -338,7 +339,7 @@ def _example_network():
 def test_reference_example_network_on_its_dataset_poses(oracle):
     """The reference's exported example network (example/model.yaml: 4->16, 16->16 x5, 16->8, 8->8 x5, 8->5) on the
     lens and camera pose of its dataset elements (example/images/lens*.yaml, rectilinear 1280x1024), with synthetic
-    BGRA images: projection on all 30 poses, probabilities on 3 of them in one batch."""
+    BGRA images: projection and probabilities on all 30 poses, classified in one batch."""
     network, meta = _example_network()
     assert meta["mesh"] == "RING6" and meta["shape"] == "SPHERE"
     heights = [p["Hoc"][2][3] for p in meta["poses"]]  # 0.78 m to 1.2 m: one mesh per height band, as the reference does
@@ -354,7 +355,7 @@ def test_reference_example_network_on_its_dataset_poses(oracle):
         views.append((np.array(p["Hoc"], np.float32), vmo.make_lens(*args), native.make_lens(*args), p))
     for Hoc, o_lens, e_lens, p in views:
         assert_projection_parity(engine(e_mesh, Hoc, e_lens), pick(o_mesh, Hoc).project(Hoc, o_lens), "example pose " + p["number"])
-    chosen = [views[i] for i in (0, 11, 29)]
+    chosen = views
     images = [wl.random_image(rng, p["width"], p["height"], 4) for _, _, _, p in chosen]
     frames = [dict(mesh=e_mesh, Hoc=H, lens=el, image=im, fourcc=wl.fourcc("BGRA")) for (H, _, el, _), im in zip(chosen, images)]
     results = engine.classify_batch(frames)

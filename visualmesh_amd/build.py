@@ -63,7 +63,6 @@ def build_hip(force=False):
         ("conv_mfma.hip", HIP_FLAGS),
         ("conv_bf16.hip", HIP_FLAGS),
         ("conv_lds.hip", HIP_FLAGS),
-        ("conv_dma.hip", HIP_FLAGS),
         ("conv_flow.hip", HIP_FLAGS),
         ("conv_narrow.hip", HIP_FLAGS),
         ("detect.hip", HIP_FLAGS),

@@ -30,6 +30,11 @@
 #ifndef VISUALMESH_ENGINE_HIP_ENGINE_HPP
 #define VISUALMESH_ENGINE_HIP_ENGINE_HPP
 
+/* VISUALMESH_DISABLE_HIP compiles the engine out, as VISUALMESH_DISABLE_OPENCL / _VULKAN do for the reference's engines
+ * (reference cpp/CMakeLists.txt:30-53, example/benchmark.cpp:141-146): cmake/HipEngine.cmake defines it unless
+ * BUILD_HIP_ENGINE is on. */
+#if !defined(VISUALMESH_DISABLE_HIP)
+
 #include <algorithm>
 #include <cstdint>
 #include <array>
@@ -631,4 +636,5 @@ namespace engine {
 }  // namespace engine
 }  // namespace visualmesh
 
+#endif  // !defined(VISUALMESH_DISABLE_HIP)
 #endif  // VISUALMESH_ENGINE_HIP_ENGINE_HPP

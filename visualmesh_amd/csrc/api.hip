@@ -102,7 +102,7 @@ struct HostLayer {
     void* d_w_mfma = nullptr;
     float* d_w_flow = nullptr; /* w_mfma in conv_flow.hip's LDS order */
     int32_t in_bf16 = 0, out_bf16 = 0, arith_bf16 = 0;
-    bool use_lds = false, use_mfma = false, use_dma = false, use_flow = false, use_narrow = false; /* which matrix-core kernels may take the layer */
+    bool use_lds = false, use_mfma = false, use_flow = false, use_narrow = false; /* which matrix-core kernels may take the layer */
     std::vector<float> h_w; /* kept until the row types are planned */
 };
 
@@ -458,7 +458,6 @@ int batch_enqueue(vmhip_batch* b) {
             if (L.arith_bf16) rc = vm_launch_conv_bf16(D, ld, b->d_act[cur].p, b->d_act[cur ^ 1].p, s, &name);
             if (rc != 0 && !L.arith_bf16 && L.use_narrow && D.row_nbl) rc = vm_launch_conv_narrow(D, ld, b->d_act[cur].as<float>(), b->d_act[cur ^ 1].as<float>(), s, &name);
             if (rc != 0 && L.use_flow && D.row_nbl) rc = vm_launch_conv_flow(D, ld, b->d_act[cur].as<float>(), b->d_act[cur ^ 1].as<float>(), s, &name);
-            if (rc != 0 && L.use_dma && D.row_nbl) rc = vm_launch_conv_dma(D, ld, b->d_act[cur].as<float>(), b->d_act[cur ^ 1].as<float>(), s, &name);
             if (rc != 0 && L.use_lds && D.row_nbl) rc = vm_launch_conv_lds(D, ld, b->d_act[cur].as<float>(), b->d_act[cur ^ 1].as<float>(), s, &name);
             if (rc != 0 && L.d_w_mfma && L.use_mfma) rc = vm_launch_conv_mfma(D, ld, b->d_act[cur].as<float>(), b->d_act[cur ^ 1].as<float>(), s, &name);
             /* the one-row-per-lane kernels only know fp32 rows */
@@ -736,13 +735,12 @@ int vmhip_engine_create(const vmhip_network* net, int32_t n_neighbours, int32_t 
     {
         /* VMHIP_CONV_KERNEL selects the kernel family for A/B runs: "rows" = one row per lane, "mfma" = matrix
          * cores gathering into registers, "lds" = matrix cores gathering from LDS (rows staged through registers),
-         * "dma" = the same with rows loaded straight into LDS, "flow" = that without barriers in the tile loop,
+         * "flow" = the same with rows loaded straight into LDS and no barriers in the tile loop,
          * wherever the shape has an instantiation; unset = the fastest measured kernel per layer shape */
         const char* pick = getenv("VMHIP_CONV_KERNEL");
         const bool rows_only = pick && std::string(pick) == "rows";
         const bool allow_lds = !rows_only && !(pick && std::string(pick) == "mfma");
         const bool force_lds = pick && std::string(pick) == "lds";
-        const bool force_dma = pick && std::string(pick) == "dma";
         const bool force_flow = pick && std::string(pick) == "flow";
         if (const char* g = getenv("VMHIP_GRAPH")) E->use_graph = atoi(g) != 0;
         if (const char* cap = getenv("VMHIP_HALO_CAP")) E->halo_cap = std::min(std::max(atoi(cap), 0), VMHIP_HALO_MAX);
@@ -768,7 +766,7 @@ int vmhip_engine_create(const vmhip_network* net, int32_t n_neighbours, int32_t 
             HostLayer& H = E->layers[l];
             H.in_bf16 = bf[l], H.out_bf16 = bf[l + 1], H.arith_bf16 = arith(l);
             const bool plain = !H.in_bf16 && !H.out_bf16 && !H.arith_bf16;
-            H.use_mfma = !rows_only && plain && vm_mfma_supported(H.c_in, H.c_out, H.slots, 0, 0, 0);
+            H.use_mfma = !rows_only && plain && vm_mfma_supported(H.c_in, H.c_out, H.slots);
             H.use_lds = allow_lds && !H.in_bf16 && !H.arith_bf16 && H.slots - 1 <= VMHIP_NBL_STRIDE && vm_lds_supported(H.c_in, H.c_out, H.slots, H.out_bf16);
             E->use_bf16 = E->use_bf16 || H.arith_bf16;
             /* Measured on the 16-frame 1280x1024 workload: the LDS gather is the faster matrix-core kernel on every
@@ -776,15 +774,14 @@ int vmhip_engine_create(const vmhip_network* net, int32_t n_neighbours, int32_t 
              * 2- and 3-class output layers are quicker with one row per lane (46 us against 56 us). */
             if (H.use_lds && !force_lds && H.c_out < 4) H.use_lds = false;
             if (H.out_bf16 && !H.arith_bf16 && !H.use_lds) return bail(VMHIP_ERR_ARGUMENT, "engine_create: no kernel writes the rows the next layer was planned to read");
-            H.use_dma = force_dma && plain && H.slots - 1 <= VMHIP_NBL_STRIDE && vm_dma_supported(H.c_in, H.c_out, H.slots);
             /* the barrier-free variant of the LDS gather is the faster one where the matrix pipe is the limit
              * (32 -> 32: 147 us against 158 us, 32 -> 16: 93 against 99) and makes no difference for 16-wide input */
-            H.use_flow = (force_flow || (allow_lds && !force_lds && !force_dma && H.c_in >= 32)) && plain && H.slots - 1 <= VMHIP_NBL_STRIDE
+            H.use_flow = (force_flow || (allow_lds && !force_lds && H.c_in >= 32)) && plain && H.slots - 1 <= VMHIP_NBL_STRIDE
                          && vm_flow_supported(H.c_in, H.c_out, H.slots);
             /* class layers (at most four output channels): the 4x4x1 matrix instruction, unless a family is forced */
-            H.use_narrow = allow_lds && !force_lds && !force_dma && plain && H.slots - 1 <= VMHIP_NBL_STRIDE
+            H.use_narrow = allow_lds && !force_lds && plain && H.slots - 1 <= VMHIP_NBL_STRIDE
                            && vm_narrow_supported(H.c_in, H.c_out, H.slots);
-            E->use_lds = E->use_lds || H.use_lds || H.use_dma || H.use_flow || H.use_narrow;
+            E->use_lds = E->use_lds || H.use_lds || H.use_flow || H.use_narrow;
             E->use_flow = E->use_flow || H.use_flow;
             if (H.arith_bf16) {
                 std::vector<unsigned char> wp(vm_bf16_weight_bytes(H.c_in, H.c_out, H.slots));
@@ -793,9 +790,9 @@ int vmhip_engine_create(const vmhip_network* net, int32_t n_neighbours, int32_t 
                 if (hipMemcpy(H.d_w_mfma, wp.data(), wp.size(), hipMemcpyHostToDevice) != hipSuccess)
                     return bail(VMHIP_ERR_HIP, "engine_create: weight upload failed");
             }
-            else if (H.use_mfma || H.use_lds || H.use_dma || H.use_flow) {
-                std::vector<unsigned char> wp(vm_mfma_weight_bytes(H.c_in, H.c_out, H.slots, 0));
-                vm_mfma_permute_weights(H.h_w.data(), H.c_in, H.c_out, H.slots, 0, wp.data());
+            else if (H.use_mfma || H.use_lds || H.use_flow) {
+                std::vector<unsigned char> wp(vm_mfma_weight_bytes(H.c_in, H.c_out, H.slots));
+                vm_mfma_permute_weights(H.h_w.data(), H.c_in, H.c_out, H.slots, wp.data());
                 if (hipMalloc(&H.d_w_mfma, wp.size()) != hipSuccess) return bail(VMHIP_ERR_HIP, "engine_create: out of device memory");
                 if (hipMemcpy(H.d_w_mfma, wp.data(), wp.size(), hipMemcpyHostToDevice) != hipSuccess)
                     return bail(VMHIP_ERR_HIP, "engine_create: weight upload failed");

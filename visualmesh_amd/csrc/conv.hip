@@ -11,6 +11,12 @@
  * vm_conv_generic_kernel: any shape, output channels in chunks of 8; the fallback for shapes that have no
  *   specialisation.
  */
+#include <atomic>
+#include <cstdio>
+#include <map>
+#include <mutex>
+#include <string>
+
 #include "vmhip_internal.h"
 
 namespace {
@@ -197,7 +203,23 @@ int vm_launch_conv(const VmBatchDev& B, const VmLayerDev& L, const float* in, fl
     ROWS_CASE(24, 24, 9)
     ROWS_CASE(24, 4, 9)
 #undef ROWS_CASE
+    /* no kernel knows this shape at compile time: one row per lane with loops over run-time widths. Said once per
+     * process, so that a network that lands here by accident (an input width that is not a multiple of four channels,
+     * more than 64 output channels, a gather of neither 7 nor 9 slots) is noticed. */
+    static std::atomic<bool> told{false};
+    if (!told.exchange(true))
+        fprintf(stderr, "visualmesh_hip: layer %d -> %d (%d gather slots) has no matrix-core kernel; it runs on the generic one-row-per-lane kernel\n",
+                L.c_in, L.c_out, L.slots);
     hipLaunchKernelGGL(vm_conv_generic_kernel, dim3(B.n_row_tiles), dim3(VMHIP_TILE), 0, stream, B, L, in, out);
     if (kernel_name) *kernel_name = "conv_generic";
     return 0;
+}
+
+const char* vm_kernel_name(const char* family, int c_in, int c_out, int slots) {
+    static std::mutex guard;
+    static std::map<std::string, std::string> names; /* node addresses of a map stay put */
+    char text[96];
+    snprintf(text, sizeof(text), "%s_%dx%ds%d", family, c_in, c_out, slots);
+    std::lock_guard<std::mutex> lock(guard);
+    return names.emplace(text, text).first->second.c_str();
 }

@@ -49,6 +49,12 @@
 #include "vmhip_internal.h"
 
 
+/* The activation code of this file is compiled three times per kernel (the usual half tile, the one with neighbours that
+ * are not staged, the last half tile of a block): no contraction of a multiplication and an addition at the compiler's
+ * discretion, which may differ between the copies - a row's result must not depend on which copy computed it. Where a
+ * fused multiply-add is wanted it is written out. */
+#pragma clang fp contract(off)
+
 namespace {
 
 typedef float v4f __attribute__((ext_vector_type(4)));
@@ -91,7 +97,7 @@ __device__ __forceinline__ void static_for(F&& body) {
 __device__ __forceinline__ float selu(float s) {
     const float lambda = 1.0507009873554804934193349852946f;
     const float alpha = 1.6732632423543772848170429916717f;
-    return lambda * (s >= 0.0f ? s : alpha * __builtin_amdgcn_exp2f(s * 1.44269504088896340736f) - alpha);
+    return lambda * (s >= 0.0f ? s : __builtin_fmaf(alpha, __builtin_amdgcn_exp2f(s * 1.44269504088896340736f), -alpha));
 }
 
 /* two floats -> two bf16 in one word, round to nearest even (v_cvt_pk_bf16_f32) */

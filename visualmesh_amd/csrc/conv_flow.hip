@@ -3,9 +3,9 @@
  * gather + dense + bias + activation in one kernel (reference engine/cpu/engine.hpp:213-264,
  * apply_activation.hpp:34-84).
  *
- * Contraction, operand layout, tile-local tables, XCD-aware persistent tile walk, the side path for neighbours that
- * are not staged, the staging by buffer_load ... lds and the two alternating row buffers are those of conv_dma.hip.
- * What differs is how the 16 waves of a block stay in step. A barrier makes all of them change phase together, so
+ * Contraction, operand layout, tile-local tables, XCD-aware persistent tile walk and the side path for neighbours that
+ * are not staged are those of conv_lds.hip; the rows go from global memory straight into LDS (buffer_load ... lds), into
+ * two alternating row buffers. What differs most is how the 16 waves of a block stay in step. A barrier makes all of them change phase together, so
  * the matrix pipe idles whenever the block applies activations, stores or waits for the barrier itself. Here two
  * counters per row buffer, kept in LDS, take its place:
  *   staged[b]   += 1 by every loader once its share of a tile's loads has landed in buffer b,

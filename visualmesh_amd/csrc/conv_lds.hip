@@ -30,33 +30,6 @@
 
 #include "vmhip_internal.h"
 
-/* Build with -DVM_LDS_TIMING to count, per phase of the tile loop, the shader clock cycles every wave spends in
- * it (first wave of every block, layers with C_IN = C_OUT = VM_LDS_TIMING; slot 7 counts tiles);
- * vm_lds_timing_read() returns and clears the sums. A development aid, compiled out otherwise. */
-#ifdef VM_LDS_TIMING
-__device__ unsigned long long vm_lds_timing[10];
-#define VM_T_DECL unsigned long long t_acc[10] = {}, t_prev = __builtin_readcyclecounter();
-#define VM_T_MARK(i)                                              \
-    {                                                             \
-        const unsigned long long t_now = __builtin_readcyclecounter(); \
-        t_acc[i] += t_now - t_prev;                               \
-        t_prev = t_now;                                           \
-    }
-#define VM_T_FLUSH                                                 \
-    if (threadIdx.x == 0 && C_IN == VM_LDS_TIMING && C_OUT == VM_LDS_TIMING) { /* wave 0 of every block, one layer shape */ \
-        for (int i = 0; i < 10; ++i) atomicAdd(&vm_lds_timing[i], t_acc[i]); \
-    }
-extern "C" int vm_lds_timing_read(unsigned long long* out) {
-    unsigned long long zero[10] = {};
-    if (hipMemcpyFromSymbol(out, HIP_SYMBOL(vm_lds_timing), sizeof(zero)) != hipSuccess) return -1;
-    return hipMemcpyToSymbol(HIP_SYMBOL(vm_lds_timing), zero, sizeof(zero)) == hipSuccess ? 0 : -1;
-}
-#else
-#define VM_T_DECL
-#define VM_T_MARK(i)
-#define VM_T_FLUSH
-#endif
-
 namespace {
 
 typedef float v4f __attribute__((ext_vector_type(4)));
@@ -120,15 +93,20 @@ __host__ __device__ constexpr int halo_rows(int c_in, int c_out, int slots) {
 }
 
 /* NW waves per block, RB row blocks of 16 rows per wave: NW * RB * 16 == VMHIP_TILE. */
-template <int C_IN, int C_OUT, int SLOTS, int NW, int HALO, int OUT_FMT>
+/* C_OUT_T > 0: that many output channels, known to the compiler. C_OUT_T < 0: -C_OUT_T column blocks of 16 and the
+ * layer's own count of output channels (L.c_out, at most 16 per block) read at run time - the instantiations that
+ * take every shape the enumerated ones leave out. */
+template <int C_IN, int C_OUT_T, int SLOTS, int NW, int HALO, int OUT_FMT>
 __global__ __launch_bounds__(NW * 64, 4) void vm_conv_lds_kernel(VmBatchDev B, VmLayerDev L, const float* __restrict__ in, float* __restrict__ out) {
-    static_assert(OUT_FMT == VM_ROWS_F32 || (OUT_FMT == VM_ROWS_BF16X2 && C_OUT % 16 == 0), "rows go out as fp32, or as hi + lo pairs of bf16 for a bf16 layer to read");
+    static_assert(OUT_FMT == VM_ROWS_F32 || (OUT_FMT == VM_ROWS_BF16X2 && C_OUT_T > 0 && C_OUT_T % 16 == 0), "rows go out as fp32, or as hi + lo pairs of bf16 for a bf16 layer to read");
+    constexpr bool ANY_WIDTH = C_OUT_T < 0;
+    const int C_OUT = ANY_WIDTH ? L.c_out : C_OUT_T;
     constexpr int RB = VMHIP_TILE / (16 * NW);
     static_assert(NW * RB * 16 == VMHIP_TILE, "a block covers one tile");
     static_assert(C_IN % 4 == 0, "rows are staged in 16-byte pieces");
     constexpr int NT = NW * 64;
     constexpr int STEPS = C_IN / 4; /* matrix steps per slot = floats in a lane's quarter row */
-    constexpr int CB = (C_OUT + 15) / 16;
+    constexpr int CB = ANY_WIDTH ? -C_OUT_T : (C_OUT_T + 15) / 16;
     constexpr int NN = SLOTS - 1;
     static_assert(NN <= VMHIP_NBL_STRIDE, "the tile-local neighbour table holds 8 entries per row");
     constexpr int RS = row_stride(C_IN);
@@ -248,13 +226,9 @@ __global__ __launch_bounds__(NW * 64, 4) void vm_conv_lds_kernel(VmBatchDev B, V
     request_positions(d_cur, nbl);
     int4 d_next = load_desc(min(next, t_last)), d_after = d_next;
     request_halo_rows(min(next, t_last));
-
-    VM_T_DECL
     while (true) {
         write_rows();
-        VM_T_MARK(0)
         __syncthreads(); /* rows (and, the first time, weights) are in LDS */
-        VM_T_MARK(1)
 
         const bool has_next = next < t_end;
         const int after = next + gx;
@@ -262,7 +236,6 @@ __global__ __launch_bounds__(NW * 64, 4) void vm_conv_lds_kernel(VmBatchDev B, V
         d_after = load_desc(min(after, t_last));
         request_halo_rows(min(after, t_last));
         __builtin_amdgcn_sched_barrier(0);
-        VM_T_MARK(2)
 
         {
             /* an empty tile (no rows in use) runs the same code on position 0 and stores nothing */
@@ -368,7 +341,6 @@ __global__ __launch_bounds__(NW * 64, 4) void vm_conv_lds_kernel(VmBatchDev B, V
             };
             if (any_far) contract(std::true_type());
             else contract(std::false_type());
-            VM_T_MARK(4)
             /* the next tile's neighbour positions: requested only now, when the operand registers are free */
             request_positions(d_next, nbl_next);
 
@@ -411,7 +383,6 @@ __global__ __launch_bounds__(NW * 64, 4) void vm_conv_lds_kernel(VmBatchDev B, V
                         for (int v = 0; v < 4; ++v) acc[rb][cb][v] = acc[rb][cb][v] / sum;
                 }
             }
-            VM_T_MARK(8)
             /* buffer stores relative to the tile's first output row; lanes without a row get an out-of-range
              * offset, which the hardware drops: no branch around the stores either */
             const __amdgpu_buffer_rsrc_t out_rsrc = make_rsrc(out + (size_t) d_cur.x * C_OUT, (uint64_t) VMHIP_TILE * C_OUT * 4);
@@ -438,27 +409,24 @@ __global__ __launch_bounds__(NW * 64, 4) void vm_conv_lds_kernel(VmBatchDev B, V
                         __builtin_amdgcn_raw_buffer_store_b64(hi, out_rsrc, valid[rb] ? at2 : 0xffffffffu, 0, 0);
                         __builtin_amdgcn_raw_buffer_store_b64(lo, out_rsrc, valid[rb] ? at2 + C_OUT * 2 : 0xffffffffu, 0, 0);
                     }
-                    else if constexpr (C_OUT % 4 == 0) {
+                    else if constexpr (!ANY_WIDTH && C_OUT_T % 4 == 0) {
+                        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, acc[rb][cb]), out_rsrc, (valid[rb] && o < C_OUT) ? at : 0xffffffffu, 0, 0);
+                    }
+                    else if (ANY_WIDTH && C_OUT % 4 == 0) { /* one uniform branch for the whole kernel: rows are whole 16-byte pieces */
                         __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, acc[rb][cb]), out_rsrc, (valid[rb] && o < C_OUT) ? at : 0xffffffffu, 0, 0);
                     }
                     else {
 #pragma unroll
                         for (int v = 0; v < 4; ++v)
-                            if (cb * 16 + v < C_OUT) /* compile-time: some lane group holds a real channel here */
+                            if (ANY_WIDTH || cb * 16 + v < C_OUT_T) /* known width: some lane group holds a real channel here */
                                 __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(acc[rb][cb][v]), out_rsrc,
                                                                       (valid[rb] && o + v < C_OUT) ? at + v * 4 : 0xffffffffu, 0, 0);
                     }
                 }
             }
         }
-
-        VM_T_MARK(5)
-#ifdef VM_LDS_TIMING
-        t_acc[7] += 1;
-#endif
         if (!has_next) break;
         __syncthreads(); /* every wave is done reading this tile's rows */
-        VM_T_MARK(6)
         d_cur = uniform(d_next);
         d_next = d_after;
 #pragma unroll
@@ -466,11 +434,11 @@ __global__ __launch_bounds__(NW * 64, 4) void vm_conv_lds_kernel(VmBatchDev B, V
         tile = next;
         next = after;
     }
-    VM_T_FLUSH
 }
 
-template <int C_IN, int C_OUT, int SLOTS, int OUT_FMT = VM_ROWS_F32>
+template <int C_IN, int C_OUT_T, int SLOTS, int OUT_FMT = VM_ROWS_F32>
 int launch_lds(const VmBatchDev& B, const VmLayerDev& L, const float* in, float* out, hipStream_t stream) {
+    constexpr int C_OUT = C_OUT_T > 0 ? C_OUT_T : -16 * C_OUT_T; /* what the LDS is sized for */
     constexpr int HALO = halo_rows(C_IN, C_OUT, SLOTS);
     constexpr size_t lds = lds_bytes(C_IN, C_OUT, SLOTS, HALO);
     static_assert(lds <= 160 * 1024, "weights and staged rows must fit the CU's LDS");
@@ -480,7 +448,7 @@ int launch_lds(const VmBatchDev& B, const VmLayerDev& L, const float* in, float*
      * per SIMD); otherwise one block of 16 waves. */
     constexpr bool single = 2 * lds > 160 * 1024;
     constexpr int NW = single ? 16 : 8;
-    auto kernel = vm_conv_lds_kernel<C_IN, C_OUT, SLOTS, NW, HALO, OUT_FMT>;
+    auto kernel = vm_conv_lds_kernel<C_IN, C_OUT_T, SLOTS, NW, HALO, OUT_FMT>;
     static std::atomic<bool> configured{false}; /* engines on several host threads may get here together */
     if (!configured) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, int(lds)) != hipSuccess) {
@@ -521,11 +489,27 @@ int launch_lds(const VmBatchDev& B, const VmLayerDev& L, const float* in, float*
 #define VM_FOR_EACH_LDS_SPLIT_SHAPE(X) \
     X(4, 64, 7)
 
+/* Every other shape with input rows of whole 16-byte pieces up to 32 channels and up to 64 output channels runs on
+ * instantiations that know the input width and the number of 16-channel column blocks, and read the exact number of
+ * output channels at run time (reference engine/opencl/operation/make_network.hpp:43-214 generates a kernel for any
+ * shape). X(C_in, column blocks, slots). */
+#define VM_LDS_ANY_WIDTHS(X, CI) X(CI, 1, 7) X(CI, 2, 7) X(CI, 3, 7) X(CI, 4, 7) X(CI, 1, 9) X(CI, 2, 9) X(CI, 3, 9) X(CI, 4, 9)
+#define VM_FOR_EACH_LDS_ANY_SHAPE(X) \
+    VM_LDS_ANY_WIDTHS(X, 4)          \
+    VM_LDS_ANY_WIDTHS(X, 8)          \
+    VM_LDS_ANY_WIDTHS(X, 12)         \
+    VM_LDS_ANY_WIDTHS(X, 16)         \
+    VM_LDS_ANY_WIDTHS(X, 20)         \
+    VM_LDS_ANY_WIDTHS(X, 24)         \
+    VM_LDS_ANY_WIDTHS(X, 28)         \
+    VM_LDS_ANY_WIDTHS(X, 32)
+
 bool vm_lds_supported(int c_in, int c_out, int slots, int out_fmt) {
 #define X(CI, CO, SL) \
     if (c_in == CI && c_out == CO && slots == SL) return true;
     if (out_fmt == VM_ROWS_F32) {
         VM_FOR_EACH_LDS_SHAPE(X)
+        return c_in % 4 == 0 && c_in >= 4 && c_in <= 32 && c_out >= 1 && c_out <= 64 && (slots == 7 || slots == 9);
     }
     else if (out_fmt == VM_ROWS_BF16X2) {
         VM_FOR_EACH_LDS_SPLIT_SHAPE(X)
@@ -554,6 +538,14 @@ int vm_launch_conv_lds(const VmBatchDev& B, const VmLayerDev& L, const float* in
         return launch_lds<CI, CO, SL>(B, L, in, out, stream);               \
     }
     VM_FOR_EACH_LDS_SHAPE(X)
+#undef X
+    const int blocks = (L.c_out + 15) / 16;
+#define X(CI, CBL, SL)                                                                       \
+    if (L.c_in == CI && blocks == CBL && L.slots == SL) {                                    \
+        if (kernel_name) *kernel_name = vm_kernel_name("conv_lds", L.c_in, L.c_out, L.slots); \
+        return launch_lds<CI, -CBL, SL>(B, L, in, out, stream);                              \
+    }
+    VM_FOR_EACH_LDS_ANY_SHAPE(X)
 #undef X
     return -1;
 }

@@ -7,18 +7,13 @@
  *   A operand: lane l supplies W[k(l / 16)][o = l % 16]
  *   B operand: lane l supplies in[src(row = l % 16)][k(l / 16)]
  *   D:         lane l holds out channels 4 * (l / 16) + {0,1,2,3} of row l % 16   -> one vector store per lane
- * Two arithmetics share the kernel:
- *   fp32  v_mfma_f32_16x16x4_f32    one float per lane and step, 4 reduction values per instruction
- *   bf16  v_mfma_f32_16x16x32_bf16  eight bf16 per lane and step, 32 reduction values, fp32 accumulation,
- *         with the weights (and, for rows stored as fp32, the inputs) carried as hi + lo pairs of bf16
+ * The instruction is v_mfma_f32_16x16x4_f32: one float per lane and step, 4 reduction values per instruction (the bf16
+ * engine's layers have a kernel of their own, conv_bf16.hip).
  * The reduction index is free to be permuted as long as both operands agree, so lane group q = l / 16 takes
  * the q-th quarter of every gathered row: a lane's inputs for one gather slot are C_IN / 4 consecutive values
  * of one source row, and step j of slot s uses the j-th register of that run. The weights are stored once, in
  * exactly the order the lanes consume them ([slot][step][column block][lane]), and live in LDS for the life of
  * a block; one LDS read feeds RB MFMAs (RB row blocks per wave).
- *
- * Activations may be stored as fp32 or bf16 independently of the arithmetic: the bf16 engine chooses per
- * layer boundary, and only a boundary stored as bf16 costs accuracy.
  *
  * The gathered rows go straight from global memory into registers in operand layout (16-byte loads, no
  * staging). Mesh order is spatially coherent (about 88 % of a row's neighbours lie in the same 256-row tile),
@@ -48,8 +43,6 @@
 namespace {
 
 typedef float v4f __attribute__((ext_vector_type(4)));
-typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
-typedef __bf16 v4bf __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ int find_frame_by_row_tile(const VmFrame* frames, int n, int tile) {
     int lo = 0, hi = n - 1;
@@ -122,99 +115,30 @@ struct OperandF32 {
     static __device__ __forceinline__ v4f accumulate(int, areg_t a, op_t b, v4f c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
 };
 
-/* bf16 matrix instructions with fp32 accumulation. Every weight is held as two bf16, w = hi + lo with
- * hi = bf16(w) and lo = bf16(w - hi), one part each in LDS, so the products carry the weights to about 16
- * significant bits. Rows stored as bf16 are used as they are (two instructions per step: hi and lo weights);
- * the only rounding such a layer adds to the fp32 result is the storage of its input rows. */
-template <int C_IN>
-struct OperandBF16 {
-    static_assert(C_IN % 32 == 0, "one step consumes 8 bf16 from each of the four lane groups");
-    static constexpr int STEPS = C_IN / 32;
-    static constexpr int PARTS = 2;
-    static constexpr int RAW = STEPS;
-    typedef v8bf areg_t;
-    typedef v8bf raw_t;
-    typedef v8bf op_t;
-    static __device__ __forceinline__ void load(const void* __restrict__ in, uint32_t row, int q, raw_t (&x)[RAW]) {
-        const uint16_t* p = reinterpret_cast<const uint16_t*>(in) + (size_t) row * C_IN + q * (C_IN / 4);
-#pragma unroll
-        for (int j = 0; j < STEPS; ++j) x[j] = *reinterpret_cast<const v8bf*>(p + j * 8);
-    }
-    static __device__ __forceinline__ void prepare(const raw_t (&x)[RAW], op_t (&b)[STEPS]) {
-#pragma unroll
-        for (int j = 0; j < STEPS; ++j) b[j] = x[j];
-    }
-    static __device__ __forceinline__ v4f accumulate(int, areg_t a, op_t b, v4f c) { return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0); }
-};
-
-/* The same bf16 matrix instructions on rows stored as fp32: each value is split in registers into
- * hi = bf16(x) and lo = bf16(x - hi) and a step issues hi*w_hi + lo*w_hi + hi*w_lo. What is dropped (lo*w_lo
- * and the rounding of lo) is about 2^-17 of a product, so this layer adds no bf16-sized error at all while the
- * matrix pipe still runs at the bf16 rate (3 instructions of K=32 against 8 fp32 instructions of K=4). */
-template <int C_IN>
-struct OperandBF16FromF32 {
-    static_assert(C_IN % 32 == 0, "one step consumes 8 values from each of the four lane groups");
-    static constexpr int STEPS = C_IN / 32;
-    static constexpr int PARTS = 2;
-    static constexpr int RAW = C_IN / 4;
-    typedef v8bf areg_t;
-    typedef float raw_t;
-    struct op_t {
-        v8bf hi, lo;
-    };
-    static __device__ __forceinline__ void load(const void* __restrict__ in, uint32_t row, int q, raw_t (&x)[RAW]) {
-        load_words<float, RAW>(reinterpret_cast<const float*>(in) + (size_t) row * C_IN + q * RAW, x);
-    }
-    static __device__ __forceinline__ void prepare(const raw_t (&x)[RAW], op_t (&b)[STEPS]) {
-#pragma unroll
-        for (int j = 0; j < STEPS; ++j) {
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const float v = x[j * 8 + e];
-                const __bf16 h = (__bf16) v; /* round to nearest even */
-                b[j].hi[e] = h;
-                b[j].lo[e] = (__bf16) (v - (float) h); /* the difference is exact in fp32 */
-            }
-        }
-    }
-    static __device__ __forceinline__ v4f accumulate(int part, areg_t a, const op_t& b, v4f c) {
-        c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b.hi, c, 0, 0, 0);
-        if (part == 0) c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b.lo, c, 0, 0, 0);
-        return c;
-    }
-};
-
-/* four consecutive output channels of one row; OUT_T is float or uint16_t (bf16 bits) */
-template <typename OUT_T, int C_OUT>
-__device__ __forceinline__ void store4(void* __restrict__ out, uint32_t row, int o, v4f v) {
-    if constexpr (sizeof(OUT_T) == 4) {
-        float* y = reinterpret_cast<float*>(out) + (size_t) row * C_OUT + o;
-        if constexpr (C_OUT % 4 == 0) {
-            if (o < C_OUT) *reinterpret_cast<float4*>(y) = make_float4(v[0], v[1], v[2], v[3]);
-        }
-        else {
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-                if (o + i < C_OUT) y[i] = v[i];
-        }
+/* four consecutive output channels of one row; C_OUT_T > 0: the row's width is known to the compiler */
+template <typename OUT_T, int C_OUT_T>
+__device__ __forceinline__ void store4(void* __restrict__ out, uint32_t row, int o, v4f v, int c_out) {
+    static_assert(sizeof(OUT_T) == 4, "rows are stored as fp32");
+    float* y = reinterpret_cast<float*>(out) + (size_t) row * c_out + o;
+    if ((C_OUT_T > 0 ? C_OUT_T : c_out) % 4 == 0) {
+        if (o < c_out) *reinterpret_cast<float4*>(y) = make_float4(v[0], v[1], v[2], v[3]);
     }
     else {
-        static_assert(sizeof(OUT_T) == 4 || C_OUT % 4 == 0, "bf16 rows are written four channels at a time");
-        if (o < C_OUT) {
-            v4bf h;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) h[i] = (__bf16) v[i]; /* round to nearest even */
-            *reinterpret_cast<v4bf*>(reinterpret_cast<uint16_t*>(out) + (size_t) row * C_OUT + o) = h;
-        }
+        for (int i = 0; i < 4; ++i)
+            if (o + i < c_out) y[i] = v[i];
     }
 }
 
 /* NW waves per block, RB row blocks of 16 rows per wave: NW * RB * 16 == VMHIP_TILE. */
-template <class OP, int C_OUT, int SLOTS, typename OUT_T, int NW, int RB>
+/* C_OUT_T > 0: that many output channels, known to the compiler. C_OUT_T < 0: -C_OUT_T column blocks of 16 and the
+ * layer's own count of output channels (L.c_out) read at run time. */
+template <class OP, int C_OUT_T, int SLOTS, typename OUT_T, int NW, int RB>
 __global__ __launch_bounds__(NW * 64) void vm_conv_mfma_kernel(VmBatchDev B, VmLayerDev L, const void* __restrict__ in, void* __restrict__ out) {
     static_assert(NW * RB * 16 == VMHIP_TILE, "a block covers one tile");
     constexpr int STEPS = OP::STEPS;
-    constexpr int CB = (C_OUT + 15) / 16; /* column blocks of 16 output channels */
+    constexpr int CB = C_OUT_T > 0 ? (C_OUT_T + 15) / 16 : -C_OUT_T; /* column blocks of 16 output channels */
+    const int C_OUT = C_OUT_T > 0 ? C_OUT_T : L.c_out;
     constexpr int NN = SLOTS - 1;
     constexpr int NBV = NN > 0 ? NN : 1;
     constexpr int PARTS = OP::PARTS;
@@ -406,7 +330,7 @@ __global__ __launch_bounds__(NW * 64) void vm_conv_mfma_kernel(VmBatchDev B, VmL
             }
             if (valid[rb]) { /* valid => src[rb][0] is the lane's own row */
 #pragma unroll
-                for (int cb = 0; cb < CB; ++cb) store4<OUT_T, C_OUT>(out, src[rb][0], cb * 16 + q * 4, acc[rb][cb]);
+                for (int cb = 0; cb < CB; ++cb) store4<OUT_T, C_OUT_T>(out, src[rb][0], cb * 16 + q * 4, acc[rb][cb], C_OUT);
             }
         }
 
@@ -431,14 +355,11 @@ __global__ __launch_bounds__(NW * 64) void vm_conv_mfma_kernel(VmBatchDev B, VmL
 
 template <class OP, int C_OUT, int SLOTS, typename OUT_T>
 int launch_mfma(const VmBatchDev& B, const VmLayerDev& L, const void* in, void* out, hipStream_t stream) {
-    constexpr int CB = (C_OUT + 15) / 16;
+    constexpr int CB = C_OUT > 0 ? (C_OUT + 15) / 16 : -C_OUT;
     constexpr size_t lds = size_t(SLOTS) * OP::STEPS * CB * OP::PARTS * 64 * sizeof(typename OP::areg_t);
     /* 8 waves x 2 row blocks: 16 accumulator registers per pair of column blocks and two input buffers per
-     * lane leave room for four waves per SIMD on the 32-wide layers, two blocks per CU. Where the weights
-     * allow only one block per CU and the kernel lives on hiding gather latency (bf16), one block of 16 waves
-     * keeps the same four waves per SIMD. */
-    constexpr bool one_big_block = OP::PARTS > 1 && lds > 80 * 1024;
-    constexpr int NW = one_big_block ? 16 : 8, RB = VMHIP_TILE / (16 * NW);
+     * lane leave room for four waves per SIMD on the 32-wide layers, two blocks per CU. */
+    constexpr int NW = 8, RB = VMHIP_TILE / (16 * NW);
     auto kernel = vm_conv_mfma_kernel<OP, C_OUT, SLOTS, OUT_T, NW, RB>;
     static std::atomic<bool> configured{false}; /* engines on several host threads may get here together */
     if (!configured) {
@@ -459,109 +380,85 @@ int launch_mfma(const VmBatchDev& B, const VmLayerDev& L, const void* in, void* 
     return 0;
 }
 
-uint16_t bf16_round(float f) {
-    uint32_t u;
-    std::memcpy(&u, &f, 4);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return uint16_t((u >> 16) | 0x40); /* NaN stays NaN */
-    u += 0x7fffu + ((u >> 16) & 1u);                                         /* round to nearest even */
-    return uint16_t(u >> 16);
-}
-
-template <int CI, int CO, int SL, int IB, int OB, int AB>
+template <int CI, int CO, int SL>
 int launch_variant(const VmBatchDev& B, const VmLayerDev& L, const void* in, void* out, hipStream_t stream) {
-    typedef typename std::conditional<OB != 0, uint16_t, float>::type out_t;
-    static_assert(AB != 0 || IB == 0, "fp32 arithmetic reads fp32 rows");
-    if constexpr (AB != 0 && IB != 0) return launch_mfma<OperandBF16<CI>, CO, SL, out_t>(B, L, in, out, stream);
-    else if constexpr (AB != 0) return launch_mfma<OperandBF16FromF32<CI>, CO, SL, out_t>(B, L, in, out, stream);
-    else return launch_mfma<OperandF32<CI>, CO, SL, out_t>(B, L, in, out, stream);
+    return launch_mfma<OperandF32<CI>, CO, SL, float>(B, L, in, out, stream);
 }
 
 }  // namespace
 
-/* Weight layouts the kernel consumes, [slot][step][column block][part][lane = q*16 + o] with, per lane,
- *   fp32 arithmetic: one part, one float,   W[slot*C_IN + q*(C_IN/4) + step][cb*16 + o]
- *   bf16 arithmetic: two parts (hi, lo), eight bf16 each, of W[slot*C_IN + q*(C_IN/4) + step*8 + e][cb*16 + o], e = 0..7
- * and zeros for padded output channels. */
-size_t vm_mfma_weight_bytes(int c_in, int c_out, int slots, int arith_bf16) {
+/* Weight layout the kernel consumes: [slot][step][column block][lane = q*16 + o], one float per lane:
+ * W[slot*C_IN + q*(C_IN/4) + step][cb*16 + o], zeros for padded output channels. */
+size_t vm_mfma_weight_bytes(int c_in, int c_out, int slots) {
     const size_t cb = (c_out + 15) / 16;
-    return arith_bf16 ? size_t(slots) * (c_in / 32) * cb * 2 * 64 * 16 : size_t(slots) * (c_in / 4) * cb * 64 * 4;
+    return size_t(slots) * (c_in / 4) * cb * 64 * 4;
 }
-void vm_mfma_permute_weights(const float* w, int c_in, int c_out, int slots, int arith_bf16, void* wp) {
+void vm_mfma_permute_weights(const float* w, int c_in, int c_out, int slots, void* wp) {
     const int CB = (c_out + 15) / 16;
     const int quarter = c_in / 4;
-    if (!arith_bf16) {
-        float* dst = reinterpret_cast<float*>(wp);
-        for (int s = 0; s < slots; ++s)
-            for (int j = 0; j < quarter; ++j)
-                for (int cb = 0; cb < CB; ++cb)
-                    for (int q = 0; q < 4; ++q)
-                        for (int o = 0; o < 16; ++o) {
-                            const int col = cb * 16 + o;
-                            const int k = s * c_in + q * quarter + j;
-                            dst[((size_t(s) * quarter + j) * CB + cb) * 64 + q * 16 + o] = col < c_out ? w[size_t(k) * c_out + col] : 0.0f;
-                        }
-        return;
-    }
-    uint16_t* dst = reinterpret_cast<uint16_t*>(wp);
-    const int steps = c_in / 32;
+    float* dst = reinterpret_cast<float*>(wp);
     for (int s = 0; s < slots; ++s)
-        for (int j = 0; j < steps; ++j)
+        for (int j = 0; j < quarter; ++j)
             for (int cb = 0; cb < CB; ++cb)
                 for (int q = 0; q < 4; ++q)
-                    for (int o = 0; o < 16; ++o)
-                        for (int e = 0; e < 8; ++e) {
-                            const int col = cb * 16 + o;
-                            const int k = s * c_in + q * quarter + j * 8 + e;
-                            const float v = col < c_out ? w[size_t(k) * c_out + col] : 0.0f;
-                            const uint16_t hi = bf16_round(v);
-                            const uint32_t hi_bits = uint32_t(hi) << 16;
-                            float hi_f;
-                            std::memcpy(&hi_f, &hi_bits, 4);
-                            const uint16_t lo = std::isfinite(v) ? bf16_round(v - hi_f) : uint16_t(0);
-                            const size_t at = ((size_t(s) * steps + j) * CB + cb) * 2;
-                            dst[((at + 0) * 64 + q * 16 + o) * 8 + e] = hi;
-                            dst[((at + 1) * 64 + q * 16 + o) * 8 + e] = lo;
-                        }
+                    for (int o = 0; o < 16; ++o) {
+                        const int col = cb * 16 + o;
+                        const int k = s * c_in + q * quarter + j;
+                        dst[((size_t(s) * quarter + j) * CB + cb) * 64 + q * 16 + o] = col < c_out ? w[size_t(k) * c_out + col] : 0.0f;
+                    }
 }
 
-/* Instantiated combinations: (C_in, C_out, gather slots, bf16 rows in, bf16 rows out, bf16 arithmetic). */
-#define VM_FOR_EACH_MFMA_VARIANT(X)                                \
-    /* fp32 rows in and out, fp32 arithmetic */                    \
-    X(4, 16, 7, 0, 0, 0)                                           \
-    X(16, 16, 7, 0, 0, 0)                                          \
-    X(16, 32, 7, 0, 0, 0)                                          \
-    X(32, 32, 7, 0, 0, 0)                                          \
-    X(32, 16, 7, 0, 0, 0)                                          \
-    X(4, 64, 7, 0, 0, 0)                                           \
-    X(64, 64, 7, 0, 0, 0)                                          \
-    X(4, 24, 9, 0, 0, 0)                                           \
-    X(24, 24, 9, 0, 0, 0)                                          \
-    /* bf16 engine: bf16 matrix instructions; rows fp32 -> fp32, fp32 -> bf16, bf16 -> fp32 (bf16 storage is \
-     * only ever chosen for every second boundary, so bf16 -> bf16 does not occur) */                          \
-    X(64, 64, 7, 0, 0, 1)                                          \
-    X(64, 64, 7, 0, 1, 1)                                          \
-    X(64, 64, 7, 1, 0, 1)
+/* Instantiated shapes: (C_in, C_out, gather slots). */
+#define VM_FOR_EACH_MFMA_VARIANT(X) \
+    X(4, 16, 7)                     \
+    X(16, 16, 7)                    \
+    X(16, 32, 7)                    \
+    X(32, 32, 7)                    \
+    X(32, 16, 7)                    \
+    X(4, 64, 7)                     \
+    X(64, 64, 7)                    \
+    X(4, 24, 9)                     \
+    X(24, 24, 9)
 
-bool vm_mfma_supported(int c_in, int c_out, int slots, int in_bf16, int out_bf16, int arith_bf16) {
-#define X(CI, CO, SL, IB, OB, AB) \
-    if (c_in == CI && c_out == CO && slots == SL && in_bf16 == IB && out_bf16 == OB && arith_bf16 == AB) return true;
+/* Every other shape with input rows of 36 to 64 channels (whole 16-byte pieces) and up to 64 output channels:
+ * instantiations that know the input width and the number of 16-channel column blocks and read the exact number of
+ * output channels at run time; narrower input rows are conv_lds.hip's. X(C_in, column blocks, slots). */
+#define VM_MFMA_ANY_WIDTHS(X, CI) X(CI, 1, 7) X(CI, 2, 7) X(CI, 3, 7) X(CI, 4, 7) X(CI, 1, 9) X(CI, 2, 9) X(CI, 3, 9) X(CI, 4, 9)
+#define VM_FOR_EACH_MFMA_ANY_SHAPE(X) \
+    VM_MFMA_ANY_WIDTHS(X, 36)         \
+    VM_MFMA_ANY_WIDTHS(X, 40)         \
+    VM_MFMA_ANY_WIDTHS(X, 44)         \
+    VM_MFMA_ANY_WIDTHS(X, 48)         \
+    VM_MFMA_ANY_WIDTHS(X, 52)         \
+    VM_MFMA_ANY_WIDTHS(X, 56)         \
+    VM_MFMA_ANY_WIDTHS(X, 60)         \
+    VM_MFMA_ANY_WIDTHS(X, 64)
+
+bool vm_mfma_supported(int c_in, int c_out, int slots) {
+#define X(CI, CO, SL) \
+    if (c_in == CI && c_out == CO && slots == SL) return true;
     VM_FOR_EACH_MFMA_VARIANT(X)
 #undef X
-    return false;
+    return c_in % 4 == 0 && c_in >= 36 && c_in <= 64 && c_out >= 1 && c_out <= 64 && (slots == 7 || slots == 9);
 }
 
 int vm_launch_conv_mfma(const VmBatchDev& B, const VmLayerDev& L, const void* in, void* out, hipStream_t stream, const char** kernel_name) {
     if (B.n_row_tiles <= 0) return 0;
-#define X(CI, CO, SL, IB, OB, AB)                                                                                      \
-    if (L.c_in == CI && L.c_out == CO && L.slots == SL && L.in_bf16 == IB && L.out_bf16 == OB && L.arith_bf16 == AB) { \
-        if (kernel_name)                                                                                               \
-            *kernel_name = AB && IB   ? (OB ? "conv_bf16x2_" #CI "x" #CO "s" #SL : "conv_bf16x2_tof32_" #CI "x" #CO "s" #SL)  \
-                           : AB       ? (OB ? "conv_bf16x3_tobf16_" #CI "x" #CO "s" #SL : "conv_bf16x3_" #CI "x" #CO "s" #SL) \
-                           : OB       ? "conv_mfma_tobf16_" #CI "x" #CO "s" #SL                                        \
-                                      : "conv_mfma_" #CI "x" #CO "s" #SL;                                              \
-        return launch_variant<CI, CO, SL, IB, OB, AB>(B, L, in, out, stream);                                          \
+    if (L.in_bf16 || L.out_bf16 || L.arith_bf16) return -1;
+#define X(CI, CO, SL)                                                     \
+    if (L.c_in == CI && L.c_out == CO && L.slots == SL) {                 \
+        if (kernel_name) *kernel_name = "conv_mfma_" #CI "x" #CO "s" #SL; \
+        return launch_variant<CI, CO, SL>(B, L, in, out, stream);         \
     }
     VM_FOR_EACH_MFMA_VARIANT(X)
+#undef X
+    const int blocks = (L.c_out + 15) / 16;
+#define X(CI, CBL, SL)                                                                        \
+    if (L.c_in == CI && blocks == CBL && L.slots == SL) {                                     \
+        if (kernel_name) *kernel_name = vm_kernel_name("conv_mfma", L.c_in, L.c_out, L.slots); \
+        return launch_variant<CI, -CBL, SL>(B, L, in, out, stream);                           \
+    }
+    VM_FOR_EACH_MFMA_ANY_SHAPE(X)
 #undef X
     return -1;
 }

@@ -10,7 +10,7 @@
  * written with one store. Per row that is 8 matrix-pipe cycles for every 64 x 4 x 1 products: no waste against
  * the 16-column instruction, which spends 5.3 times more on a 3-channel layer.
  *
- * Staging follows conv_dma.hip: rows travel from global memory straight into LDS (buffer_load ... lds), tile-local tables, XCD-aware persistent tile walk, a side path for
+ * Staging follows conv_flow.hip: rows travel from global memory straight into LDS (buffer_load ... lds), tile-local tables, XCD-aware persistent tile walk, a side path for
  * neighbours that are not staged. A lane reads its whole source row from LDS per gather slot.
  */
 #include <cstdlib>
@@ -278,7 +278,7 @@ __global__ __launch_bounds__(NW * 64) void vm_conv_narrow_kernel(VmBatchDev B, V
         else contract(std::false_type());
 
         /* ---- every wave is done reading this buffer (with two buffers also: the next tile is complete and visible,
-         * see conv_dma.hip) ---- */
+         * see conv_flow.hip) ---- */
         if (NBUFS == 2) wait_all_loads();
         __syncthreads();
 

@@ -191,6 +191,9 @@ void vm_launch_detect(const VmBatchDev& B, const VmDetectDev& D, int clusters, h
 /* packed: 5 * total_d + 7 * total_c words (detect.hip says in which order) */
 void vm_launch_detect_pack(const VmBatchDev& B, const VmDetectDev& D, uint32_t* packed, int total_d, int total_c, hipStream_t stream);
 
+/* "<family>_<c_in>x<c_out>s<slots>" as a string that stays valid (the profile of a run names its kernels) */
+const char* vm_kernel_name(const char* family, int c_in, int c_out, int slots);
+
 /* launchers, one per kernel; all asynchronous on `stream` */
 void vm_launch_libm(int which, const float* x, float* y, int n, hipStream_t stream);
 void vm_launch_copy_probe(const void* src, void* dst, size_t bytes, hipStream_t stream);
@@ -203,9 +206,9 @@ int vm_launch_conv(const VmBatchDev& B, const VmLayerDev& L, const float* in, fl
                    const char** kernel_name);
 
 /* matrix-core variant (conv_mfma.hip); launch returns a negative value if the combination has no instantiation */
-bool vm_mfma_supported(int c_in, int c_out, int slots, int in_bf16, int out_bf16, int arith_bf16);
-size_t vm_mfma_weight_bytes(int c_in, int c_out, int slots, int arith_bf16);
-void vm_mfma_permute_weights(const float* w, int c_in, int c_out, int slots, int arith_bf16, void* wp);
+bool vm_mfma_supported(int c_in, int c_out, int slots);
+size_t vm_mfma_weight_bytes(int c_in, int c_out, int slots);
+void vm_mfma_permute_weights(const float* w, int c_in, int c_out, int slots, void* wp);
 int vm_launch_conv_mfma(const VmBatchDev& B, const VmLayerDev& L, const void* in, void* out, hipStream_t stream,
                         const char** kernel_name);
 
@@ -248,11 +251,7 @@ __device__ __forceinline__ __attribute__((ext_vector_type(4))) uint32_t vm_load_
     }
 }
 
-/* the same with rows brought into LDS by buffer_load ... lds and two alternating row buffers (conv_dma.hip) */
-bool vm_dma_supported(int c_in, int c_out, int slots);
-int vm_launch_conv_dma(const VmBatchDev& B, const VmLayerDev& L, const float* in, float* out, hipStream_t stream,
-                       const char** kernel_name);
-/* the same with LDS counters in place of the tile loop's barriers, so that the waves of a block run freely between
+/* the same with rows brought into LDS by buffer_load ... lds, two alternating row buffers and LDS counters in place of the tile loop's barriers, so that the waves of a block run freely between
  * "my tile is staged" and "my buffer may be refilled" (conv_flow.hip) */
 bool vm_flow_supported(int c_in, int c_out, int slots);
 /* host side: w_mfma (fp32, vm_mfma_permute_weights' order) rearranged into that kernel's LDS order; same size */
@@ -263,7 +262,7 @@ int vm_launch_conv_flow(const VmBatchDev& B, const VmLayerDev& L, const float* i
 hipError_t vm_flow_set_poll_limit(int polls); /* process wide; tests of the give-up path only */
 
 /* layers with at most four output channels on v_mfma_f32_4x4x1 (64 rows x 4 channels per instruction), staged like
- * conv_dma.hip (conv_narrow.hip); reads the plain row-major weights */
+ * conv_flow.hip (conv_narrow.hip); reads the plain row-major weights */
 bool vm_narrow_supported(int c_in, int c_out, int slots);
 int vm_launch_conv_narrow(const VmBatchDev& B, const VmLayerDev& L, const float* in, float* out, hipStream_t stream,
                           const char** kernel_name);
