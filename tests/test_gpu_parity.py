@@ -148,6 +148,31 @@ def test_config4_and_5_full_size_frame(oracle):
         assert_classification_parity(got, want, tol, label)
 
 
+@pytest.mark.parametrize("index", [1, 3])
+def test_layer_shapes_outside_the_enumerated_ones(oracle, index):
+    """A network whose widths no kernel was written for, 4 -> 48 -> 40 -> 12 -> 5, on configuration 1's Ring6 and
+    configuration 3's NMGrid8 geometry: every layer still runs on a matrix-core kernel (the instantiations that read
+    the number of output channels at run time: conv_lds for input rows up to 32 channels, conv_mfma above), within
+    1e-4 of the oracle (reference engine/opencl/operation/make_network.hpp:43-214 generates a kernel for any shape)."""
+    cfg = wl.config(index, n_frames=1)
+    nn = wl.N_NEIGHBOURS[cfg.model]
+    rng = np.random.default_rng(123)
+    net = wl.glorot_network(rng, [3, 48, 40, 12, 5], nn, wl.SELU if index == 1 else wl.RELU)
+    o_lens, e_lens = lens_pair(cfg)
+    o_mesh, e_mesh = meshes_for(cfg, oracle)
+    engine = eng.Engine(net, cfg.model)
+    f = cfg.frames[0]
+    got = engine(e_mesh, f["Hoc"], e_lens, f["image"], cfg.fourcc)
+    engine.profile(True)
+    engine.run()
+    names = [n for n, _, _ in engine.profile_read() if n.startswith("conv")]
+    s = nn + 1
+    assert names == ["conv_lds_4x48s%d" % s, "conv_mfma_48x40s%d" % s, "conv_mfma_40x12s%d" % s, "conv_lds_12x5s%d" % s], names
+    want = pick(o_mesh, f["Hoc"]).classify(f["Hoc"], o_lens, f["image"], cfg.fourcc, vmo.Network(net))
+    assert got["cls"].shape[1] == 5
+    assert_classification_parity(got, want, PROB_TOL, "4->48->40->12->5 on cfg%d" % index)
+
+
 def test_class_layers_use_the_4x4_matrix_instruction(oracle):
     """The output layers of configurations 1 to 3 (16 -> 2, 16 -> 3, 24 -> 4) run on the kernel built on
     v_mfma_f32_4x4x1 by default; their probabilities are covered by the configuration tests above, this one pins
