@@ -165,7 +165,7 @@ def workload_name(cfg, n_frames, table):
         {0: "Ring6", 1: "NMGrid8"}[cfg.model], "->".join(["4"] + [str(t[1]) for t in table]))
 
 
-def measure(cfg, engine, frames, steps, warmup, settle_s, events=True):
+def measure(cfg, engine, frames, steps, warmup, settle_s, events=True, stream_ceiling=True):
     """Stages `frames` (inputs resident in HBM from then on), lets the clocks settle, then W untimed and K timed passes.
     -> dict with the throughput, the dominant kernel's roofline (timed live with HIP events on the engine's stream in the
     timed passes) and every graph-convolution kernel's (from one fully bracketed, untimed pass)."""
@@ -240,6 +240,24 @@ def measure(cfg, engine, frames, steps, warmup, settle_s, events=True):
             entry = conv_roofline(name, ms / launches_per_step[name], rows)[0]
             conv_rooflines[name] = dict(bound=entry["bound"], achieved=entry["achieved"], unit=entry["unit"], frac=entry["frac"],
                                         avg_launch_ms=ms / launches_per_step[name])
+    # The layers bound by memory, against what the memory system gives a kernel that does nothing but read and write
+    # their bytes (same rows, same bytes per row in and out, whole cache lines, no gather, no arithmetic): the ceiling
+    # that a copy-like kernel of that shape reaches on this device, next to the 8 TB/s on the data sheet.
+    if stream_ceiling:
+        from visualmesh_amd import native
+        for name, entry in conv_rooflines.items():
+            if entry["bound"] != "hbm":
+                continue
+            shape = name.split("_")[-1]
+            c_in, rest = shape.split("x")
+            c_out, slots = rest.split("s")
+            s_in = 2 if name.startswith("conv_bf16_bf16_") else 4
+            s_out = 2 if "_tobf16_" in name else 4
+            read_b, write_b = int(c_in) * s_in + 4 * (int(slots) - 1), int(c_out) * s_out
+            ms = native.stream_probe(rows, read_b, write_b)
+            ceiling = (read_b + write_b) * ((rows + 63) // 64 * 64) / (ms * 1e-3) / 1e9
+            entry["stream_ceiling_GBps"] = ceiling
+            entry["frac_of_stream_ceiling"] = entry["achieved"] / ceiling
     return dict(value=nodes * steps / elapsed, frames_per_s=len(frames) * steps / elapsed, ms_per_step=elapsed * 1e3 / steps, nodes=nodes,
                 settle_passes=settle_passes, settle_ms=settle_ms, roofline=roofline, kernel_ms_per_step=dict(sorted(kernel_ms_per_step.items())),
                 conv_rooflines=conv_rooflines)
@@ -391,7 +409,7 @@ def main():
                 continue
             heavy = index in (4, 5)
             c, e, _, _, fr = build_workload(index)
-            r = measure(c, e, fr, 10 if heavy else 300, 2 if heavy else 30, 0.1 if heavy else args.settle, events=True)
+            r = measure(c, e, fr, 10 if heavy else 300, 2 if heavy else 30, 0.1 if heavy else args.settle, events=True, stream_ceiling=not heavy)
             others[c.name] = dict(workload=workload_name(c, len(fr), layer_table(c, wl.N_NEIGHBOURS[c.model])), dtype="bf16" if c.precision == "bf16" else "f32",
                                   nodes_per_s=r["value"], frames_per_s=r["frames_per_s"], ms_per_step=r["ms_per_step"], steps=10 if heavy else 300,
                                   visible_nodes_per_batch=r["nodes"], roofline=r["roofline"], conv_rooflines=r["conv_rooflines"])

@@ -299,6 +299,12 @@ int vmhip_selftest_libm(int32_t which, const float* x, float* y, int32_t n);
  * use it as the dispatch of known size that hardware memory counters are scaled by; it also gives the
  * practical copy bandwidth of the device. */
 int vmhip_selftest_copy(int64_t bytes, int32_t repeats, float* ms);
+/* Diagnostic with no counterpart in the reference: a graph-convolution layer reduced to its memory traffic - `rows` rows
+ * (a multiple of 64), `read_bytes_per_row` read and `write_bytes_per_row` written (multiples of 4), whole cache lines,
+ * no arithmetic - run `repeats` times; the average milliseconds per launch go to *ms. What it reaches is what the memory
+ * system gives a kernel with that mix of reads and writes at best: the ceiling the gather-bound layers are measured
+ * against next to the 8 TB/s peak. */
+int vmhip_selftest_stream(int64_t rows, int32_t read_bytes_per_row, int32_t write_bytes_per_row, int32_t repeats, float* ms);
 
 #ifdef __cplusplus
 }

@@ -1302,6 +1302,36 @@ int vmhip_selftest_copy(int64_t bytes, int32_t repeats, float* ms) {
     return VMHIP_OK;
 }
 
+int vmhip_selftest_stream(int64_t rows, int32_t read_bytes_per_row, int32_t write_bytes_per_row, int32_t repeats, float* ms) {
+    if (rows <= 0 || rows % 64 != 0 || read_bytes_per_row <= 0 || read_bytes_per_row % 4 != 0 || write_bytes_per_row <= 0 || write_bytes_per_row % 4 != 0
+        || repeats <= 0)
+        return fail(VMHIP_ERR_ARGUMENT, "selftest_stream: bad arguments");
+    void *src = nullptr, *dst = nullptr;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    const size_t rd = size_t(rows) * read_bytes_per_row, wr = size_t(rows) * write_bytes_per_row;
+    hipError_t e = hipMalloc(&src, rd);
+    if (e == hipSuccess) e = hipMalloc(&dst, wr);
+    if (e == hipSuccess) e = hipMemset(src, 1, rd);
+    if (e == hipSuccess) e = hipEventCreate(&e0);
+    if (e == hipSuccess) e = hipEventCreate(&e1);
+    if (e == hipSuccess) {
+        vm_launch_stream_probe(src, dst, size_t(rows), read_bytes_per_row, write_bytes_per_row, nullptr); /* warm-up */
+        e = hipEventRecord(e0, nullptr);
+        for (int i = 0; i < repeats && e == hipSuccess; ++i) vm_launch_stream_probe(src, dst, size_t(rows), read_bytes_per_row, write_bytes_per_row, nullptr);
+        if (e == hipSuccess) e = hipEventRecord(e1, nullptr);
+        if (e == hipSuccess) e = hipEventSynchronize(e1);
+        float total = 0.0f;
+        if (e == hipSuccess) e = hipEventElapsedTime(&total, e0, e1);
+        if (ms) *ms = total / float(repeats);
+    }
+    if (e0) (void) hipEventDestroy(e0);
+    if (e1) (void) hipEventDestroy(e1);
+    if (src) (void) hipFree(src);
+    if (dst) (void) hipFree(dst);
+    if (e != hipSuccess) return fail(VMHIP_ERR_HIP, std::string("selftest_stream: ") + hipGetErrorString(e));
+    return VMHIP_OK;
+}
+
 int vmhip_classify_batch(vmhip_engine* E, const vmhip_frame* frames, int32_t n_frames, vmhip_result* results) {
     if (!E) return fail(VMHIP_ERR_ARGUMENT, "classify_batch: null engine");
     ensure_scratch(E);

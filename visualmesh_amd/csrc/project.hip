@@ -103,6 +103,25 @@ __global__ __launch_bounds__(256) void vm_copy_probe_kernel(const float4* __rest
     for (size_t i = (size_t) blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t) gridDim.x * blockDim.x) dst[i] = src[i];
 }
 
+/* A layer reduced to its memory traffic: every wave takes 64 rows at a time, reads their read_vec 16-byte pieces and
+ * writes their write_vec 16-byte pieces (per 64 rows), both as whole cache lines, with nothing in between but an xor
+ * that keeps the reads alive. What this reaches for a layer's mix of bytes read and written is what the memory system
+ * gives a kernel of that shape at best. */
+__global__ __launch_bounds__(256) void vm_stream_probe_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst, size_t groups, int read_vec, int write_vec) {
+    const int lane = threadIdx.x & 63;
+    const size_t wave = ((size_t) blockIdx.x * blockDim.x + threadIdx.x) >> 6, n_waves = ((size_t) gridDim.x * blockDim.x) >> 6;
+    for (size_t g = wave; g < groups; g += n_waves) {
+        uint4 acc = make_uint4(0, 0, 0, 0);
+        const uint4* in = src + g * (size_t) read_vec;
+        for (int i = lane; i < read_vec; i += 64) {
+            const uint4 v = in[i];
+            acc.x ^= v.x, acc.y ^= v.y, acc.z ^= v.z, acc.w ^= v.w;
+        }
+        uint4* o = dst + g * (size_t) write_vec;
+        for (int i = lane; i < write_vec; i += 64) o[i] = acc;
+    }
+}
+
 __global__ void vm_reset_kernel(VmBatchDev B) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < B.n_frames) {
@@ -738,6 +757,10 @@ void vm_launch_copy_probe(const void* src, void* dst, size_t bytes, hipStream_t 
     const size_t n = bytes / 16;
     hipLaunchKernelGGL(vm_copy_probe_kernel, dim3(256 * 16), dim3(256), 0, stream, reinterpret_cast<const float4*>(src),
                        reinterpret_cast<float4*>(dst), n);
+}
+void vm_launch_stream_probe(const void* src, void* dst, size_t rows, int read_bytes_per_row, int write_bytes_per_row, hipStream_t stream) {
+    hipLaunchKernelGGL(vm_stream_probe_kernel, dim3(256 * 16), dim3(256), 0, stream, reinterpret_cast<const uint4*>(src), reinterpret_cast<uint4*>(dst),
+                       rows / 64, read_bytes_per_row * 4, write_bytes_per_row * 4);
 }
 void vm_launch_reset(const VmBatchDev& B, hipStream_t stream) {
     hipLaunchKernelGGL(vm_reset_kernel, dim3((B.n_frames + 63) / 64), dim3(64), 0, stream, B);

@@ -197,6 +197,8 @@ const char* vm_kernel_name(const char* family, int c_in, int c_out, int slots);
 /* launchers, one per kernel; all asynchronous on `stream` */
 void vm_launch_libm(int which, const float* x, float* y, int n, hipStream_t stream);
 void vm_launch_copy_probe(const void* src, void* dst, size_t bytes, hipStream_t stream);
+/* rows: a multiple of 64; bytes per row: multiples of 4 (64 rows are whole 16-byte pieces then) */
+void vm_launch_stream_probe(const void* src, void* dst, size_t rows, int read_bytes_per_row, int write_bytes_per_row, hipStream_t stream);
 void vm_launch_reset(const VmBatchDev& B, hipStream_t stream);
 void vm_launch_project(const VmBatchDev& B, hipStream_t stream);
 void vm_launch_compact(const VmBatchDev& B, float* feat, int classify, hipStream_t stream);

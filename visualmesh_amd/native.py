@@ -25,7 +25,7 @@ HIP_SYMBOLS = [
     "vmhip_last_error", "vmhip_engine_create", "vmhip_engine_destroy", "vmhip_engine_n_classes", "vmhip_mesh_upload",
     "vmhip_mesh_release", "vmhip_project", "vmhip_classify", "vmhip_classify_batch", "vmhip_batch_create",
     "vmhip_batch_destroy", "vmhip_mesh_attach_tree", "vmhip_batch_stage", "vmhip_batch_ranges", "vmhip_batch_export", "vmhip_batch_run", "vmhip_batch_run_async", "vmhip_batch_wait", "vmhip_batch_counts", "vmhip_batch_fetch", "vmhip_batch_fetch_async", "vmhip_batch_fetch_wait", "vmhip_batch_detect", "vmhip_host_alloc", "vmhip_host_free",
-    "vmhip_batch_profile", "vmhip_batch_profile_read", "vmhip_selftest_libm", "vmhip_selftest_copy", "vmhip_project_noalloc", "vmhip_debug_set", "vmhip_batch_guard_stats",
+    "vmhip_batch_profile", "vmhip_batch_profile_read", "vmhip_selftest_libm", "vmhip_selftest_copy", "vmhip_selftest_stream", "vmhip_project_noalloc", "vmhip_debug_set", "vmhip_batch_guard_stats",
 ]
 
 
@@ -157,6 +157,7 @@ def hip():
                                            C.POINTER(C.c_int64)]
     L.vmhip_selftest_libm.argtypes = [C.c_int32, C.POINTER(C.c_float), C.POINTER(C.c_float), C.c_int32]
     L.vmhip_selftest_copy.argtypes = [C.c_int64, C.c_int32, C.POINTER(C.c_float)]
+    L.vmhip_selftest_stream.argtypes = [C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.POINTER(C.c_float)]
     L.vmhip_debug_set.argtypes = [C.c_int32, C.c_double]
     L.vmhip_batch_guard_stats.argtypes = [vp, C.POINTER(C.c_int64), C.POINTER(C.c_int64), C.POINTER(C.c_int64), C.POINTER(C.c_int64)]
     L.vmhip_project_noalloc.argtypes = [vp, C.POINTER(C.c_float), C.POINTER(Lens), C.POINTER(C.c_int32), C.c_int32, C.c_int32,
@@ -182,6 +183,13 @@ def copy_probe(nbytes=1 << 30, repeats=5):
     """average milliseconds of a plain device copy kernel of nbytes (read nbytes + write nbytes)"""
     ms = C.c_float(0.0)
     hip_check(hip().vmhip_selftest_copy(nbytes, repeats, C.byref(ms)))
+    return float(ms.value)
+
+
+def stream_probe(rows, read_bytes_per_row, write_bytes_per_row, repeats=20):
+    """average milliseconds of a kernel that only reads and writes a layer's bytes (rows: rounded up to 64)"""
+    ms = C.c_float(0.0)
+    hip_check(hip().vmhip_selftest_stream((int(rows) + 63) // 64 * 64, read_bytes_per_row, write_bytes_per_row, repeats, C.byref(ms)))
     return float(ms.value)
 
 
