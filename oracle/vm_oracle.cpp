@@ -1,14 +1,17 @@
 /*
- * vm_oracle.cpp - CPU restatement of the reference Visual Mesh inference path, fp32 only.
+ * vm_oracle.cpp - CPU restatement of the reference Visual Mesh inference path for one Scalar type:
+ * `real` is float (libvm_oracle.so) or, compiled with -DVMO_REAL=double, double (libvm_oracle_f64.so).
  *
  * TEST INFRASTRUCTURE ONLY: the checker for the HIP engine and the timed CPU baseline. The shipped
  * engine never links or loads this file.
  *
  * Every function names the reference file:line it follows (paths relative to the reference's
- * cpp/visualmesh/). The arithmetic is written out for Scalar=float with the exact operand types and
- * evaluation order of the reference, because the node order, the lookup ranges and the visible set
- * all hang on last-bit fp32 comparisons. Build with -O2 -ffp-contract=off, no -march=native, no
- * -ffast-math (see Makefile), so that every float operation is a single IEEE-754 binary32 operation.
+ * cpp/visualmesh/). The arithmetic is written out with the exact operand types and evaluation order
+ * the reference's templates have for Scalar=real (where the reference mixes a double literal into a
+ * Scalar expression the promotion to double and the rounding back are spelled out; for real=double
+ * they change nothing), because the node order, the lookup ranges and the visible set all hang on
+ * last-bit comparisons. Build with -O2 -ffp-contract=off, no -march=native, no -ffast-math (see
+ * Makefile), so that every operation on reals is a single IEEE-754 operation of that type.
  *
  * Parity status: every function here is pinned bit-for-bit against the compiled reference headers
  * (_ref/libvm_ref.so, tests/test_oracle_vs_reference.py) wherever the reference tree is mounted, and
@@ -32,19 +35,21 @@
 #include <utility>
 #include <vector>
 
+typedef vmo_real real;
+
 namespace {
 
-typedef std::array<float, 3> V3;
-typedef std::array<float, 2> V2;
+typedef std::array<real, 3> V3;
+typedef std::array<real, 2> V2;
 
 /* utility/math.hpp:145-164: dot is the recursion a[L-1]*b[L-1] + dot_{L-2}, i.e. for three
  * components a2*b2 + (a1*b1 + a0*b0). */
-inline float dot3(const V3& a, const V3& b) { return a[2] * b[2] + (a[1] * b[1] + a[0] * b[0]); }
-inline float dot2(const V2& a, const V2& b) { return a[1] * b[1] + a[0] * b[0]; }
+inline real dot3(const V3& a, const V3& b) { return a[2] * b[2] + (a[1] * b[1] + a[0] * b[0]); }
+inline real dot2(const V2& a, const V2& b) { return a[1] * b[1] + a[0] * b[0]; }
 /* utility/math.hpp:166-175 */
-inline float norm3(const V3& a) { return std::sqrt(dot3(a, a)); }
+inline real norm3(const V3& a) { return std::sqrt(dot3(a, a)); }
 inline V3 normalise3(const V3& a) {
-    const float len = 1.0f / norm3(a);
+    const real len = real(1.0) / norm3(a);
     return V3{{a[0] * len, a[1] * len, a[2] * len}};
 }
 /* utility/math.hpp:177-184 */
@@ -58,7 +63,7 @@ struct M3 {
 inline V3 mul(const M3& m, const V3& v) { return V3{{dot3(m.r[0], v), dot3(m.r[1], v), dot3(m.r[2], v)}}; }
 
 /* Rco = block<3,3>(transpose(Hoc)) : engine/cpu/engine.hpp:95, mesh.hpp:507 */
-inline M3 rco_from_hoc(const float* H) {
+inline M3 rco_from_hoc(const real* H) {
     M3 m;
     for (int i = 0; i < 3; ++i)
         for (int j = 0; j < 3; ++j) m.r[i][j] = H[j * 4 + i];
@@ -68,92 +73,92 @@ inline M3 rco_from_hoc(const float* H) {
 /* ------------------------------------------------------------------ shapes */
 struct Shape {
     int kind;
-    float r;
+    real r;
     /* geometry/Sphere.hpp:66-68, geometry/Circle.hpp:72-74 */
-    float phi(float n, float h) const {
-        if (kind == VMO_SHAPE_SPHERE) return -std::atan(std::sinh(n * std::log1p(-2.0f * r / h)));
-        return std::atan((2.0f * n * r) / h);
+    real phi(real n, real h) const {
+        if (kind == VMO_SHAPE_SPHERE) return -std::atan(std::sinh(n * std::log1p(-real(2.0) * r / h)));
+        return std::atan((real(2.0) * n * r) / h);
     }
     /* geometry/Sphere.hpp:80-82, geometry/Circle.hpp:85-87 */
-    float n(float phi_, float h) const {
-        if (kind == VMO_SHAPE_SPHERE) return std::asinh(std::tan(-phi_)) / std::log1p(-2.0f * r / h);
-        return (h * std::tan(phi_)) / (2.0f * r);
+    real n(real phi_, real h) const {
+        if (kind == VMO_SHAPE_SPHERE) return std::asinh(std::tan(-phi_)) / std::log1p(-real(2.0) * r / h);
+        return (h * std::tan(phi_)) / (real(2.0) * r);
     }
     /* geometry/Sphere.hpp:97-99, geometry/Circle.hpp:101-103 */
-    float k(float h0, float h1) const {
+    real k(real h0, real h1) const {
         if (kind == VMO_SHAPE_SPHERE)
             return (std::log(h1 - 2 * r) - std::log(h1)) / (std::log(h0 - 2 * r) - std::log(h0));
         return h0 / h1;
     }
     /* geometry/Sphere.hpp:106-108, geometry/Circle.hpp:110-112 */
-    float c() const { return kind == VMO_SHAPE_SPHERE ? r : 0.0f; }
+    real c() const { return kind == VMO_SHAPE_SPHERE ? r : real(0.0); }
     /* geometry/Sphere.hpp:124-130, geometry/Circle.hpp:128-134. The first arm divides in double
-     * (the literal 1.0), the conditional's common type is double, the return rounds to float. */
-    float theta(float n, float h) const {
-        const double v = n <= 0.5 ? double(float(2.0 * M_PI)) / (1.0 + double(n * 2.0f))
-                                  : double(2.0f * std::asin(r / ((h - r) * std::tan(phi(n, h)))));
-        return float(v);
+     * (the literal 1.0), the conditional's common type is double, the return rounds to real. */
+    real theta(real n, real h) const {
+        const double v = n <= 0.5 ? double(real(2.0 * M_PI)) / (1.0 + double(n * real(2.0)))
+                                  : double(real(2.0) * std::asin(r / ((h - r) * std::tan(phi(n, h)))));
+        return real(v);
     }
 };
 
 /* ------------------------------------------------------------------ lens maths */
-/* utility/projection.hpp:104-120: the literal 1.0 makes the bracket a double sum of float terms. */
-inline float distort(float r, const float* k) {
-    const float ik0 = -k[0];
-    const float ik1 = 3.0f * (k[0] * k[0]) - k[1];
-    const float ik2 = -12.0f * (k[0] * k[0]) * k[0] + 8.0f * k[0] * k[1];
-    const float ik3 = 55.0f * (k[0] * k[0]) * (k[0] * k[0]) - 55.0f * (k[0] * k[0]) * k[1] + 5.0f * (k[1] * k[1]);
+/* utility/projection.hpp:104-120: the literal 1.0 makes the bracket a double sum of real terms. */
+inline real distort(real r, const real* k) {
+    const real ik0 = -k[0];
+    const real ik1 = real(3.0) * (k[0] * k[0]) - k[1];
+    const real ik2 = -real(12.0) * (k[0] * k[0]) * k[0] + real(8.0) * k[0] * k[1];
+    const real ik3 = real(55.0) * (k[0] * k[0]) * (k[0] * k[0]) - real(55.0) * (k[0] * k[0]) * k[1] + real(5.0) * (k[1] * k[1]);
     const double s = 1.0 + double(ik0 * (r * r)) + double(ik1 * ((r * r) * (r * r)))
                      + double(ik2 * ((r * r) * (r * r)) * (r * r))
                      + double(ik3 * ((r * r) * (r * r)) * ((r * r) * (r * r)));
-    return float(double(r) * s);
+    return real(double(r) * s);
 }
 /* utility/projection.hpp:138-144 */
-inline float undistort(float r, const float* k) {
-    return float(double(r) * (1.0 + double(k[0] * (r * r)) + double(k[1] * ((r * r) * (r * r)))));
+inline real undistort(real r, const real* k) {
+    return real(double(r) * (1.0 + double(k[0] * (r * r)) + double(k[1] * ((r * r) * (r * r)))));
 }
 
 /* utility/projection.hpp:162-187 */
 inline V2 project(const V3& ray, const vmo_lens& lens) {
-    const float f = lens.focal_length;
-    const float theta = std::acos(ray[0]);
-    const float rsin_theta = 1.0f / std::sqrt(1.0f - ray[0] * ray[0]);
-    float r_u;
+    const real f = lens.focal_length;
+    const real theta = std::acos(ray[0]);
+    const real rsin_theta = real(1.0) / std::sqrt(real(1.0) - ray[0] * ray[0]);
+    real r_u;
     switch (lens.projection) {
-        case VMO_RECTILINEAR: r_u = f * std::tan(std::min(std::max(theta, 0.0f), float(M_PI_2))); break;
-        case VMO_EQUISOLID: r_u = 2.0f * f * std::sin(theta * 0.5f); break;
+        case VMO_RECTILINEAR: r_u = f * std::tan(std::min(std::max(theta, real(0.0)), real(M_PI_2))); break;
+        case VMO_EQUISOLID: r_u = real(2.0) * f * std::sin(theta * real(0.5)); break;
         case VMO_EQUIDISTANT: r_u = f * theta; break;
         default: throw std::runtime_error("Cannot project: Unknown lens type");
     }
-    const float r_d = distort(r_u, lens.k);
-    V2 screen = ray[0] >= 1 ? V2{{0.0f, 0.0f}} : V2{{r_d * ray[1] * rsin_theta, r_d * ray[2] * rsin_theta}};
-    const float cx = float(lens.width) * 0.5f, cy = float(lens.height) * 0.5f;
+    const real r_d = distort(r_u, lens.k);
+    V2 screen = ray[0] >= 1 ? V2{{real(0.0), real(0.0)}} : V2{{r_d * ray[1] * rsin_theta, r_d * ray[2] * rsin_theta}};
+    const real cx = real(lens.width) * real(0.5), cy = real(lens.height) * real(0.5);
     return V2{{(cx - screen[0]) - lens.centre[0], (cy - screen[1]) - lens.centre[1]}};
 }
 
 /* utility/projection.hpp:204-225 */
 inline V3 unproject(const V2& px, const vmo_lens& lens) {
-    const V2 screen{{float(lens.width) * 0.5f - (px[0] + lens.centre[0]),
-                     float(lens.height) * 0.5f - (px[1] + lens.centre[1])}};
-    const float f = lens.focal_length;
-    const float r_d = std::sqrt(dot2(screen, screen));
-    if (r_d == 0) return V3{{1.0f, 0.0f, 0.0f}};
-    const float r_u = undistort(r_d, lens.k);
-    float theta;
+    const V2 screen{{real(lens.width) * real(0.5) - (px[0] + lens.centre[0]),
+                     real(lens.height) * real(0.5) - (px[1] + lens.centre[1])}};
+    const real f = lens.focal_length;
+    const real r_d = std::sqrt(dot2(screen, screen));
+    if (r_d == 0) return V3{{real(1.0), real(0.0), real(0.0)}};
+    const real r_u = undistort(r_d, lens.k);
+    real theta;
     switch (lens.projection) {
         case VMO_RECTILINEAR: theta = std::atan(r_u / f); break;
-        case VMO_EQUISOLID: theta = 2.0f * std::asin(r_u / (2.0f * f)); break;
+        case VMO_EQUISOLID: theta = real(2.0) * std::asin(r_u / (real(2.0) * f)); break;
         case VMO_EQUIDISTANT: theta = r_u / f; break;
         default: throw std::runtime_error("Cannot project: Unknown lens type");
     }
-    const float sin_theta = std::sin(theta);
+    const real sin_theta = std::sin(theta);
     return V3{{std::cos(theta), sin_theta * screen[0] / r_d, sin_theta * screen[1] / r_d}};
 }
 
 /* ------------------------------------------------------------------ cones */
 struct Cone {
     V3 axis;
-    float cos_t;
+    real cos_t;
 };
 /* utility/cone.hpp:32-34, :46-48, :61-66, :80-98 */
 inline Cone cone0() { return Cone{V3{{0, 0, 0}}, 1}; }
@@ -165,15 +170,15 @@ inline Cone cone2(const V3& p1, const V3& p2) {
 inline Cone cone3(const V3& p1, const V3& p2, const V3& p3) {
     /* invert(): utility/math.hpp:275-301 */
     const V3 m[3] = {p1, p2, p3};
-    const float det = (m[0][0] * (m[1][1] * m[2][2] - m[2][1] * m[1][2]) - m[0][1] * (m[1][0] * m[2][2] - m[1][2] * m[2][0])
+    const real det = (m[0][0] * (m[1][1] * m[2][2] - m[2][1] * m[1][2]) - m[0][1] * (m[1][0] * m[2][2] - m[1][2] * m[2][0])
                        + m[0][2] * (m[1][0] * m[2][1] - m[1][1] * m[2][0]));
     V3 im[3];
     if (det == 0) {
-        const float nan = std::numeric_limits<float>::quiet_NaN();
+        const real nan = std::numeric_limits<real>::quiet_NaN();
         im[0] = im[1] = im[2] = V3{{nan, nan, nan}};
     }
     else {
-        const float idet = 1.0f / det;
+        const real idet = real(1.0) / det;
         im[0] = V3{{(m[1][1] * m[2][2] - m[2][1] * m[1][2]) * idet, (m[0][2] * m[2][1] - m[0][1] * m[2][2]) * idet,
                     (m[0][1] * m[1][2] - m[0][2] * m[1][1]) * idet}};
         im[1] = V3{{(m[1][2] * m[2][0] - m[1][0] * m[2][2]) * idet, (m[0][0] * m[2][2] - m[0][2] * m[2][0]) * idet,
@@ -188,7 +193,7 @@ inline Cone cone3(const V3& p1, const V3& p2, const V3& p3) {
 
 struct BspCone {
     V3 axis;
-    float cos_t, sin_t;
+    real cos_t, sin_t;
 };
 
 }  // namespace
@@ -196,7 +201,7 @@ struct BspCone {
 /* ------------------------------------------------------------------ mesh */
 struct vmo_mesh {
     int nn = 0;
-    float h = 0, max_distance = 0;
+    real h = 0, max_distance = 0;
     std::vector<V3> rays;
     std::vector<int> nbr; /* [n][nn], global indices, n_nodes means "no neighbour" */
     struct Bsp {
@@ -211,16 +216,16 @@ struct vmo_mesh {
 namespace {
 
 /* model/polar_map.hpp:41-43, :56-72 */
-V3 polar_map(const Shape& s, float h, float n, float m) {
-    const float phi = s.phi(std::abs(n), h);
-    const float d_theta = s.theta(std::abs(n), h);
-    const float theta = float(double(d_theta * m) + (n < 0 ? M_PI : 0.0));
+V3 polar_map(const Shape& s, real h, real n, real m) {
+    const real phi = s.phi(std::abs(n), h);
+    const real d_theta = s.theta(std::abs(n), h);
+    const real theta = real(double(d_theta * m) + (n < 0 ? M_PI : 0.0));
     return V3{{std::cos(theta) * std::sin(phi), std::sin(theta) * std::sin(phi), -std::cos(phi)}};
 }
 
 /* model/ring6.hpp:50-69 */
 std::array<int, 6> ring6_neighbours(int i, int p, int c, int n) {
-    const float f = float(i) / float(c);
+    const real f = real(i) / real(c);
     const int l = i > 0 ? i - 1 : c - 1;
     const int r = i + 1 < c ? i + 1 : 0;
     const int tl = (int(f * n) % n) + c;
@@ -231,29 +236,29 @@ std::array<int, 6> ring6_neighbours(int i, int p, int c, int n) {
 }
 
 /* model/ring_base.hpp:53-115 with Ring = Ring6 */
-void generate_ring6(vmo_mesh& mesh, const Shape& shape, float h, float k, float max_distance) {
+void generate_ring6(vmo_mesh& mesh, const Shape& shape, real h, real k, real max_distance) {
     const int N = 6;
     mesh.nn = N;
-    const float jump = float(1.0 / double(k));
-    const float two_pi = float(2.0 * M_PI);
+    const real jump = real(1.0 / double(k));
+    const real two_pi = real(2.0 * M_PI);
     int start = 1;
 
-    mesh.rays.push_back(V3{{0.0f, 0.0f, -1.0f}});
+    mesh.rays.push_back(V3{{real(0.0), real(0.0), -real(1.0)}});
     mesh.nbr.resize(N, 0);
     const int n_first = int(std::ceil((k * two_pi) / shape.theta(jump, h)));
-    const float first_jump = float(n_first) / float(N);
+    const real first_jump = real(n_first) / real(N);
     for (unsigned int i = 0; i < unsigned(N); ++i) mesh.nbr[i] = int(i * first_jump) + start;
 
     for (int i = 1; h * std::tan(shape.phi(i * jump, h)) < max_distance; ++i) {
-        const float n_p = (i - 1) * jump;
-        const float n_c = i * jump;
-        const float n_n = (i + 1) * jump;
+        const real n_p = (i - 1) * jump;
+        const real n_c = i * jump;
+        const real n_n = (i + 1) * jump;
 
-        const float s_p = i == 1 ? 1.0f : k * two_pi / shape.theta(n_p, h);
-        const float s_c = k * two_pi / shape.theta(n_c, h);
-        const float s_n = k * two_pi / shape.theta(n_n, h);
+        const real s_p = i == 1 ? real(1.0) : k * two_pi / shape.theta(n_p, h);
+        const real s_c = k * two_pi / shape.theta(n_c, h);
+        const real s_n = k * two_pi / shape.theta(n_n, h);
 
-        const float m_jump = s_c / (k * std::ceil(s_c));
+        const real m_jump = s_c / (k * std::ceil(s_c));
 
         start = int(mesh.rays.size());
         const int ip = int(std::ceil(s_p)), ic = int(std::ceil(s_c)), in = int(std::ceil(s_n));
@@ -269,33 +274,33 @@ void generate_ring6(vmo_mesh& mesh, const Shape& shape, float h, float k, float 
 }
 
 /* model/nmgrid_map.hpp:33-64 */
-V3 nm_xyz(const Shape& s, float h, float n, float h_n) {
-    const float c = s.c();
-    const float x = (h_n - c) * std::tan(s.phi(n, h_n));
-    const float y = std::sqrt((h_n - c) * (h_n - c) - (h - c) * (h - c));
+V3 nm_xyz(const Shape& s, real h, real n, real h_n) {
+    const real c = s.c();
+    const real x = (h_n - c) * std::tan(s.phi(n, h_n));
+    const real y = std::sqrt((h_n - c) * (h_n - c) - (h - c) * (h - c));
     return V3{{x, y, c - h}};
 }
-float nm_guess_m(const Shape& s, float h, float n, float h_n) {
-    const float c = s.c();
+real nm_guess_m(const Shape& s, real h, real n, real h_n) {
+    const real c = s.c();
     const V3 v = nm_xyz(s, h, n, h_n);
-    const float h_m = std::sqrt(v[0] * v[0] + v[2] * v[2]) + c;
-    const float phi_m = std::acos(std::sqrt((v[0] * v[0] + v[2] * v[2]) / (v[0] * v[0] + v[1] * v[1] + v[2] * v[2])));
+    const real h_m = std::sqrt(v[0] * v[0] + v[2] * v[2]) + c;
+    const real phi_m = std::acos(std::sqrt((v[0] * v[0] + v[2] * v[2]) / (v[0] * v[0] + v[1] * v[1] + v[2] * v[2])));
     return s.n(phi_m, h_m);
 }
 /* model/nmgrid_map.hpp:95-131: bisection on the plane height of the first coordinate */
-V3 nmgrid_map(const Shape& s, float h, float nm0, float nm1) {
-    const float n = std::abs(nm0);
-    const float m = std::abs(nm1);
-    const float c = s.c();
-    float lo = h;
-    float hi = (h - c) / std::cos(s.phi(m, h)) + c;
-    float h_n = float(double(lo + hi) * 0.5);
+V3 nmgrid_map(const Shape& s, real h, real nm0, real nm1) {
+    const real n = std::abs(nm0);
+    const real m = std::abs(nm1);
+    const real c = s.c();
+    real lo = h;
+    real hi = (h - c) / std::cos(s.phi(m, h)) + c;
+    real h_n = real(double(lo + hi) * 0.5);
     while (true) {
         if (h_n == lo || h_n == hi) break;
-        const float m_g = nm_guess_m(s, h, n, h_n);
+        const real m_g = nm_guess_m(s, h, n, h_n);
         (m_g > m ? hi : lo) = h_n;
         if (double(h_n) == double(lo + hi) * 0.5) break;
-        h_n = float(double(lo + hi) * 0.5);
+        h_n = real(double(lo + hi) * 0.5);
     }
     V3 v = nm_xyz(s, h, n, h_n);
     v[0] *= nm0 >= 0 ? 1 : -1;
@@ -305,11 +310,11 @@ V3 nmgrid_map(const Shape& s, float h, float nm0, float nm1) {
 
 /* model/grid_base.hpp:78-144 with Map = NMGridMap, 8 neighbours. The flood fill order (LIFO stack,
  * offsets in the table's order) fixes the node order; the containers only answer membership. */
-void generate_nmgrid8(vmo_mesh& mesh, const Shape& shape, float h, float k, float max_distance) {
+void generate_nmgrid8(vmo_mesh& mesh, const Shape& shape, real h, real k, real max_distance) {
     const int N = 8;
     mesh.nn = N;
     static const int off[8][2] = {{-1, 0}, {-1, 1}, {0, 1}, {1, 1}, {1, 0}, {1, -1}, {0, -1}, {-1, -1}};
-    const float jump = float(1.0 / double(k));
+    const real jump = real(1.0 / double(k));
     typedef std::pair<int, int> C2;
     std::map<C2, int> locations;
     std::set<C2> seen;
@@ -319,9 +324,9 @@ void generate_nmgrid8(vmo_mesh& mesh, const Shape& shape, float h, float k, floa
     while (!stack.empty()) {
         const C2 e = stack.back();
         stack.pop_back();
-        const float nm0 = float(e.first) * jump, nm1 = float(e.second) * jump;
+        const real nm0 = real(e.first) * jump, nm1 = real(e.second) * jump;
         const V3 vec = nmgrid_map(shape, h, nm0, nm1);
-        const float distance = std::sqrt(dot2(V2{{vec[0], vec[1]}}, V2{{vec[0], vec[1]}}));
+        const real distance = std::sqrt(dot2(V2{{vec[0], vec[1]}}, V2{{vec[0], vec[1]}}));
         if (distance <= max_distance) {
             locations.emplace(e, int(mesh.rays.size()));
             mesh.rays.push_back(normalise3(vec));
@@ -362,7 +367,7 @@ BspCone bounding_cone(const vmo_mesh& mesh, It start, It end) {
             }
         }
     }
-    return BspCone{cone.axis, cone.cos_t, std::sqrt(1.0f - cone.cos_t * cone.cos_t)};
+    return BspCone{cone.axis, cone.cos_t, std::sqrt(real(1.0) - cone.cos_t * cone.cos_t)};
 }
 
 /* mesh.hpp:135-248. std::partition / std::sort / std::max_element on std::vector<int>::iterator, as in
@@ -381,8 +386,8 @@ int build_bsp(vmo_mesh& mesh, It start, It end, int min_points, int offset) {
 
     if (mesh.bsp.empty()) {
         It max_phi_element = std::max_element(start, end, [&R](const int& a, const int& b) { return R[a][2] < R[b][2]; });
-        const float cone_cos = -R[*max_phi_element][2];
-        const float cone_sin = std::sqrt(1 - cone_cos * cone_cos);
+        const real cone_cos = -R[*max_phi_element][2];
+        const real cone_sin = std::sqrt(1 - cone_cos * cone_cos);
         It mid = std::partition(start, end, [&R](const int& a) { return R[a][1] > 0; });
         mesh.bsp.push_back(vmo_mesh::Bsp{offset, count, {-1, -1}, BspCone{V3{{0, 0, -1}}, cone_cos, cone_sin}});
         const int c0 = build_bsp(mesh, start, mid, min_points, 0);
@@ -394,16 +399,16 @@ int build_bsp(vmo_mesh& mesh, It start, It end, int min_points, int offset) {
 
     const BspCone cone = bounding_cone(mesh, start, end);
 
-    float min_phi = std::numeric_limits<float>::max();
-    float max_phi = std::numeric_limits<float>::lowest();
-    float min_theta = std::numeric_limits<float>::max();
-    float max_theta = std::numeric_limits<float>::lowest();
-    float sum_theta = 0, sum_phi = 0;
+    real min_phi = std::numeric_limits<real>::max();
+    real max_phi = std::numeric_limits<real>::lowest();
+    real min_theta = std::numeric_limits<real>::max();
+    real max_theta = std::numeric_limits<real>::lowest();
+    real sum_theta = 0, sum_phi = 0;
     int count_theta = 0, count_phi = 0;
     for (It it = start; it != end; ++it) {
         const V3& ray = R[*it];
-        const float phi = ray[2];
-        const float theta = ray[0] / std::sqrt(1 - ray[2] * ray[2]);
+        const real phi = ray[2];
+        const real theta = ray[0] / std::sqrt(1 - ray[2] * ray[2]);
         min_phi = std::min(min_phi, phi);
         max_phi = std::max(max_phi, phi);
         sum_phi += phi;
@@ -415,8 +420,8 @@ int build_bsp(vmo_mesh& mesh, It start, It end, int min_points, int offset) {
             count_theta += 1;
         }
     }
-    const float split_phi = sum_phi / count_phi;
-    const float split_theta = sum_theta / count_theta;
+    const real split_phi = sum_phi / count_phi;
+    const real split_theta = sum_theta / count_theta;
 
     It mid = max_phi - min_phi > max_theta - min_theta
                ? std::partition(start, end, [&R, &split_phi](const int& a) { return R[a][2] > split_phi; })
@@ -464,11 +469,11 @@ void finish_mesh(vmo_mesh& mesh) {
 }
 
 /* mesh.hpp:265-349 */
-void screen_edges(const float* H, const vmo_lens& lens, BspCone edges[4]) {
+void screen_edges(const real* H, const vmo_lens& lens, BspCone edges[4]) {
     M3 Roc;
     for (int i = 0; i < 3; ++i)
         for (int j = 0; j < 3; ++j) Roc.r[i][j] = H[i * 4 + j];
-    const V2 dims{{float(lens.width) - 1.0f, float(lens.height) - 1.0f}};
+    const V2 dims{{real(lens.width) - real(1.0), real(lens.height) - real(1.0)}};
     const V3 rN[4] = {
       mul(Roc, unproject(V2{{1, 1}}, lens)),
       mul(Roc, unproject(V2{{dims[0], 1}}, lens)),
@@ -485,7 +490,7 @@ void screen_edges(const float* H, const vmo_lens& lens, BspCone edges[4]) {
         }
         case VMO_EQUIDISTANT:
         case VMO_EQUISOLID: {
-            const V2 centre{{dims[0] * 0.5f + lens.centre[0], dims[1] * 0.5f + lens.centre[1]}};
+            const V2 centre{{dims[0] * real(0.5) + lens.centre[0], dims[1] * real(0.5) + lens.centre[1]}};
             const V3 rE[4] = {
               mul(Roc, unproject(V2{{centre[0], 1}}, lens)),
               mul(Roc, unproject(V2{{dims[0], centre[1]}}, lens)),
@@ -494,7 +499,7 @@ void screen_edges(const float* H, const vmo_lens& lens, BspCone edges[4]) {
             };
             const Cone c[4] = {cone3(rN[1], rE[0], rN[0]), cone3(rN[2], rE[1], rN[1]), cone3(rN[3], rE[2], rN[2]),
                                cone3(rN[0], rE[3], rN[3])};
-            for (int i = 0; i < 4; ++i) edges[i] = BspCone{c[i].axis, c[i].cos_t, std::sqrt(1.0f - c[i].cos_t * c[i].cos_t)};
+            for (int i = 0; i < 4; ++i) edges[i] = BspCone{c[i].axis, c[i].cos_t, std::sqrt(real(1.0) - c[i].cos_t * c[i].cos_t)};
             return;
         }
         default: throw std::runtime_error("Unknown lens type");
@@ -505,7 +510,7 @@ void screen_edges(const float* H, const vmo_lens& lens, BspCone edges[4]) {
 std::pair<bool, bool> check_on_screen(const M3& Rco, const BspCone& cone, const vmo_lens& lens, const BspCone edges[4]) {
     const V2 px = project(mul(Rco, cone.axis), lens);
     const bool axis_on_screen = 0 <= px[0] && px[0] + 1 <= lens.width && 0 <= px[1] && px[1] + 1 <= lens.height;
-    float angles[4];
+    real angles[4];
     bool contains[4];
     for (int i = 0; i < 4; ++i) {
         angles[i] = dot3(cone.axis, edges[i].axis);
@@ -520,9 +525,9 @@ std::pair<bool, bool> check_on_screen(const M3& Rco, const BspCone& cone, const 
 }
 
 /* mesh.hpp:499-595 */
-std::vector<std::pair<int, int>> lookup(const vmo_mesh& mesh, const float* H, const vmo_lens& lens) {
-    const float cos_fov = std::cos(lens.fov * 0.5f);
-    const float sin_fov = std::sin(lens.fov * 0.5f);
+std::vector<std::pair<int, int>> lookup(const vmo_mesh& mesh, const real* H, const vmo_lens& lens) {
+    const real cos_fov = std::cos(lens.fov * real(0.5));
+    const real sin_fov = std::sin(lens.fov * real(0.5));
     const M3 Rco = rco_from_hoc(H);
     const V3 rXCo = Rco.r[0];
     BspCone edges[4];
@@ -538,7 +543,7 @@ std::vector<std::pair<int, int>> lookup(const vmo_mesh& mesh, const float* H, co
         const vmo_mesh::Bsp& elem = mesh.bsp[i];
         const BspCone& cone = elem.cone;
 
-        const float delta = dot3(rXCo, cone.axis);
+        const real delta = dot3(rXCo, cone.axis);
         bool outside = delta < cos_fov * cone.cos_t - sin_fov * cone.sin_t;
         bool inside = delta > cos_fov * cone.cos_t + sin_fov * cone.sin_t;
         if (!outside && inside) {
@@ -608,7 +613,7 @@ inline int idot25(const int* p, const int* k) {
 }
 
 /* engine/cpu/bayer.hpp:95-108: integer dot, C++ truncating division by 64, no clamp, alpha 255 */
-void demosaic(const int* p, BayerType type, float* out) {
+void demosaic(const int* p, BayerType type, real* out) {
     int o[4];
     switch (type) {
         case BT_R: o[0] = p[12], o[1] = idot25(p, G_R) / 64, o[2] = idot25(p, B_R) / 64; break;
@@ -617,12 +622,12 @@ void demosaic(const int* p, BayerType type, float* out) {
         default: o[0] = idot25(p, R_B) / 64, o[1] = idot25(p, G_B) / 64, o[2] = p[12]; break;
     }
     o[3] = 255;
-    const float s = float(1.0 / 255.0);
-    for (int i = 0; i < 4; ++i) out[i] = float(o[i]) * s;
+    const real s = real(1.0 / 255.0);
+    for (int i = 0; i < 4; ++i) out[i] = real(o[i]) * s;
 }
 
 /* engine/cpu/bayer.hpp:122-158 */
-int bayer_get_pixel(int px, int py, const uint8_t* image, int W, int H, uint32_t format, float* out) {
+int bayer_get_pixel(int px, int py, const uint8_t* image, int W, int H, uint32_t format, real* out) {
     int patch[25];
     for (int y = 0; y < 5; ++y) {
         const int yc = std::min(std::max(py - 2 + y, 0), H - 1);
@@ -644,13 +649,13 @@ int bayer_get_pixel(int px, int py, const uint8_t* image, int W, int H, uint32_t
 }
 
 /* engine/cpu/pixel.hpp:43-102 */
-int get_pixel(int x, int y, const uint8_t* im, int W, int H, uint32_t format, float* o) {
-    const float s = float(1.0 / 255.0);
+int get_pixel(int x, int y, const uint8_t* im, int W, int H, uint32_t format, real* o) {
+    const real s = real(1.0 / 255.0);
     if (format == cc("GRBG") || format == cc("RGGB") || format == cc("GBRG") || format == cc("BGGR"))
         return bayer_get_pixel(x, y, im, W, H, format, o);
     if (format == cc("BGR3") || format == cc("BGR8")) {
         const int c = (y * W + x) * 3;
-        o[0] = im[c + 2] * s, o[1] = im[c + 1] * s, o[2] = im[c + 0] * s, o[3] = 1.0f;
+        o[0] = im[c + 2] * s, o[1] = im[c + 1] * s, o[2] = im[c + 0] * s, o[3] = real(1.0);
         return VMO_OK;
     }
     if (format == cc("BGRA")) {
@@ -660,7 +665,7 @@ int get_pixel(int x, int y, const uint8_t* im, int W, int H, uint32_t format, fl
     }
     if (format == cc("RGB3") || format == cc("RGB8")) {
         const int c = (y * W + x) * 3;
-        o[0] = im[c + 0] * s, o[1] = im[c + 1] * s, o[2] = im[c + 2] * s, o[3] = 1.0f;
+        o[0] = im[c + 0] * s, o[1] = im[c + 1] * s, o[2] = im[c + 2] * s, o[3] = real(1.0);
         return VMO_OK;
     }
     if (format == cc("RGBA")) {
@@ -670,46 +675,46 @@ int get_pixel(int x, int y, const uint8_t* im, int W, int H, uint32_t format, fl
     }
     if (format == cc("GRAY") || format == cc("GREY") || format == cc("Y8  ")) {
         const int c = y * W + x;
-        o[0] = o[1] = o[2] = im[c] * s, o[3] = 1.0f;
+        o[0] = o[1] = o[2] = im[c] * s, o[3] = real(1.0);
         return VMO_OK;
     }
     return VMO_ERR_FORMAT;
 }
 
 /* engine/cpu/pixel.hpp:115-144 */
-int interpolate(const float* P, const uint8_t* im, int W, int H, uint32_t format, float* out) {
-    const float x = P[0], y = P[1];
+int interpolate(const real* P, const uint8_t* im, int W, int H, uint32_t format, real* out) {
+    const real x = P[0], y = P[1];
     const int x1 = std::max(int(std::floor(P[0])), 0);
     const int y1 = std::max(int(std::floor(P[1])), 0);
     const int x2 = std::min(x1 + 1, W - 1);
     const int y2 = std::min(y1 + 1, H - 1);
-    float Q1[4], Q2[4], Q3[4], Q4[4];
+    real Q1[4], Q2[4], Q3[4], Q4[4];
     int rc;
     if ((rc = get_pixel(x1, y1, im, W, H, format, Q1)) != VMO_OK) return rc;
     if ((rc = get_pixel(x2, y1, im, W, H, format, Q2)) != VMO_OK) return rc;
     if ((rc = get_pixel(x1, y2, im, W, H, format, Q3)) != VMO_OK) return rc;
     if ((rc = get_pixel(x2, y2, im, W, H, format, Q4)) != VMO_OK) return rc;
-    const float wx_a = (x2 - x) / (x2 - x1), wx_b = (x - x1) / (x2 - x1);
-    const float wy_a = (y2 - y) / (y2 - y1), wy_b = (y - y1) / (y2 - y1);
+    const real wx_a = (x2 - x) / (x2 - x1), wx_b = (x - x1) / (x2 - x1);
+    const real wy_a = (y2 - y) / (y2 - y1), wy_b = (y - y1) / (y2 - y1);
     for (int c = 0; c < 4; ++c) {
-        const float R1 = Q1[c] * wx_a + Q2[c] * wx_b;
-        const float R2 = Q3[c] * wx_a + Q4[c] * wx_b;
+        const real R1 = Q1[c] * wx_a + Q2[c] * wx_b;
+        const real R2 = Q3[c] * wx_a + Q4[c] * wx_b;
         out[c] = R1 * wy_a + R2 * wy_b;
     }
     return VMO_OK;
 }
 
 /* engine/cpu/apply_activation.hpp:34-84 */
-void apply_activation(int fn, float* d, size_t n_rows, int dims) {
+void apply_activation(int fn, real* d, size_t n_rows, int dims) {
     const size_t total = n_rows * size_t(dims);
     switch (fn) {
         case VMO_SELU: {
-            const float lambda = 1.0507009873554804934193349852946;
-            const float alpha = 1.6732632423543772848170429916717;
+            const real lambda = 1.0507009873554804934193349852946;
+            const real alpha = 1.6732632423543772848170429916717;
             for (size_t i = 0; i < total; ++i) d[i] = lambda * (d[i] >= 0 ? d[i] : alpha * std::exp(d[i]) - alpha);
         } break;
         case VMO_RELU:
-            for (size_t i = 0; i < total; ++i) d[i] = std::max(d[i], 0.0f);
+            for (size_t i = 0; i < total; ++i) d[i] = std::max(d[i], real(0.0));
             break;
         case VMO_TANH:
             for (size_t i = 0; i < total; ++i) d[i] = std::tanh(d[i]);
@@ -717,8 +722,8 @@ void apply_activation(int fn, float* d, size_t n_rows, int dims) {
         case VMO_SOFTMAX:
             for (size_t i = 0; i < total; ++i) d[i] = std::exp(d[i]);
             for (size_t r = 0; r < n_rows; ++r) {
-                float* row = d + r * dims;
-                float sum = 0.0f;
+                real* row = d + r * dims;
+                real sum = real(0.0);
                 for (int j = 0; j < dims; ++j) sum = sum + row[j];
                 for (int j = 0; j < dims; ++j) row[j] = row[j] / sum;
             }
@@ -728,7 +733,7 @@ void apply_activation(int fn, float* d, size_t n_rows, int dims) {
 }
 
 /* engine/cpu/engine.hpp:84-147 */
-int project_mesh(const vmo_mesh& mesh, const float* H, const vmo_lens& lens, int cap, float* px_out, int32_t* nb_out,
+int project_mesh(const vmo_mesh& mesh, const real* H, const vmo_lens& lens, int cap, real* px_out, int32_t* nb_out,
                  int32_t* gidx_out) {
     const std::vector<std::pair<int, int>> ranges = lookup(mesh, H, lens);
     const M3 Rco = rco_from_hoc(H);
@@ -760,20 +765,20 @@ int project_mesh(const vmo_mesh& mesh, const float* H, const vmo_lens& lens, int
 /* engine/cpu/engine.hpp:180-273, with input/output as locals so every call starts from empty buffers
  * (the reference keeps them as members and never clears input, which makes every call after the first on
  * one engine object wrong; a fresh reference engine per call is what this equals). */
-int classify_mesh(const vmo_mesh& mesh, const float* H, const vmo_lens& lens, const void* image, uint32_t format,
-                  const vmo_network* net, int cap, float* px, int32_t* nb, int32_t* gidx, float* cls) {
+int classify_mesh(const vmo_mesh& mesh, const real* H, const vmo_lens& lens, const void* image, uint32_t format,
+                  const vmo_network* net, int cap, real* px, int32_t* nb, int32_t* gidx, real* cls) {
     const int V = project_mesh(mesh, H, lens, cap, px, nb, gidx);
     if (V <= 0) return V;
     const int nn = mesh.nn;
     const size_t n_points = size_t(V) + 1;
     const uint8_t* im = reinterpret_cast<const uint8_t*>(image);
 
-    std::vector<float> input(n_points * 4), output;
+    std::vector<real> input(n_points * 4), output;
     for (int i = 0; i < V; ++i) {
         const int rc = interpolate(px + 2 * size_t(i), im, lens.width, lens.height, format, &input[size_t(i) * 4]);
         if (rc != VMO_OK) return rc;
     }
-    for (int c = 0; c < 4; ++c) input[size_t(V) * 4 + c] = -1.0f;
+    for (int c = 0; c < 4; ++c) input[size_t(V) * 4 + c] = -real(1.0);
 
     int in_dims = 4;
     int layer_index = 0;
@@ -782,10 +787,10 @@ int classify_mesh(const vmo_mesh& mesh, const float* H, const vmo_lens& lens, co
         const int gathered = in_dims * (nn + 1);
         output.resize(n_points * gathered);
         for (size_t i = 0; i < n_points; ++i) {
-            float* o = &output[i * gathered];
-            std::memcpy(o, &input[i * in_dims], sizeof(float) * in_dims);
+            real* o = &output[i * gathered];
+            std::memcpy(o, &input[i * in_dims], sizeof(real) * in_dims);
             for (int j = 0; j < nn; ++j)
-                std::memcpy(o + (j + 1) * in_dims, &input[size_t(nb[i * nn + j]) * in_dims], sizeof(float) * in_dims);
+                std::memcpy(o + (j + 1) * in_dims, &input[size_t(nb[i * nn + j]) * in_dims], sizeof(real) * in_dims);
         }
         std::swap(input, output);
         in_dims = gathered;
@@ -795,15 +800,15 @@ int classify_mesh(const vmo_mesh& mesh, const float* H, const vmo_lens& lens, co
             if (L.n_in != in_dims) return VMO_ERR_ARG;
             const int out_dims = L.n_out;
             /* transposed copy, engine/cpu/engine.hpp:57-71 */
-            std::vector<float> wT(size_t(out_dims) * in_dims);
+            std::vector<real> wT(size_t(out_dims) * in_dims);
             for (int t = 0; t < in_dims; ++t)
                 for (int j = 0; j < out_dims; ++j) wT[size_t(j) * in_dims + t] = L.weights[size_t(t) * out_dims + j];
             output.resize(n_points * out_dims);
             for (size_t i = 0; i < n_points; ++i) {
-                const float* in = &input[i * in_dims];
+                const real* in = &input[i * in_dims];
                 for (int j = 0; j < out_dims; ++j) {
-                    const float* w = &wT[size_t(j) * in_dims];
-                    float acc = L.biases[j]; /* std::inner_product: acc = acc + a*b, in order */
+                    const real* w = &wT[size_t(j) * in_dims];
+                    real acc = L.biases[j]; /* std::inner_product: acc = acc + a*b, in order */
                     for (int t = 0; t < in_dims; ++t) acc = acc + in[t] * w[t];
                     output[i * out_dims + j] = acc;
                 }
@@ -813,7 +818,7 @@ int classify_mesh(const vmo_mesh& mesh, const float* H, const vmo_lens& lens, co
             in_dims = out_dims;
         }
     }
-    std::memcpy(cls, input.data(), sizeof(float) * n_points * in_dims);
+    std::memcpy(cls, input.data(), sizeof(real) * n_points * in_dims);
     return V;
 }
 
@@ -821,7 +826,7 @@ int classify_mesh(const vmo_mesh& mesh, const float* H, const vmo_lens& lens, co
 
 /* ------------------------------------------------------------------ C interface */
 struct vmo_visualmesh {
-    std::map<float, vmo_mesh*> luts;
+    std::map<real, vmo_mesh*> luts;
     std::vector<vmo_mesh*> ordered;
 };
 
@@ -829,7 +834,7 @@ extern "C" {
 
 const char* vmo_name(void) { return "oracle"; }
 
-vmo_mesh* vmo_mesh_create(int model, int shape, float radius, float h, float k, float max_distance) {
+vmo_mesh* vmo_mesh_create(int model, int shape, real radius, real h, real k, real max_distance) {
     if ((model != VMO_MODEL_RING6 && model != VMO_MODEL_NMGRID8) || (shape != VMO_SHAPE_SPHERE && shape != VMO_SHAPE_CIRCLE))
         return nullptr;
     vmo_mesh* m = new vmo_mesh();
@@ -849,12 +854,12 @@ vmo_mesh* vmo_mesh_create(int model, int shape, float radius, float h, float k, 
 void vmo_mesh_destroy(vmo_mesh* m) { delete m; }
 int vmo_mesh_n_nodes(const vmo_mesh* m) { return m->n(); }
 int vmo_mesh_n_neighbours(const vmo_mesh* m) { return m->nn; }
-float vmo_mesh_h(const vmo_mesh* m) { return m->h; }
-void vmo_mesh_copy(const vmo_mesh* m, float* rays, int32_t* neighbours) {
-    if (rays) std::memcpy(rays, m->rays.data(), sizeof(float) * 3 * m->rays.size());
+real vmo_mesh_h(const vmo_mesh* m) { return m->h; }
+void vmo_mesh_copy(const vmo_mesh* m, real* rays, int32_t* neighbours) {
+    if (rays) std::memcpy(rays, m->rays.data(), sizeof(real) * 3 * m->rays.size());
     if (neighbours) std::memcpy(neighbours, m->nbr.data(), sizeof(int32_t) * m->nbr.size());
 }
-int vmo_mesh_lookup(const vmo_mesh* m, const float* Hoc16, const vmo_lens* lens, int32_t* ranges, int cap) {
+int vmo_mesh_lookup(const vmo_mesh* m, const real* Hoc16, const vmo_lens* lens, int32_t* ranges, int cap) {
     try {
         const std::vector<std::pair<int, int>> r = lookup(*m, Hoc16, *lens);
         for (int i = 0; i < int(r.size()) && i < cap; ++i) {
@@ -866,11 +871,11 @@ int vmo_mesh_lookup(const vmo_mesh* m, const float* Hoc16, const vmo_lens* lens,
 }
 
 /* visualmesh.hpp:64-96 */
-vmo_visualmesh* vmo_visualmesh_create(int model, int shape, float radius, float min_h, float max_h, float k,
-                                      float max_error, float max_distance) {
+vmo_visualmesh* vmo_visualmesh_create(int model, int shape, real radius, real min_h, real max_h, real k,
+                                      real max_error, real max_distance) {
     vmo_visualmesh* v = new vmo_visualmesh();
     const Shape s{shape, radius};
-    auto add = [&](float h) {
+    auto add = [&](real h) {
         if (v->luts.count(h)) return true; /* std::map::insert keeps the first */
         vmo_mesh* m = vmo_mesh_create(model, shape, radius, h, k, max_distance);
         if (!m) return false;
@@ -882,10 +887,10 @@ vmo_visualmesh* vmo_visualmesh_create(int model, int shape, float radius, float 
     stack.push_back(V2{{min_h, max_h}});
     while (ok && !stack.empty()) {
         const V2 range = stack.back();
-        const float h = (range[0] + range[1]) / 2;
+        const real h = (range[0] + range[1]) / 2;
         stack.pop_back();
-        const float lower_err = std::abs(k - k * s.k(range[0], h));
-        const float upper_err = std::abs(k - k * s.k(range[1], h));
+        const real lower_err = std::abs(k - k * s.k(range[0], h));
+        const real upper_err = std::abs(k - k * s.k(range[1], h));
         if (lower_err > max_error || upper_err > max_error) {
             ok = add(h);
             stack.push_back(V2{{range[0], h}});
@@ -907,7 +912,7 @@ void vmo_visualmesh_destroy(vmo_visualmesh* v) {
 int vmo_visualmesh_n_meshes(const vmo_visualmesh* v) { return int(v->ordered.size()); }
 const vmo_mesh* vmo_visualmesh_mesh(const vmo_visualmesh* v, int i) { return v->ordered[i]; }
 /* visualmesh.hpp:122-135 */
-const vmo_mesh* vmo_visualmesh_height(const vmo_visualmesh* v, float h) {
+const vmo_mesh* vmo_visualmesh_height(const vmo_visualmesh* v, real h) {
     auto it = v->luts.lower_bound(h);
     if (it == v->luts.begin()) return it->second;
     if (it == v->luts.end()) return v->luts.rbegin()->second;
@@ -915,37 +920,37 @@ const vmo_mesh* vmo_visualmesh_height(const vmo_visualmesh* v, float h) {
     return std::abs(it->first - h) < std::abs(pv->first - h) ? it->second : pv->second;
 }
 
-int vmo_project(const vmo_mesh* m, const float* Hoc16, const vmo_lens* lens, int cap, float* px, int32_t* nb,
+int vmo_project(const vmo_mesh* m, const real* Hoc16, const vmo_lens* lens, int cap, real* px, int32_t* nb,
                 int32_t* gidx) {
     try {
         return project_mesh(*m, Hoc16, *lens, cap, px, nb, gidx);
     } catch (...) { return VMO_ERR_LENS; }
 }
-int vmo_classify(const vmo_mesh* m, const float* Hoc16, const vmo_lens* lens, const void* image, uint32_t fourcc,
-                 const vmo_network* net, int cap, float* px, int32_t* nb, int32_t* gidx, float* cls) {
+int vmo_classify(const vmo_mesh* m, const real* Hoc16, const vmo_lens* lens, const void* image, uint32_t fourcc,
+                 const vmo_network* net, int cap, real* px, int32_t* nb, int32_t* gidx, real* cls) {
     try {
         return classify_mesh(*m, Hoc16, *lens, image, fourcc, net, cap, px, nb, gidx, cls);
     } catch (...) { return VMO_ERR_LENS; }
 }
 
-void vmo_fn_project(const float* r, const vmo_lens* lens, float* px2) {
+void vmo_fn_project(const real* r, const vmo_lens* lens, real* px2) {
     const V2 p = project(V3{{r[0], r[1], r[2]}}, *lens);
     px2[0] = p[0], px2[1] = p[1];
 }
-void vmo_fn_unproject(const float* px2, const vmo_lens* lens, float* ray3) {
+void vmo_fn_unproject(const real* px2, const vmo_lens* lens, real* ray3) {
     const V3 r = unproject(V2{{px2[0], px2[1]}}, *lens);
     ray3[0] = r[0], ray3[1] = r[1], ray3[2] = r[2];
 }
-int vmo_fn_interpolate(const float* px2, const void* image, int width, int height, uint32_t fourcc, float* out4) {
+int vmo_fn_interpolate(const real* px2, const void* image, int width, int height, uint32_t fourcc, real* out4) {
     return interpolate(px2, reinterpret_cast<const uint8_t*>(image), width, height, fourcc, out4);
 }
-int vmo_fn_get_pixel(int x, int y, const void* image, int width, int height, uint32_t fourcc, float* out4) {
+int vmo_fn_get_pixel(int x, int y, const void* image, int width, int height, uint32_t fourcc, real* out4) {
     return get_pixel(x, y, reinterpret_cast<const uint8_t*>(image), width, height, fourcc, out4);
 }
-void vmo_fn_activation(int activation, float* data, int n_rows, int dims) {
+void vmo_fn_activation(int activation, real* data, int n_rows, int dims) {
     apply_activation(activation, data, size_t(n_rows), dims);
 }
-float vmo_fn_shape(int shape, float radius, int which, float a, float b) {
+real vmo_fn_shape(int shape, real radius, int which, real a, real b) {
     const Shape s{shape, radius};
     switch (which) {
         case 0: return s.phi(a, b);
@@ -955,7 +960,7 @@ float vmo_fn_shape(int shape, float radius, int which, float a, float b) {
         default: return s.c();
     }
 }
-void vmo_fn_libm(int which, const float* x, float* y, int n) {
+void vmo_fn_libm(int which, const real* x, real* y, int n) {
     for (int i = 0; i < n; ++i)
         y[i] = which == 0 ? std::acos(x[i]) : which == 1 ? std::sin(x[i]) : which == 2 ? std::tan(x[i]) : std::sqrt(x[i]);
 }

@@ -27,3 +27,20 @@ def reference():
     if ref is None:
         pytest.skip("oracle/_ref/libvm_ref.so is not built (needs the reference tree)")
     return ref
+
+
+@pytest.fixture(scope="session")
+def oracle64():
+    """the restatement compiled for Scalar = double"""
+    from oracle import vmo
+    return vmo.load("oracle", real="f64")
+
+
+@pytest.fixture(scope="session")
+def reference64():
+    """the reference's headers instantiated with Scalar = double"""
+    from oracle import vmo
+    ref = vmo.load("reference", real="f64")
+    if ref is None:
+        pytest.skip("oracle/_ref/libvm_ref_f64.so is not built (needs the reference tree)")
+    return ref

@@ -18,6 +18,8 @@ def bits_equal(a, b):
         return False
     if a.dtype == np.float32:
         return np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    if a.dtype == np.float64:
+        return np.array_equal(a.view(np.uint64), b.view(np.uint64))
     return np.array_equal(a, b)
 
 

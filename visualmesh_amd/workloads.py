@@ -21,8 +21,8 @@ def fourcc(s):
     return b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24)
 
 
-def make_hoc(height, pitch, roll=0.0, yaw=0.0):
-    """Camera-to-observation-plane transform, row major 4x4 float32.
+def make_hoc(height, pitch, roll=0.0, yaw=0.0, dtype=np.float32):
+    """Camera-to-observation-plane transform, row major 4x4 (float32 unless dtype says otherwise).
 
     Rotation = Rz(yaw) . Ry(pitch) . Rx(roll); the camera looks along its own x axis (y left, z up), so a
     positive pitch tilts the optical axis down towards the observation plane. Translation = (0, 0, height).
@@ -36,7 +36,7 @@ def make_hoc(height, pitch, roll=0.0, yaw=0.0):
     H = np.eye(4)
     H[:3, :3] = Rz @ Ry @ Rx
     H[2, 3] = height
-    return H.astype(np.float32)
+    return H.astype(dtype)
 
 
 def random_image(rng, width, height, bytes_per_pixel):
