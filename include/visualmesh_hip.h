@@ -43,8 +43,10 @@ enum {
 enum { VMHIP_RECTILINEAR = 0, VMHIP_EQUISOLID = 1, VMHIP_EQUIDISTANT = 2 };
 /* Same numbering as the reference's ActivationFunction (network_structure.hpp:34-39). */
 enum { VMHIP_SELU = 0, VMHIP_RELU = 1, VMHIP_SOFTMAX = 2, VMHIP_TANH = 3 };
-/* Arithmetic of the graph-convolution layers. Projection and sampling are always fp32. */
-enum { VMHIP_FP32 = 0, VMHIP_BF16 = 1 };
+/* Arithmetic of the graph-convolution layers of a float engine (vmhip_engine_create); its projection and sampling are
+ * always fp32. VMHIP_FP64 names the arithmetic of the double engines further down, which have entry points of their own
+ * (every number they take or return is a double, so the structures differ): vmhip_engine_create refuses it and says so. */
+enum { VMHIP_FP32 = 0, VMHIP_BF16 = 1, VMHIP_FP64 = 2 };
 
 /* POD mirror of visualmesh::Lens<float> (reference lens.hpp:41-52). */
 typedef struct vmhip_lens {
@@ -305,6 +307,68 @@ int vmhip_selftest_copy(int64_t bytes, int32_t repeats, float* ms);
  * system gives a kernel with that mix of reads and writes at best: the ceiling the gather-bound layers are measured
  * against next to the 8 TB/s peak. */
 int vmhip_selftest_stream(int64_t rows, int32_t read_bytes_per_row, int32_t write_bytes_per_row, int32_t repeats, float* ms);
+
+/* ---- Scalar = double ----
+ * The reference's engines and meshes are templates over Scalar (engine/cpu/engine.hpp:49-50, mesh.hpp:56; the training
+ * op registers float and double, tensorflow/lookup.cpp:255-278). These entry points are what Engine<double> binds: the
+ * same path as vmhip_project / vmhip_classify with every stage in fp64 on the device - projection, the strict on-screen
+ * filter, compaction, the neighbourhood table, sampling, and the layers on the fp64 matrix cores. The mesh must be the
+ * one Mesh<double, Model> generates (a double mesh is not the float mesh rounded: ring sizes come from ceil() of
+ * quotients in Scalar), the ranges what its lookup returns. One frame per call; structures and meanings mirror the float
+ * ones above. Layers may have any number of inputs; a softmax layer at most 128 outputs. */
+typedef struct vmhip_lens_f64 {
+    int32_t width, height;
+    int32_t projection;
+    double focal_length;
+    double centre[2];
+    double k[2];
+    double fov;
+} vmhip_lens_f64;
+typedef struct vmhip_layer_f64 {
+    int32_t n_in, n_out;
+    int32_t activation;
+    const double* weights; /* [n_in][n_out] row major */
+    const double* biases;  /* [n_out] */
+} vmhip_layer_f64;
+typedef struct vmhip_network_f64 {
+    int32_t n_groups;
+    const int32_t* group_sizes;
+    const vmhip_layer_f64* layers;
+} vmhip_network_f64;
+typedef struct vmhip_engine_f64 vmhip_engine_f64;
+typedef struct vmhip_mesh_f64 vmhip_mesh_f64;
+typedef struct vmhip_frame_f64 {
+    const vmhip_mesh_f64* mesh;
+    double Rco[9];         /* row major; Rco[i][j] = Hoc[j][i] */
+    vmhip_lens_f64 lens;
+    const int32_t* ranges; /* n_ranges pairs (first, one-past-last), ascending and disjoint */
+    int32_t n_ranges;
+    const void* image;     /* NULL when only projecting */
+    uint32_t fourcc;
+} vmhip_frame_f64;
+typedef struct vmhip_result_f64 {
+    int32_t capacity;  /* in nodes: at least the sum of the range lengths */
+    int32_t n_visible; /* written by the library */
+    double* pixel_coordinates; /* [capacity][2] */
+    int32_t* global_indices;   /* [capacity] */
+    int32_t* neighbourhood;    /* [capacity+1][n_neighbours] */
+    double* classifications;   /* [capacity+1][n_classes]; may be NULL when projecting */
+} vmhip_result_f64;
+/* Replaces cpu::Engine<double>'s constructor (reference engine/cpu/engine.hpp:57-71). */
+int vmhip_engine_create_f64(const vmhip_network_f64* net, int32_t n_neighbours, vmhip_engine_f64** out);
+void vmhip_engine_destroy_f64(vmhip_engine_f64* engine);
+int32_t vmhip_engine_n_classes_f64(const vmhip_engine_f64* engine);
+/* rays[n_nodes][3] of doubles, neighbours[n_nodes][n_neighbours] as for vmhip_mesh_upload */
+int vmhip_mesh_upload_f64(const double* rays, const int32_t* neighbours, int32_t n_nodes, int32_t n_neighbours,
+                          vmhip_mesh_f64** out);
+void vmhip_mesh_release_f64(vmhip_mesh_f64* mesh);
+/* Replace cpu::Engine<double>::operator()(mesh, Hoc, lens) and (mesh, Hoc, lens, image, format)
+ * (reference engine/cpu/engine.hpp:84-147, :180-273). */
+int vmhip_project_f64(vmhip_engine_f64* engine, const vmhip_frame_f64* frame, vmhip_result_f64* result);
+int vmhip_classify_f64(vmhip_engine_f64* engine, const vmhip_frame_f64* frame, vmhip_result_f64* result);
+/* What the edge guard of a double engine did since the engine was made (see vmhip_batch_guard_stats): near-edge nodes
+ * the device listed, device decisions the host overruled. Either pointer may be NULL. */
+int vmhip_engine_guard_stats_f64(const vmhip_engine_f64* engine, int64_t* listed, int64_t* overruled);
 
 #ifdef __cplusplus
 }

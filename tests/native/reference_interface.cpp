@@ -15,21 +15,22 @@
 #include "visualmesh/utility/fourcc.hpp"
 #include "visualmesh/visualmesh.hpp"
 
-int main() {
-    using Scalar = float;
-    visualmesh::geometry::Sphere<Scalar> shape(0.0949f);
-    visualmesh::Mesh<Scalar, visualmesh::model::Ring6> mesh(shape, 1.2f, 6.0f, 5.0f);
-    visualmesh::VisualMesh<Scalar, visualmesh::model::Ring6> heights(shape, 0.8f, 1.5f, 6.0f, 0.5f, 5.0f);
+/* the same calls for both Scalars the reference's engines are instantiated with (engine/cpu/engine.hpp:49-50) */
+template <typename Scalar>
+int use_engine() {
+    visualmesh::geometry::Sphere<Scalar> shape(Scalar(0.0949));
+    visualmesh::Mesh<Scalar, visualmesh::model::Ring6> mesh(shape, Scalar(1.2), Scalar(6.0), Scalar(5.0));
+    visualmesh::VisualMesh<Scalar, visualmesh::model::Ring6> heights(shape, Scalar(0.8), Scalar(1.5), Scalar(6.0), Scalar(0.5), Scalar(5.0));
     visualmesh::NetworkStructure<Scalar> network;
     visualmesh::engine::hip::Engine<Scalar> engine(network);
-    visualmesh::mat4<Scalar> Hoc = {{{{1, 0, 0, 0}}, {{0, 1, 0, 0}}, {{0, 0, 1, 1.2f}}, {{0, 0, 0, 1}}}};
+    visualmesh::mat4<Scalar> Hoc = {{{{1, 0, 0, 0}}, {{0, 1, 0, 0}}, {{0, 0, 1, Scalar(1.2)}}, {{0, 0, 0, 1}}}};
     visualmesh::Lens<Scalar> lens;
     lens.dimensions = {{1280, 1024}};
     lens.projection = visualmesh::EQUISOLID;
     lens.focal_length = 420;
     lens.centre = {{0, 0}};
     lens.k = {{0, 0}};
-    lens.fov = 3.14159265f;
+    lens.fov = Scalar(3.14159265);
     std::vector<uint8_t> image(1280 * 1024 * 4);
     visualmesh::ProjectedMesh<Scalar, visualmesh::model::Ring6<Scalar>::N_NEIGHBOURS> projected = engine(mesh, Hoc, lens);
     auto projected_too = engine.project(mesh, Hoc, lens);
@@ -41,3 +42,5 @@ int main() {
     return int(projected.global_indices.size() + projected_too.global_indices.size() + classified.global_indices.size()
                + by_height.global_indices.size() + projected_by_height.global_indices.size());
 }
+
+int main() { return use_engine<float>() + use_engine<double>(); }

@@ -47,6 +47,25 @@ def test_struct_layouts_match_the_header():
     assert native.Detections.node.offset == 16 and native.Detections.cluster_centre.offset == 64
 
 
+def test_double_struct_layouts_match_the_header(tmp_path):
+    """the _f64 structures as the C compiler lays them out against the ctypes mirrors, and the double host library"""
+    import subprocess
+    src = tmp_path / "layout.c"
+    src.write_text('#include <stdio.h>\n#include <stddef.h>\n#include "visualmesh_hip.h"\nint main(void) { printf("%zu %zu %zu %zu %zu %zu %zu %zu\\n", '
+                   'sizeof(vmhip_lens_f64), sizeof(vmhip_layer_f64), sizeof(vmhip_network_f64), sizeof(vmhip_frame_f64), sizeof(vmhip_result_f64), '
+                   'offsetof(vmhip_frame_f64, lens), offsetof(vmhip_frame_f64, ranges), offsetof(vmhip_frame_f64, fourcc)); return 0; }\n')
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", "-std=c99", "-I" + os.path.join(ROOT, "include"), str(src), "-o", str(exe)], check=True)
+    got = [int(v) for v in subprocess.run([str(exe)], stdout=subprocess.PIPE, universal_newlines=True, check=True).stdout.split()]
+    want = [ctypes.sizeof(native.Lens64), ctypes.sizeof(native.Layer64), ctypes.sizeof(native.NetworkC64), ctypes.sizeof(native.Frame64),
+            ctypes.sizeof(native.Result64), native.Frame64.lens.offset, native.Frame64.ranges.offset, native.Frame64.fourcc.offset]
+    assert got == want
+    lib = native.host64()
+    for name in ("vmh_mesh_create", "vmh_mesh_lookup", "vmh_visualmesh_create", "vmh_engine_create", "vmh_engine_project", "vmh_engine_classify",
+                 "vmh_engine_guard_stats"):
+        assert hasattr(lib, name)
+
+
 def build_integration_snippet(directory):
     """the reference's call sites with the engine type changed, compiled as C++14 against the host headers and linked
     with the HIP library; returns the executable"""

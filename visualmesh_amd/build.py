@@ -24,11 +24,14 @@ ARCH = "gfx950"
 # Packed-fp32 instructions are switched off for all device code.
 HIP_FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC", "-I" + INCLUDE, "-I" + CSRC,
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument", "-Wno-inline-asm"]
-# Host code that must reproduce the reference's fp32 arithmetic: one IEEE operation per step.
-HOST_EXACT_FLAGS = ["-std=c++14", "-O2", "-ffp-contract=off", "-fPIC", "-Wall", "-Wextra"]
+# Host code that must reproduce the reference's arithmetic: one IEEE operation per step, and sin(x), cos(x) as the two
+# C library calls the sources write (merged into sincos() by the compiler, their double results differ in the last bit
+# for some arguments).
+HOST_EXACT_FLAGS = ["-std=c++14", "-O2", "-ffp-contract=off", "-fno-builtin-sin", "-fno-builtin-cos", "-fPIC", "-Wall", "-Wextra"]
 
 HIP_LIB = os.path.join(LIB, "libvisualmesh_hip.so")
 HOST_LIB = os.path.join(LIB, "libvisualmesh_host.so")
+HOST_LIB_F64 = os.path.join(LIB, "libvisualmesh_host_f64.so")
 
 
 def _run(cmd):
@@ -67,6 +70,8 @@ def build_hip(force=False):
         ("conv_narrow.hip", HIP_FLAGS),
         ("detect.hip", HIP_FLAGS),
         ("noalloc.hip", HIP_FLAGS),
+        # the double engine: its projection keeps the reference's operation order too
+        ("f64.hip", HIP_FLAGS + ["-ffp-contract=off"]),
         ("api.hip", HIP_FLAGS),
     ]
     for name, flags in units:
@@ -90,9 +95,10 @@ def build_host(force=False):
     small C interface so that Python tests and the benchmark drive the real C++ host code."""
     os.makedirs(LIB, exist_ok=True)
     src = os.path.join(PKG, "capi", "host_capi.cpp")
-    if force or _stale(HOST_LIB, [src, HIP_LIB] + _headers()):
-        _run([CXX] + HOST_EXACT_FLAGS + ["-I" + CPP, "-I" + INCLUDE, "-shared", src, "-o", HOST_LIB,
-                                         "-L" + LIB, "-lvisualmesh_hip", "-Wl,-rpath,$ORIGIN", "-pthread"])
+    for target, defines in ((HOST_LIB, []), (HOST_LIB_F64, ["-DVMH_DOUBLE"])):  # Scalar = float, Scalar = double
+        if force or _stale(target, [src, HIP_LIB] + _headers()):
+            _run([CXX] + HOST_EXACT_FLAGS + defines + ["-I" + CPP, "-I" + INCLUDE, "-shared", src, "-o", target,
+                                                       "-L" + LIB, "-lvisualmesh_hip", "-Wl,-rpath,$ORIGIN", "-pthread"])
     return HOST_LIB
 
 

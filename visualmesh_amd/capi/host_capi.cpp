@@ -5,6 +5,10 @@
  *
  * Functions return a count / 0 on success or a negative status (the VMHIP_ERR_* values);
  * vmh_last_error() holds the message of the last failure on the calling thread.
+ *
+ * Compiled twice: as it stands for Scalar = float (libvisualmesh_host.so), and with -DVMH_DOUBLE for Scalar = double
+ * (libvisualmesh_host_f64.so: the same names with `real` = double and the _f64 structures of visualmesh_hip.h; the
+ * parts of Engine<float> that Engine<double> does not offer - staged batches, lookup graphs, model files - are left out).
  */
 #include <cstring>
 #include <memory>
@@ -22,35 +26,49 @@
 #include "visualmesh/utility/load_model.hpp"
 #include "visualmesh/visualmesh.hpp"
 
+#if defined(VMH_DOUBLE)
+typedef double real;
+typedef vmhip_lens_f64 vmh_lens_t;
+typedef vmhip_layer_f64 vmh_layer_t;
+typedef vmhip_network_f64 vmh_network_t;
+#else
+typedef float real;
+typedef vmhip_lens vmh_lens_t;
+typedef vmhip_layer vmh_layer_t;
+typedef vmhip_network vmh_network_t;
+#endif
+
 using namespace visualmesh;
 using geometry::Circle;
 using geometry::Sphere;
 using model::NMGrid8;
 using model::Ring6;
-typedef engine::hip::Engine<float> HipEngine;
+typedef engine::hip::Engine<real> HipEngine;
 
 enum { VMH_RING6 = 0, VMH_NMGRID8 = 1 };
 enum { VMH_SPHERE = 0, VMH_CIRCLE = 1 };
 
 struct vmh_mesh {
-    const Mesh<float, Ring6>* r6 = nullptr;
-    const Mesh<float, NMGrid8>* g8 = nullptr;
-    std::unique_ptr<Mesh<float, Ring6>> own_r6;
-    std::unique_ptr<Mesh<float, NMGrid8>> own_g8;
+    const Mesh<real, Ring6>* r6 = nullptr;
+    const Mesh<real, NMGrid8>* g8 = nullptr;
+    std::unique_ptr<Mesh<real, Ring6>> own_r6;
+    std::unique_ptr<Mesh<real, NMGrid8>> own_g8;
 };
 struct vmh_visualmesh {
-    std::unique_ptr<VisualMesh<float, Ring6>> r6;
-    std::unique_ptr<VisualMesh<float, NMGrid8>> g8;
+    std::unique_ptr<VisualMesh<real, Ring6>> r6;
+    std::unique_ptr<VisualMesh<real, NMGrid8>> g8;
     std::vector<std::unique_ptr<vmh_mesh>> views;  // ascending height
 };
+#if !defined(VMH_DOUBLE)
 struct vmh_model {
-    ModelFile<float> file;
+    ModelFile<real> file;
 };
+#endif
 struct vmh_engine {
     int model;
     std::unique_ptr<HipEngine> engine;
-    std::vector<ClassifiedMesh<float, 6>> fetched6;
-    std::vector<ClassifiedMesh<float, 8>> fetched8;
+    std::vector<ClassifiedMesh<real, 6>> fetched6;
+    std::vector<ClassifiedMesh<real, 8>> fetched8;
 };
 
 namespace {
@@ -70,8 +88,8 @@ int report(const std::exception& e) {
         return report(e);               \
     }
 
-Lens<float> to_lens(const vmhip_lens* l) {
-    Lens<float> lens;
+Lens<real> to_lens(const vmh_lens_t* l) {
+    Lens<real> lens;
     lens.dimensions = {{l->width, l->height}};
     lens.projection = LensProjection(l->projection);
     lens.focal_length = l->focal_length;
@@ -80,21 +98,21 @@ Lens<float> to_lens(const vmhip_lens* l) {
     lens.fov = l->fov;
     return lens;
 }
-mat4<float> to_hoc(const float* H) {
-    mat4<float> m;
+mat4<real> to_hoc(const real* H) {
+    mat4<real> m;
     for (int i = 0; i < 4; ++i)
         for (int j = 0; j < 4; ++j) m[i][j] = H[i * 4 + j];
     return m;
 }
-NetworkStructure<float> to_network(const vmhip_network* net) {
-    NetworkStructure<float> s;
+NetworkStructure<real> to_network(const vmh_network_t* net) {
+    NetworkStructure<real> s;
     int li = 0;
     for (int g = 0; net && g < net->n_groups; ++g) {
         s.emplace_back();
         for (int l = 0; l < net->group_sizes[g]; ++l, ++li) {
-            const vmhip_layer& L = net->layers[li];
-            Layer<float> layer;
-            layer.weights.assign(L.n_in, std::vector<float>(L.n_out));
+            const vmh_layer_t& L = net->layers[li];
+            Layer<real> layer;
+            layer.weights.assign(L.n_in, std::vector<real>(L.n_out));
             for (int t = 0; t < L.n_in; ++t)
                 for (int j = 0; j < L.n_out; ++j) layer.weights[t][j] = L.weights[size_t(t) * L.n_out + j];
             layer.biases.assign(L.biases, L.biases + L.n_out);
@@ -106,7 +124,7 @@ NetworkStructure<float> to_network(const vmhip_network* net) {
 }
 
 template <typename M>
-void copy_nodes(const M& mesh, float* rays, int32_t* nbr) {
+void copy_nodes(const M& mesh, real* rays, int32_t* nbr) {
     const int nn = M::N_NEIGHBOURS;
     for (size_t i = 0; i < mesh.nodes.size(); ++i) {
         if (rays)
@@ -117,7 +135,7 @@ void copy_nodes(const M& mesh, float* rays, int32_t* nbr) {
 }
 
 template <typename R>
-int export_result(const R& r, int cap, float* px, int32_t* nb, int32_t* gidx) {
+int export_result(const R& r, int cap, real* px, int32_t* nb, int32_t* gidx) {
     const int V = int(r.global_indices.size());
     if (V > cap) {
         g_error = "result capacity too small";
@@ -126,7 +144,7 @@ int export_result(const R& r, int cap, float* px, int32_t* nb, int32_t* gidx) {
     /* an empty projection still has its null row (the caller's table holds cap + 1 rows); an empty classification has none */
     if (nb && !r.neighbourhood.empty()) std::memcpy(nb, r.neighbourhood.data(), sizeof(r.neighbourhood[0]) * r.neighbourhood.size());
     if (V == 0) return 0;
-    if (px) std::memcpy(px, r.pixel_coordinates.data(), sizeof(float) * 2 * V);
+    if (px) std::memcpy(px, r.pixel_coordinates.data(), sizeof(real) * 2 * V);
     if (gidx) std::memcpy(gidx, r.global_indices.data(), sizeof(int32_t) * V);
     return V;
 }
@@ -136,18 +154,18 @@ extern "C" {
 
 const char* vmh_last_error(void) { return g_error.c_str(); }
 
-vmh_mesh* vmh_mesh_create(int model, int shape, float radius, float h, float k, float max_distance) {
+vmh_mesh* vmh_mesh_create(int model, int shape, real radius, real h, real k, real max_distance) {
     try {
         std::unique_ptr<vmh_mesh> m(new vmh_mesh());
         if (model == VMH_RING6) {
-            if (shape == VMH_SPHERE) m->own_r6.reset(new Mesh<float, Ring6>(Sphere<float>(radius), h, k, max_distance));
-            else if (shape == VMH_CIRCLE) m->own_r6.reset(new Mesh<float, Ring6>(Circle<float>(radius), h, k, max_distance));
+            if (shape == VMH_SPHERE) m->own_r6.reset(new Mesh<real, Ring6>(Sphere<real>(radius), h, k, max_distance));
+            else if (shape == VMH_CIRCLE) m->own_r6.reset(new Mesh<real, Ring6>(Circle<real>(radius), h, k, max_distance));
             else return nullptr;
             m->r6 = m->own_r6.get();
         }
         else if (model == VMH_NMGRID8) {
-            if (shape == VMH_SPHERE) m->own_g8.reset(new Mesh<float, NMGrid8>(Sphere<float>(radius), h, k, max_distance));
-            else if (shape == VMH_CIRCLE) m->own_g8.reset(new Mesh<float, NMGrid8>(Circle<float>(radius), h, k, max_distance));
+            if (shape == VMH_SPHERE) m->own_g8.reset(new Mesh<real, NMGrid8>(Sphere<real>(radius), h, k, max_distance));
+            else if (shape == VMH_CIRCLE) m->own_g8.reset(new Mesh<real, NMGrid8>(Circle<real>(radius), h, k, max_distance));
             else return nullptr;
             m->g8 = m->own_g8.get();
         }
@@ -161,12 +179,12 @@ vmh_mesh* vmh_mesh_create(int model, int shape, float radius, float h, float k, 
 void vmh_mesh_destroy(vmh_mesh* m) { delete m; }
 int vmh_mesh_n_nodes(const vmh_mesh* m) { return m->r6 ? int(m->r6->nodes.size()) : int(m->g8->nodes.size()); }
 int vmh_mesh_n_neighbours(const vmh_mesh* m) { return m->r6 ? 6 : 8; }
-float vmh_mesh_h(const vmh_mesh* m) { return m->r6 ? m->r6->h : m->g8->h; }
-void vmh_mesh_copy(const vmh_mesh* m, float* rays, int32_t* neighbours) {
+real vmh_mesh_h(const vmh_mesh* m) { return m->r6 ? m->r6->h : m->g8->h; }
+void vmh_mesh_copy(const vmh_mesh* m, real* rays, int32_t* neighbours) {
     if (m->r6) copy_nodes(*m->r6, rays, neighbours);
     else copy_nodes(*m->g8, rays, neighbours);
 }
-int vmh_mesh_lookup(const vmh_mesh* m, const float* Hoc16, const vmhip_lens* lens, int32_t* ranges, int cap) {
+int vmh_mesh_lookup(const vmh_mesh* m, const real* Hoc16, const vmh_lens_t* lens, int32_t* ranges, int cap) {
     GUARD({
         const auto r = m->r6 ? m->r6->lookup(to_hoc(Hoc16), to_lens(lens)) : m->g8->lookup(to_hoc(Hoc16), to_lens(lens));
         for (int i = 0; i < int(r.size()) && i < cap; ++i) {
@@ -177,13 +195,13 @@ int vmh_mesh_lookup(const vmh_mesh* m, const float* Hoc16, const vmhip_lens* len
     })
 }
 
-vmh_visualmesh* vmh_visualmesh_create(int model, int shape, float radius, float min_h, float max_h, float k, float max_error,
-                                      float max_distance) {
+vmh_visualmesh* vmh_visualmesh_create(int model, int shape, real radius, real min_h, real max_h, real k, real max_error,
+                                      real max_distance) {
     try {
         std::unique_ptr<vmh_visualmesh> v(new vmh_visualmesh());
         if (model == VMH_RING6) {
-            if (shape == VMH_SPHERE) v->r6.reset(new VisualMesh<float, Ring6>(Sphere<float>(radius), min_h, max_h, k, max_error, max_distance));
-            else v->r6.reset(new VisualMesh<float, Ring6>(Circle<float>(radius), min_h, max_h, k, max_error, max_distance));
+            if (shape == VMH_SPHERE) v->r6.reset(new VisualMesh<real, Ring6>(Sphere<real>(radius), min_h, max_h, k, max_error, max_distance));
+            else v->r6.reset(new VisualMesh<real, Ring6>(Circle<real>(radius), min_h, max_h, k, max_error, max_distance));
             for (const auto& kv : v->r6->meshes()) {
                 std::unique_ptr<vmh_mesh> view(new vmh_mesh());
                 view->r6 = &kv.second;
@@ -191,8 +209,8 @@ vmh_visualmesh* vmh_visualmesh_create(int model, int shape, float radius, float 
             }
         }
         else if (model == VMH_NMGRID8) {
-            if (shape == VMH_SPHERE) v->g8.reset(new VisualMesh<float, NMGrid8>(Sphere<float>(radius), min_h, max_h, k, max_error, max_distance));
-            else v->g8.reset(new VisualMesh<float, NMGrid8>(Circle<float>(radius), min_h, max_h, k, max_error, max_distance));
+            if (shape == VMH_SPHERE) v->g8.reset(new VisualMesh<real, NMGrid8>(Sphere<real>(radius), min_h, max_h, k, max_error, max_distance));
+            else v->g8.reset(new VisualMesh<real, NMGrid8>(Circle<real>(radius), min_h, max_h, k, max_error, max_distance));
             for (const auto& kv : v->g8->meshes()) {
                 std::unique_ptr<vmh_mesh> view(new vmh_mesh());
                 view->g8 = &kv.second;
@@ -209,14 +227,14 @@ vmh_visualmesh* vmh_visualmesh_create(int model, int shape, float radius, float 
 void vmh_visualmesh_destroy(vmh_visualmesh* v) { delete v; }
 int vmh_visualmesh_n_meshes(const vmh_visualmesh* v) { return int(v->views.size()); }
 const vmh_mesh* vmh_visualmesh_mesh(const vmh_visualmesh* v, int i) { return v->views[i].get(); }
-const vmh_mesh* vmh_visualmesh_height(const vmh_visualmesh* v, float h) {
+const vmh_mesh* vmh_visualmesh_height(const vmh_visualmesh* v, real h) {
     const void* picked = v->r6 ? static_cast<const void*>(&v->r6->height(h)) : static_cast<const void*>(&v->g8->height(h));
     for (const auto& view : v->views)
         if (static_cast<const void*>(view->r6) == picked || static_cast<const void*>(view->g8) == picked) return view.get();
     return nullptr;
 }
 
-int vmh_engine_create(const vmhip_network* net, int model, int precision, vmh_engine** out) {
+int vmh_engine_create(const vmh_network_t* net, int model, int precision, vmh_engine** out) {
     GUARD({
         std::unique_ptr<vmh_engine> e(new vmh_engine());
         e->model = model;
@@ -227,7 +245,7 @@ int vmh_engine_create(const vmhip_network* net, int model, int precision, vmh_en
 }
 void vmh_engine_destroy(vmh_engine* e) { delete e; }
 
-int vmh_engine_project(vmh_engine* e, const vmh_mesh* m, const float* Hoc16, const vmhip_lens* lens, int cap, float* px,
+int vmh_engine_project(vmh_engine* e, const vmh_mesh* m, const real* Hoc16, const vmh_lens_t* lens, int cap, real* px,
                        int32_t* nb, int32_t* gidx) {
     GUARD({
         if (m->r6) return export_result(e->engine->project(*m->r6, to_hoc(Hoc16), to_lens(lens)), cap, px, nb, gidx);
@@ -235,24 +253,33 @@ int vmh_engine_project(vmh_engine* e, const vmh_mesh* m, const float* Hoc16, con
     })
 }
 
-int vmh_engine_classify(vmh_engine* e, const vmh_mesh* m, const float* Hoc16, const vmhip_lens* lens, const void* image,
-                        uint32_t fourcc, int cap, float* px, int32_t* nb, int32_t* gidx, float* cls) {
+int vmh_engine_classify(vmh_engine* e, const vmh_mesh* m, const real* Hoc16, const vmh_lens_t* lens, const void* image,
+                        uint32_t fourcc, int cap, real* px, int32_t* nb, int32_t* gidx, real* cls) {
     GUARD({
         if (m->r6) {
             const auto r = (*e->engine)(*m->r6, to_hoc(Hoc16), to_lens(lens), image, fourcc);
             const int V = export_result(r, cap, px, nb, gidx);
-            if (V > 0 && cls) std::memcpy(cls, r.classifications.data(), sizeof(float) * r.classifications.size());
+            if (V > 0 && cls) std::memcpy(cls, r.classifications.data(), sizeof(real) * r.classifications.size());
             return V;
         }
         const auto r = (*e->engine)(*m->g8, to_hoc(Hoc16), to_lens(lens), image, fourcc);
         const int V = export_result(r, cap, px, nb, gidx);
-        if (V > 0 && cls) std::memcpy(cls, r.classifications.data(), sizeof(float) * r.classifications.size());
+        if (V > 0 && cls) std::memcpy(cls, r.classifications.data(), sizeof(real) * r.classifications.size());
         return V;
     })
 }
 
+#if defined(VMH_DOUBLE)
+int vmh_engine_guard_stats(vmh_engine* e, int64_t* listed, int64_t* overruled) {
+    GUARD({
+        const auto stats = e->engine->guard_stats();
+        *listed = stats.first, *overruled = stats.second;
+        return 0;
+    })
+}
+#else
 /* staged batch: all frames must use meshes of the engine's model */
-int vmh_engine_stage(vmh_engine* e, int n, const vmh_mesh* const* meshes, const float* Hoc16s, const vmhip_lens* lenses,
+int vmh_engine_stage(vmh_engine* e, int n, const vmh_mesh* const* meshes, const real* Hoc16s, const vmh_lens_t* lenses,
                      const void* const* images, const uint32_t* fourccs) {
     GUARD({
         if (e->model == VMH_RING6) {
@@ -299,22 +326,22 @@ int vmh_engine_fetch(vmh_engine* e) {
     })
 }
 /* copies frame i of the last fetch */
-int vmh_engine_result(vmh_engine* e, int i, int cap, float* px, int32_t* nb, int32_t* gidx, float* cls) {
+int vmh_engine_result(vmh_engine* e, int i, int cap, real* px, int32_t* nb, int32_t* gidx, real* cls) {
     GUARD({
         if (e->model == VMH_RING6) {
             const auto& r = e->fetched6.at(i);
             const int V = export_result(r, cap, px, nb, gidx);
-            if (V > 0 && cls) std::memcpy(cls, r.classifications.data(), sizeof(float) * r.classifications.size());
+            if (V > 0 && cls) std::memcpy(cls, r.classifications.data(), sizeof(real) * r.classifications.size());
             return V;
         }
         const auto& r = e->fetched8.at(i);
         const int V = export_result(r, cap, px, nb, gidx);
-        if (V > 0 && cls) std::memcpy(cls, r.classifications.data(), sizeof(float) * r.classifications.size());
+        if (V > 0 && cls) std::memcpy(cls, r.classifications.data(), sizeof(real) * r.classifications.size());
         return V;
     })
 }
 /* lookup_graph() of staged frame i: returns its number of points; copies when the arrays hold that many rows */
-int vmh_engine_lookup_graph(vmh_engine* e, int i, int same_edges, int cap, float* vectors, int32_t* graph, float* pixels) {
+int vmh_engine_lookup_graph(vmh_engine* e, int i, int same_edges, int cap, real* vectors, int32_t* graph, real* pixels) {
     GUARD({
         typedef HipEngine E;
         const E::EdgeType edges = same_edges ? E::SAME : E::HARD;
@@ -323,9 +350,9 @@ int vmh_engine_lookup_graph(vmh_engine* e, int i, int same_edges, int cap, float
             const auto& g = all.at(i);
             const int n = int(g.vectors.size());
             if (n <= cap && n > 0) {
-                std::memcpy(vectors, g.vectors.data(), sizeof(float) * 3 * n);
+                std::memcpy(vectors, g.vectors.data(), sizeof(real) * 3 * n);
                 std::memcpy(graph, g.graph.data(), sizeof(int32_t) * 7 * n);
-                if (pixels) std::memcpy(pixels, g.pixel_coordinates.data(), sizeof(float) * 2 * n);
+                if (pixels) std::memcpy(pixels, g.pixel_coordinates.data(), sizeof(real) * 2 * n);
             }
             return n;
         }
@@ -333,9 +360,9 @@ int vmh_engine_lookup_graph(vmh_engine* e, int i, int same_edges, int cap, float
         const auto& g = all.at(i);
         const int n = int(g.vectors.size());
         if (n <= cap && n > 0) {
-            std::memcpy(vectors, g.vectors.data(), sizeof(float) * 3 * n);
+            std::memcpy(vectors, g.vectors.data(), sizeof(real) * 3 * n);
             std::memcpy(graph, g.graph.data(), sizeof(int32_t) * 9 * n);
-            if (pixels) std::memcpy(pixels, g.pixel_coordinates.data(), sizeof(float) * 2 * n);
+            if (pixels) std::memcpy(pixels, g.pixel_coordinates.data(), sizeof(real) * 2 * n);
         }
         return n;
     })
@@ -355,7 +382,7 @@ int vmh_engine_cache_info(vmh_engine* e, uint64_t* bytes) {
 vmh_model* vmh_model_load(const char* path) {
     try {
         std::unique_ptr<vmh_model> m(new vmh_model());
-        m->file = load_model_file<float>(path);
+        m->file = load_model_file<real>(path);
         return m.release();
     } catch (const std::exception& e) {
         report(e);
@@ -364,7 +391,7 @@ vmh_model* vmh_model_load(const char* path) {
 }
 void vmh_model_free(vmh_model* m) { delete m; }
 /* names are copied into caller buffers of `cap` bytes */
-int vmh_model_info(const vmh_model* m, char* mesh, char* shape, int cap, float* radius, float* intersections) {
+int vmh_model_info(const vmh_model* m, char* mesh, char* shape, int cap, real* radius, real* intersections) {
     GUARD({
         if (cap <= 0) throw std::invalid_argument("model_info: no room for the names");
         std::strncpy(mesh, m->file.mesh.c_str(), size_t(cap) - 1);
@@ -379,21 +406,21 @@ int vmh_model_group_size(const vmh_model* m, int group) {
     GUARD({ return int(m->file.network.at(group).size()); })
 }
 /* sizes of a layer; weights (row major [n_in][n_out]) and biases are copied when the pointers are not null */
-int vmh_model_layer(const vmh_model* m, int group, int layer, int* n_in, int* n_out, int* activation, float* weights, float* biases) {
+int vmh_model_layer(const vmh_model* m, int group, int layer, int* n_in, int* n_out, int* activation, real* weights, real* biases) {
     GUARD({
-        const Layer<float>& l = m->file.network.at(group).at(layer);
+        const Layer<real>& l = m->file.network.at(group).at(layer);
         *n_in = int(l.weights.size());
         *n_out = int(l.biases.size());
         *activation = int(l.activation);
         if (weights)
-            for (size_t r = 0; r < l.weights.size(); ++r) std::memcpy(weights + r * l.biases.size(), l.weights[r].data(), sizeof(float) * l.biases.size());
-        if (biases) std::memcpy(biases, l.biases.data(), sizeof(float) * l.biases.size());
+            for (size_t r = 0; r < l.weights.size(); ++r) std::memcpy(weights + r * l.biases.size(), l.weights[r].data(), sizeof(real) * l.biases.size());
+        if (biases) std::memcpy(biases, l.biases.data(), sizeof(real) * l.biases.size());
         return 0;
     })
 }
-int vmh_lens_load(const char* path, int width, int height, vmhip_lens* lens, float* Hoc16) {
+int vmh_lens_load(const char* path, int width, int height, vmh_lens_t* lens, real* Hoc16) {
     GUARD({
-        const LensFile<float> f = load_lens<float>(path, width, height);
+        const LensFile<real> f = load_lens<real>(path, width, height);
         lens->width = width;
         lens->height = height;
         lens->projection = int(f.lens.projection);
@@ -406,4 +433,5 @@ int vmh_lens_load(const char* path, int width, int height, vmhip_lens* lens, flo
         return 0;
     })
 }
+#endif  // !VMH_DOUBLE
 }

@@ -33,17 +33,18 @@
 namespace visualmesh {
 namespace detail {
 
-    class ConeTree {
+    template <typename T>
+    class ConeTreeT {
     public:
         struct Element {
             int first, last;  ///< node range [first, last) in sorted order
             int child[2];     ///< -1, -1 for a leaf
-            Cone cone;
+            ConeT<T> cone;
         };
 
         /// Builds the tree over `rays` (generation order) and returns the sorted order:
         /// order[new_position] = generation index.
-        std::vector<int> build(const std::vector<f3>& rays) {
+        std::vector<int> build(const std::vector<vec3<T>>& rays) {
             rays_ = &rays;
             std::vector<int> order(rays.size());
             std::iota(order.begin(), order.end(), 0);
@@ -68,25 +69,25 @@ namespace detail {
         /// four cones (or planes) along the screen edges. visible_ranges() works these out for itself; a walk that
         /// runs elsewhere (on the device) is handed them.
         struct Parameters {
-            float cos_half_fov, sin_half_fov;
-            Cone edges[4];
+            T cos_half_fov, sin_half_fov;
+            ConeT<T> edges[4];
         };
-        static Parameters lookup_parameters(const mat4<float>& Hoc, const Lens<float>& lens) {
+        static Parameters lookup_parameters(const mat4<T>& Hoc, const Lens<T>& lens) {
             Parameters p;
-            p.cos_half_fov = std::cos(lens.fov * 0.5f);
-            p.sin_half_fov = std::sin(lens.fov * 0.5f);
+            p.cos_half_fov = std::cos(lens.fov * T(0.5));
+            p.sin_half_fov = std::sin(lens.fov * T(0.5));
             screen_edges(Hoc, lens, p.edges);
             return p;
         }
 
         /// On-screen candidate ranges. ray_at(i) returns the unit vector of node i in sorted order.
         template <typename RayAt>
-        std::vector<std::pair<int, int>> visible_ranges(const RayAt& ray_at, const mat4<float>& Hoc, const Lens<float>& lens) const {
-            const float cos_half_fov = std::cos(lens.fov * 0.5f);
-            const float sin_half_fov = std::sin(lens.fov * 0.5f);
-            const mat3<float> Rco = rotation_co(Hoc);
-            const f3 optical_axis = Rco[0];
-            Cone edges[4];
+        std::vector<std::pair<int, int>> visible_ranges(const RayAt& ray_at, const mat4<T>& Hoc, const Lens<T>& lens) const {
+            const T cos_half_fov = std::cos(lens.fov * T(0.5));
+            const T sin_half_fov = std::sin(lens.fov * T(0.5));
+            const mat3<T> Rco = rotation_co(Hoc);
+            const vec3<T> optical_axis = Rco[0];
+            ConeT<T> edges[4];
             screen_edges(Hoc, lens, edges);
 
             std::vector<std::pair<int, int>> ranges;
@@ -105,7 +106,7 @@ namespace detail {
                 todo.pop_back();
 
                 // field-of-view cone first: cos(a -/+ b) by the compound angle formula
-                const float along = dot(optical_axis, e.cone.axis);
+                const T along = dot(optical_axis, e.cone.axis);
                 bool outside = along < cos_half_fov * e.cone.c - sin_half_fov * e.cone.s;
                 bool inside = along > cos_half_fov * e.cone.c + sin_half_fov * e.cone.s;
                 if (!outside && inside) cone_on_screen(Rco, e.cone, lens, edges, inside, outside);
@@ -122,8 +123,8 @@ namespace detail {
                 }
                 else if (e.child[0] < 0) {
                     for (int i = e.first; i < e.last; ++i) {
-                        const f3 ray = ray_at(i);
-                        const f2 px = project(apply(Rco, ray), lens);
+                        const vec3<T> ray = ray_at(i);
+                        const vec2<T> px = project(apply(Rco, ray), lens);
                         const bool on_screen = dot(optical_axis, ray) > cos_half_fov && 0 <= px[0] && px[0] + 1 <= lens.dimensions[0]
                                                && 0 <= px[1] && px[1] + 1 <= lens.dimensions[1];
                         if (on_screen) {
@@ -150,9 +151,9 @@ namespace detail {
     private:
         typedef std::vector<int>::iterator Iter;
 
-        Cone enclose(Iter begin, Iter end) const {
-            const std::vector<f3>& R = *rays_;
-            Cone k = cone_through();
+        ConeT<T> enclose(Iter begin, Iter end) const {
+            const std::vector<vec3<T>>& R = *rays_;
+            ConeT<T> k = cone_through<T>();
             for (Iter a = begin; a < end; ++a) {
                 if (!(dot(k.axis, R[*a]) < k.c)) continue;
                 k = cone_through(R[*a]);
@@ -168,7 +169,7 @@ namespace detail {
         }
 
         int split(Iter begin, Iter end, int offset) {
-            const std::vector<f3>& R = *rays_;
+            const std::vector<vec3<T>>& R = *rays_;
             const int count = int(std::distance(begin, end));
             if (count == 0) throw std::runtime_error("We tried to make a tree with no nodes");
             const int leaf_size = 8;
@@ -183,10 +184,10 @@ namespace detail {
             if (elements_.empty()) {
                 // root: the cone around straight-down that reaches the highest node; children = sign of y
                 Iter top = std::max_element(begin, end, [&R](const int& a, const int& b) { return R[a][2] < R[b][2]; });
-                const float c = -R[*top][2];
-                const float s = std::sqrt(1 - c * c);
+                const T c = -R[*top][2];
+                const T s = std::sqrt(1 - c * c);
                 Iter mid = std::partition(begin, end, [&R](const int& a) { return R[a][1] > 0; });
-                elements_.push_back(Element{offset, count, {-1, -1}, Cone{f3{{0, 0, -1}}, c, s}});
+                elements_.push_back(Element{offset, count, {-1, -1}, ConeT<T>{vec3<T>{{0, 0, -1}}, c, s}});
                 const int left = split(begin, mid, 0);
                 const int right = split(mid, end, int(std::distance(begin, mid)));
                 elements_[0].child[0] = left;
@@ -194,17 +195,17 @@ namespace detail {
                 return 0;
             }
 
-            const Cone cone = enclose(begin, end);
+            const ConeT<T> cone = enclose(begin, end);
 
             // extents of z ("phi") and of x / sqrt(1 - z^2) ("theta"); split the wider one at its mean
-            float z_min = std::numeric_limits<float>::max(), z_max = std::numeric_limits<float>::lowest();
-            float t_min = std::numeric_limits<float>::max(), t_max = std::numeric_limits<float>::lowest();
-            float z_sum = 0, t_sum = 0;
+            T z_min = std::numeric_limits<T>::max(), z_max = std::numeric_limits<T>::lowest();
+            T t_min = std::numeric_limits<T>::max(), t_max = std::numeric_limits<T>::lowest();
+            T z_sum = 0, t_sum = 0;
             int z_count = 0, t_count = 0;
             for (Iter it = begin; it != end; ++it) {
-                const f3& ray = R[*it];
-                const float z = ray[2];
-                const float t = ray[0] / std::sqrt(1 - ray[2] * ray[2]);
+                const vec3<T>& ray = R[*it];
+                const T z = ray[2];
+                const T t = ray[0] / std::sqrt(1 - ray[2] * ray[2]);
                 z_min = std::min(z_min, z);
                 z_max = std::max(z_max, z);
                 z_sum += z;
@@ -216,8 +217,8 @@ namespace detail {
                     t_count += 1;
                 }
             }
-            const float z_split = z_sum / z_count;
-            const float t_split = t_sum / t_count;
+            const T z_split = z_sum / z_count;
+            const T t_split = t_sum / t_count;
             Iter mid = z_max - z_min > t_max - t_min
                          ? std::partition(begin, end, [&R, &z_split](const int& a) { return R[a][2] > z_split; })
                          : std::partition(begin, end, [&R, &t_split](const int& a) {
@@ -234,28 +235,28 @@ namespace detail {
         }
 
         /// Four cones (fisheye) or planes (rectilinear) hugging the image edges, in observation-plane space.
-        static void screen_edges(const mat4<float>& Hoc, const Lens<float>& lens, Cone (&edges)[4]) {
-            const mat3<float> Roc = rotation_oc(Hoc);
+        static void screen_edges(const mat4<T>& Hoc, const Lens<T>& lens, ConeT<T> (&edges)[4]) {
+            const mat3<T> Roc = rotation_oc(Hoc);
             // one pixel inside the border
-            const f2 far{{float(lens.dimensions[0]) - 1.0f, float(lens.dimensions[1]) - 1.0f}};
-            const f3 corner[4] = {
-              apply(Roc, unproject(f2{{1, 1}}, lens)),
-              apply(Roc, unproject(f2{{far[0], 1}}, lens)),
-              apply(Roc, unproject(f2{{far[0], far[1]}}, lens)),
-              apply(Roc, unproject(f2{{1, far[1]}}, lens)),
+            const vec2<T> far{{T(lens.dimensions[0]) - T(1.0), T(lens.dimensions[1]) - T(1.0)}};
+            const vec3<T> corner[4] = {
+              apply(Roc, unproject(vec2<T>{{1, 1}}, lens)),
+              apply(Roc, unproject(vec2<T>{{far[0], 1}}, lens)),
+              apply(Roc, unproject(vec2<T>{{far[0], far[1]}}, lens)),
+              apply(Roc, unproject(vec2<T>{{1, far[1]}}, lens)),
             };
             switch (lens.projection) {
                 case RECTILINEAR:
-                    for (int i = 0; i < 4; ++i) edges[i] = Cone{unit(cross(corner[(i + 1) & 3], corner[i])), 0, 1};
+                    for (int i = 0; i < 4; ++i) edges[i] = ConeT<T>{unit(cross(corner[(i + 1) & 3], corner[i])), 0, 1};
                     return;
                 case EQUIDISTANT:
                 case EQUISOLID: {
-                    const f2 mid{{far[0] * 0.5f + lens.centre[0], far[1] * 0.5f + lens.centre[1]}};
-                    const f3 edge_mid[4] = {
-                      apply(Roc, unproject(f2{{mid[0], 1}}, lens)),
-                      apply(Roc, unproject(f2{{far[0], mid[1]}}, lens)),
-                      apply(Roc, unproject(f2{{mid[0], far[1]}}, lens)),
-                      apply(Roc, unproject(f2{{1, mid[1]}}, lens)),
+                    const vec2<T> mid{{far[0] * T(0.5) + lens.centre[0], far[1] * T(0.5) + lens.centre[1]}};
+                    const vec3<T> edge_mid[4] = {
+                      apply(Roc, unproject(vec2<T>{{mid[0], 1}}, lens)),
+                      apply(Roc, unproject(vec2<T>{{far[0], mid[1]}}, lens)),
+                      apply(Roc, unproject(vec2<T>{{mid[0], far[1]}}, lens)),
+                      apply(Roc, unproject(vec2<T>{{1, mid[1]}}, lens)),
                     };
                     for (int i = 0; i < 4; ++i) edges[i] = with_sine(cone_through(corner[(i + 1) & 3], edge_mid[i], corner[i]));
                     return;
@@ -264,12 +265,12 @@ namespace detail {
             }
         }
 
-        static void cone_on_screen(const mat3<float>& Rco, const Cone& cone, const Lens<float>& lens, const Cone (&edges)[4],
+        static void cone_on_screen(const mat3<T>& Rco, const ConeT<T>& cone, const Lens<T>& lens, const ConeT<T> (&edges)[4],
                                    bool& inside, bool& outside) {
-            const f2 px = project(apply(Rco, cone.axis), lens);
+            const vec2<T> px = project(apply(Rco, cone.axis), lens);
             const bool axis_on_screen =
               0 <= px[0] && px[0] + 1 <= lens.dimensions[0] && 0 <= px[1] && px[1] + 1 <= lens.dimensions[1];
-            float along[4];
+            T along[4];
             bool beyond = false;
             for (int i = 0; i < 4; ++i) {
                 along[i] = dot(cone.axis, edges[i].axis);
@@ -287,8 +288,10 @@ namespace detail {
         }
 
         std::vector<Element> elements_;
-        const std::vector<f3>* rays_ = nullptr;
+        const std::vector<vec3<T>>* rays_ = nullptr;
     };
+
+    typedef ConeTreeT<float> ConeTree;
 
 }  // namespace detail
 }  // namespace visualmesh

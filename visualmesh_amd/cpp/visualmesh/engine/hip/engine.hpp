@@ -88,11 +88,12 @@ namespace engine {
             throw std::system_error(code, hip_error_category(), what);
         }
 
-        enum class Precision { FP32 = VMHIP_FP32, BF16 = VMHIP_BF16 };
+        enum class Precision { FP32 = VMHIP_FP32, BF16 = VMHIP_BF16, FP64 = VMHIP_FP64 };
 
+        /// Engine<float> is the template below; Engine<double> is the specialisation at the end of this file.
         template <typename Scalar>
         class Engine {
-            static_assert(std::is_same<Scalar, float>::value, "the HIP engine computes in float");
+            static_assert(std::is_same<Scalar, float>::value, "Scalar is float (this template) or double (the specialisation below)");
 
         public:
             /// One frame of a batch.
@@ -630,6 +631,246 @@ namespace engine {
             bool device_lookup_ = false;
             mutable size_t cache_bytes_ = 0, cache_limit_ = size_t(8) << 30;
             mutable std::vector<FrameData> staged_;
+        };
+
+        /**
+         * Scalar = double (the reference's engines are templates over Scalar, engine/cpu/engine.hpp:49-50): the reference
+         * interface - construction from a NetworkStructure<double>, projection and classification of a
+         * Mesh<double, Model> or VisualMesh<double, Model> - with every stage in fp64 on the device. It is the engine for
+         * callers that need the reference's double results; the batch pipeline, the lookup on the device and the
+         * detections of Engine<float> are not offered here. One frame per call.
+         */
+        template <>
+        class Engine<double> {
+            typedef double Scalar;
+
+        public:
+            template <template <typename> class Model>
+            struct Frame {
+                const Mesh<Scalar, Model>* mesh;
+                mat4<Scalar> Hoc;
+                Lens<Scalar> lens;
+                const void* image;
+                uint32_t format;
+            };
+
+            Engine(const NetworkStructure<Scalar>& structure = {}, Precision precision = Precision::FP64) {
+                if (precision != Precision::FP64) throw std::invalid_argument("Engine<double> computes in fp64");
+                for (const auto& group : structure) {
+                    group_sizes_.push_back(int32_t(group.size()));
+                    for (const auto& layer : group) {
+                        FlatLayer flat;
+                        flat.n_in = int32_t(layer.weights.size());
+                        flat.n_out = int32_t(layer.biases.size());
+                        flat.activation = int32_t(layer.activation);
+                        flat.weights.reserve(size_t(flat.n_in) * flat.n_out);
+                        for (const auto& row : layer.weights) {
+                            if (int32_t(row.size()) != flat.n_out) throw std::invalid_argument("ragged weight matrix");
+                            flat.weights.insert(flat.weights.end(), row.begin(), row.end());
+                        }
+                        flat.biases = layer.biases;
+                        layers_.push_back(std::move(flat));
+                    }
+                }
+            }
+            ~Engine() { release(); }
+            Engine(const Engine&) = delete;
+            Engine& operator=(const Engine&) = delete;
+
+            template <template <typename> class Model>
+            ProjectedMesh<Scalar, Model<Scalar>::N_NEIGHBOURS> operator()(const Mesh<Scalar, Model>& mesh, const mat4<Scalar>& Hoc,
+                                                                          const Lens<Scalar>& lens) const {
+                constexpr int N = Model<Scalar>::N_NEIGHBOURS;
+                ProjectedMesh<Scalar, N> out;
+                std::array<int, N> null_row;
+                null_row.fill(0);
+                std::vector<int32_t> ranges;
+                vmhip_frame_f64 f = describe(mesh, Hoc, lens, nullptr, 0, ranges);
+                const int candidates = count(ranges);
+                vmhip_result_f64 r{};
+                if (candidates > 0) {
+                    out.pixel_coordinates.resize(candidates);
+                    out.global_indices.resize(candidates);
+                    out.neighbourhood.resize(size_t(candidates) + 1);
+                    r.capacity = candidates;
+                    r.pixel_coordinates = reinterpret_cast<double*>(out.pixel_coordinates.data());
+                    r.global_indices = out.global_indices.data();
+                    r.neighbourhood = reinterpret_cast<int32_t*>(out.neighbourhood.data());
+                    throw_on_error(vmhip_project_f64(handle(N), &f, &r));
+                }
+                /* nothing visible: the neighbourhood table is its null row alone, pointing at itself (reference
+                 * engine/cpu/engine.hpp:127-143 with n_points = 0) */
+                out.pixel_coordinates.resize(r.n_visible);
+                out.global_indices.resize(r.n_visible);
+                out.neighbourhood.resize(size_t(r.n_visible) + 1);
+                if (r.n_visible == 0) out.neighbourhood[0] = null_row;
+                return out;
+            }
+            template <template <typename> class Model>
+            ProjectedMesh<Scalar, Model<Scalar>::N_NEIGHBOURS> operator()(const VisualMesh<Scalar, Model>& mesh, const mat4<Scalar>& Hoc,
+                                                                          const Lens<Scalar>& lens) const {
+                return operator()(mesh.height(Hoc[2][3]), Hoc, lens);
+            }
+            template <typename AnyMesh>
+            auto project(const AnyMesh& mesh, const mat4<Scalar>& Hoc, const Lens<Scalar>& lens) const
+              -> decltype(this->operator()(mesh, Hoc, lens)) {
+                return operator()(mesh, Hoc, lens);
+            }
+
+            template <template <typename> class Model>
+            ClassifiedMesh<Scalar, Model<Scalar>::N_NEIGHBOURS> operator()(const Mesh<Scalar, Model>& mesh, const mat4<Scalar>& Hoc,
+                                                                           const Lens<Scalar>& lens, const void* image,
+                                                                           const uint32_t& format) const {
+                constexpr int N = Model<Scalar>::N_NEIGHBOURS;
+                ClassifiedMesh<Scalar, N> out;
+                std::vector<int32_t> ranges;
+                vmhip_frame_f64 f = describe(mesh, Hoc, lens, image, format, ranges);
+                const int candidates = count(ranges);
+                vmhip_engine_f64* e = handle(N);
+                const int classes = vmhip_engine_n_classes_f64(e);
+                vmhip_result_f64 r{};
+                out.pixel_coordinates.resize(candidates);
+                out.global_indices.resize(candidates);
+                out.neighbourhood.resize(size_t(candidates) + 1);
+                out.classifications.resize((size_t(candidates) + 1) * classes);
+                r.capacity = candidates;
+                r.pixel_coordinates = reinterpret_cast<double*>(out.pixel_coordinates.data());
+                r.global_indices = out.global_indices.data();
+                r.neighbourhood = reinterpret_cast<int32_t*>(out.neighbourhood.data());
+                r.classifications = out.classifications.data();
+                /* called with no candidates too, so that an unsupported format throws as in the reference */
+                throw_on_error(vmhip_classify_f64(e, &f, &r));
+                if (r.n_visible == 0) return ClassifiedMesh<Scalar, N>();  // reference engine/cpu/engine.hpp:193
+                out.pixel_coordinates.resize(r.n_visible);
+                out.global_indices.resize(r.n_visible);
+                out.neighbourhood.resize(size_t(r.n_visible) + 1);
+                out.classifications.resize((size_t(r.n_visible) + 1) * classes);
+                return out;
+            }
+            template <template <typename> class Model>
+            ClassifiedMesh<Scalar, Model<Scalar>::N_NEIGHBOURS> operator()(const VisualMesh<Scalar, Model>& mesh, const mat4<Scalar>& Hoc,
+                                                                           const Lens<Scalar>& lens, const void* image,
+                                                                           const uint32_t& format) const {
+                return operator()(mesh.height(Hoc[2][3]), Hoc, lens, image, format);
+            }
+            /// Independent frames, one after the other.
+            template <template <typename> class Model>
+            std::vector<ClassifiedMesh<Scalar, Model<Scalar>::N_NEIGHBOURS>> classify(const std::vector<Frame<Model>>& frames) const {
+                std::vector<ClassifiedMesh<Scalar, Model<Scalar>::N_NEIGHBOURS>> out;
+                out.reserve(frames.size());
+                for (const auto& f : frames) out.push_back(operator()(*f.mesh, f.Hoc, f.lens, f.image, f.format));
+                return out;
+            }
+
+            /// What the edge guard did since the engine was made: near-edge nodes the device listed and device decisions
+            /// the host overruled.
+            std::pair<int64_t, int64_t> guard_stats() const {
+                int64_t listed = 0, overruled = 0;
+                if (engine_) throw_on_error(vmhip_engine_guard_stats_f64(engine_, &listed, &overruled));
+                return std::make_pair(listed, overruled);
+            }
+            void clear_cache() {
+                for (auto& kv : meshes_) vmhip_mesh_release_f64(kv.second.device);
+                meshes_.clear();
+            }
+
+        private:
+            struct FlatLayer {
+                int32_t n_in, n_out, activation;
+                std::vector<double> weights, biases;
+            };
+            struct MeshEntry {
+                const void* nodes;
+                size_t count;
+                uint64_t fingerprint;
+                vmhip_mesh_f64* device;
+            };
+
+            static int count(const std::vector<int32_t>& ranges) {
+                int n = 0;
+                for (size_t i = 0; i + 1 < ranges.size(); i += 2) n += ranges[i + 1] - ranges[i];
+                return n;
+            }
+
+            vmhip_engine_f64* handle(int n_neighbours) const {
+                if (engine_ && engine_nn_ == n_neighbours) return engine_;
+                if (engine_) throw std::invalid_argument("this engine was already used with a different neighbour count");
+                std::vector<vmhip_layer_f64> flat(layers_.size());
+                for (size_t i = 0; i < layers_.size(); ++i)
+                    flat[i] = vmhip_layer_f64{layers_[i].n_in, layers_[i].n_out, layers_[i].activation, layers_[i].weights.data(),
+                                              layers_[i].biases.data()};
+                vmhip_network_f64 net{int32_t(group_sizes_.size()), group_sizes_.data(), flat.data()};
+                throw_on_error(vmhip_engine_create_f64(&net, n_neighbours, &engine_));
+                engine_nn_ = n_neighbours;
+                return engine_;
+            }
+
+            /// The device copy of a mesh, keyed like Engine<float>'s cache: address, node storage, node count and a
+            /// fingerprint of the content.
+            template <template <typename> class Model>
+            vmhip_mesh_f64* device_mesh(const Mesh<Scalar, Model>& mesh) const {
+                constexpr int N = Model<Scalar>::N_NEIGHBOURS;
+                const size_t n = mesh.nodes.size();
+                uint64_t fingerprint = 1469598103934665603ull;
+                for (size_t k = 0; k < 64 && n > 0; ++k) {
+                    const unsigned char* bytes = reinterpret_cast<const unsigned char*>(&mesh.nodes[(k * (n - 1)) / 63]);
+                    for (size_t b = 0; b < sizeof(mesh.nodes[0]); ++b) fingerprint = (fingerprint ^ bytes[b]) * 1099511628211ull;
+                }
+                auto it = meshes_.find(&mesh);
+                if (it != meshes_.end() && it->second.nodes == mesh.nodes.data() && it->second.count == n && it->second.fingerprint == fingerprint)
+                    return it->second.device;
+                if (it != meshes_.end()) {
+                    vmhip_mesh_release_f64(it->second.device);
+                    meshes_.erase(it);
+                }
+                std::vector<double> rays(n * 3);
+                std::vector<int32_t> nbr(n * N);
+                for (size_t i = 0; i < n; ++i) {
+                    for (int c = 0; c < 3; ++c) rays[i * 3 + c] = mesh.nodes[i].ray[c];
+                    for (int t = 0; t < N; ++t) nbr[i * N + t] = mesh.nodes[i].neighbours[t];
+                }
+                vmhip_mesh_f64* dev = nullptr;
+                throw_on_error(vmhip_mesh_upload_f64(rays.data(), nbr.data(), int32_t(n), N, &dev));
+                meshes_[&mesh] = MeshEntry{mesh.nodes.data(), n, fingerprint, dev};
+                return dev;
+            }
+
+            template <template <typename> class Model>
+            vmhip_frame_f64 describe(const Mesh<Scalar, Model>& mesh, const mat4<Scalar>& Hoc, const Lens<Scalar>& lens, const void* image,
+                                     uint32_t format, std::vector<int32_t>& ranges) const {
+                const auto found = mesh.lookup(Hoc, lens);
+                ranges.resize(found.size() * 2);
+                for (size_t i = 0; i < found.size(); ++i) ranges[2 * i] = found[i].first, ranges[2 * i + 1] = found[i].second;
+                vmhip_frame_f64 f;
+                std::memset(&f, 0, sizeof(f));
+                f.mesh = device_mesh(mesh);
+                for (int i = 0; i < 3; ++i)
+                    for (int j = 0; j < 3; ++j) f.Rco[i * 3 + j] = Hoc[j][i];
+                f.lens.width = lens.dimensions[0];
+                f.lens.height = lens.dimensions[1];
+                f.lens.projection = int32_t(lens.projection);
+                f.lens.focal_length = lens.focal_length;
+                f.lens.centre[0] = lens.centre[0], f.lens.centre[1] = lens.centre[1];
+                f.lens.k[0] = lens.k[0], f.lens.k[1] = lens.k[1];
+                f.lens.fov = lens.fov;
+                f.ranges = ranges.data();
+                f.n_ranges = int32_t(found.size());
+                f.image = image;
+                f.fourcc = format;
+                return f;
+            }
+
+            void release() {
+                clear_cache();
+                if (engine_) vmhip_engine_destroy_f64(engine_);
+                engine_ = nullptr;
+            }
+
+            std::vector<int32_t> group_sizes_;
+            std::vector<FlatLayer> layers_;
+            mutable vmhip_engine_f64* engine_ = nullptr;
+            mutable int engine_nn_ = -1;
+            mutable std::map<const void*, MeshEntry> meshes_;
         };
 
     }  // namespace hip

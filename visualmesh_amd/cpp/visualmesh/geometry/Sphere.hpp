@@ -1,6 +1,6 @@
 /*
  * Sphere of radius r resting on the observation plane: the shape functions a mesh generator needs
- * (reference geometry/Sphere.hpp:55-134). fp32 only; operand types follow the reference so that the
+ * (reference geometry/Sphere.hpp:55-134). Operand types follow the reference for Scalar = float and double alike so that the
  * generated mesh is bit-identical.
  */
 #ifndef VISUALMESH_GEOMETRY_SPHERE_HPP
@@ -14,13 +14,12 @@ namespace geometry {
 
     template <typename Scalar>
     struct Sphere {
-        static_assert(std::is_same<Scalar, float>::value, "the host mesh code is written for float");
         explicit Sphere(const Scalar& radius) : r(radius) {}
 
         /// angle from straight down to the centre of the n-th object
-        Scalar phi(const Scalar& n, const Scalar& h) const { return -std::atan(std::sinh(n * std::log1p(-2.0f * r / h))); }
+        Scalar phi(const Scalar& n, const Scalar& h) const { return -std::atan(std::sinh(n * std::log1p(-Scalar(2.0) * r / h))); }
         /// inverse of phi
-        Scalar n(const Scalar& phi_, const Scalar& h) const { return std::asinh(std::tan(-phi_)) / std::log1p(-2.0f * r / h); }
+        Scalar n(const Scalar& phi_, const Scalar& h) const { return std::asinh(std::tan(-phi_)) / std::log1p(-Scalar(2.0) * r / h); }
         /// ratio of intersections seen from h1 versus h0
         Scalar k(const Scalar& h0, const Scalar& h1) const {
             return (std::log(h1 - 2 * r) - std::log(h1)) / (std::log(h0 - 2 * r) - std::log(h0));
@@ -30,9 +29,9 @@ namespace geometry {
         /// angular width of the object at ring n. Below n = 0.5 it is interpolated from 2 pi to pi; that arm
         /// divides in double and both arms meet in double before the result is rounded.
         Scalar theta(const Scalar& n, const Scalar& h) const {
-            const double v = n <= 0.5 ? double(float(2.0 * M_PI)) / (1.0 + double(n * 2.0f))
-                                      : double(2.0f * std::asin(r / ((h - r) * std::tan(phi(n, h)))));
-            return float(v);
+            const double v = n <= 0.5 ? double(Scalar(2.0 * M_PI)) / (1.0 + double(n * Scalar(2.0)))
+                                      : double(Scalar(2.0) * std::asin(r / ((h - r) * std::tan(phi(n, h)))));
+            return Scalar(v);
         }
 
         Scalar r;

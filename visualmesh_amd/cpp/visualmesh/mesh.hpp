@@ -20,7 +20,6 @@ namespace visualmesh {
 
 template <typename Scalar, template <typename> class Model>
 class Mesh {
-    static_assert(std::is_same<Scalar, float>::value, "the host mesh code is written for float");
 
 public:
     static constexpr int N_NEIGHBOURS = Model<Scalar>::N_NEIGHBOURS;
@@ -37,7 +36,7 @@ public:
       : h(h), max_distance(max_distance) {
         std::vector<node_type> generated = Model<Scalar>::generate(shape, h, k, max_distance);
         const int n = int(generated.size());
-        std::vector<detail::f3> rays(n);
+        std::vector<vec3<Scalar>> rays(n);
         for (int i = 0; i < n; ++i) rays[i] = generated[i].ray;
 
         const std::vector<int> order = tree_.build(rays);
@@ -55,20 +54,19 @@ public:
 
     /// Index ranges [first, last) of nodes that may be on screen, ascending and disjoint.
     std::vector<std::pair<int, int>> lookup(const mat4<Scalar>& Hoc, const Lens<Scalar>& lens) const {
-        return tree_.visible_ranges([this](int i) -> const detail::f3& { return nodes[i].ray; }, Hoc, lens);
+        return tree_.visible_ranges([this](int i) -> const vec3<Scalar>& { return nodes[i].ray; }, Hoc, lens);
     }
 
-    /// The cone tree behind lookup(), for engines that walk it themselves.
-    /// The cone tree, for walks that run elsewhere (the HIP engine's lookup on the device)
+    /// The cone tree behind lookup(), for walks that run elsewhere (the HIP engine's lookup on the device)
 #define VISUALMESH_MESH_HAS_CONE_TREE 1
-    const detail::ConeTree& tree() const { return tree_; }
+    const detail::ConeTreeT<Scalar>& tree() const { return tree_; }
 
     Scalar h;                      ///< camera height this mesh was generated for
     Scalar max_distance;           ///< reach of the mesh
     std::vector<node_type> nodes;  ///< nodes in cone-tree order
 
 private:
-    detail::ConeTree tree_;
+    detail::ConeTreeT<Scalar> tree_;
 };
 
 }  // namespace visualmesh

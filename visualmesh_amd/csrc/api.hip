@@ -676,6 +676,11 @@ int ensure_scratch(vmhip_engine* E) {
 }  // namespace
 
 int vm_set_error(int code, const char* message) { return fail(code, message); }
+bool vm_decode_fourcc(uint32_t fourcc, int* fmt, int* bytes_per_pixel) { return decode_fourcc(fourcc, fmt, bytes_per_pixel); }
+void vm_debug_knobs(double* projection_error, double* edge_band) {
+    *projection_error = double(g_debug_px_error.load());
+    *edge_band = double(g_debug_edge_band.load());
+}
 
 extern "C" {
 
@@ -685,6 +690,8 @@ int vmhip_engine_create(const vmhip_network* net, int32_t n_neighbours, int32_t 
     if (!out) return fail(VMHIP_ERR_ARGUMENT, "engine_create: null output");
     *out = nullptr;
     if (n_neighbours < 0 || n_neighbours > 16) return fail(VMHIP_ERR_ARGUMENT, "engine_create: unsupported neighbour count");
+    if (precision == VMHIP_FP64)
+        return fail(VMHIP_ERR_ARGUMENT, "engine_create: a double engine takes double weights: use vmhip_engine_create_f64 and the other _f64 entry points");
     if (precision != VMHIP_FP32 && precision != VMHIP_BF16) return fail(VMHIP_ERR_ARGUMENT, "engine_create: unknown precision");
     int n_dev = 0;
     HIP_TRY(hipGetDeviceCount(&n_dev));

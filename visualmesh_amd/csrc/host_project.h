@@ -1,4 +1,5 @@
-/* Host-side lens projection in the reference's fp32 arithmetic (host_project.cpp). Plain C++, no HIP. */
+/* Host-side lens projection in the reference's arithmetic for Scalar = float and, with the _f64 names, double
+ * (host_project.cpp). Plain C++, no HIP. */
 #ifndef VMHIP_HOST_PROJECT_H
 #define VMHIP_HOST_PROJECT_H
 
@@ -7,5 +8,8 @@
 int vm_host_on_screen(const float* Rco, const float* ray, int projection, float focal, const float* centre,
                       const float* ik, int width, int height, float* px_out);
 void vm_host_inverse_coefficients(const float* k, float* ik);
+int vm_host_on_screen_f64(const double* Rco, const double* ray, int projection, double focal, const double* centre,
+                          const double* ik, int width, int height, double* px_out);
+void vm_host_inverse_coefficients_f64(const double* k, double* ik);
 
 #endif

@@ -289,5 +289,9 @@ struct vmhip_mesh {
  * the calling thread's message for vmhip_last_error and returns code. */
 hipError_t vm_noalloc_setup(void);
 int vm_set_error(int code, const char* message);
+/* fourcc -> sampling kind (VMHIP_FMT_*) and bytes per pixel; false for a code the reference's pixel.hpp does not take */
+bool vm_decode_fourcc(uint32_t fourcc, int* fmt, int* bytes_per_pixel);
+/* the test knobs VMHIP_DEBUG_PROJECTION_ERROR and VMHIP_DEBUG_EDGE_BAND as they stand */
+void vm_debug_knobs(double* projection_error, double* edge_band);
 
 #endif

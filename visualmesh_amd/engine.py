@@ -345,3 +345,123 @@ def load_lens(path, width, height):
     Hoc = np.zeros((4, 4), np.float32)
     native.host_check(lib.vmh_lens_load(str(path).encode(), width, height, C.byref(lens), _fp(Hoc)))
     return lens, Hoc
+
+
+# ---------------------------------------------------------------------------------------------- Scalar = double
+def _dp(a):
+    return a.ctypes.data_as(C.POINTER(C.c_double))
+
+
+class Mesh64:
+    """Mesh<double, Model> of the C++ host code"""
+
+    def __init__(self, model=None, shape=None, radius=None, h=None, k=None, max_distance=None, _ptr=None):
+        self._lib = native.host64()
+        self._owned = _ptr is None
+        if _ptr is None:
+            _ptr = self._lib.vmh_mesh_create(model, shape, radius, h, k, max_distance)
+            if not _ptr:
+                raise RuntimeError("mesh construction failed: " + self._lib.vmh_last_error().decode())
+        self.ptr = _ptr
+        self.n_nodes = self._lib.vmh_mesh_n_nodes(_ptr)
+        self.n_neighbours = self._lib.vmh_mesh_n_neighbours(_ptr)
+        self.h = self._lib.vmh_mesh_h(_ptr)
+        self._arrays = None
+
+    def __del__(self):
+        if getattr(self, "_owned", False) and self.ptr:
+            self._lib.vmh_mesh_destroy(self.ptr)
+            self.ptr = None
+
+    def arrays(self):
+        """(rays[n,3] float64, neighbours[n,nn] int32) in mesh order"""
+        if self._arrays is None:
+            rays = np.zeros((self.n_nodes, 3), np.float64)
+            nbr = np.zeros((self.n_nodes, self.n_neighbours), np.int32)
+            self._lib.vmh_mesh_copy(self.ptr, _dp(rays), _ip(nbr))
+            self._arrays = (rays, nbr)
+        return self._arrays
+
+    def lookup(self, Hoc, lens):
+        H = np.ascontiguousarray(Hoc, dtype=np.float64)
+        cap = 4096
+        while True:
+            r = np.zeros((cap, 2), np.int32)
+            n = native.host_check(self._lib.vmh_mesh_lookup(self.ptr, _dp(H), C.byref(lens), _ip(r), cap), self._lib)
+            if n <= cap:
+                return r[:n].copy()
+            cap = n
+
+    def height(self, h):
+        return self
+
+
+class VisualMesh64:
+    """VisualMesh<double, Model> of the C++ host code"""
+
+    def __init__(self, model, shape, radius, min_h, max_h, k, max_error, max_distance):
+        self._lib = native.host64()
+        self.ptr = self._lib.vmh_visualmesh_create(model, shape, radius, min_h, max_h, k, max_error, max_distance)
+        if not self.ptr:
+            raise RuntimeError("visual mesh construction failed: " + self._lib.vmh_last_error().decode())
+        n = self._lib.vmh_visualmesh_n_meshes(self.ptr)
+        self.meshes = [Mesh64(_ptr=self._lib.vmh_visualmesh_mesh(self.ptr, i)) for i in range(n)]
+        self._by_ptr = {m.ptr: m for m in self.meshes}
+
+    def __del__(self):
+        if getattr(self, "ptr", None):
+            self._lib.vmh_visualmesh_destroy(self.ptr)
+            self.ptr = None
+
+    def height(self, h):
+        return self._by_ptr[self._lib.vmh_visualmesh_height(self.ptr, float(h))]
+
+
+class Engine64:
+    """visualmesh::engine::hip::Engine<double> for meshes of one model (0 = Ring6, 1 = NMGrid8)."""
+
+    def __init__(self, network_groups, model):
+        self._lib = native.host64()
+        self.network = network_groups if isinstance(network_groups, native.Network64) else native.Network64(network_groups)
+        self.model = model
+        p = C.c_void_p()
+        native.host_check(self._lib.vmh_engine_create(C.byref(self.network.c), model, native.FP64, C.byref(p)), self._lib)
+        self.ptr = p
+
+    def __del__(self):
+        if getattr(self, "ptr", None):
+            self._lib.vmh_engine_destroy(self.ptr)
+            self.ptr = None
+
+    def _buffers(self, mesh, Hoc, lens):
+        m = mesh.height(float(Hoc[2][3]))
+        H = np.ascontiguousarray(Hoc, dtype=np.float64)
+        r = m.lookup(H, lens)
+        cap = int((r[:, 1] - r[:, 0]).sum()) if len(r) else 0
+        return m, H, cap, np.zeros((max(cap, 1), 2), np.float64), np.zeros((cap + 1, m.n_neighbours), np.int32), np.zeros(max(cap, 1), np.int32)
+
+    def project(self, mesh, Hoc, lens):
+        m, H, cap, px, nb, gidx = self._buffers(mesh, Hoc, lens)
+        V = native.host_check(self._lib.vmh_engine_project(self.ptr, m.ptr, _dp(H), C.byref(lens), cap, _dp(px), _ip(nb), _ip(gidx)), self._lib)
+        return dict(px=px[:V].copy(), nb=nb[:V + 1].copy(), gidx=gidx[:V].copy())
+
+    def classify(self, mesh, Hoc, lens, image, fcc):
+        m, H, cap, px, nb, gidx = self._buffers(mesh, Hoc, lens)
+        cls = np.zeros((cap + 1, self.network.n_out), np.float64)
+        img = np.ascontiguousarray(image)
+        V = native.host_check(self._lib.vmh_engine_classify(self.ptr, m.ptr, _dp(H), C.byref(lens), img.ctypes.data, fcc, cap,
+                                                            _dp(px), _ip(nb), _ip(gidx), _dp(cls)), self._lib)
+        if V == 0:
+            return dict(px=px[:0], nb=nb[:0], gidx=gidx[:0], cls=cls[:0])
+        return dict(px=px[:V].copy(), nb=nb[:V + 1].copy(), gidx=gidx[:V].copy(), cls=cls[:V + 1].copy())
+
+    def __call__(self, mesh, Hoc, lens, image=None, fcc=None):
+        if image is None:
+            return self.project(mesh, Hoc, lens)
+        return self.classify(mesh, Hoc, lens, image, fcc)
+
+    def guard_stats(self):
+        """dict(listed, overruled): near-edge nodes the device listed, device decisions the host overruled"""
+        a, b = C.c_int64(0), C.c_int64(0)
+        native.host_check(self._lib.vmh_engine_guard_stats(self.ptr, C.byref(a), C.byref(b)), self._lib)
+        return dict(listed=a.value, overruled=b.value)

@@ -1,8 +1,9 @@
 """ctypes bindings of the two native libraries.
 
-    hip()   libvisualmesh_hip.so   the C ABI of include/visualmesh_hip.h (kernels + device state)
-    host()  libvisualmesh_host.so  the C++ host code (Mesh, VisualMesh, visualmesh::engine::hip::Engine)
-                                   behind a small C interface
+    hip()    libvisualmesh_hip.so       the C ABI of include/visualmesh_hip.h (kernels + device state)
+    host()   libvisualmesh_host.so      the C++ host code (Mesh, VisualMesh, visualmesh::engine::hip::Engine)
+                                        behind a small C interface, instantiated for Scalar = float
+    host64() libvisualmesh_host_f64.so  the same for Scalar = double (Mesh<double, ...>, Engine<double>)
 
 There is no fallback: if a library has not been built, loading raises, and every call that needs a GPU
 fails with the library's own error when none is present.
@@ -15,9 +16,10 @@ import numpy as np
 PKG = os.path.dirname(os.path.abspath(__file__))
 HIP_LIB = os.path.join(PKG, "lib", "libvisualmesh_hip.so")
 HOST_LIB = os.path.join(PKG, "lib", "libvisualmesh_host.so")
+HOST_LIB_F64 = os.path.join(PKG, "lib", "libvisualmesh_host_f64.so")
 
 OK, ERR_HIP, ERR_FORMAT, ERR_LENS, ERR_ARGUMENT, ERR_CAPACITY = 0, -1, -2, -3, -4, -5
-FP32, BF16 = 0, 1
+FP32, BF16, FP64 = 0, 1, 2
 DEBUG_FLOW_POLL_LIMIT, DEBUG_PROJECTION_ERROR, DEBUG_EDGE_BAND = 0, 1, 2
 
 # every symbol include/visualmesh_hip.h declares
@@ -26,6 +28,8 @@ HIP_SYMBOLS = [
     "vmhip_mesh_release", "vmhip_project", "vmhip_classify", "vmhip_classify_batch", "vmhip_batch_create",
     "vmhip_batch_destroy", "vmhip_mesh_attach_tree", "vmhip_batch_stage", "vmhip_batch_ranges", "vmhip_batch_export", "vmhip_batch_run", "vmhip_batch_run_async", "vmhip_batch_wait", "vmhip_batch_counts", "vmhip_batch_fetch", "vmhip_batch_fetch_async", "vmhip_batch_fetch_wait", "vmhip_batch_detect", "vmhip_host_alloc", "vmhip_host_free",
     "vmhip_batch_profile", "vmhip_batch_profile_read", "vmhip_selftest_libm", "vmhip_selftest_copy", "vmhip_selftest_stream", "vmhip_project_noalloc", "vmhip_debug_set", "vmhip_batch_guard_stats",
+    "vmhip_engine_create_f64", "vmhip_engine_destroy_f64", "vmhip_engine_n_classes_f64", "vmhip_mesh_upload_f64", "vmhip_mesh_release_f64",
+    "vmhip_project_f64", "vmhip_classify_f64", "vmhip_engine_guard_stats_f64",
 ]
 
 
@@ -82,8 +86,42 @@ class Result(C.Structure):
                 ("classifications", C.POINTER(C.c_float))]
 
 
+class Lens64(C.Structure):
+    """vmhip_lens_f64"""
+    _fields_ = [("width", C.c_int32), ("height", C.c_int32), ("projection", C.c_int32), ("focal_length", C.c_double),
+                ("centre", C.c_double * 2), ("k", C.c_double * 2), ("fov", C.c_double)]
+
+
+def make_lens64(width, height, projection, focal_length, fov, centre=(0.0, 0.0), k=(0.0, 0.0)):
+    return Lens64(width, height, projection, focal_length, (C.c_double * 2)(*centre), (C.c_double * 2)(*k), fov)
+
+
+class Layer64(C.Structure):
+    _fields_ = [("n_in", C.c_int32), ("n_out", C.c_int32), ("activation", C.c_int32), ("weights", C.POINTER(C.c_double)),
+                ("biases", C.POINTER(C.c_double))]
+
+
+class NetworkC64(C.Structure):
+    _fields_ = [("n_groups", C.c_int32), ("group_sizes", C.POINTER(C.c_int32)), ("layers", C.POINTER(Layer64))]
+
+
+class Frame64(C.Structure):
+    _fields_ = [("mesh", C.c_void_p), ("Rco", C.c_double * 9), ("lens", Lens64), ("ranges", C.POINTER(C.c_int32)),
+                ("n_ranges", C.c_int32), ("image", C.c_void_p), ("fourcc", C.c_uint32)]
+
+
+class Result64(C.Structure):
+    _fields_ = [("capacity", C.c_int32), ("n_visible", C.c_int32), ("pixel_coordinates", C.POINTER(C.c_double)),
+                ("global_indices", C.POINTER(C.c_int32)), ("neighbourhood", C.POINTER(C.c_int32)),
+                ("classifications", C.POINTER(C.c_double))]
+
+
 def _fp(a):
     return a.ctypes.data_as(C.POINTER(C.c_float))
+
+
+def _dp(a):
+    return a.ctypes.data_as(C.POINTER(C.c_double))
 
 
 def _ip(a):
@@ -109,8 +147,28 @@ class Network:
         self.n_out = groups[-1][-1][0].shape[1] if groups else 4
 
 
+class Network64:
+    """list of groups, group = list of (weights[n_in, n_out], biases[n_out], activation) -> vmhip_network_f64"""
+
+    def __init__(self, groups):
+        self.groups = groups
+        self._keep = []
+        layers = []
+        for g in groups:
+            for (w, b, act) in g:
+                w = np.ascontiguousarray(w, dtype=np.float64)
+                b = np.ascontiguousarray(b, dtype=np.float64)
+                self._keep += [w, b]
+                layers.append(Layer64(w.shape[0], w.shape[1], act, _dp(w), _dp(b)))
+        self._layers = (Layer64 * max(len(layers), 1))(*layers)
+        self._sizes = (C.c_int32 * max(len(groups), 1))(*[len(g) for g in groups])
+        self.c = NetworkC64(len(groups), self._sizes, self._layers)
+        self.n_out = groups[-1][-1][0].shape[1] if groups else 4
+
+
 _hip = None
 _host = None
+_host64 = None
 
 
 def hip():
@@ -162,6 +220,17 @@ def hip():
     L.vmhip_batch_guard_stats.argtypes = [vp, C.POINTER(C.c_int64), C.POINTER(C.c_int64), C.POINTER(C.c_int64), C.POINTER(C.c_int64)]
     L.vmhip_project_noalloc.argtypes = [vp, C.POINTER(C.c_float), C.POINTER(Lens), C.POINTER(C.c_int32), C.c_int32, C.c_int32,
                                         C.POINTER(ProjectionDevice), vp]
+    dp = C.POINTER(C.c_double)
+    L.vmhip_engine_create_f64.argtypes = [C.POINTER(NetworkC64), C.c_int32, C.POINTER(vp)]
+    L.vmhip_engine_destroy_f64.argtypes = [vp]
+    L.vmhip_engine_destroy_f64.restype = None
+    L.vmhip_engine_n_classes_f64.argtypes = [vp]
+    L.vmhip_mesh_upload_f64.argtypes = [dp, C.POINTER(C.c_int32), C.c_int32, C.c_int32, C.POINTER(vp)]
+    L.vmhip_mesh_release_f64.argtypes = [vp]
+    L.vmhip_mesh_release_f64.restype = None
+    L.vmhip_project_f64.argtypes = [vp, C.POINTER(Frame64), C.POINTER(Result64)]
+    L.vmhip_classify_f64.argtypes = [vp, C.POINTER(Frame64), C.POINTER(Result64)]
+    L.vmhip_engine_guard_stats_f64.argtypes = [vp, C.POINTER(C.c_int64), C.POINTER(C.c_int64)]
     _hip = L
     return L
 
@@ -272,9 +341,50 @@ def host():
     return L
 
 
-def host_check(rc):
+def host64():
+    """libvisualmesh_host_f64.so (Scalar = double) with argument types set."""
+    global _host64
+    if _host64 is not None:
+        return _host64
+    hip()
+    if not os.path.exists(HOST_LIB_F64):
+        raise FileNotFoundError(HOST_LIB_F64 + " is not built: run `python -m visualmesh_amd.build`")
+    L = C.CDLL(HOST_LIB_F64)
+    vp, dp, ip = C.c_void_p, C.POINTER(C.c_double), C.POINTER(C.c_int32)
+    L.vmh_last_error.restype = C.c_char_p
+    L.vmh_mesh_create.restype = vp
+    L.vmh_mesh_create.argtypes = [C.c_int, C.c_int, C.c_double, C.c_double, C.c_double, C.c_double]
+    L.vmh_mesh_destroy.argtypes = [vp]
+    L.vmh_mesh_destroy.restype = None
+    L.vmh_mesh_n_nodes.argtypes = [vp]
+    L.vmh_mesh_n_neighbours.argtypes = [vp]
+    L.vmh_mesh_h.argtypes = [vp]
+    L.vmh_mesh_h.restype = C.c_double
+    L.vmh_mesh_copy.argtypes = [vp, dp, ip]
+    L.vmh_mesh_copy.restype = None
+    L.vmh_mesh_lookup.argtypes = [vp, dp, C.POINTER(Lens64), ip, C.c_int]
+    L.vmh_visualmesh_create.restype = vp
+    L.vmh_visualmesh_create.argtypes = [C.c_int, C.c_int] + [C.c_double] * 6
+    L.vmh_visualmesh_destroy.argtypes = [vp]
+    L.vmh_visualmesh_destroy.restype = None
+    L.vmh_visualmesh_n_meshes.argtypes = [vp]
+    L.vmh_visualmesh_mesh.restype = vp
+    L.vmh_visualmesh_mesh.argtypes = [vp, C.c_int]
+    L.vmh_visualmesh_height.restype = vp
+    L.vmh_visualmesh_height.argtypes = [vp, C.c_double]
+    L.vmh_engine_create.argtypes = [C.POINTER(NetworkC64), C.c_int, C.c_int, C.POINTER(vp)]
+    L.vmh_engine_destroy.argtypes = [vp]
+    L.vmh_engine_destroy.restype = None
+    L.vmh_engine_project.argtypes = [vp, vp, dp, C.POINTER(Lens64), C.c_int, dp, ip, ip]
+    L.vmh_engine_classify.argtypes = [vp, vp, dp, C.POINTER(Lens64), vp, C.c_uint32, C.c_int, dp, ip, ip, dp]
+    L.vmh_engine_guard_stats.argtypes = [vp, C.POINTER(C.c_int64), C.POINTER(C.c_int64)]
+    _host64 = L
+    return L
+
+
+def host_check(rc, lib=None):
     if rc < 0:
-        msg = host().vmh_last_error().decode()
+        msg = (lib or host()).vmh_last_error().decode()
         if rc == ERR_FORMAT:
             raise ValueError(msg)
         raise VisualMeshError(rc, msg)
