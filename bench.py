@@ -265,11 +265,16 @@ def measure(cfg, engine, frames, steps, warmup, settle_s, events=True, stream_ce
 
 def pinned_copies(cfg, mesh, lens):
     from visualmesh_amd import native
-    held = []
-    for f in cfg.frames:
-        a = native.pinned_empty(f["image"].shape, f["image"].dtype)
+    # one page-locked allocation for all the batch's images, as a ring of camera buffers would be: images that adjoin
+    # in memory go up in one copy
+    sizes = [int(f["image"].nbytes) for f in cfg.frames]
+    block = native.pinned_empty((sum(sizes),), np.uint8)
+    held, at = [], 0
+    for f, n in zip(cfg.frames, sizes):
+        a = block[at:at + n].view(f["image"].dtype).reshape(f["image"].shape)
         a[...] = f["image"]
         held.append(a)
+        at += n
     return held, [dict(mesh=mesh, Hoc=f["Hoc"], lens=lens, image=a, fourcc=cfg.fourcc) for f, a in zip(cfg.frames, held)]
 
 
@@ -290,7 +295,7 @@ def end_to_end(cfg, mesh, lens, nodes, batches):
         for step in range(n + 2):
             if step < n:
                 e = engines[step % 3]
-                e.stage(frames)
+                e.stage(frames, wait=False)  # the images are page-locked and stay as they are
                 e.run_async()
             if 1 <= step <= n:
                 e = engines[(step - 1) % 3]

@@ -167,6 +167,12 @@ int vmhip_classify_batch(vmhip_engine* engine, const vmhip_frame* frames, int32_
 int vmhip_batch_create(vmhip_engine* engine, vmhip_batch** out);
 void vmhip_batch_destroy(vmhip_batch* batch);
 int vmhip_batch_stage(vmhip_batch* batch, const vmhip_frame* frames, int32_t n_frames, int32_t classify);
+/* vmhip_batch_stage without the wait for its copies: they are queued on the engine's stream ahead of the run and the call
+ * returns, so a caller that rotates engines (one staging, one running, one copying out) is not held up for the 2 ms
+ * that 84 MB of images take to cross the bus. The frames' images must be page-locked (vmhip_host_alloc) for the copies
+ * to run on their own, and must stay untouched until the batch's next vmhip_batch_run or vmhip_batch_wait has returned.
+ * No counterpart in the reference, whose OpenCL engine copies the image inside the call (engine/opencl/engine.hpp:307-315). */
+int vmhip_batch_stage_async(vmhip_batch* batch, const vmhip_frame* frames, int32_t n_frames, int32_t classify);
 /* The lookup ranges of a staged frame, as pairs (first, one-past-last): the caller's own, or what the lookup on the
  * device produced. Returns their number (ranges may be NULL to ask for it only) or a negative status. */
 int vmhip_batch_ranges(const vmhip_batch* batch, int32_t frame, int32_t* ranges, int32_t capacity);

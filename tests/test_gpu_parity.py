@@ -663,16 +663,24 @@ def test_results_into_page_locked_memory(oracle):
                 assert np.array_equal(a[key], b[key]), key
 
 
-def test_fetch_in_two_halves_and_three_engines_in_rotation(oracle):
+@pytest.mark.parametrize("stage_waits", [True, False], ids=["stage", "stage_async"])
+def test_fetch_in_two_halves_and_three_engines_in_rotation(oracle, stage_waits):
     """vmhip_batch_fetch_async / vmhip_batch_fetch_wait: three engines in rotation, one staging, one running and one
     copying its results out at any time; every batch must give the oracle's results, and a batch whose fetch is in
-    flight must refuse to be staged, run or fetched again."""
+    flight must refuse to be staged, run or fetched again. With stage_async the uploads are only queued (from page-locked
+    images) and a batch staged twice in a row must end up with the second set of frames."""
     cfg = wl.config(2, n_frames=6)
     o_lens, e_lens = lens_pair(cfg)
     o_mesh, e_mesh = meshes_for(cfg, oracle)
     engines = [eng.Engine(cfg.network, cfg.model) for _ in range(3)]
     groups = [cfg.frames[0:2], cfg.frames[2:4], cfg.frames[4:6]]
-    staged = [[dict(mesh=e_mesh, Hoc=f["Hoc"], lens=e_lens, image=f["image"], fourcc=cfg.fourcc) for f in g] for g in groups]
+    images = {}
+    for g in groups:
+        for f in g:
+            held = native.pinned_empty(f["image"].shape, f["image"].dtype)
+            held[...] = f["image"]
+            images[id(f)] = held
+    staged = [[dict(mesh=e_mesh, Hoc=f["Hoc"], lens=e_lens, image=images[id(f)], fourcc=cfg.fourcc) for f in g] for g in groups]
     net = vmo.Network(cfg.network)
     wants = [[pick(o_mesh, f["Hoc"]).classify(f["Hoc"], o_lens, f["image"], cfg.fourcc, net) for f in g] for g in groups]
     results = {}
@@ -680,7 +688,9 @@ def test_fetch_in_two_halves_and_three_engines_in_rotation(oracle):
     for step in range(3 + 2):          # every engine's group once, then the pipeline drains
         if step < 3:
             e = engines[step]
-            e.stage(staged[step])
+            if not stage_waits and step == 0:
+                e.stage(staged[2], wait=False)  # overwritten by the next stage before any run
+            e.stage(staged[step], wait=stage_waits)
             e.run_async()
         if 1 <= step <= 3:
             e = engines[step - 1]

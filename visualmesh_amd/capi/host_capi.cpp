@@ -278,9 +278,9 @@ int vmh_engine_guard_stats(vmh_engine* e, int64_t* listed, int64_t* overruled) {
     })
 }
 #else
-/* staged batch: all frames must use meshes of the engine's model */
+/* staged batch: all frames must use meshes of the engine's model; wait = 0 queues the copies and returns (stage_async) */
 int vmh_engine_stage(vmh_engine* e, int n, const vmh_mesh* const* meshes, const real* Hoc16s, const vmh_lens_t* lenses,
-                     const void* const* images, const uint32_t* fourccs) {
+                     const void* const* images, const uint32_t* fourccs, int wait) {
     GUARD({
         if (e->model == VMH_RING6) {
             std::vector<HipEngine::Frame<Ring6>> frames(n);
@@ -288,7 +288,8 @@ int vmh_engine_stage(vmh_engine* e, int n, const vmh_mesh* const* meshes, const 
                 if (!meshes[i]->r6) throw std::invalid_argument("mesh model does not match the engine");
                 frames[i] = HipEngine::Frame<Ring6>{meshes[i]->r6, to_hoc(Hoc16s + 16 * i), to_lens(lenses + i), images[i], fourccs[i]};
             }
-            e->engine->stage(frames);
+            if (wait) e->engine->stage(frames);
+            else e->engine->stage_async(frames);
         }
         else {
             std::vector<HipEngine::Frame<NMGrid8>> frames(n);
@@ -296,7 +297,8 @@ int vmh_engine_stage(vmh_engine* e, int n, const vmh_mesh* const* meshes, const 
                 if (!meshes[i]->g8) throw std::invalid_argument("mesh model does not match the engine");
                 frames[i] = HipEngine::Frame<NMGrid8>{meshes[i]->g8, to_hoc(Hoc16s + 16 * i), to_lens(lenses + i), images[i], fourccs[i]};
             }
-            e->engine->stage(frames);
+            if (wait) e->engine->stage(frames);
+            else e->engine->stage_async(frames);
         }
         return 0;
     })

@@ -238,6 +238,18 @@ namespace engine {
             /// Copy the frames' inputs to the device (images, poses, lenses, lookup ranges).
             template <template <typename> class Model>
             void stage(const std::vector<Frame<Model>>& frames) const {
+                stage_frames(frames, true);
+            }
+            /// The same without waiting for the copies: they are queued ahead of the run and the call returns. The
+            /// images must be page-locked (vmhip_host_alloc) and stay untouched until run() or wait() has returned.
+            template <template <typename> class Model>
+            void stage_async(const std::vector<Frame<Model>>& frames) const {
+                stage_frames(frames, false);
+            }
+
+        private:
+            template <template <typename> class Model>
+            void stage_frames(const std::vector<Frame<Model>>& frames, bool wait_for_copies) const {
                 constexpr int N = Model<Scalar>::N_NEIGHBOURS;
                 staged_since_ = ++clock_;
                 staged_.assign(frames.size(), FrameData());
@@ -276,8 +288,12 @@ namespace engine {
                 staging_ = false;
                 vmhip_engine* e = handle(N);
                 if (!batch_) throw_on_error(vmhip_batch_create(e, &batch_));
-                if (!flat.empty()) throw_on_error(vmhip_batch_stage(batch_, flat.data(), int32_t(flat.size()), 1));
+                if (!flat.empty())
+                    throw_on_error(wait_for_copies ? vmhip_batch_stage(batch_, flat.data(), int32_t(flat.size()), 1)
+                                                   : vmhip_batch_stage_async(batch_, flat.data(), int32_t(flat.size()), 1));
             }
+
+        public:
             /// Run the staged frames on the device and wait; may be called repeatedly.
             void run() const {
                 if (batch_ && !staged_.empty()) throw_on_error(vmhip_batch_run(batch_));

@@ -140,6 +140,11 @@ struct vmhip_batch {
     void* h_pin = nullptr;
     size_t h_pin_cap = 0;
     std::vector<uint64_t> h_force_valid, h_force_keep;
+    /* pinned home of the frame descriptions and range tables a stage uploads: they must outlive a stage that does not
+     * wait for its copies */
+    void* h_stage = nullptr;
+    size_t h_stage_cap = 0;
+    bool stage_pending = false; /* copies of the last stage may still be reading h_stage (and the caller's images) */
     bool have_run = false;
     bool in_flight = false;     /* vmhip_batch_run_async without its vmhip_batch_wait */
     bool fetching = false;      /* vmhip_batch_fetch_async without its vmhip_batch_fetch_wait */
@@ -186,6 +191,8 @@ struct vmhip_batch {
         for (DevBuf* b : all) b->release();
         if (h_pin) (void) hipHostFree(h_pin);
         h_pin = nullptr, h_pin_cap = 0;
+        if (h_stage) (void) hipHostFree(h_stage);
+        h_stage = nullptr, h_stage_cap = 0;
         if (h_detect) (void) hipHostFree(h_detect);
         h_detect = nullptr, h_detect_cap = 0;
         for (hipEvent_t e : events) (void) hipEventDestroy(e);
@@ -195,9 +202,13 @@ struct vmhip_batch {
 
 namespace {
 
-int batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int32_t classify) {
+int batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int32_t classify, bool wait) {
     vmhip_engine* E = b->engine;
     if (!frames || n_frames <= 0) return fail(VMHIP_ERR_ARGUMENT, "stage: no frames");
+    if (b->stage_pending) { /* staged twice without a run between: the first stage's copies still read h_stage */
+        HIP_TRY(hipStreamSynchronize(E->stream));
+        b->stage_pending = false;
+    }
     b->have_run = false;
     b->classify = classify ? 1 : 0;
     b->frames.assign(n_frames, HostFrame());
@@ -326,25 +337,46 @@ int batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int
     b->drop_graph(); /* pointers and sizes baked into a captured run are no longer valid */
 
     /* fill in device pointers and upload */
-    std::vector<int32_t> h_ranges(std::max<size_t>(range_ints, 1));
+    const size_t n_range_ints = std::max<size_t>(range_ints, 1);
+    {
+        const size_t need = align_up(sizeof(VmFrame) * size_t(n_frames), 64) + 4 * n_range_ints;
+        if (need > b->h_stage_cap) {
+            if (b->h_stage) HIP_TRY(hipHostFree(b->h_stage));
+            b->h_stage = nullptr, b->h_stage_cap = 0;
+            HIP_TRY(hipHostMalloc(&b->h_stage, need + need / 4, hipHostMallocDefault));
+            b->h_stage_cap = need + need / 4;
+        }
+    }
+    VmFrame* h_frames = static_cast<VmFrame*>(b->h_stage);
+    int32_t* h_ranges = reinterpret_cast<int32_t*>(static_cast<char*>(b->h_stage) + align_up(sizeof(VmFrame) * size_t(n_frames), 64));
     size_t range_off = 0, image_off = 0, lookup_off = 0;
-    std::vector<VmFrame> h_frames(n_frames);
+    const uint8_t* run_src = nullptr; /* the run of adjoining images not yet copied */
+    size_t run_dst = 0, run_bytes = 0;
     for (int f = 0; f < n_frames; ++f) {
         HostFrame& hf = b->frames[f];
         VmFrame& d = hf.dev;
         const int R = d.n_ranges;
         d.range_first = b->d_ranges.as<int32_t>() + range_off;
-        std::copy(hf.first.begin(), hf.first.end(), h_ranges.begin() + range_off);
+        std::copy(hf.first.begin(), hf.first.end(), h_ranges + range_off);
         range_off += R;
         d.range_prefix = b->d_ranges.as<int32_t>() + range_off;
-        std::copy(hf.prefix.begin(), hf.prefix.end(), h_ranges.begin() + range_off);
+        std::copy(hf.prefix.begin(), hf.prefix.end(), h_ranges + range_off);
         range_off += size_t(R) + 1;
         if (classify) {
             int fmt, bpp;
             decode_fourcc(frames[f].fourcc, &fmt, &bpp);
             const size_t bytes = size_t(d.width) * d.height * bpp;
             d.image = b->d_images.as<uint8_t>() + image_off;
-            HIP_TRY(hipMemcpyAsync(b->d_images.as<uint8_t>() + image_off, frames[f].image, bytes, hipMemcpyHostToDevice, E->stream));
+            /* images that follow one another in the caller's memory (a ring of camera buffers in one allocation) and on
+             * the device go up as one copy: a few large copies cross the bus faster than many small ones */
+            const uint8_t* src = static_cast<const uint8_t*>(frames[f].image);
+            if (run_bytes > 0 && src == run_src + run_bytes && image_off == run_dst + run_bytes) {
+                run_bytes += bytes;
+            }
+            else {
+                if (run_bytes > 0) HIP_TRY(hipMemcpyAsync(b->d_images.as<uint8_t>() + run_dst, run_src, run_bytes, hipMemcpyHostToDevice, E->stream));
+                run_src = src, run_dst = image_off, run_bytes = bytes;
+            }
             image_off += align_up(bytes, 256);
         }
         d.r_lookup = b->d_lookup.as<uint2>() + lookup_off;
@@ -353,13 +385,18 @@ int batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int
         d.force_keep = b->d_force_keep.as<uint64_t>();
         h_frames[f] = d;
     }
-    HIP_TRY(hipMemcpyAsync(b->d_frames.p, h_frames.data(), sizeof(VmFrame) * n_frames, hipMemcpyHostToDevice, E->stream));
-    HIP_TRY(hipMemcpyAsync(b->d_ranges.p, h_ranges.data(), sizeof(int32_t) * h_ranges.size(), hipMemcpyHostToDevice, E->stream));
+    if (run_bytes > 0) HIP_TRY(hipMemcpyAsync(b->d_images.as<uint8_t>() + run_dst, run_src, run_bytes, hipMemcpyHostToDevice, E->stream));
+    HIP_TRY(hipMemcpyAsync(b->d_frames.p, h_frames, sizeof(VmFrame) * n_frames, hipMemcpyHostToDevice, E->stream));
+    HIP_TRY(hipMemcpyAsync(b->d_ranges.p, h_ranges, sizeof(int32_t) * n_range_ints, hipMemcpyHostToDevice, E->stream));
     HIP_TRY(hipMemsetAsync(b->d_force_valid.p, 0, 8 * std::max<size_t>(words, 1), E->stream));
     HIP_TRY(hipMemsetAsync(b->d_force_keep.p, 0, 8 * std::max<size_t>(words, 1), E->stream));
     b->h_force_valid.assign(std::max<size_t>(words, 1), 0);
     b->h_force_keep.assign(std::max<size_t>(words, 1), 0);
-    HIP_TRY(hipStreamSynchronize(E->stream)); /* the host vectors above go out of scope */
+    /* a stage that waits returns with the caller's images read; one that does not leaves its copies on the stream,
+     * ahead of the run's kernels: the tables they read live in h_stage, the images must stay as they are until the
+     * run has been waited for */
+    if (wait) HIP_TRY(hipStreamSynchronize(E->stream));
+    b->stage_pending = !wait;
 
     VmBatchDev& D = b->dev;
     D.frames = b->d_frames.as<VmFrame>();
@@ -601,6 +638,7 @@ int batch_complete(vmhip_batch* b) {
         if (rc < 0) return rc;
         if (rc == 0) {
             b->have_run = true;
+            b->stage_pending = false; /* the stream has been waited for */
             ++b->run_serial;
             return VMHIP_OK;
         }
@@ -1001,16 +1039,22 @@ static int lookup_on_device(vmhip_batch* b, const vmhip_frame* frames, int32_t n
     return VMHIP_OK;
 }
 
-int vmhip_batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int32_t classify) {
+static int stage_entry(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int32_t classify, bool wait) {
     if (!b) return fail(VMHIP_ERR_ARGUMENT, "batch_stage: null batch");
     if (b->in_flight) return fail(VMHIP_ERR_ARGUMENT, "batch_stage: a run of this batch is still in flight (vmhip_batch_wait first)");
     if (b->fetching) return fail(VMHIP_ERR_ARGUMENT, "batch_stage: a fetch of this batch is still in flight (vmhip_batch_fetch_wait first)");
     if (!frames || n_frames <= 0) return fail(VMHIP_ERR_ARGUMENT, "stage: no frames");
     std::vector<vmhip_frame> patched;
     int rc = lookup_on_device(b, frames, n_frames, patched);
-    if (rc == VMHIP_OK) rc = batch_stage(b, patched.data(), n_frames, classify);
+    if (rc == VMHIP_OK) rc = batch_stage(b, patched.data(), n_frames, classify, wait);
     if (rc != VMHIP_OK) b->frames.clear();
     return rc;
+}
+int vmhip_batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int32_t classify) {
+    return stage_entry(b, frames, n_frames, classify, true);
+}
+int vmhip_batch_stage_async(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int32_t classify) {
+    return stage_entry(b, frames, n_frames, classify, false);
 }
 int vmhip_batch_run(vmhip_batch* b) {
     if (!b) return fail(VMHIP_ERR_ARGUMENT, "batch_run: null batch");

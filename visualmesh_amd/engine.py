@@ -144,8 +144,10 @@ class Engine:
         return self.classify(mesh, Hoc, lens, image, fcc)
 
     # ---- staged batches
-    def stage(self, frames):
-        """frames: list of dict(mesh=Mesh|VisualMesh, Hoc, lens, image, fourcc); copies the inputs to the device"""
+    def stage(self, frames, wait=True):
+        """frames: list of dict(mesh=Mesh|VisualMesh, Hoc, lens, image, fourcc); copies the inputs to the device.
+        wait=False queues the copies ahead of the run and returns (Engine::stage_async): the images must then be
+        page-locked (native.pinned_empty) and stay untouched until run() or wait() has returned."""
         n = len(frames)
         meshes = [self._pick(f["mesh"], f["Hoc"]) for f in frames]
         mesh_ptrs = (C.c_void_p * n)(*[m.ptr for m in meshes])
@@ -154,8 +156,9 @@ class Engine:
         images = [np.ascontiguousarray(f["image"]) for f in frames]
         image_ptrs = (C.c_void_p * n)(*[im.ctypes.data for im in images])
         fccs = (C.c_uint32 * n)(*[f["fourcc"] for f in frames])
-        native.host_check(self._lib.vmh_engine_stage(self.ptr, n, mesh_ptrs, _fp(H), lenses, image_ptrs, fccs))
+        native.host_check(self._lib.vmh_engine_stage(self.ptr, n, mesh_ptrs, _fp(H), lenses, image_ptrs, fccs, int(bool(wait))))
         self._staged = meshes
+        self._staged_images = images  # an asynchronous stage still reads them
 
     def run(self):
         native.host_check(self._lib.vmh_engine_run(self.ptr))
