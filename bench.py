@@ -300,7 +300,7 @@ def end_to_end(cfg, mesh, lens, nodes, batches):
             if 1 <= step <= n:
                 e = engines[(step - 1) % 3]
                 e.wait()
-                e.fetch_pinned(wait=False)
+                e.fetch_pinned(wait=False)  # one copy per array: these interleave with the next batch's upload (one 50 MB copy does not)
             if step >= 2:
                 engines[(step - 2) % 3].fetch_wait()
 
@@ -365,14 +365,14 @@ def main():
     if not args.no_pcie:
         held, pinned_frames = pinned_copies(cfg, mesh, lens)
         for _ in range(2):
-            engine.stage(pinned_frames), engine.run(), engine.fetch_pinned()
+            engine.stage(pinned_frames), engine.run(), engine.fetch_packed()
         passes = 5
         t0 = time.perf_counter()
         for _ in range(passes):
-            engine.stage(pinned_frames), engine.run(), engine.fetch_pinned()
+            engine.stage(pinned_frames), engine.run(), engine.fetch_packed()
         dt = (time.perf_counter() - t0) / passes
         pcie = dict(ms_per_batch=dt * 1e3, nodes_per_s=nodes / dt, frames_per_s=len(frames) / dt,
-                    what="stage from page-locked images + run + fetch into page-locked arrays, one engine, serial")
+                    what="stage from page-locked images + run + fetch (all frames' arrays gathered on the device, one copy into a page-locked block), one engine, serial")
         del held, pinned_frames
         e2e = end_to_end(cfg, mesh, lens, nodes, 12 if big else 60)
 

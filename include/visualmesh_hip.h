@@ -212,6 +212,15 @@ int vmhip_batch_fetch(vmhip_batch* batch, vmhip_result* results);
  * arrays must not be touched. */
 int vmhip_batch_fetch_async(vmhip_batch* batch, vmhip_result* results);
 int vmhip_batch_fetch_wait(vmhip_batch* batch);
+/* vmhip_batch_fetch_async as one transfer: a kernel gathers the arrays of all frames into one block on the device and a
+ * single copy brings it into `block` (page-locked memory from vmhip_host_alloc, at least vmhip_batch_fetch_packed_size()
+ * bytes, which is known once the run has been waited for); results[i] is filled in by the library with n_visible,
+ * capacity = n_visible and pointers into `block` (NULL for a frame that sees nothing, and for classifications after a
+ * projection-only run). 64 copies of 0.8 MB on average become one of 50 MB for a 16-frame batch, which crosses the bus in
+ * two thirds of the time. Finished by vmhip_batch_fetch_wait like vmhip_batch_fetch_async. No counterpart in the
+ * reference. */
+size_t vmhip_batch_fetch_packed_size(const vmhip_batch* batch);
+int vmhip_batch_fetch_packed_async(vmhip_batch* batch, void* block, size_t bytes, vmhip_result* results);
 
 /* vmhip_project for callers that cannot allocate: code under HIP graph capture, serving loops that must not call
  * hipMalloc, harnesses that forbid it. No counterpart in the reference. The call only launches kernels on hip_stream

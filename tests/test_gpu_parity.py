@@ -1,6 +1,8 @@
 """HIP engine against the CPU oracle on the benchmark configurations, through the C++ engine and so
 through the C ABI. Gates: visible-node indices and neighbour tables bit-exact, pixel coordinates within
 1e-3 px, fp32 class probabilities within 1e-4 absolute."""
+import math
+
 import numpy as np
 import pytest
 
@@ -661,6 +663,36 @@ def test_results_into_page_locked_memory(oracle):
             assert len(a["gidx"]) > 1000
             for key in ("px", "nb", "gidx", "cls"):
                 assert np.array_equal(a[key], b[key]), key
+        # the same as one transfer: gathered into one block on the device, one copy, views into the block
+        packed = engine.fetch_packed()
+        assert len(packed) == len(chosen)
+        for a, b in zip(plain, packed):
+            for key in ("px", "nb", "gidx", "cls"):
+                assert a[key].dtype == b[key].dtype and np.array_equal(a[key], b[key]), key
+
+
+def test_packed_fetch_of_mixed_frames(oracle):
+    """vmhip_batch_fetch_packed_async on a batch whose frames differ in mesh model (6 and 8 neighbours, so the device's
+    neighbourhood rows are strided for the 6-neighbour frames), with a frame that sees nothing in the middle, and after a
+    projection-only run (no classifications)."""
+    rng = np.random.default_rng(4)
+    lens = native.make_lens(320, 256, wl.EQUISOLID, 105.0, math.pi)
+    m6 = eng.Mesh(wl.RING6, wl.SPHERE, 0.0949, 1.0, 3.0, 8.0)
+    img = wl.random_image(rng, 320, 256, 4)
+    down = wl.make_hoc(1.0, math.radians(35), 0.03, -0.02)
+    narrow = native.make_lens(320, 256, wl.RECTILINEAR, 175.0, 1.9)
+    up = wl.make_hoc(1.0, math.radians(-80), 0.0, 0.0)
+    engine = eng.Engine([], wl.RING6)
+    frames = [dict(mesh=m6, Hoc=down, lens=lens, image=img, fourcc=wl.fourcc("RGBA")),
+              dict(mesh=m6, Hoc=up, lens=narrow, image=img, fourcc=wl.fourcc("RGBA")),
+              dict(mesh=m6, Hoc=wl.make_hoc(1.0, math.radians(50), 0.0, 0.3), lens=lens, image=img, fourcc=wl.fourcc("RGBA"))]
+    engine.stage(frames)
+    engine.run()
+    plain, packed = engine.fetch(), engine.fetch_packed()
+    assert len(plain[1]["gidx"]) == 0 and len(packed[1]["gidx"]) == 0 and len(plain[0]["gidx"]) > 100
+    for a, b in zip(plain, packed):
+        for key in ("px", "nb", "gidx", "cls"):
+            assert np.array_equal(a[key], b[key]), key
 
 
 @pytest.mark.parametrize("stage_waits", [True, False], ids=["stage", "stage_async"])

@@ -352,6 +352,13 @@ namespace engine {
             void fetch_wait() const {
                 if (batch_ && !staged_.empty()) throw_on_error(vmhip_batch_fetch_wait(batch_));
             }
+            /// fetch_into_async as one transfer: all frames' arrays are gathered on the device and come home in a single copy
+            /// into `block` (page-locked, at least packed_size() bytes); results[i] point into it. Finished by fetch_wait().
+            size_t packed_size() const { return batch_ ? vmhip_batch_fetch_packed_size(batch_) : 0; }
+            void fetch_packed_async(void* block, size_t bytes, std::vector<vmhip_result>& results) const {
+                results.assign(staged_.size(), vmhip_result{});
+                if (!results.empty()) throw_on_error(vmhip_batch_fetch_packed_async(batch_, block, bytes, results.data()));
+            }
             /// The nodes of one class among the results of the last run, picked and clustered on the device so that
             /// only they are downloaded (the reference's consumers walk the whole ClassifiedMesh on the host,
             /// example/draw.hpp:41-59).

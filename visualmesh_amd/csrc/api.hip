@@ -144,6 +144,8 @@ struct vmhip_batch {
      * wait for its copies */
     void* h_stage = nullptr;
     size_t h_stage_cap = 0;
+    void* h_pack = nullptr; /* pinned home of the segment table of a packed fetch */
+    size_t h_pack_cap = 0;
     bool stage_pending = false; /* copies of the last stage may still be reading h_stage (and the caller's images) */
     bool have_run = false;
     bool in_flight = false;     /* vmhip_batch_run_async without its vmhip_batch_wait */
@@ -168,7 +170,7 @@ struct vmhip_batch {
 
     VmBatchDev dev{};
     DevBuf d_frames, d_ranges, d_images, d_cand_px, d_cand_g, d_cand_keep, d_tile_count, d_force_valid, d_force_keep, d_frame_V,
-      d_amb_list, d_row_px, d_row_gidx, d_row_nb, d_row_nbl, d_tile_halo, d_tile_desc, d_row_nbl_h, d_tile_note_h, d_active_h, d_act[2], d_lookup, d_epoch, d_detect, d_detect_packed, d_lookup_ws, d_export;
+      d_amb_list, d_row_px, d_row_gidx, d_row_nb, d_row_nbl, d_tile_halo, d_tile_desc, d_row_nbl_h, d_tile_note_h, d_active_h, d_act[2], d_lookup, d_epoch, d_detect, d_detect_packed, d_lookup_ws, d_export, d_fetch_packed;
     std::vector<std::vector<int32_t>> device_ranges; /* per frame: the ranges a lookup on the device produced */
     void* h_detect = nullptr; /* pinned landing area of vmhip_batch_detect */
     size_t h_detect_cap = 0;
@@ -186,13 +188,15 @@ struct vmhip_batch {
         DevBuf* all[] = {&d_frames, &d_ranges, &d_images, &d_cand_px, &d_cand_g, &d_cand_keep, &d_tile_count, &d_force_valid,
                          &d_force_keep, &d_frame_V, &d_amb_list, &d_row_px, &d_row_gidx, &d_row_nb,
                          &d_row_nbl, &d_tile_halo, &d_tile_desc, &d_row_nbl_h, &d_tile_note_h, &d_active_h, &d_epoch,
-                         &d_act[0], &d_act[1], &d_lookup, &d_detect, &d_detect_packed, &d_lookup_ws, &d_export};
+                         &d_act[0], &d_act[1], &d_lookup, &d_detect, &d_detect_packed, &d_lookup_ws, &d_export, &d_fetch_packed};
         drop_graph();
         for (DevBuf* b : all) b->release();
         if (h_pin) (void) hipHostFree(h_pin);
         h_pin = nullptr, h_pin_cap = 0;
         if (h_stage) (void) hipHostFree(h_stage);
         h_stage = nullptr, h_stage_cap = 0;
+        if (h_pack) (void) hipHostFree(h_pack);
+        h_pack = nullptr, h_pack_cap = 0;
         if (h_detect) (void) hipHostFree(h_detect);
         h_detect = nullptr, h_detect_cap = 0;
         for (hipEvent_t e : events) (void) hipEventDestroy(e);
@@ -519,17 +523,18 @@ int batch_request_verdict(vmhip_batch* b) {
     vmhip_engine* E = b->engine;
     const int n = int(b->frames.size());
     constexpr int HEAD = vmhip_batch::AMB_HEAD;
-    int32_t* pin_counts = reinterpret_cast<int32_t*>(b->h_pin);
+    /* a kernel stores them into the page-locked landing area: small copies would wait in the copy engine's queue behind
+     * whatever another engine is downloading */
+    void* dev_view = nullptr;
+    HIP_TRY(hipHostGetDevicePointer(&dev_view, b->h_pin, 0));
+    int32_t* pin_counts = reinterpret_cast<int32_t*>(dev_view);
     int2* pin_amb = reinterpret_cast<int2*>(pin_counts + 2 * n);
-    HIP_TRY(hipMemcpyAsync(pin_counts, b->d_frame_V.p, 8 * size_t(n), hipMemcpyDeviceToHost, E->stream));
-    HIP_TRY(hipMemcpy2DAsync(pin_amb, sizeof(int2) * HEAD, b->d_amb_list.p, sizeof(int2) * VMHIP_AMB_CAP, sizeof(int2) * HEAD, n,
-                             hipMemcpyDeviceToHost, E->stream));
+    uint32_t* pin_timeouts = reinterpret_cast<uint32_t*>(pin_amb + size_t(n) * HEAD);
     /* the barrier-free convolution kernel bounds its waits; a wait that ran out (never in a correct run) means
      * the results of this run cannot be trusted */
-    uint32_t* pin_timeouts = reinterpret_cast<uint32_t*>(pin_amb + size_t(n) * HEAD);
-    unsigned int* d_timeouts = (E->use_flow && b->classify) ? b->dev.flow_timeouts : nullptr;
-    *pin_timeouts = 0;
-    if (d_timeouts) HIP_TRY(hipMemcpyAsync(pin_timeouts, d_timeouts, 4, hipMemcpyDeviceToHost, E->stream));
+    const unsigned int* d_timeouts = (E->use_flow && b->classify) ? b->dev.flow_timeouts : nullptr;
+    vm_launch_publish(b->d_frame_V.as<int32_t>(), 2 * n, b->d_amb_list.as<int2>(), VMHIP_AMB_CAP, HEAD, n, d_timeouts, pin_counts, pin_amb, pin_timeouts, E->stream);
+    HIP_TRY(hipGetLastError());
     return VMHIP_OK;
 }
 
@@ -691,6 +696,83 @@ int batch_fetch_enqueue(vmhip_batch* b, vmhip_result* results) {
         if (R.classifications && b->classify)
             HIP_TRY(hipMemcpyAsync(R.classifications, b->final_act + base * C, 4 * size_t(V + 1) * C, hipMemcpyDeviceToHost, s));
     }
+    return VMHIP_OK;
+}
+
+/* where frame f's arrays lie in the block of a packed fetch: pixels, indices, neighbourhood, classifications, each at a
+ * multiple of 256 bytes; returns the block's size */
+size_t packed_layout(const vmhip_batch* b, std::vector<size_t>* offsets) {
+    const int n = int(b->frames.size());
+    const int C = b->engine->n_classes;
+    size_t at = 0;
+    if (offsets) offsets->assign(size_t(n) * 4, 0);
+    for (int f = 0; f < n; ++f) {
+        const size_t V = size_t(b->h_V[f]);
+        if (V == 0) continue;
+        const size_t sizes[4] = {8 * V, 4 * V, 4 * (V + 1) * size_t(b->frames[f].dev.nn), b->classify ? 4 * (V + 1) * size_t(C) : 0};
+        for (int k = 0; k < 4; ++k) {
+            if (offsets) (*offsets)[size_t(f) * 4 + k] = at;
+            at += align_up(sizes[k], 256);
+        }
+    }
+    return at;
+}
+
+/* vmhip_batch_fetch_packed_async: one kernel gathers every frame's arrays into one device block, one copy brings it home */
+int batch_fetch_packed_enqueue(vmhip_batch* b, void* block, size_t bytes, vmhip_result* results) {
+    if (!b->have_run) return fail(VMHIP_ERR_ARGUMENT, "fetch: no completed run");
+    if (!results || !block) return fail(VMHIP_ERR_ARGUMENT, "fetch_packed: null block or results");
+    if (b->fetching) return fail(VMHIP_ERR_ARGUMENT, "fetch: a fetch of this batch is still in flight (vmhip_batch_fetch_wait first)");
+    vmhip_engine* E = b->engine;
+    hipStream_t s = E->stream;
+    const int n = int(b->frames.size());
+    const int C = E->n_classes;
+    std::vector<size_t> offsets;
+    const size_t total = packed_layout(b, &offsets);
+    if (bytes < total) return fail(VMHIP_ERR_CAPACITY, "fetch_packed: the block is smaller than vmhip_batch_fetch_packed_size says");
+    const size_t table_bytes = sizeof(VmPackSegment) * size_t(n) * 4;
+    if (table_bytes > b->h_pack_cap) {
+        if (b->h_pack) HIP_TRY(hipHostFree(b->h_pack));
+        b->h_pack = nullptr, b->h_pack_cap = 0;
+        HIP_TRY(hipHostMalloc(&b->h_pack, table_bytes, hipHostMallocDefault));
+        b->h_pack_cap = table_bytes;
+    }
+    VmPackSegment* seg = static_cast<VmPackSegment*>(b->h_pack);
+    int n_seg = 0, n_chunks = 0;
+    uint8_t* host = static_cast<uint8_t*>(block);
+    for (int f = 0; f < n; ++f) {
+        const VmFrame& d = b->frames[f].dev;
+        vmhip_result& R = results[f];
+        const size_t V = size_t(b->h_V[f]);
+        R.capacity = R.n_visible = int32_t(V);
+        R.pixel_coordinates = nullptr, R.global_indices = nullptr, R.neighbourhood = nullptr, R.classifications = nullptr;
+        if (V == 0) continue;
+        const size_t base = size_t(d.row_base), stride = size_t(b->dev.nb_stride);
+        const size_t* at = &offsets[size_t(f) * 4];
+        auto add = [&](const void* src, size_t dst_offset, size_t nbytes, size_t row_bytes, size_t src_stride) {
+            seg[n_seg++] = VmPackSegment{static_cast<const uint8_t*>(src), dst_offset, nbytes, row_bytes, src_stride, n_chunks};
+            n_chunks += int((nbytes + VM_PACK_CHUNK - 1) / VM_PACK_CHUNK);
+        };
+        add(b->dev.row_px + base, at[0], 8 * V, 8, 8);
+        add(b->dev.row_gidx + base, at[1], 4 * V, 4, 4);
+        add(b->dev.row_nb + base * stride, at[2], 4 * (V + 1) * size_t(d.nn), 4 * size_t(d.nn), 4 * stride);
+        R.pixel_coordinates = reinterpret_cast<float*>(host + at[0]);
+        R.global_indices = reinterpret_cast<int32_t*>(host + at[1]);
+        R.neighbourhood = reinterpret_cast<int32_t*>(host + at[2]);
+        if (b->classify) {
+            add(b->final_act + base * C, at[3], 4 * (V + 1) * size_t(C), 4 * size_t(C), 4 * size_t(C));
+            R.classifications = reinterpret_cast<float*>(host + at[3]);
+        }
+    }
+    if (total == 0) return VMHIP_OK;
+    HIP_TRY(b->d_fetch_packed.reserve(total));
+    /* the kernel reads the table where it lies, in page-locked host memory: an upload would wait in the copy engine's
+     * queue behind the images another engine is staging. The table is not touched again before vmhip_batch_fetch_wait. */
+    void* seg_dev = nullptr;
+    HIP_TRY(hipHostGetDevicePointer(&seg_dev, seg, 0));
+    vm_launch_fetch_pack(static_cast<const VmPackSegment*>(seg_dev), n_seg, n_chunks, b->d_fetch_packed.p, s);
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipMemcpyAsync(block, b->d_fetch_packed.p, total, hipMemcpyDeviceToHost, s));
     return VMHIP_OK;
 }
 
@@ -1136,6 +1218,20 @@ int vmhip_batch_fetch_async(vmhip_batch* b, vmhip_result* results) {
     const int rc = batch_fetch_enqueue(b, results);
     if (rc != VMHIP_OK) {
         (void) hipStreamSynchronize(b->engine->stream); /* copies queued before the failure write into the caller's arrays */
+        return rc;
+    }
+    b->fetching = true;
+    return VMHIP_OK;
+}
+size_t vmhip_batch_fetch_packed_size(const vmhip_batch* b) {
+    if (!b || !b->have_run) return 0;
+    return packed_layout(b, nullptr);
+}
+int vmhip_batch_fetch_packed_async(vmhip_batch* b, void* block, size_t bytes, vmhip_result* results) {
+    if (!b) return fail(VMHIP_ERR_ARGUMENT, "batch_fetch_packed_async: null batch");
+    const int rc = batch_fetch_packed_enqueue(b, block, bytes, results);
+    if (rc != VMHIP_OK) {
+        (void) hipStreamSynchronize(b->engine->stream);
         return rc;
     }
     b->fetching = true;

@@ -238,7 +238,41 @@ __global__ __launch_bounds__(DETECT_THREADS) void vm_detect_pack_kernel(VmBatchD
     }
 }
 
+/* The results of all frames gathered into one block for a single download: segment g is `bytes` bytes at `src`, made of rows
+ * of `row_bytes` that lie `src_stride` bytes apart (equal for a contiguous array), and goes to dst + dst_offset; the segments'
+ * chunks of VM_PACK_CHUNK bytes are numbered through chunk_first. All sizes and offsets are multiples of 4, dst offsets of 256. */
+__global__ __launch_bounds__(256) void vm_fetch_pack_kernel(const VmPackSegment* __restrict__ segments, int n_segments, uint8_t* __restrict__ dst) {
+    int lo = 0, hi = n_segments - 1;
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (segments[mid].chunk_first <= (int) blockIdx.x) lo = mid;
+        else hi = mid - 1;
+    }
+    const VmPackSegment g = segments[lo];
+    const size_t begin = (size_t) ((int) blockIdx.x - g.chunk_first) * VM_PACK_CHUNK;
+    const size_t end = begin + VM_PACK_CHUNK < g.bytes ? begin + VM_PACK_CHUNK : g.bytes;
+    uint8_t* out = dst + g.dst_offset;
+    if (g.row_bytes == g.src_stride && (reinterpret_cast<uintptr_t>(g.src) & 15) == 0) {
+        const size_t vec_end = begin + ((end - begin) & ~(size_t) 15);
+        for (size_t at = begin + (size_t) threadIdx.x * 16; at < vec_end; at += 256 * 16)
+            *reinterpret_cast<uint4*>(out + at) = *reinterpret_cast<const uint4*>(g.src + at);
+        for (size_t at = vec_end + (size_t) threadIdx.x * 4; at < end; at += 256 * 4)
+            *reinterpret_cast<uint32_t*>(out + at) = *reinterpret_cast<const uint32_t*>(g.src + at);
+    }
+    else {
+        for (size_t at = begin + (size_t) threadIdx.x * 4; at < end; at += 256 * 4) {
+            const size_t row = at / g.row_bytes, in_row = at - row * g.row_bytes;
+            *reinterpret_cast<uint32_t*>(out + at) = *reinterpret_cast<const uint32_t*>(g.src + row * g.src_stride + in_row);
+        }
+    }
+}
+
 }  // namespace
+
+void vm_launch_fetch_pack(const VmPackSegment* segments, int n_segments, int n_chunks, void* dst, hipStream_t stream) {
+    if (n_segments <= 0 || n_chunks <= 0) return;
+    hipLaunchKernelGGL(vm_fetch_pack_kernel, dim3(n_chunks), dim3(256), 0, stream, segments, n_segments, static_cast<uint8_t*>(dst));
+}
 
 void vm_launch_detect_pack(const VmBatchDev& B, const VmDetectDev& D, uint32_t* packed, int total_d, int total_c, hipStream_t stream) {
     if (B.n_frames <= 0) return;

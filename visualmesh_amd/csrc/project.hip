@@ -122,6 +122,20 @@ __global__ __launch_bounds__(256) void vm_stream_probe_kernel(const uint4* __res
     }
 }
 
+/* What the host needs of a pass, written by the device straight into page-locked host memory (block f: the head of frame
+ * f's ambiguity list; block 0 also the counts and the convolution kernel's count of waits that ran out). A copy engine is
+ * not involved, so the few hundred bytes never queue behind another engine's 50 MB download. */
+__global__ __launch_bounds__(64) void vm_publish_kernel(const int32_t* __restrict__ counts, int n_counts, const int2* __restrict__ amb_list, int amb_stride,
+                                                        int amb_head, const unsigned int* __restrict__ timeouts, int32_t* host_counts, int2* host_amb,
+                                                        uint32_t* host_timeouts) {
+    const int f = blockIdx.x;
+    for (int t = threadIdx.x; t < amb_head; t += 64) host_amb[(size_t) f * amb_head + t] = amb_list[(size_t) f * amb_stride + t];
+    if (f == 0) {
+        for (int t = threadIdx.x; t < n_counts; t += 64) host_counts[t] = counts[t];
+        if (threadIdx.x == 0) *host_timeouts = timeouts ? *timeouts : 0u;
+    }
+}
+
 __global__ void vm_reset_kernel(VmBatchDev B) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < B.n_frames) {
@@ -761,6 +775,11 @@ void vm_launch_copy_probe(const void* src, void* dst, size_t bytes, hipStream_t 
 void vm_launch_stream_probe(const void* src, void* dst, size_t rows, int read_bytes_per_row, int write_bytes_per_row, hipStream_t stream) {
     hipLaunchKernelGGL(vm_stream_probe_kernel, dim3(256 * 16), dim3(256), 0, stream, reinterpret_cast<const uint4*>(src), reinterpret_cast<uint4*>(dst),
                        rows / 64, read_bytes_per_row * 4, write_bytes_per_row * 4);
+}
+void vm_launch_publish(const int32_t* counts, int n_counts, const int2* amb_list, int amb_stride, int amb_head, int n_frames, const unsigned int* timeouts,
+                       int32_t* host_counts, int2* host_amb, uint32_t* host_timeouts, hipStream_t stream) {
+    hipLaunchKernelGGL(vm_publish_kernel, dim3(n_frames > 0 ? n_frames : 1), dim3(64), 0, stream, counts, n_counts, amb_list, amb_stride, amb_head, timeouts, host_counts,
+                       host_amb, host_timeouts);
 }
 void vm_launch_reset(const VmBatchDev& B, hipStream_t stream) {
     hipLaunchKernelGGL(vm_reset_kernel, dim3((B.n_frames + 63) / 64), dim3(64), 0, stream, B);

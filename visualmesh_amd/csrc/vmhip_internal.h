@@ -190,6 +190,15 @@ void vm_detect_carve(void* workspace, size_t rows, int n_frames, VmDetectDev* D)
 void vm_launch_detect(const VmBatchDev& B, const VmDetectDev& D, int clusters, hipStream_t stream);
 /* packed: 5 * total_d + 7 * total_c words (detect.hip says in which order) */
 void vm_launch_detect_pack(const VmBatchDev& B, const VmDetectDev& D, uint32_t* packed, int total_d, int total_c, hipStream_t stream);
+/* one array of one frame on its way into the block of vmhip_batch_fetch_packed_async (detect.hip: vm_fetch_pack_kernel) */
+#define VM_PACK_CHUNK 16384
+struct VmPackSegment {
+    const uint8_t* src;
+    size_t dst_offset, bytes;        /* multiples of 256 and of 4 */
+    size_t row_bytes, src_stride;    /* equal for a contiguous array */
+    int32_t chunk_first;             /* number of the segment's first chunk of VM_PACK_CHUNK bytes */
+};
+void vm_launch_fetch_pack(const VmPackSegment* segments, int n_segments, int n_chunks, void* dst, hipStream_t stream);
 
 /* "<family>_<c_in>x<c_out>s<slots>" as a string that stays valid (the profile of a run names its kernels) */
 const char* vm_kernel_name(const char* family, int c_in, int c_out, int slots);
@@ -200,6 +209,10 @@ void vm_launch_copy_probe(const void* src, void* dst, size_t bytes, hipStream_t 
 /* rows: a multiple of 64; bytes per row: multiples of 4 (64 rows are whole 16-byte pieces then) */
 void vm_launch_stream_probe(const void* src, void* dst, size_t rows, int read_bytes_per_row, int write_bytes_per_row, hipStream_t stream);
 void vm_launch_reset(const VmBatchDev& B, hipStream_t stream);
+/* counts[n_counts], the first amb_head entries of every frame's ambiguity list and the timeout count, stored by the device
+ * into page-locked host memory (device-visible pointers) */
+void vm_launch_publish(const int32_t* counts, int n_counts, const int2* amb_list, int amb_stride, int amb_head, int n_frames, const unsigned int* timeouts,
+                       int32_t* host_counts, int2* host_amb, uint32_t* host_timeouts, hipStream_t stream);
 void vm_launch_project(const VmBatchDev& B, hipStream_t stream);
 void vm_launch_compact(const VmBatchDev& B, float* feat, int classify, hipStream_t stream);
 void vm_launch_neighbourhood(const VmBatchDev& B, hipStream_t stream); /* also the tile-local tables if B.row_nbl */

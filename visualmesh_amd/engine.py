@@ -250,6 +250,40 @@ class Engine:
             self._raw_results = raw  # the copies read this table's pointers only at the call, but keep it with the arrays
         return out
 
+    def fetch_packed(self, wait=True):
+        """fetch_pinned() as one transfer (vmhip_batch_fetch_packed_async): a kernel gathers all frames' arrays into one block on
+        the device and a single copy brings it into one page-locked block of the engine's; the arrays returned are views into
+        it, valid after fetch_wait() (or at once with wait=True) and until the next fetch_packed()."""
+        lib = native.hip()
+        n = len(self._staged)
+        need = int(lib.vmhip_batch_fetch_packed_size(self.native_batch()))
+        block = getattr(self, "_packed_block", None)
+        if block is None or block.nbytes < need:
+            block = self._packed_block = native.pinned_empty((need + need // 8 + 256,), np.uint8)
+        raw = (native.Result * n)()
+        native.hip_check(lib.vmhip_batch_fetch_packed_async(self.native_batch(), block.ctypes.data, block.nbytes, raw))
+        n_out = self.network.n_out
+        out = []
+        base = block.ctypes.data
+        for i in range(n):
+            V = raw[i].n_visible
+            nn = self._staged[i].n_neighbours
+            if V == 0:
+                out.append(dict(px=np.zeros((0, 2), np.float32), nb=np.zeros((0, nn), np.int32), gidx=np.zeros(0, np.int32), cls=np.zeros((0, n_out), np.float32)))
+                continue
+
+            def view(pointer, count, dtype, shape):
+                at = C.cast(pointer, C.c_void_p).value - base
+                return block[at:at + count * 4].view(dtype).reshape(shape)
+
+            out.append(dict(px=view(raw[i].pixel_coordinates, 2 * V, np.float32, (V, 2)), gidx=view(raw[i].global_indices, V, np.int32, (V,)),
+                            nb=view(raw[i].neighbourhood, (V + 1) * nn, np.int32, (V + 1, nn)),
+                            cls=view(raw[i].classifications, (V + 1) * n_out, np.float32, (V + 1, n_out))))
+        self._raw_results = raw
+        if wait:
+            self.fetch_wait()
+        return out
+
     def fetch_wait(self):
         """finishes fetch_pinned(wait=False): the arrays it returned are valid from here on"""
         native.hip_check(native.hip().vmhip_batch_fetch_wait(self.native_batch()))

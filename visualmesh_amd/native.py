@@ -26,7 +26,7 @@ DEBUG_FLOW_POLL_LIMIT, DEBUG_PROJECTION_ERROR, DEBUG_EDGE_BAND = 0, 1, 2
 HIP_SYMBOLS = [
     "vmhip_last_error", "vmhip_engine_create", "vmhip_engine_destroy", "vmhip_engine_n_classes", "vmhip_mesh_upload",
     "vmhip_mesh_release", "vmhip_project", "vmhip_classify", "vmhip_classify_batch", "vmhip_batch_create",
-    "vmhip_batch_destroy", "vmhip_mesh_attach_tree", "vmhip_batch_stage", "vmhip_batch_stage_async", "vmhip_batch_ranges", "vmhip_batch_export", "vmhip_batch_run", "vmhip_batch_run_async", "vmhip_batch_wait", "vmhip_batch_counts", "vmhip_batch_fetch", "vmhip_batch_fetch_async", "vmhip_batch_fetch_wait", "vmhip_batch_detect", "vmhip_host_alloc", "vmhip_host_free",
+    "vmhip_batch_destroy", "vmhip_mesh_attach_tree", "vmhip_batch_stage", "vmhip_batch_stage_async", "vmhip_batch_ranges", "vmhip_batch_export", "vmhip_batch_run", "vmhip_batch_run_async", "vmhip_batch_wait", "vmhip_batch_counts", "vmhip_batch_fetch", "vmhip_batch_fetch_async", "vmhip_batch_fetch_wait", "vmhip_batch_fetch_packed_size", "vmhip_batch_fetch_packed_async", "vmhip_batch_detect", "vmhip_host_alloc", "vmhip_host_free",
     "vmhip_batch_profile", "vmhip_batch_profile_read", "vmhip_selftest_libm", "vmhip_selftest_copy", "vmhip_selftest_stream", "vmhip_project_noalloc", "vmhip_debug_set", "vmhip_batch_guard_stats",
     "vmhip_engine_create_f64", "vmhip_engine_destroy_f64", "vmhip_engine_n_classes_f64", "vmhip_mesh_upload_f64", "vmhip_mesh_release_f64",
     "vmhip_project_f64", "vmhip_classify_f64", "vmhip_engine_guard_stats_f64",
@@ -201,6 +201,9 @@ def hip():
     L.vmhip_batch_fetch.argtypes = [vp, C.POINTER(Result)]
     L.vmhip_batch_fetch_async.argtypes = [vp, C.POINTER(Result)]
     L.vmhip_batch_fetch_wait.argtypes = [vp]
+    L.vmhip_batch_fetch_packed_size.argtypes = [vp]
+    L.vmhip_batch_fetch_packed_size.restype = C.c_size_t
+    L.vmhip_batch_fetch_packed_async.argtypes = [vp, vp, C.c_size_t, C.POINTER(Result)]
     L.vmhip_batch_run_async.argtypes = [vp]
     L.vmhip_batch_export.argtypes = [vp, C.c_int32, C.POINTER(LookupExport)]
     L.vmhip_batch_ranges.argtypes = [vp, C.c_int32, C.POINTER(C.c_int32), C.c_int32]
