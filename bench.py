@@ -348,6 +348,29 @@ def main():
     from visualmesh_amd import workloads as wl
 
     cfg, engine, mesh, lens, frames = build_workload(args.config, args.frames)
+    # PCIe-inclusive figures (never `value`), measured before anything else runs in this process: an engine that has
+    # made some hundred passes and is then left idle slows the copies of the other engines in the process (2.5-2.6 ms per
+    # batch in the rotation below against 1.86 ms on the same box; not a graph, event or stream-count effect, and gone once
+    # that engine is destroyed), so these figures are taken with only their own engines alive.
+    # Serial: images in page-locked host memory -> stage + run + fetch of the whole classified mesh into one page-locked
+    # block, one engine, the three steps one after the other. Pipelined: end_to_end() above.
+    pcie, e2e = None, None
+    if not args.no_pcie:
+        held, pinned_frames = pinned_copies(cfg, mesh, lens)
+        for _ in range(2):
+            engine.stage(pinned_frames), engine.run(), engine.fetch_packed()
+        nodes = int(engine.counts().sum())
+        passes = 5
+        t0 = time.perf_counter()
+        for _ in range(passes):
+            engine.stage(pinned_frames), engine.run(), engine.fetch_packed()
+        dt = (time.perf_counter() - t0) / passes
+        pcie = dict(ms_per_batch=dt * 1e3, nodes_per_s=nodes / dt, frames_per_s=len(frames) / dt,
+                    what="stage from page-locked images + run + fetch (all frames' arrays gathered on the device, one copy into a page-locked block), one engine, serial")
+        del held, pinned_frames, engine
+        e2e = end_to_end(cfg, mesh, lens, nodes, 12 if big else 60)
+        cfg, engine, mesh, lens, frames = build_workload(args.config, args.frames)
+
     nn = wl.N_NEIGHBOURS[cfg.model]
     m = measure(cfg, engine, frames, args.steps, args.warmup, args.settle, events=not args.no_events)
     nodes = m["nodes"]
@@ -357,24 +380,6 @@ def main():
     if not args.no_copy_probe:
         nbytes = 1 << 30
         copy_gbs = 2 * nbytes / (native.copy_probe(nbytes, 5) * 1e-3) / 1e9
-
-    # PCIe-inclusive figures (never `value`). Serial: images in page-locked host memory -> stage + run + fetch of the
-    # whole classified mesh into page-locked host arrays, one engine, the three steps one after the other. Pipelined:
-    # end_to_end() above.
-    pcie, e2e = None, None
-    if not args.no_pcie:
-        held, pinned_frames = pinned_copies(cfg, mesh, lens)
-        for _ in range(2):
-            engine.stage(pinned_frames), engine.run(), engine.fetch_packed()
-        passes = 5
-        t0 = time.perf_counter()
-        for _ in range(passes):
-            engine.stage(pinned_frames), engine.run(), engine.fetch_packed()
-        dt = (time.perf_counter() - t0) / passes
-        pcie = dict(ms_per_batch=dt * 1e3, nodes_per_s=nodes / dt, frames_per_s=len(frames) / dt,
-                    what="stage from page-locked images + run + fetch (all frames' arrays gathered on the device, one copy into a page-locked block), one engine, serial")
-        del held, pinned_frames
-        e2e = end_to_end(cfg, mesh, lens, nodes, 12 if big else 60)
 
     cpu = None
     if not args.no_cpu:
