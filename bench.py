@@ -348,10 +348,10 @@ def main():
     from visualmesh_amd import workloads as wl
 
     cfg, engine, mesh, lens, frames = build_workload(args.config, args.frames)
-    # PCIe-inclusive figures (never `value`), measured before anything else runs in this process: an engine that has
-    # made some hundred passes and is then left idle slows the copies of the other engines in the process (2.5-2.6 ms per
-    # batch in the rotation below against 1.86 ms on the same box; not a graph, event or stream-count effect, and gone once
-    # that engine is destroyed), so these figures are taken with only their own engines alive.
+    # PCIe-inclusive figures (never `value`), measured before anything else runs in this process: with an engine alive
+    # that ran a few passes before the rotation's engines were made, the rotation below takes 2.5-2.6 ms per batch instead
+    # of 1.86 ms on the same box (not a graph, event or stream-count effect; engines made the other way round, or that
+    # engine destroyed first, and it is gone), so these figures are taken with only their own engines alive.
     # Serial: images in page-locked host memory -> stage + run + fetch of the whole classified mesh into one page-locked
     # block, one engine, the three steps one after the other. Pipelined: end_to_end() above.
     pcie, e2e = None, None
