@@ -219,6 +219,34 @@ def test_bf16_engine(oracle):
     assert worst > PROB_TOL  # two boundaries are stored as bf16: an error this small would mean they were not
 
 
+@pytest.mark.parametrize("hidden", [3, 10])
+def test_bf16_engine_on_other_depths(oracle, hidden):
+    """The plan for the rows between bf16 layers - at most two boundaries rounded to bf16, every second one, the others
+    hi + lo pairs - was tuned on configuration 5's six layers. What a rounding costs grows with the depth of the network
+    (a single one, anywhere, already 0.8-1.5e-2 with ten 64-wide layers), so networks with more than five bf16 layers get
+    no rounded boundary. A shallower (three 64-wide layers) and a deeper (ten) network on configuration 1's geometry must
+    stay inside the same 1e-2 gate."""
+    cfg = wl.config(1, n_frames=1)
+    rng = np.random.default_rng(500 + hidden)
+    net = wl.glorot_network(rng, [3] + [64] * hidden + [4], 6, wl.SELU)
+    o_lens, e_lens = lens_pair(cfg)
+    o_mesh, e_mesh = meshes_for(cfg, oracle)
+    engine = eng.Engine(net, cfg.model, precision=native.BF16)
+    f = cfg.frames[0]
+    got = engine(e_mesh, f["Hoc"], e_lens, f["image"], cfg.fourcc)
+    engine.stage([dict(mesh=e_mesh, Hoc=f["Hoc"], lens=e_lens, image=f["image"], fourcc=cfg.fourcc)])
+    engine.profile(True)
+    engine.run()
+    names = [n for n, _, _ in engine.profile_read() if n.startswith("conv")]
+    assert len(names) == hidden + 1 and all(n.startswith("conv_bf16_") for n in names[1:hidden]), names
+    rounded = sum("_tobf16_" in n for n in names)
+    assert rounded == (1 if hidden == 3 else 0), names
+    want = o_mesh.classify(f["Hoc"], o_lens, f["image"], cfg.fourcc, vmo.Network(net))
+    worst = float(np.abs(got["cls"] - want["cls"]).max())
+    print("bf16, %d hidden layers: %d boundaries as bf16, worst absolute probability error %.3e" % (hidden, rounded, worst), flush=True)
+    assert_classification_parity(got, want, BF16_TOL if rounded else 1e-3, "bf16, %d hidden layers" % hidden)
+
+
 @pytest.mark.parametrize("variant", ["halo8", "fp32_rows_in", "relu_tanh", "selu_last"])
 def test_bf16_layer_variants(oracle, variant, monkeypatch):
     """The bf16 layers' less travelled paths on configuration 1's geometry, each within 1e-2 of the fp32 oracle:

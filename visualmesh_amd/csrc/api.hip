@@ -857,8 +857,12 @@ int vmhip_engine_create(const vmhip_network* net, int32_t n_neighbours, int32_t 
      * bf16-sized error). One rounded boundary moves the final probabilities of a 6 x 64 network by up to ~4.6e-3,
      * n of them by about sqrt(n) times that (two: 7.2e-3, all five: 1.03e-2, measured on full-size frames), so to stay
      * inside the 1e-2 gate with margin every second boundary between bf16 layers is rounded and never more than two
-     * in a network, however deep. A bf16 layer behind a kernel that cannot write hi + lo rows reads fp32 rows and
-     * splits them in registers. */
+     * in a network. What one rounding costs grows with the depth of the network, wherever it sits (a single rounded
+     * boundary: 5-7e-3 with six 64-wide layers, 0.8-1.5e-2 with ten, 1.1-2.2e-2 with fourteen, on random networks), so
+     * a network with more than five bf16 layers gets none: all its boundaries are hi + lo pairs (1e-4 with ten layers,
+     * 1.6e-4 with fourteen). A bf16 layer behind a kernel that cannot write hi + lo rows reads fp32 rows and splits
+     * them in registers. VMHIP_BF16_ROUNDED=n (at most n rounded boundaries) and VMHIP_BF16_ROUNDED_AT=mask (bit l:
+     * the rows entering layer l) override the plan for measurements. */
     {
         /* VMHIP_CONV_KERNEL selects the kernel family for A/B runs: "rows" = one row per lane, "mfma" = matrix
          * cores gathering into registers, "lds" = matrix cores gathering from LDS (rows staged through registers),
@@ -878,13 +882,19 @@ int vmhip_engine_create(const vmhip_network* net, int32_t n_neighbours, int32_t 
             for (int l = 0; l < n; ++l)
                 ar[l] = (E->layers[l].slots - 1 <= VMHIP_NBL_STRIDE && vm_bf16_supported(E->layers[l].c_in, E->layers[l].c_out, E->layers[l].slots)) ? 1 : 0;
             int eligible = 0, rounded = 0;
+            int n_bf16 = 0;
+            for (int l = 0; l < n; ++l) n_bf16 += ar[l];
+            int max_rounded = n_bf16 <= 5 ? 2 : 0;
+            if (const char* r = getenv("VMHIP_BF16_ROUNDED")) max_rounded = std::max(atoi(r), 0);
             for (int l = 1; l < n; ++l) {
                 if (!ar[l]) continue;
                 ++eligible;
                 const HostLayer& P = E->layers[l - 1];
                 const bool splits = ar[l - 1] || (allow_lds && P.slots - 1 <= VMHIP_NBL_STRIDE && vm_lds_supported(P.c_in, P.c_out, P.slots, VM_ROWS_BF16X2));
                 if (!splits) continue; /* the layer before writes fp32 rows */
-                if (ar[l - 1] && eligible % 2 == 0 && rounded < 2) bf[l] = VM_ROWS_BF16, ++rounded;
+                bool round_here = ar[l - 1] && eligible % 2 == 0 && rounded < max_rounded;
+                if (const char* at = getenv("VMHIP_BF16_ROUNDED_AT")) round_here = ar[l - 1] && ((strtoul(at, nullptr, 0) >> l) & 1ul);
+                if (round_here) bf[l] = VM_ROWS_BF16, ++rounded;
                 else bf[l] = VM_ROWS_BF16X2;
             }
         }
