@@ -108,3 +108,30 @@ def test_engine_can_be_compiled_out():
     done = subprocess.run(["g++", "-std=c++14", "-fsyntax-only", "-DVISUALMESH_DISABLE_HIP", "-I" + os.path.join(ROOT, "visualmesh_amd", "cpp"), "-x", "c++", "-"],
                           input=src, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, universal_newlines=True)
     assert done.returncode == 0, done.stdout[-2000:]
+
+
+def test_bf16_kernels_with_weights_in_accumulation_registers_do_not_spill(tmp_path):
+    """conv_bf16.hip places the weights of most instantiations in accumulation registers (an "a" constraint); the ones that
+    spill to scratch memory gave wrong results that way and are excluded in the source (tanh, fp32 rows in). The excluded
+    set must cover every instantiation that spills: compile the file to assembly with the library's flags and check each
+    kernel's scratch segment against where its matrix instructions read the weights from."""
+    import subprocess
+    from visualmesh_amd import build as vm_build
+    out = tmp_path / "conv_bf16.s"
+    flags = [f for f in vm_build.HIP_FLAGS if f != "-fPIC"]
+    subprocess.run([vm_build.HIPCC] + flags + ["-S", "--cuda-device-only", "-o", str(out), os.path.join(vm_build.CSRC, "conv_bf16.hip")],
+                   check=True, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
+    text = out.read_text()
+    checked = 0
+    for m in re.finditer(r"\n(_ZN12_GLOBAL__N_119vm_conv_bf16_kernelILi7ELi(\d)ELi(\d)ELi(\d)EEEv\S+?):", text):
+        name, rows_in, activation = m.group(1), int(m.group(2)), int(m.group(4))
+        body = text[m.end():text.index(".Lfunc_end", m.end())]
+        from_agprs = sum(1 for line in body.splitlines() if line.strip().startswith("v_mfma") and line.split(",")[1].strip().startswith("a["))
+        total = sum(1 for line in body.splitlines() if line.strip().startswith("v_mfma"))
+        scratch = int(re.search(r"\.private_segment_fixed_size:\s+(\d+)", text[text.index(".name:           " + name):]).group(1))
+        expected_in_agprs = rows_in != 0 and activation != 3
+        assert (from_agprs > total // 2) == expected_in_agprs, (name, from_agprs, total)
+        if expected_in_agprs:
+            assert scratch == 0, name + " spills with its weights in accumulation registers"
+        checked += 1
+    assert checked == 36

@@ -232,13 +232,24 @@ __global__ __launch_bounds__(256) void vm_conv_bf16_kernel(VmBatchDev B, VmLayer
                 for (int p = 0; p < 2; ++p) w[s][j][p] = wp[((s * 4 + j) * 2 + p) * 64];
     }
     if (threadIdx.x < CH) b_lds[threadIdx.x] = L.b[threadIdx.x];
-    /* every load the compiler knows of returns before the first one it does not know of is issued */
+    /* Every load the compiler knows of returns before the first one it does not know of is issued. The same statements
+     * say where the weights live: in accumulation registers ("a"), from which the matrix instruction reads them as well
+     * as from vector registers. Left to itself the compiler keeps the 224 weight registers in the vector file and moves
+     * everything else in and out of accumulation registers around each use (822 such moves in the kernel against 176, a
+     * sixth of its instructions; 4-5 % of its time). Only the instantiations that fit the register file get this: the
+     * ones that spill to scratch memory (tanh, fp32 rows in) gave wrong results with it and keep the weights where the
+     * compiler puts them; tests/test_abi.py checks that no instantiation with weights in accumulation registers has a
+     * scratch segment. */
+    constexpr bool WEIGHTS_IN_AGPRS = IN_FMT != VM_ROWS_F32 && ACT != VMHIP_TANH;
 #pragma unroll
     for (int s = 0; s < SLOTS; ++s)
 #pragma unroll
         for (int j = 0; j < 4; ++j)
 #pragma unroll
-            for (int p = 0; p < 2; ++p) asm volatile("" : "+v"(w[s][j][p]));
+            for (int p = 0; p < 2; ++p) {
+                if constexpr (WEIGHTS_IN_AGPRS) asm volatile("" : "+a"(w[s][j][p]));
+                else asm volatile("" : "+v"(w[s][j][p]));
+            }
 
     const uint32_t total_rows = (uint32_t) B.n_row_tiles * VMHIP_TILE;
     const v4u note_rsrc = raw_rsrc(B.tile_note_h, (uint64_t) n_tiles * NOTE * 4);
