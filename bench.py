@@ -288,23 +288,18 @@ def end_to_end(cfg, mesh, lens, nodes, batches):
     from visualmesh_amd import native
     from visualmesh_amd import workloads as wl
     precision = native.BF16 if cfg.precision == "bf16" else native.FP32
-    engines = [eng.Engine(cfg.network, cfg.model, precision) for _ in range(3)]
+    pipe = eng.Pipeline(cfg.network, cfg.model, precision)  # visualmesh::engine::hip::Pipeline<float>
     held, frames = pinned_copies(cfg, mesh, lens)
 
     def rotate(n):
-        for step in range(n + 2):
-            if step < n:
-                e = engines[step % 3]
-                e.stage(frames, wait=False)  # the images are page-locked and stay as they are
-                e.run_async()
-            if 1 <= step <= n:
-                e = engines[(step - 1) % 3]
-                e.wait()
-                e.fetch_pinned(wait=False)  # one copy per array: these interleave with the next batch's upload (one 50 MB copy does not)
-            if step >= 2:
-                engines[(step - 2) % 3].fetch_wait()
+        returned = 0
+        for _ in range(n):
+            returned += pipe.submit(frames, arrays=False) is not None  # stage_async + run_async; wait + fetch of the batch before; results of the one before that
+        while pipe.flush(arrays=False) is not None:
+            returned += 1
+        assert returned == n
 
-    rotate(6)  # buffers allocated, graphs captured
+    rotate(6)  # buffers allocated
     t0 = time.perf_counter()
     rotate(batches)
     dt = (time.perf_counter() - t0) / batches

@@ -699,6 +699,51 @@ def test_results_into_page_locked_memory(oracle):
                 assert a[key].dtype == b[key].dtype and np.array_equal(a[key], b[key]), key
 
 
+def test_pipeline_of_three_engines(oracle):
+    """Pipeline<float>: batches of different sizes through submit() (one frame that sees nothing among them), the results
+    of batch k come back from the submit of batch k + 2 or from flush(), every one the oracle's; a single batch drains
+    with flush() alone."""
+    cfg = wl.config(2, n_frames=7)
+    o_lens, e_lens = lens_pair(cfg)
+    o_mesh, e_mesh = meshes_for(cfg, oracle)
+    net = vmo.Network(cfg.network)
+    images = []
+    for f in cfg.frames:
+        held = native.pinned_empty(f["image"].shape, f["image"].dtype)
+        held[...] = f["image"]
+        images.append(held)
+    frames = [dict(mesh=e_mesh, Hoc=f["Hoc"], lens=e_lens, image=im, fourcc=cfg.fourcc) for f, im in zip(cfg.frames, images)]
+    up = dict(mesh=e_mesh, Hoc=wl.make_hoc(1.0, math.radians(-85), 0.0, 0.0), lens=native.make_lens(1280, 1024, wl.RECTILINEAR, 700.0, 1.6),
+              image=images[0], fourcc=cfg.fourcc)
+    wants = [pick(o_mesh, f["Hoc"]).classify(f["Hoc"], o_lens, f["image"], cfg.fourcc, net) for f in cfg.frames]
+    batches = [[0, 1], [2], [3, "up", 4], [5, 6], [1]]
+    pipe = eng.Pipeline(cfg.network, cfg.model)
+    got = []
+    for b in batches:
+        done = pipe.submit([up if i == "up" else frames[i] for i in b])
+        if done is not None:
+            got.append([{k: v.copy() for k, v in r.items()} for r in done])
+    assert len(got) == len(batches) - 2
+    while True:
+        done = pipe.flush()
+        if done is None:
+            break
+        got.append([{k: v.copy() for k, v in r.items()} for r in done])
+    assert len(got) == len(batches)
+    for b, results in zip(batches, got):
+        assert len(results) == len(b)
+        for i, r in zip(b, results):
+            if i == "up":
+                assert len(r["gidx"]) == 0
+            else:
+                assert_classification_parity(r, wants[i], PROB_TOL, "pipeline frame %d" % i)
+    single = eng.Pipeline(cfg.network, cfg.model)
+    assert single.submit([frames[0]]) is None
+    done = single.flush()
+    assert done is not None and single.flush() is None
+    assert_classification_parity(done[0], wants[0], PROB_TOL, "pipeline of one batch")
+
+
 def test_packed_fetch_of_mixed_frames(oracle):
     """vmhip_batch_fetch_packed_async on a batch whose frames differ in mesh model (6 and 8 neighbours, so the device's
     neighbourhood rows are strided for the 6-neighbour frames), with a frame that sees nothing in the middle, and after a

@@ -435,5 +435,57 @@ int vmh_lens_load(const char* path, int width, int height, vmh_lens_t* lens, rea
         return 0;
     })
 }
+
+/* ---- Pipeline<float>: three engines in rotation ---- */
+struct vmh_pipeline {
+    int model;
+    std::unique_ptr<engine::hip::Pipeline<real>> pipe;
+    const std::vector<vmhip_result>* done = nullptr;
+};
+int vmh_pipeline_create(const vmh_network_t* net, int model, int precision, vmh_pipeline** out) {
+    GUARD({
+        std::unique_ptr<vmh_pipeline> p(new vmh_pipeline());
+        p->model = model;
+        p->pipe.reset(new engine::hip::Pipeline<real>(to_network(net), engine::hip::Precision(precision)));
+        *out = p.release();
+        return 0;
+    })
+}
+void vmh_pipeline_destroy(vmh_pipeline* p) { delete p; }
+/* queues a batch (n = 0: drains instead); returns the number of frames of the batch whose results are ready (read them with
+ * vmh_pipeline_result before the next call but one), 0 if none is, or a negative status */
+int vmh_pipeline_submit(vmh_pipeline* p, int n, const vmh_mesh* const* meshes, const real* Hoc16s, const vmh_lens_t* lenses,
+                        const void* const* images, const uint32_t* fourccs) {
+    GUARD({
+        if (n == 0) p->done = p->pipe->flush();
+        else if (p->model == VMH_RING6) {
+            std::vector<HipEngine::Frame<Ring6>> frames(n);
+            for (int i = 0; i < n; ++i) {
+                if (!meshes[i]->r6) throw std::invalid_argument("mesh model does not match the pipeline");
+                frames[i] = HipEngine::Frame<Ring6>{meshes[i]->r6, to_hoc(Hoc16s + 16 * i), to_lens(lenses + i), images[i], fourccs[i]};
+            }
+            p->done = p->pipe->submit<Ring6>(frames);
+        }
+        else {
+            std::vector<HipEngine::Frame<NMGrid8>> frames(n);
+            for (int i = 0; i < n; ++i) {
+                if (!meshes[i]->g8) throw std::invalid_argument("mesh model does not match the pipeline");
+                frames[i] = HipEngine::Frame<NMGrid8>{meshes[i]->g8, to_hoc(Hoc16s + 16 * i), to_lens(lenses + i), images[i], fourccs[i]};
+            }
+            p->done = p->pipe->submit<NMGrid8>(frames);
+        }
+        return p->done ? int(p->done->size()) : 0;
+    })
+}
+/* frame i of the ready batch: its visible count and the arrays (inside the pipeline's page-locked memory) */
+int vmh_pipeline_result(vmh_pipeline* p, int i, real** px, int32_t** gidx, int32_t** nb, real** cls) {
+    GUARD({
+        if (!p->done) throw std::invalid_argument("pipeline_result: no batch is ready");
+        const vmhip_result& r = p->done->at(size_t(i));
+        *px = r.pixel_coordinates, *gidx = r.global_indices, *nb = r.neighbourhood, *cls = r.classifications;
+        return r.capacity;
+    })
+}
+int vmh_pipeline_n_classes(vmh_pipeline* p) { return p->pipe->engine(0).n_classes(); }
 #endif  // !VMH_DOUBLE
 }

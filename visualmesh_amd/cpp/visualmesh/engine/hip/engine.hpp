@@ -42,6 +42,7 @@
 #include <thread>
 #include <cstring>
 #include <map>
+#include <memory>
 #include <stdexcept>
 #include <string>
 #include <system_error>
@@ -462,6 +463,8 @@ namespace engine {
             bool device_lookup() const { return device_lookup_; }
             /// The batch object behind stage/run/fetch, for profiling hooks.
             vmhip_batch* native_batch() const { return batch_; }
+            /// Width of the classification rows (known once the engine has been used; -1 before).
+            int n_classes() const { return engine_ ? int(vmhip_engine_n_classes(engine_)) : -1; }
 
             /// Forget the device copies of all meshes (same purpose as the reference OpenCL engine's
             /// clear_cache, engine/opencl/engine.hpp:559-572). Not needed for correctness: a cached copy is only
@@ -894,6 +897,121 @@ namespace engine {
             mutable vmhip_engine_f64* engine_ = nullptr;
             mutable int engine_nn_ = -1;
             mutable std::map<const void*, MeshEntry> meshes_;
+        };
+
+        /**
+         * Three engines taking turns, so that the upload of one batch, the kernels of the one before and the download of
+         * the one before that run at the same time: what a caller otherwise writes by hand with stage_async / run_async /
+         * wait / fetch_into_async / fetch_wait on three Engine objects. No counterpart in the reference, whose benchmark
+         * runs one frame at a time per engine (example/benchmark.cpp:50-58).
+         *
+         *     Pipeline<float> pipe(network);
+         *     for (;;) { if (auto* done = pipe.submit(next_frames())) consume(*done); }   // results of the batch two submits ago
+         *     while (auto* done = pipe.flush()) consume(*done);
+         *
+         * The frames' images must lie in page-locked memory (vmhip_host_alloc; a batch's images in one allocation go up as one
+         * copy) and stay untouched until the next submit() or flush() has returned. The results returned point into page-locked
+         * memory of the pipeline and stay valid until two more calls of submit() or flush().
+         */
+        template <typename Scalar>
+        class Pipeline {
+            static_assert(std::is_same<Scalar, float>::value, "the pipeline drives Engine<float>");
+
+        public:
+            explicit Pipeline(const NetworkStructure<Scalar>& structure = {}, Precision precision = Precision::FP32) {
+                for (Slot& s : slots_) s.engine.reset(new Engine<Scalar>(structure, precision));
+            }
+            ~Pipeline() {
+                for (Slot& s : slots_) {
+                    try {
+                        if (s.running) s.engine->wait();
+                        if (s.fetching) s.engine->fetch_wait();
+                    } catch (...) {
+                    }
+                    if (s.block) vmhip_host_free(s.block);
+                }
+            }
+            Pipeline(const Pipeline&) = delete;
+            Pipeline& operator=(const Pipeline&) = delete;
+
+            /// Queue a batch; returns the results of the batch submitted two calls earlier (one entry per frame of that batch:
+            /// n_visible and pointers as in vmhip_result), or nullptr while the pipeline fills.
+            template <template <typename> class Model>
+            const std::vector<vmhip_result>* submit(const std::vector<typename Engine<Scalar>::template Frame<Model>>& frames) {
+                Slot& now = slots_[step_ % 3];
+                now.engine->stage_async(frames);
+                now.engine->run_async();
+                now.running = true;
+                now.neighbours = Model<Scalar>::N_NEIGHBOURS;
+                return advance();
+            }
+            /// Drain: the results of the batches still in flight, oldest first, then nullptr.
+            const std::vector<vmhip_result>* flush() {
+                for (int turn = 0; turn < 2; ++turn) {
+                    bool in_flight = false;
+                    for (const Slot& s : slots_) in_flight = in_flight || s.running || s.fetching;
+                    if (!in_flight) return nullptr;
+                    if (const std::vector<vmhip_result>* done = advance()) return done;
+                }
+                return nullptr;
+            }
+            /// The engines, e.g. to set a cache limit or the lookup on the device on all three.
+            Engine<Scalar>& engine(int i) { return *slots_[i % 3].engine; }
+
+        private:
+            struct Slot {
+                std::unique_ptr<Engine<Scalar>> engine;
+                bool running = false, fetching = false;
+                int neighbours = 0;
+                void* block = nullptr;
+                size_t block_bytes = 0;
+                std::vector<vmhip_result> results;
+            };
+            static size_t pad(size_t n) { return (n + 255) / 256 * 256; }
+
+            const std::vector<vmhip_result>* advance() {
+                Slot& previous = slots_[(step_ + 2) % 3];  // submitted one call ago: its kernels finish, its download starts
+                Slot& oldest = slots_[(step_ + 1) % 3];    // submitted two calls ago: its download finishes
+                ++step_;
+                if (previous.running) {
+                    previous.engine->wait();
+                    previous.running = false;
+                    const std::vector<int32_t> visible = previous.engine->visible_counts();
+                    const size_t classes = size_t(previous.engine->n_classes()), nn = size_t(previous.neighbours);
+                    size_t need = 0;
+                    for (int32_t v : visible)
+                        if (v > 0) need += pad(8 * size_t(v)) + pad(4 * size_t(v)) + pad(4 * (size_t(v) + 1) * nn) + pad(4 * (size_t(v) + 1) * classes);
+                    if (need > previous.block_bytes) {
+                        if (previous.block) vmhip_host_free(previous.block);
+                        previous.block = vmhip_host_alloc(need + need / 8);
+                        previous.block_bytes = previous.block ? need + need / 8 : 0;
+                        if (!previous.block) throw std::system_error(VMHIP_ERR_HIP, hip_error_category(), "Pipeline: no page-locked memory for the results");
+                    }
+                    previous.results.assign(visible.size(), vmhip_result{});
+                    char* at = static_cast<char*>(previous.block);
+                    for (size_t i = 0; i < visible.size(); ++i) {
+                        const size_t v = size_t(visible[i]);
+                        vmhip_result& r = previous.results[i];
+                        r.capacity = int32_t(v);
+                        if (v == 0) continue;
+                        r.pixel_coordinates = reinterpret_cast<float*>(at), at += pad(8 * v);
+                        r.global_indices = reinterpret_cast<int32_t*>(at), at += pad(4 * v);
+                        r.neighbourhood = reinterpret_cast<int32_t*>(at), at += pad(4 * (v + 1) * nn);
+                        r.classifications = reinterpret_cast<float*>(at), at += pad(4 * (v + 1) * classes);
+                    }
+                    previous.engine->fetch_into_async(previous.results);
+                    previous.fetching = true;
+                }
+                if (oldest.fetching) {
+                    oldest.engine->fetch_wait();
+                    oldest.fetching = false;
+                    return &oldest.results;
+                }
+                return nullptr;
+            }
+
+            std::array<Slot, 3> slots_;
+            size_t step_ = 0;
         };
 
     }  // namespace hip

@@ -346,6 +346,68 @@ class Engine:
         return native.profile_read(self.native_batch())
 
 
+class Pipeline:
+    """visualmesh::engine::hip::Pipeline<float>: three engines in rotation behind one submit() call. submit(frames) queues a
+    batch (images in page-locked memory, untouched until the next call returns) and returns the results of the batch
+    submitted two calls earlier, or None while the pipeline fills; flush() drains (None when empty). The arrays returned
+    are views into the pipeline's page-locked memory, valid until two more calls."""
+
+    def __init__(self, network_groups, model, precision=native.FP32):
+        self._lib = native.host()
+        self.network = network_groups if isinstance(network_groups, Network) else Network(network_groups)
+        self.model = model
+        p = C.c_void_p()
+        native.host_check(self._lib.vmh_pipeline_create(C.byref(self.network.c), model, precision, C.byref(p)))
+        self.ptr = p
+        self._neighbours = []   # per batch in flight: the frames' neighbour counts
+        self._keep = []         # per batch in flight: what the asynchronous stage still reads
+
+    def __del__(self):
+        if getattr(self, "ptr", None):
+            self._lib.vmh_pipeline_destroy(self.ptr)
+            self.ptr = None
+
+    def _results(self, n_done, arrays=True):
+        if n_done == 0:
+            return None
+        nns = self._neighbours.pop(0)
+        self._keep.pop(0)
+        if not arrays:
+            return n_done
+        n_out = self.network.n_out
+        out = []
+        for i in range(n_done):
+            px, gidx, nb, cls = C.POINTER(C.c_float)(), C.POINTER(C.c_int32)(), C.POINTER(C.c_int32)(), C.POINTER(C.c_float)()
+            V = native.host_check(self._lib.vmh_pipeline_result(self.ptr, i, C.byref(px), C.byref(gidx), C.byref(nb), C.byref(cls)))
+            nn = nns[i]
+            if V == 0:
+                out.append(dict(px=np.zeros((0, 2), np.float32), nb=np.zeros((0, nn), np.int32), gidx=np.zeros(0, np.int32), cls=np.zeros((0, n_out), np.float32)))
+                continue
+            out.append(dict(px=np.ctypeslib.as_array(px, (V, 2)), gidx=np.ctypeslib.as_array(gidx, (V,)),
+                            nb=np.ctypeslib.as_array(nb, (V + 1, nn)), cls=np.ctypeslib.as_array(cls, (V + 1, n_out))))
+        return out
+
+    def submit(self, frames, arrays=True):
+        """arrays=False: the number of frames of the finished batch instead of numpy views of its results (a caller that
+        only counts, like a benchmark loop, saves the time numpy takes to wrap 4 arrays per frame)"""
+        n = len(frames)
+        meshes = [f["mesh"].height(float(f["Hoc"][2][3])) for f in frames]
+        mesh_ptrs = (C.c_void_p * n)(*[m.ptr for m in meshes])
+        H = np.ascontiguousarray(np.stack([np.asarray(f["Hoc"], dtype=np.float32) for f in frames]))
+        lenses = (Lens * n)(*[f["lens"] for f in frames])
+        images = [np.ascontiguousarray(f["image"]) for f in frames]
+        image_ptrs = (C.c_void_p * n)(*[im.ctypes.data for im in images])
+        fccs = (C.c_uint32 * n)(*[f["fourcc"] for f in frames])
+        self._neighbours.append([m.n_neighbours for m in meshes])
+        self._keep.append(images)
+        return self._results(native.host_check(self._lib.vmh_pipeline_submit(self.ptr, n, mesh_ptrs, _fp(H), lenses, image_ptrs, fccs)), arrays)
+
+    def flush(self, arrays=True):
+        if not self._neighbours:
+            return None
+        return self._results(native.host_check(self._lib.vmh_pipeline_submit(self.ptr, 0, None, None, None, None, None)), arrays)
+
+
 def load_model(path):
     """An exported model file through the C++ reader (visualmesh::load_model_file): dict(mesh, shape, radius,
     intersections, network) with network = list of groups of (weights[n_in, n_out], biases[n_out], activation)."""

@@ -341,6 +341,13 @@ def host():
     L.vmh_model_layer.argtypes = [vp, C.c_int, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_int),
                                   C.POINTER(C.c_float), C.POINTER(C.c_float)]
     L.vmh_lens_load.argtypes = [C.c_char_p, C.c_int, C.c_int, C.POINTER(Lens), C.POINTER(C.c_float)]
+    fpp, ipp = C.POINTER(C.POINTER(C.c_float)), C.POINTER(C.POINTER(C.c_int32))
+    L.vmh_pipeline_create.argtypes = [C.POINTER(NetworkC), C.c_int, C.c_int, C.POINTER(vp)]
+    L.vmh_pipeline_destroy.argtypes = [vp]
+    L.vmh_pipeline_destroy.restype = None
+    L.vmh_pipeline_submit.argtypes = [vp, C.c_int, C.POINTER(vp), C.POINTER(C.c_float), C.POINTER(Lens), C.POINTER(vp), C.POINTER(C.c_uint32)]
+    L.vmh_pipeline_result.argtypes = [vp, C.c_int, fpp, ipp, ipp, fpp]
+    L.vmh_pipeline_n_classes.argtypes = [vp]
     _host = L
     return L
 
