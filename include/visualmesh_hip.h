@@ -232,7 +232,7 @@ int vmhip_batch_fetch_packed_async(vmhip_batch* batch, void* block, size_t bytes
  *                 the mesh or not summing to n_candidates (then nothing else is written)
  *   pixel_coordinates [capacity][2], global_indices [capacity], neighbourhood [capacity+1][n_neighbours]
  *                 as in vmhip_result; all four are required. With visible nodes the null row follows them.
- * The workspace is one array of fixed size inside the library (15.5 MB per device, held until the process ends), so
+ * The workspace is one array of fixed size inside the library (11.3 MB per device, held until the process ends), so
  * sizes are limited as below and VMHIP_ERR_CAPACITY says which limit a call exceeds; calls that overlap on one
  * device race on that array, calls on one stream do not. The on-screen decisions are the device's own: they equal the
  * host's bit for bit where the host's C library is the one the device arithmetic reproduces (glibc's), and the
@@ -298,8 +298,10 @@ int vmhip_batch_profile_read(vmhip_batch* batch, int32_t max_slots, int32_t* n_s
  *                                 device's lens arithmetic differed from the host's: the host's re-decision of near-edge
  *                                 nodes must then overrule the device (read when a batch is staged; 0 = off)
  *   VMHIP_DEBUG_EDGE_BAND         width in pixels of the band along the screen edges inside which nodes are re-decided
- *                                 on the host (read when a batch is staged; <= 0 restores the default, 1/64) */
-enum { VMHIP_DEBUG_FLOW_POLL_LIMIT = 0, VMHIP_DEBUG_PROJECTION_ERROR = 1, VMHIP_DEBUG_EDGE_BAND = 2 };
+ *                                 on the host (read when a batch is staged; <= 0 restores the default, 1/64)
+ *   VMHIP_DEBUG_WIDE_OFFSETS      non-zero: the neighbourhood kernel addresses its tables with 64-bit offsets, as it does by
+ *                                 itself for a batch with a table of 4 GiB or more (read when a batch is staged; 0 = off) */
+enum { VMHIP_DEBUG_FLOW_POLL_LIMIT = 0, VMHIP_DEBUG_PROJECTION_ERROR = 1, VMHIP_DEBUG_EDGE_BAND = 2, VMHIP_DEBUG_WIDE_OFFSETS = 3 };
 int vmhip_debug_set(int32_t what, double value);
 /* What the edge guard did in the runs of a batch since it was staged: near-edge nodes the device listed (summed over
  * frames and passes), the most it listed for one frame in one pass, device decisions the host overruled, passes

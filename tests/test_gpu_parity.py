@@ -64,7 +64,8 @@ def test_config3_bayer(oracle):
 
 def test_device_libm_matches_host(oracle):
     """The device's acosf/sinf/tanf/sqrtf must return the host C library's bits (a dense sample here; the
-    same source is compared exhaustively on the CPU in test_libm_exact.py)."""
+    same source is compared exhaustively on the CPU in test_libm_exact.py). The square root is the compiler's
+    sequence on the device and not the header's own arithmetic, so it is compared exhaustively here."""
     import ctypes as C
     from visualmesh_amd import native
     L = native.hip()
@@ -76,15 +77,101 @@ def test_device_libm_matches_host(oracle):
         "sin": (1, np.concatenate([rng.uniform(0, np.pi / 2, n).astype(np.float32), np.geomspace(1e-7, 1.6, 4096).astype(np.float32)])),
         "tan": (2, np.concatenate([rng.uniform(0, np.pi / 2, n).astype(np.float32), (np.float32(np.pi / 2) - np.geomspace(1e-7, 1, 4096)).astype(np.float32),
                                    np.array([np.float32(np.pi / 2)], np.float32)])),
-        "sqrt": (3, rng.uniform(0, 4, n).astype(np.float32)),
     }
-    for name, (which, x) in cases.items():
+
+    def all_cases():
+        for name, (which, x) in cases.items():
+            yield name, which, x
+        # the square root over every float from zero to four, denormals included (the projection takes roots of values in [0, 1])
+        step = 1 << 26
+        for first in range(0, 0x40800000 + 1, step):
+            yield "sqrt from bit pattern %#x" % first, 3, np.arange(first, min(first + step, 0x40800000 + 1), dtype=np.uint32).view(np.float32)
+
+    for name, which, x in all_cases():
         x = np.ascontiguousarray(x)
         y = np.zeros_like(x)
         native.hip_check(L.vmhip_selftest_libm(which, x.ctypes.data_as(C.POINTER(C.c_float)), y.ctypes.data_as(C.POINTER(C.c_float)), x.size))
-        want = oracle.fn_libm(name, x)
+        want = oracle.fn_libm(name.split()[0], x)
         bad = np.flatnonzero(y.view(np.uint32) != want.view(np.uint32))
         assert bad.size == 0, "%s: %d of %d differ, e.g. x=%r device=%r host=%r" % (name, bad.size, x.size, x[bad[0]], y[bad[0]], want[bad[0]])
+
+
+def test_reverse_lookup_across_a_restart_of_the_run_stamp(oracle):
+    """A reverse-lookup entry holds an 8-bit run stamp above the row, and an engine's table is cleared when the stamps
+    start again after 255 runs. One view stamps its nodes, then another view runs 600 times on the same engine: no run
+    may take an entry of the first view (or of itself, 255 runs earlier) for current."""
+    mesh = eng.Mesh(wl.RING6, wl.SPHERE, 0.0949, 1.0, 3.0, 8.0)
+    lens = native.make_lens(320, 256, wl.RECTILINEAR, 180.0, math.pi / 2)
+    first_view = wl.make_hoc(1.0, math.radians(50.0), math.radians(-4.0), math.radians(1.0))
+    views = [wl.make_hoc(1.0, math.radians(55.0), math.radians(3.0), math.radians(40.0)),
+             wl.make_hoc(1.0, math.radians(42.0), math.radians(-2.0), math.radians(65.0))]
+    engine = eng.Engine([], wl.RING6)
+    a = engine.project(mesh, first_view, lens)
+    assert len(a["gidx"]) > 100
+    o_mesh = oracle.mesh(wl.RING6, wl.SPHERE, 0.0949, 1.0, 3.0, 8.0)
+    o_lens = vmo.make_lens(320, 256, wl.RECTILINEAR, 180.0, math.pi / 2)
+    want = []
+    for Hoc in views:
+        o = o_mesh.project(Hoc, o_lens)
+        assert 100 < len(o["gidx"]) and not set(o["gidx"]) >= set(a["gidx"])  # the first view has nodes of its own
+        want.append(o)
+    for run in range(600):
+        got = engine.project(mesh, views[run & 1], lens)
+        assert np.array_equal(got["gidx"], want[run & 1]["gidx"]), "run %d: visible nodes differ" % run
+        assert np.array_equal(got["nb"], want[run & 1]["nb"]), "run %d: neighbourhood differs" % run
+
+
+def test_neighbourhood_of_meshes_with_other_neighbour_counts(oracle):
+    """The neighbourhood kernel has instantiations for 4, 6 and 8 neighbours per node and a general one. Meshes with 5
+    and with 12 columns of neighbours (the nodes of a real mesh, so that the lookup is a real one; the columns random,
+    "no neighbour" included) go through vmhip_project, and the table must be what engine/cpu/engine.hpp:127-143 defines:
+    the row of every neighbour that is on screen, the null row for the others."""
+    import ctypes as C
+    L = native.hip()
+    rng = np.random.default_rng(12)
+    mesh = eng.Mesh(wl.RING6, wl.SPHERE, 0.0949, 1.0, 3.0, 8.0)
+    rays, _ = mesh.arrays()
+    lens = native.make_lens(320, 256, wl.EQUISOLID, 105.0, math.pi)
+    Hoc = np.ascontiguousarray(wl.make_hoc(1.0, math.radians(40.0), 0.02, 0.3), dtype=np.float32)
+    ranges = np.ascontiguousarray(mesh.lookup(Hoc, lens), dtype=np.int32)
+    n_cand = int((ranges[:, 1] - ranges[:, 0]).sum())
+    Rco = np.ascontiguousarray(Hoc[:3, :3].T)
+    empty = native.Network([])
+    for nn in (5, 12, 4):
+        nbr = np.ascontiguousarray(rng.integers(0, mesh.n_nodes + 1, (mesh.n_nodes, nn)), dtype=np.int32)
+        engine, handle = C.c_void_p(), C.c_void_p()
+        native.hip_check(L.vmhip_engine_create(C.byref(empty.c), nn, native.FP32, C.byref(engine)))
+        native.hip_check(L.vmhip_mesh_upload(rays.ctypes.data_as(C.POINTER(C.c_float)), nbr.ctypes.data_as(C.POINTER(C.c_int32)), mesh.n_nodes, nn, C.byref(handle)))
+        px = np.zeros((n_cand, 2), np.float32)
+        gidx = np.zeros(n_cand, np.int32)
+        nb = np.full((n_cand + 1, nn), -1, np.int32)
+        frame = native.Frame(handle, (C.c_float * 9)(*Rco.ravel()), lens, ranges.ctypes.data_as(C.POINTER(C.c_int32)), len(ranges), None, 0, None)
+        result = native.Result(n_cand, 0, px.ctypes.data_as(C.POINTER(C.c_float)), gidx.ctypes.data_as(C.POINTER(C.c_int32)),
+                               nb.ctypes.data_as(C.POINTER(C.c_int32)), None)
+        for _ in range(2):  # the second run finds the first run's stamps in the table
+            native.hip_check(L.vmhip_project(engine, C.byref(frame), C.byref(result)))
+        V = result.n_visible
+        assert V > 500
+        row_of = np.full(mesh.n_nodes + 1, V, np.int32)
+        row_of[gidx[:V]] = np.arange(V, dtype=np.int32)
+        want = np.concatenate([row_of[nbr[gidx[:V]]], np.full((1, nn), V, np.int32)])
+        assert np.array_equal(nb[:V + 1], want), "%d neighbours per node" % nn
+        L.vmhip_mesh_release(handle)
+        L.vmhip_engine_destroy(engine)
+
+
+def test_neighbourhood_kernel_with_64_bit_offsets(oracle):
+    """A batch with a table of 4 GiB or more takes the instantiations of the neighbourhood kernel that address with
+    64-bit offsets; the knob forces them onto ordinary frames: projection only (no tile-local tables), a network with
+    six neighbours per node, and a batch whose frames differ in their neighbour count (the general instantiation)."""
+    lib = native.hip()
+    native.hip_check(lib.vmhip_debug_set(native.DEBUG_WIDE_OFFSETS, 1))
+    try:
+        test_config1_projection_only(oracle)
+        _run_config(oracle, 1, 1, batch=False)
+        test_neighbourhood_of_meshes_with_other_neighbour_counts(oracle)
+    finally:
+        native.hip_check(lib.vmhip_debug_set(native.DEBUG_WIDE_OFFSETS, 0))
 
 
 def test_pixels_and_inputs_bit_exact(oracle):
@@ -745,9 +832,8 @@ def test_pipeline_of_three_engines(oracle):
 
 
 def test_packed_fetch_of_mixed_frames(oracle):
-    """vmhip_batch_fetch_packed_async on a batch whose frames differ in mesh model (6 and 8 neighbours, so the device's
-    neighbourhood rows are strided for the 6-neighbour frames), with a frame that sees nothing in the middle, and after a
-    projection-only run (no classifications)."""
+    """vmhip_batch_fetch_packed_async on a batch whose frames differ in lens and view, with a frame that sees nothing in
+    the middle, and after a projection-only run (no classifications)."""
     rng = np.random.default_rng(4)
     lens = native.make_lens(320, 256, wl.EQUISOLID, 105.0, math.pi)
     m6 = eng.Mesh(wl.RING6, wl.SPHERE, 0.0949, 1.0, 3.0, 8.0)

@@ -106,6 +106,12 @@ def test_projection_without_allocation_matches_vmhip_project():
     want, got, _ = _both_ways(L, engine, handles[0], big, Hoc_big, lens_big)
     _assert_same(want, got, "third call")
 
+    # The reverse lookup carries an 8-bit run stamp: after 255 calls the count starts again and the table is cleared on the
+    # device. The big mesh's entries, stamped by the call above, must not look current again to any later call.
+    for call in range(300):
+        want, got, (ranges, n_cand) = _both_ways(L, engine, handles[1], small, Hoc_small, lens_small)
+        _assert_same(want, got, "call %d on the smaller input" % call)
+
     # a range table that does not sum to the stated candidate count is rejected on the device, nothing else is written
     d_ranges = native.pinned_empty(ranges.shape, np.int32)
     d_ranges[...] = ranges

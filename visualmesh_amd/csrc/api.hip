@@ -20,6 +20,7 @@ thread_local std::string g_error;
 
 /* test knobs (vmhip_debug_set); read when a batch is staged */
 std::atomic<float> g_debug_px_error{0.0f};
+std::atomic<bool> g_debug_wide_offsets{false};
 std::atomic<float> g_debug_edge_band{VMHIP_AMB_EPS_DEFAULT};
 
 int fail(int code, const std::string& msg) {
@@ -155,6 +156,7 @@ struct vmhip_batch {
     int32_t detect_class = -1, detect_arg_max = 0, detect_clusters = 0;
     float detect_threshold = 0.0f;
     uint32_t epoch = 0; /* host mirror of the device run stamp */
+    int stamp_row_bits = 0; /* how the reverse-lookup entries of the table on the device are split (VmBatchDev::stamp_row_bits) */
     /* what the edge guard did since the batch was staged (vmhip_batch_guard_stats) */
     int64_t reruns = 0, overruled = 0, amb_seen = 0, amb_most = 0;
     /* the kernel sequence of a run, captured once per staged batch and replayed (no profiling, VMHIP_GRAPH != 0) */
@@ -218,8 +220,9 @@ int batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int
     b->frames.assign(n_frames, HostFrame());
 
     /* validate and place */
-    size_t cand_tiles = 0, row_tiles = 0, range_ints = 0, image_bytes = 0, lookup_entries = 0;
-    int32_t nb_stride = 1;
+    size_t cand_tiles = 0, row_tiles = 0, range_ints = 0, image_bytes = 0, lookup_entries = 0, max_cand = 0;
+    uint64_t widest_mesh = 0; /* most neighbour table entries of a frame's mesh */
+    int32_t nb_stride = 1, uniform_nn = 0;
     for (int f = 0; f < n_frames; ++f) {
         const vmhip_frame& in = frames[f];
         HostFrame& hf = b->frames[f];
@@ -280,7 +283,10 @@ int batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int
         range_ints += size_t(in.n_ranges) * 2 + 1;
         if (classify) image_bytes += align_up(size_t(in.lens.width) * in.lens.height * bpp, 256);
         lookup_entries += size_t(in.mesh->n_nodes) + 1;
+        max_cand = std::max(max_cand, size_t(total));
+        widest_mesh = std::max(widest_mesh, uint64_t(in.mesh->n_nodes) * uint64_t(in.mesh->nn));
         nb_stride = std::max(nb_stride, in.mesh->nn);
+        uniform_nn = (f == 0 || uniform_nn == in.mesh->nn) ? in.mesh->nn : 0;
     }
     b->cand_total = cand_tiles * VMHIP_TILE;
     b->row_total = row_tiles * VMHIP_TILE;
@@ -327,16 +333,24 @@ int batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int
         HIP_TRY(b->d_tile_note_h.reserve(4 * 2 * row_tiles * VMHIP_NOTE_WORDS));
         HIP_TRY(b->d_active_h.reserve(4 * (size_t(n_frames) + 1)));
     }
-    HIP_TRY(b->d_lookup.reserve(sizeof(uint2) * lookup_entries));
-    if (b->d_lookup.grew) {
-        /* a fresh reverse-lookup table holds no valid stamp; epochs start above zero */
-        HIP_TRY(hipMemsetAsync(b->d_lookup.p, 0, b->d_lookup.cap, E->stream));
-    }
+    HIP_TRY(b->d_lookup.reserve(sizeof(uint32_t) * lookup_entries));
     b->lookup_total = lookup_entries;
     if (!b->d_epoch.p) {
         HIP_TRY(b->d_epoch.reserve(256));
         HIP_TRY(hipMemsetAsync(b->d_epoch.p, 0, 256, E->stream));
         b->epoch = 0;
+    }
+    /* a reverse-lookup entry: the run's stamp above the node's row. 24 bits of row serve every frame below 2^24
+     * candidates and leave 255 runs between two clears of the table; a larger frame takes the bits it needs from the stamp */
+    int row_bits = 24;
+    while (row_bits < 31 && (max_cand >> row_bits) != 0) ++row_bits;
+    if (b->d_lookup.grew || row_bits != b->stamp_row_bits) {
+        /* a fresh table, or one whose entries were split differently, holds no valid stamp: zero everywhere, and the
+         * runs count from one again */
+        HIP_TRY(hipMemsetAsync(b->d_lookup.p, 0, b->d_lookup.cap, E->stream));
+        HIP_TRY(hipMemsetAsync(b->d_epoch.p, 0, 4, E->stream));
+        b->epoch = 0;
+        b->stamp_row_bits = row_bits;
     }
     b->drop_graph(); /* pointers and sizes baked into a captured run are no longer valid */
 
@@ -383,7 +397,7 @@ int batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int
             }
             image_off += align_up(bytes, 256);
         }
-        d.r_lookup = b->d_lookup.as<uint2>() + lookup_off;
+        d.r_lookup = b->d_lookup.as<uint32_t>() + lookup_off;
         lookup_off += size_t(d.n_nodes) + 1;
         d.force_valid = b->d_force_valid.as<uint64_t>();
         d.force_keep = b->d_force_keep.as<uint64_t>();
@@ -426,6 +440,11 @@ int batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int
     D.row_nbl_h = half_tables ? b->d_row_nbl_h.as<uint16_t>() : nullptr;
     D.tile_note_h = half_tables ? b->d_tile_note_h.as<uint32_t>() : nullptr;
     D.epoch = b->d_epoch.as<uint32_t>();
+    D.stamp_row_bits = b->stamp_row_bits;
+    D.uniform_nn = uniform_nn;
+    /* 32-bit byte offsets into a frame's part of every table the neighbourhood kernel touches (4-byte entries of the
+     * mesh's neighbour table and of the output table, 16-byte rows of the tile-local table), unless one is too large */
+    D.wide_offsets = (widest_mesh >= (1ull << 30) || (uint64_t(max_cand) + 1) * uint64_t(std::max(nb_stride, 4)) >= (1ull << 30) || g_debug_wide_offsets.load()) ? 1 : 0;
     D.flow_timeouts = b->d_epoch.as<unsigned int>() + 16; /* same zeroed block, a cache line of its own */
     D.amb_eps = g_debug_edge_band.load();
     D.px_error = g_debug_px_error.load();
@@ -608,7 +627,7 @@ int batch_verify(vmhip_batch* b) {
 /* puts one pass over the staged frames, and the download of its verdict, on the engine's stream */
 int batch_launch(vmhip_batch* b) {
     vmhip_engine* E = b->engine;
-    if (b->epoch == 0xffffffffu) { /* the device stamp is about to wrap: old stamps could look current again */
+    if (b->epoch >= (0xffffffffu >> b->stamp_row_bits)) { /* the stamp has used all its bits: old stamps could look current again */
         HIP_TRY(hipMemsetAsync(b->d_lookup.p, 0, b->d_lookup.cap, E->stream));
         HIP_TRY(hipMemsetAsync(b->d_epoch.p, 0, 4, E->stream));
         b->epoch = 0;
@@ -1400,6 +1419,7 @@ int vmhip_debug_set(int32_t what, double value) {
             return VMHIP_OK;
         }
         case VMHIP_DEBUG_PROJECTION_ERROR: g_debug_px_error.store(float(value)); return VMHIP_OK;
+        case VMHIP_DEBUG_WIDE_OFFSETS: g_debug_wide_offsets.store(value != 0.0); return VMHIP_OK;
         case VMHIP_DEBUG_EDGE_BAND: g_debug_edge_band.store(value <= 0.0 ? VMHIP_AMB_EPS_DEFAULT : float(value)); return VMHIP_OK;
         default: return fail(VMHIP_ERR_ARGUMENT, "debug_set: unknown knob");
     }

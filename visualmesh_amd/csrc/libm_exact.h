@@ -42,12 +42,14 @@ VM_HD float vm_bits_float(uint32_t u) {
     memcpy(&f, &u, 4);
     return f;
 }
-/* Correctly rounded square root. The device's single-precision square root instruction is only
- * accurate to an ulp, so the device takes the double-precision root (correctly rounded) and rounds it
- * once more: with 53 >= 2*24 + 2 significand bits that double rounding cannot change the result. */
+/* Correctly rounded square root. The device's square root instruction alone is only accurate to an ulp; what the
+ * compiler makes of sqrtf() in device code (HIP's default: correctly rounded division and square root) is that
+ * instruction followed by a choice among the result and its two neighbours by the sign of their exact residuals
+ * x - s * s', which is the correctly rounded root, denormals included. The GPU test of this header compares it with
+ * the host's over every float from zero to four. */
 VM_HD float vm_sqrtf(float x) {
 #if defined(__HIP_DEVICE_COMPILE__)
-    return (float) sqrt((double) x);
+    return __builtin_sqrtf(x);
 #else
     return sqrtf(x);
 #endif

@@ -41,11 +41,16 @@ constexpr size_t AT_TILE_COUNT = AT_CAND_KEEP + up256(MAX_CAND / 8);
 constexpr size_t AT_NO_FORCE = AT_TILE_COUNT + up256(4 * (MAX_CAND / VMHIP_TILE)); /* stays zero: no forced decisions */
 constexpr size_t AT_AMB_LIST = AT_NO_FORCE + up256(MAX_CAND / 8);
 constexpr size_t AT_LOOKUP = AT_AMB_LIST + up256(sizeof(int2) * VMHIP_AMB_CAP);
-constexpr size_t SCRATCH_BYTES = AT_LOOKUP + up256(sizeof(uint2) * (MAX_NODES + 1));
+constexpr size_t SCRATCH_BYTES = AT_LOOKUP + up256(sizeof(uint32_t) * (MAX_NODES + 1));
+
+/* a reverse-lookup entry: 8 bits of run stamp above 24 bits of row */
+constexpr int STAMP_ROW_BITS = 24;
+constexpr uint32_t STAMP_LAST = 0xffffffffu >> STAMP_ROW_BITS;
+static_assert(MAX_CAND < (size_t(1) << STAMP_ROW_BITS), "a row fits the entry");
 
 }  // namespace
 
-/* The workspace of vmhip_project_noalloc, 15.5 MB, held by every device the library runs on until the process ends.
+/* The workspace of vmhip_project_noalloc, 11.3 MB, held by every device the library runs on until the process ends.
  * In host code this name is a handle, not an address: the address on a device comes from hipGetSymbolAddress
  * (vm_noalloc_setup) and is what every launch below is given. */
 static __device__ __align__(256) unsigned char scratch[SCRATCH_BYTES];
@@ -70,9 +75,9 @@ __global__ __launch_bounds__(PREPARE_THREADS) void vm_noalloc_prepare_kernel(VmF
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     if (tid == 0) {
         bad = 0;
-        uint32_t e = header->epoch + 1u;
-        header->wrapped = e == 0u ? 1u : 0u;
-        header->epoch = e == 0u ? 1u : e;
+        const uint32_t e = header->epoch + 1u;
+        header->wrapped = e > STAMP_LAST ? 1u : 0u;
+        header->epoch = e > STAMP_LAST ? 1u : e;
         header->amb_count = 0;
     }
     __syncthreads();
@@ -121,11 +126,11 @@ __global__ __launch_bounds__(PREPARE_THREADS) void vm_noalloc_prepare_kernel(VmF
     }
 }
 
-/* Second kernel of a call: does nothing unless the run stamp wrapped, then it clears the reverse lookup table so that
- * stamps of four thousand million calls ago cannot look current. */
-__global__ __launch_bounds__(256) void vm_noalloc_wrap_kernel(const Header* header, uint2* lookup, size_t entries) {
+/* Second kernel of a call: does nothing unless the run stamp started again from one (every 255 calls), then it clears the
+ * reverse lookup table so that stamps of 255 calls ago cannot look current. */
+__global__ __launch_bounds__(256) void vm_noalloc_wrap_kernel(const Header* header, uint32_t* lookup, size_t entries) {
     if (header->wrapped == 0u) return;
-    for (size_t i = (size_t) blockIdx.x * blockDim.x + threadIdx.x; i < entries; i += (size_t) gridDim.x * blockDim.x) lookup[i] = make_uint2(0u, 0u);
+    for (size_t i = (size_t) blockIdx.x * blockDim.x + threadIdx.x; i < entries; i += (size_t) gridDim.x * blockDim.x) lookup[i] = 0u;
 }
 
 }  // namespace
@@ -177,7 +182,7 @@ extern "C" int vmhip_project_noalloc(const vmhip_mesh* mesh, const float* Rco, c
     VmFrame* d_frame = reinterpret_cast<VmFrame*>(ws + AT_FRAME);
     int32_t* range_first = reinterpret_cast<int32_t*>(ws + AT_RANGE_FIRST);
     int32_t* range_prefix = reinterpret_cast<int32_t*>(ws + AT_RANGE_PREFIX);
-    uint2* lookup = reinterpret_cast<uint2*>(ws + AT_LOOKUP);
+    uint32_t* lookup = reinterpret_cast<uint32_t*>(ws + AT_LOOKUP);
 
     VmFrame F{};
     F.rays = mesh->d_rays;
@@ -207,6 +212,9 @@ extern "C" int vmhip_project_noalloc(const vmhip_mesh* mesh, const float* Rco, c
     B.n_cand_tiles = (n_candidates + VMHIP_TILE - 1) / VMHIP_TILE;
     B.n_row_tiles = n_candidates > 0 ? (n_candidates + 1 + VMHIP_TILE - 1) / VMHIP_TILE : 0;
     B.epoch = &header->epoch;
+    B.stamp_row_bits = STAMP_ROW_BITS;
+    B.uniform_nn = mesh->nn;
+    B.wide_offsets = uint64_t(mesh->n_nodes) * uint64_t(mesh->nn) >= (1ull << 30) ? 1 : 0; /* the output tables are far below 4 GiB */
     B.cand_px = reinterpret_cast<float2*>(ws + AT_CAND_PX);
     B.cand_g = reinterpret_cast<int32_t*>(ws + AT_CAND_G);
     B.cand_keep = reinterpret_cast<uint64_t*>(ws + AT_CAND_KEEP);

@@ -19,11 +19,35 @@
  */
 #include "vmhip_internal.h"
 
+#include <type_traits>
+
 #pragma clang fp contract(off)
 
 #include "libm_exact.h"
 
 namespace {
+
+/* A pointer that was itself read from memory (a frame's tables, its image) is taken for one that might point into
+ * LDS, and what it points to is then read through the slower generic path with a 64-bit vector address. These casts
+ * say that it points to device memory. */
+#define VM_GLOBAL __attribute__((address_space(1)))
+template <typename T>
+__device__ __forceinline__ const VM_GLOBAL T* in_device_memory(const T* p) {
+    return (const VM_GLOBAL T*) p;
+}
+template <typename T>
+__device__ __forceinline__ VM_GLOBAL T* in_device_memory(T* p) {
+    return (VM_GLOBAL T*) p;
+}
+/* base[index] with the offset in Off's width */
+template <typename T, typename Off>
+__device__ __forceinline__ T read_element(const T* base, Off index) {
+    return *reinterpret_cast<const VM_GLOBAL T*>((const VM_GLOBAL char*) reinterpret_cast<const char*>(base) + index * (Off) sizeof(T));
+}
+template <typename T, typename Off>
+__device__ __forceinline__ void write_element(T* base, Off index, const T& value) {
+    *reinterpret_cast<VM_GLOBAL T*>((VM_GLOBAL char*) reinterpret_cast<char*>(base) + index * (Off) sizeof(T)) = value;
+}
 
 __device__ __forceinline__ int find_frame_by_cand_tile(const VmFrame* frames, int n, int tile) {
     int lo = 0, hi = n - 1;
@@ -55,6 +79,30 @@ __device__ __forceinline__ int cand_to_global(const VmFrame& F, int p) {
     return F.range_first[lo] + (p - F.range_prefix[lo]);
 }
 
+/* The same for the 64 consecutive slots of a wave (p = the wave's first slot + lane): the range of the first slot is
+ * found once, by a search on wave-uniform values that the scalar unit carries out; a lane then steps forward over the
+ * range boundaries that lie between the first slot and its own - rarely more than one or two. */
+__device__ __forceinline__ int cand_to_global_wave(const VmFrame& F, int p, int lane) {
+    const int p0 = __builtin_amdgcn_readfirstlane(p - lane);
+    int lo = 0, hi = F.n_ranges - 1;
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (F.range_prefix[mid] <= p0) lo = mid;
+        else hi = mid - 1;
+    }
+    lo = __builtin_amdgcn_readfirstlane(lo);
+    const VM_GLOBAL int32_t* const prefix = in_device_memory(F.range_prefix);
+    const int n_ranges = F.n_ranges;
+    int start = prefix[lo];
+    while (lo + 1 < n_ranges) {
+        const int next = prefix[lo + 1];
+        if (next > p) break;
+        start = next;
+        ++lo;
+    }
+    return in_device_memory(F.range_first)[lo] + (p - start);
+}
+
 /* Lens projection, reference utility/projection.hpp:162-187 with utility/math.hpp's dot order. */
 __device__ __forceinline__ float2 project_ray(const VmFrame& F, float rx, float ry, float rz) {
     const float c0 = F.Rco[2] * rz + (F.Rco[1] * ry + F.Rco[0] * rx);
@@ -74,11 +122,17 @@ __device__ __forceinline__ float2 project_ray(const VmFrame& F, float rx, float 
     else {
         r_u = F.focal * theta;
     }
-    /* distortion polynomial: a double sum of float terms (the reference's literal 1.0) */
+    /* distortion polynomial: a double sum of float terms (the reference's literal 1.0). Without distortion every term
+     * is a zero and the sum is exactly 1.0 unless a power of r_u overflowed (zero times infinity), so that a lens without
+     * coefficients skips the double-precision steps and gets the same bits. */
     const float r2 = r_u * r_u;
-    const double s = 1.0 + (double) (F.ik[0] * r2) + (double) (F.ik[1] * (r2 * r2)) + (double) (F.ik[2] * (r2 * r2) * r2)
-                     + (double) (F.ik[3] * (r2 * r2) * (r2 * r2));
-    const float r_d = (float) ((double) r_u * s);
+    float r_d = r_u;
+    const bool undistorted = F.ik[0] == 0.0f && F.ik[1] == 0.0f && F.ik[2] == 0.0f && F.ik[3] == 0.0f;
+    if (!undistorted || !((r2 * r2) * (r2 * r2) < __builtin_inff())) {
+        const double s = 1.0 + (double) (F.ik[0] * r2) + (double) (F.ik[1] * (r2 * r2)) + (double) (F.ik[2] * (r2 * r2) * r2)
+                         + (double) (F.ik[3] * (r2 * r2) * (r2 * r2));
+        r_d = (float) ((double) r_u * s);
+    }
 
     float sx = 0.0f, sy = 0.0f;
     if (!(c0 >= 1.0f)) {
@@ -397,8 +451,11 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_project_kernel(VmBatchDev B) {
     bool keep = false;
     float2 px = make_float2(0.0f, 0.0f);
     if (valid) {
-        const int g = cand_to_global(F, p);
-        const float* r = F.rays + (size_t) g * 3;
+        /* the host's overruling decisions for this wave's candidates: read ahead of the arithmetic they do not depend on */
+        const size_t word = (size_t) (F.cand_base + p) >> 6;
+        const uint64_t force_valid = in_device_memory(F.force_valid)[word];
+        const int g = cand_to_global_wave(F, p, threadIdx.x & 63);
+        const VM_GLOBAL float* r = in_device_memory(F.rays) + (size_t) g * 3;
         px = project_ray(F, r[0], r[1], r[2]);
         px.x += B.px_error, px.y += B.px_error; /* zero outside tests of the edge guard */
         const float W = (float) F.width, H = (float) F.height;
@@ -409,10 +466,9 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_project_kernel(VmBatchDev B) {
         const float d = fminf(fminf(fabsf(px.x), fabsf(px.x + 1.0f - W)), fminf(fabsf(px.y), fabsf(px.y + 1.0f - H)));
         const bool ambiguous = !(d >= B.amb_eps);
 
-        const size_t word = (size_t) (F.cand_base + p) >> 6;
         const uint64_t bit = 1ull << (threadIdx.x & 63);
-        const bool forced = (F.force_valid[word] & bit) != 0;
-        if (forced) { keep = (F.force_keep[word] & bit) != 0; }
+        const bool forced = (force_valid & bit) != 0;
+        if (forced) { keep = (in_device_memory(F.force_keep)[word] & bit) != 0; }
         else if (ambiguous) {
             const int slot = atomicAdd(&B.amb_count[f], 1);
             if (slot < VMHIP_AMB_CAP) B.amb_list[(size_t) f * VMHIP_AMB_CAP + slot] = make_int2(p, keep ? 1 : 0);
@@ -443,25 +499,25 @@ __device__ __forceinline__ float4 texel_packed(const VmFrame& F, int x, int y) {
     float4 o;
     switch (F.fmt) {
         case VMHIP_FMT_RGBA: {
-            const uint32_t v = reinterpret_cast<const uint32_t*>(F.image)[idx];
+            const uint32_t v = in_device_memory(reinterpret_cast<const uint32_t*>(F.image))[idx];
             o = make_float4((float) (v & 0xff) * INV255, (float) ((v >> 8) & 0xff) * INV255,
                             (float) ((v >> 16) & 0xff) * INV255, (float) (v >> 24) * INV255);
         } break;
         case VMHIP_FMT_BGRA: {
-            const uint32_t v = reinterpret_cast<const uint32_t*>(F.image)[idx];
+            const uint32_t v = in_device_memory(reinterpret_cast<const uint32_t*>(F.image))[idx];
             o = make_float4((float) ((v >> 16) & 0xff) * INV255, (float) ((v >> 8) & 0xff) * INV255,
                             (float) (v & 0xff) * INV255, (float) (v >> 24) * INV255);
         } break;
         case VMHIP_FMT_RGB3: {
-            const uint8_t* b = F.image + idx * 3;
+            const VM_GLOBAL uint8_t* b = in_device_memory(F.image) + idx * 3;
             o = make_float4((float) b[0] * INV255, (float) b[1] * INV255, (float) b[2] * INV255, 1.0f);
         } break;
         case VMHIP_FMT_BGR3: {
-            const uint8_t* b = F.image + idx * 3;
+            const VM_GLOBAL uint8_t* b = in_device_memory(F.image) + idx * 3;
             o = make_float4((float) b[2] * INV255, (float) b[1] * INV255, (float) b[0] * INV255, 1.0f);
         } break;
         default: { /* GRAY */
-            const float v = (float) F.image[idx] * INV255;
+            const float v = (float) in_device_memory(F.image)[idx] * INV255;
             o = make_float4(v, v, v, 1.0f);
         } break;
     }
@@ -523,7 +579,7 @@ __device__ __forceinline__ float4 sample_image(const VmFrame& F, float2 px) {
 #pragma unroll
             for (int c = 0; c < 6; ++c) {
                 const int xc = min(max(x1 - 2 + c, 0), F.width - 1);
-                u[r][c] = F.image[(size_t) yc * F.width + xc];
+                u[r][c] = in_device_memory(F.image)[(size_t) yc * F.width + xc];
             }
         }
         /* x2 == x1 or y2 == y1 only on the last column/row, which the filter excludes; handle anyway */
@@ -596,7 +652,7 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_compact_kernel(VmBatchDev B, fl
         const float2 px = B.cand_px[(size_t) F.cand_base + p];
         B.row_px[row] = px;
         B.row_gidx[row] = g;
-        F.r_lookup[g] = make_uint2(*B.epoch, (uint32_t) local);
+        in_device_memory(F.r_lookup)[g] = (*B.epoch << B.stamp_row_bits) | (uint32_t) local;
         if (classify) feat[row] = sample_image(F, px);
     }
     if (t_local == F.cand_tiles - 1 && threadIdx.x == 0) {
@@ -613,9 +669,15 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_compact_kernel(VmBatchDev B, fl
  * other tiles are deduplicated through an open-addressing hash in LDS, numbered densely in table order (the
  * halo slots), and every neighbour is rewritten as a position in "own tile rows, then halo slots". Which row
  * gets which halo slot depends on the order the atomics land in and may differ from run to run; the rows that a
- * slot stands for, and so every result computed through the tables, do not. */
+ * slot stands for, and so every result computed through the tables, do not.
+ *
+ * WIDE = false addresses the frame's tables with 32-bit byte offsets from wave-uniform bases (an address is then a
+ * scalar register pair plus one vector register, and the 64-bit vector arithmetic that was a third of this kernel's
+ * instructions is gone); the host picks WIDE = true for a batch with a table of 4 GiB or more. */
 #define NB_HASH 2048 /* >= the most out-of-tile neighbours a tile can have (256 rows x 8) */
+template <bool WIDE, int NN>
 __global__ __launch_bounds__(VMHIP_TILE) void vm_neighbourhood_kernel(VmBatchDev B) {
+    using Off = typename std::conditional<WIDE, size_t, uint32_t>::type;
     __shared__ __align__(16) uint32_t h_key[NB_HASH];
     __shared__ uint16_t h_dense[NB_HASH];
     __shared__ int wave_total[VMHIP_TILE / 64];
@@ -625,13 +687,14 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_neighbourhood_kernel(VmBatchDev
     const int f = find_frame_by_row_tile(B.frames, B.n_frames, tile);
     const VmFrame& F = B.frames[f];
     const int V = B.frame_V[f];
-    const int nn = F.nn;
+    /* the frame's fields as values: read through F again after a store, they would be fetched again */
+    const int nn = NN > 0 ? NN : F.nn, n_nodes = F.n_nodes, row_base = F.row_base;
     const int row0 = (tile - F.row_tile0) * VMHIP_TILE;
     const bool tables = B.row_nbl != nullptr;
-    const uint32_t epoch = *B.epoch;
+    const uint32_t epoch = *B.epoch, row_mask = (1u << B.stamp_row_bits) - 1u;
     const int n_rows = max(0, min(VMHIP_TILE, V + 1 - row0));
     if (n_rows == 0) {
-        if (tables && threadIdx.x == 0) B.tile_desc[tile] = make_int4(F.row_base + row0, 0, 0, F.row_base);
+        if (tables && threadIdx.x == 0) B.tile_desc[tile] = make_int4(row_base + row0, 0, 0, row_base);
         return;
     }
     constexpr uint32_t EMPTY = 0xffffffffu;
@@ -641,59 +704,74 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_neighbourhood_kernel(VmBatchDev
         __syncthreads();
     }
 
-    /* (row, neighbour) items are dealt round-robin to the threads; a thread keeps its items' results in registers
-     * between the passes (the tables are only built for nn <= VMHIP_NBL_STRIDE, so at most 8 items per thread) */
+    /* the frame's parts of the tables, wave-uniform */
+    const int32_t* const gidx = B.row_gidx + row_base;
+    int32_t* const nb_out = B.row_nb + (size_t) row_base * B.nb_stride;
+    const int32_t* const nbr = F.nbr;
+    const uint32_t* const lookup = F.r_lookup;
+    const Off nb_stride = (Off) B.nb_stride;
+
+    /* (row, neighbour) items are dealt round-robin to the threads, VMHIP_TILE at a time, so that a thread has at most nn
+     * of them; it takes them MAX_ITEMS at a time and keeps their results in registers between the passes (the tables
+     * are only built for nn <= VMHIP_NBL_STRIDE, one round). NN > 0: every frame of the batch has NN neighbours per node, and
+     * the rounds have no idle items; NN = 0: whatever the frame has, eight at a time, with the
+     * item -> row division by nn as a multiplication by ceil(2^32 / nn), exact while item * nn < 2^32. */
     const int n_items = n_rows * nn;
-    constexpr int MAX_ITEMS = VMHIP_NBL_STRIDE;
-    int outs[MAX_ITEMS];
-    auto resolve = [&](int it) {
-        const int i = row0 + it / nn;
-        const int j = it - (it / nn) * nn;
-        int out = V;
-        if (i < V) {
-            const int g = B.row_gidx[(size_t) F.row_base + i];
-            const int gn = F.nbr[(size_t) g * nn + j];
-            const uint2 e = F.r_lookup[min(gn, F.n_nodes)];
-            out = e.x == epoch ? (int) e.y : V;
+    const uint32_t nn_magic = nn > 1 ? 0xffffffffu / (uint32_t) nn + 1u : 0u;
+    auto row_of = [&](int it) { return NN > 0 ? it / (NN > 0 ? NN : 1) : nn > 1 ? (int) __umulhi((uint32_t) it, nn_magic) : it; };
+    constexpr int MAX_ITEMS = NN > 0 ? NN : VMHIP_NBL_STRIDE;
+    int item_row[MAX_ITEMS], item_slot[MAX_ITEMS], outs[MAX_ITEMS];
+
+    /* Items k0 .. k0 + MAX_ITEMS - 1 of this thread. The three dependent reads of an item (row -> node, node -> neighbour
+     * node, neighbour node -> its row) go level by level over all the items, so that the items' reads are in flight together
+     * and no store or branch stands between them: an item that does not exist, or that belongs to the null row, reads what
+     * the frame's last row reads, and its result is not used. */
+    auto resolve = [&](int k0) {
+        bool live[MAX_ITEMS];
+        uint32_t stamp[MAX_ITEMS];
+#pragma unroll
+        for (int k = 0; k < MAX_ITEMS; ++k) {
+            const int it = threadIdx.x + (k0 + k) * VMHIP_TILE;
+            const int r = row_of(it);
+            item_row[k] = row0 + r;
+            item_slot[k] = it - r * nn;
+            live[k] = it < n_items;
+            stamp[k] = 0u; /* zero carries no run's stamp: runs count from one */
         }
-        B.row_nb[((size_t) F.row_base + i) * B.nb_stride + j] = out;
-        return out;
+        if (V > 0) {
+            int node[MAX_ITEMS];
+#pragma unroll
+            for (int k = 0; k < MAX_ITEMS; ++k) node[k] = read_element(gidx, (Off) min(item_row[k], V - 1));
+#pragma unroll
+            for (int k = 0; k < MAX_ITEMS; ++k) node[k] = min(read_element(nbr, (Off) node[k] * (Off) nn + (Off) item_slot[k]), n_nodes);
+#pragma unroll
+            for (int k = 0; k < MAX_ITEMS; ++k) stamp[k] = read_element(lookup, (Off) node[k]);
+        }
+#pragma unroll
+        for (int k = 0; k < MAX_ITEMS; ++k) {
+            outs[k] = -1;
+            if (live[k]) {
+                const bool found = item_row[k] < V && (stamp[k] >> B.stamp_row_bits) == epoch;
+                const int out = found ? (int) (stamp[k] & row_mask) : V;
+                write_element(nb_out, (Off) item_row[k] * nb_stride + (Off) item_slot[k], out);
+                outs[k] = out;
+            }
+        }
     };
     if (!tables) {
-        for (int it = threadIdx.x; it < n_items; it += VMHIP_TILE) resolve(it);
+        for (int k0 = 0; k0 < nn; k0 += MAX_ITEMS) resolve(k0);
         return;
     }
-    /* the three dependent reads of an item (row -> node, node -> neighbour node, neighbour node -> its row), level by
-     * level over all of the thread's items, so that the items' reads are in flight together and no store stands
-     * between them */
-    int item_row[MAX_ITEMS], item_slot[MAX_ITEMS], node[MAX_ITEMS];
+    resolve(0);
 #pragma unroll
     for (int k = 0; k < MAX_ITEMS; ++k) {
-        const int it = threadIdx.x + k * VMHIP_TILE;
-        item_row[k] = row0 + it / nn;
-        item_slot[k] = it - (it / nn) * nn;
-        node[k] = (it < n_items && item_row[k] < V) ? B.row_gidx[(size_t) F.row_base + item_row[k]] : -1;
-    }
-#pragma unroll
-    for (int k = 0; k < MAX_ITEMS; ++k) node[k] = node[k] >= 0 ? min(F.nbr[(size_t) node[k] * nn + item_slot[k]], F.n_nodes) : -1;
-    uint2 stamp[MAX_ITEMS];
-#pragma unroll
-    for (int k = 0; k < MAX_ITEMS; ++k) stamp[k] = node[k] >= 0 ? F.r_lookup[node[k]] : make_uint2(epoch + 1u, 0u);
-#pragma unroll
-    for (int k = 0; k < MAX_ITEMS; ++k) {
-        const int it = threadIdx.x + k * VMHIP_TILE;
-        outs[k] = -1;
-        if (it < n_items) {
-            const int out = stamp[k].x == epoch ? (int) stamp[k].y : V;
-            B.row_nb[((size_t) F.row_base + item_row[k]) * B.nb_stride + item_slot[k]] = out;
-            outs[k] = out;
-            if (out < row0 || out >= row0 + VMHIP_TILE) {
-                uint32_t slot = hash((uint32_t) out);
-                while (true) {
-                    const uint32_t prev = atomicCAS(&h_key[slot], EMPTY, (uint32_t) out);
-                    if (prev == EMPTY || prev == (uint32_t) out) break;
-                    slot = (slot + 1) & (NB_HASH - 1);
-                }
+        const int out = outs[k];
+        if (out >= 0 && (out < row0 || out >= row0 + VMHIP_TILE)) {
+            uint32_t slot = hash((uint32_t) out);
+            while (true) {
+                const uint32_t prev = atomicCAS(&h_key[slot], EMPTY, (uint32_t) out);
+                if (prev == EMPTY || prev == (uint32_t) out) break;
+                slot = (slot + 1) & (NB_HASH - 1);
             }
         }
     }
@@ -725,22 +803,22 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_neighbourhood_kernel(VmBatchDev
         total += wave_total[w];
     }
     const int cap = B.halo_cap;
+    uint32_t* const tile_halo = B.tile_halo + (size_t) tile * VMHIP_HALO_MAX;
     if (mine > 0) {
 #pragma unroll
         for (int k = 0; k < PER; ++k) {
             if (keys[k] != EMPTY) {
                 h_dense[threadIdx.x * PER + k] = (uint16_t) min(before, 0xffff);
-                if (before < cap) B.tile_halo[(size_t) tile * VMHIP_HALO_MAX + before] = (uint32_t) F.row_base + keys[k];
+                if (before < cap) tile_halo[before] = (uint32_t) row_base + keys[k];
                 ++before;
             }
         }
     }
-    if (threadIdx.x == 0) B.tile_desc[tile] = make_int4(F.row_base + row0, n_rows, min(total, cap), F.row_base);
+    if (threadIdx.x == 0) B.tile_desc[tile] = make_int4(row_base + row0, n_rows, min(total, cap), row_base);
     __syncthreads();
 
 #pragma unroll
     for (int k = 0; k < MAX_ITEMS; ++k) {
-        const int it = threadIdx.x + k * VMHIP_TILE;
         const int out = outs[k];
         if (out >= 0) {
             uint32_t local;
@@ -753,13 +831,16 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_neighbourhood_kernel(VmBatchDev
                 const int dense = h_dense[slot];
                 local = dense < cap ? (uint32_t) (VMHIP_TILE + dense) : VMHIP_NBL_FAR;
             }
-            nbl_rows[it / nn][it - (it / nn) * nn] = (uint16_t) local;
+            nbl_rows[item_row[k] - row0][item_slot[k]] = (uint16_t) local;
         }
     }
     __syncthreads();
     /* one 16-byte store per row (entries past nn are never read) */
-    if ((int) threadIdx.x < n_rows)
-        *reinterpret_cast<uint4*>(B.row_nbl + ((size_t) F.row_base + row0 + threadIdx.x) * VMHIP_NBL_STRIDE) = *reinterpret_cast<const uint4*>(nbl_rows[threadIdx.x]);
+    if ((int) threadIdx.x < n_rows) {
+        uint16_t* const nbl_out = B.row_nbl + (size_t) row_base * VMHIP_NBL_STRIDE;
+        typedef unsigned int row_words __attribute__((ext_vector_type(4)));
+        write_element(reinterpret_cast<row_words*>(nbl_out), (Off) (row0 + threadIdx.x), *reinterpret_cast<const row_words*>(nbl_rows[threadIdx.x]));
+    }
 }
 
 }  // namespace
@@ -802,6 +883,18 @@ void vm_launch_lookup(const VmLookupFrame* frames, int n_frames, hipStream_t str
     if (n_frames > 0) hipLaunchKernelGGL(vm_lookup_kernel, dim3(n_frames), dim3(LOOKUP_THREADS), 0, stream, frames);
 }
 
+template <bool WIDE>
+static void launch_neighbourhood(const VmBatchDev& B, hipStream_t stream) {
+    const dim3 grid(B.n_row_tiles), block(VMHIP_TILE);
+    switch (B.uniform_nn) {
+        case 4: hipLaunchKernelGGL((vm_neighbourhood_kernel<WIDE, 4>), grid, block, 0, stream, B); break;
+        case 6: hipLaunchKernelGGL((vm_neighbourhood_kernel<WIDE, 6>), grid, block, 0, stream, B); break;
+        case 8: hipLaunchKernelGGL((vm_neighbourhood_kernel<WIDE, 8>), grid, block, 0, stream, B); break;
+        default: hipLaunchKernelGGL((vm_neighbourhood_kernel<WIDE, 0>), grid, block, 0, stream, B); break;
+    }
+}
 void vm_launch_neighbourhood(const VmBatchDev& B, hipStream_t stream) {
-    if (B.n_row_tiles > 0) hipLaunchKernelGGL(vm_neighbourhood_kernel, dim3(B.n_row_tiles), dim3(VMHIP_TILE), 0, stream, B);
+    if (B.n_row_tiles <= 0) return;
+    if (B.wide_offsets) launch_neighbourhood<true>(B, stream);
+    else launch_neighbourhood<false>(B, stream);
 }

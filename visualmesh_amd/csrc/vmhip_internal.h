@@ -64,7 +64,7 @@ struct VmFrame {
     /* mesh */
     const float* rays;     /* [n_nodes][3] */
     const int32_t* nbr;    /* [n_nodes][nn] */
-    uint2* r_lookup;       /* [n_nodes+1] {epoch, local row}; entry n_nodes is never stamped */
+    uint32_t* r_lookup;    /* [n_nodes+1] run stamp above the local row (VmBatchDev::stamp_row_bits); entry n_nodes is never stamped */
     int32_t n_nodes;
     int32_t nn;
     /* pose + lens */
@@ -93,6 +93,11 @@ struct VmBatchDev {
     int32_t n_frames;
     int32_t n_cand_tiles, n_row_tiles;
     uint32_t* epoch;      /* device word: the run's stamp for the reverse lookup; the reset kernel increments it */
+    int32_t uniform_nn;     /* neighbours per node if every frame of the batch has the same number, else 0 */
+    int32_t wide_offsets;   /* a frame's part of a table reaches 4 GiB: the neighbourhood kernel addresses with 64-bit offsets */
+    int32_t stamp_row_bits; /* a reverse-lookup entry is (stamp << stamp_row_bits) | local row: 24 bits of row unless a frame
+                             * has 2^24 candidates or more; the stamp counts from 1 to 2^(32 - stamp_row_bits) - 1 and the table
+                             * is cleared before it starts again */
     /* candidate space */
     float2* cand_px;
     int32_t* cand_g;      /* the candidate's node (global index), worked out once by the projection */
