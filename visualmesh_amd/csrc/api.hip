@@ -294,7 +294,9 @@ int batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int
 
     /* device workspace */
     HIP_TRY(b->d_frames.reserve(sizeof(VmFrame) * n_frames));
-    HIP_TRY(b->d_ranges.reserve(sizeof(int32_t) * std::max<size_t>(range_ints, 1)));
+    /* the range tables, then the tile tables: {frame, first range} per candidate tile (on an 8-byte boundary), frame per row tile */
+    const size_t tile_table_at = align_up(std::max<size_t>(range_ints, 1), 2), n_table_ints = tile_table_at + 2 * cand_tiles + row_tiles;
+    HIP_TRY(b->d_ranges.reserve(sizeof(int32_t) * n_table_ints));
     HIP_TRY(b->d_images.reserve(std::max<size_t>(image_bytes, 256)));
     HIP_TRY(b->d_cand_px.reserve(sizeof(float2) * std::max<size_t>(b->cand_total, 1)));
     HIP_TRY(b->d_cand_g.reserve(4 * std::max<size_t>(b->cand_total, 1)));
@@ -355,9 +357,8 @@ int batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int
     b->drop_graph(); /* pointers and sizes baked into a captured run are no longer valid */
 
     /* fill in device pointers and upload */
-    const size_t n_range_ints = std::max<size_t>(range_ints, 1);
     {
-        const size_t need = align_up(sizeof(VmFrame) * size_t(n_frames), 64) + 4 * n_range_ints;
+        const size_t need = align_up(sizeof(VmFrame) * size_t(n_frames), 64) + 4 * n_table_ints;
         if (need > b->h_stage_cap) {
             if (b->h_stage) HIP_TRY(hipHostFree(b->h_stage));
             b->h_stage = nullptr, b->h_stage_cap = 0;
@@ -402,10 +403,19 @@ int batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int
         d.force_valid = b->d_force_valid.as<uint64_t>();
         d.force_keep = b->d_force_keep.as<uint64_t>();
         h_frames[f] = d;
+        /* the tiles of this frame: a candidate tile's first candidate lies in range r, prefix[r] <= first < prefix[r + 1] */
+        int32_t* const cand_info = h_ranges + tile_table_at + 2 * size_t(d.cand_tile0);
+        int r = 0;
+        for (int t = 0; t < d.cand_tiles; ++t) {
+            while (r + 1 < R && hf.prefix[size_t(r) + 1] <= int64_t(t) * VMHIP_TILE) ++r;
+            cand_info[2 * t] = f;
+            cand_info[2 * t + 1] = r;
+        }
+        std::fill_n(h_ranges + tile_table_at + 2 * cand_tiles + size_t(d.row_tile0), size_t(d.row_tiles), f);
     }
     if (run_bytes > 0) HIP_TRY(hipMemcpyAsync(b->d_images.as<uint8_t>() + run_dst, run_src, run_bytes, hipMemcpyHostToDevice, E->stream));
     HIP_TRY(hipMemcpyAsync(b->d_frames.p, h_frames, sizeof(VmFrame) * n_frames, hipMemcpyHostToDevice, E->stream));
-    HIP_TRY(hipMemcpyAsync(b->d_ranges.p, h_ranges, sizeof(int32_t) * n_range_ints, hipMemcpyHostToDevice, E->stream));
+    HIP_TRY(hipMemcpyAsync(b->d_ranges.p, h_ranges, sizeof(int32_t) * n_table_ints, hipMemcpyHostToDevice, E->stream));
     HIP_TRY(hipMemsetAsync(b->d_force_valid.p, 0, 8 * std::max<size_t>(words, 1), E->stream));
     HIP_TRY(hipMemsetAsync(b->d_force_keep.p, 0, 8 * std::max<size_t>(words, 1), E->stream));
     b->h_force_valid.assign(std::max<size_t>(words, 1), 0);
@@ -442,6 +452,8 @@ int batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int
     D.epoch = b->d_epoch.as<uint32_t>();
     D.stamp_row_bits = b->stamp_row_bits;
     D.uniform_nn = uniform_nn;
+    D.cand_tile_info = reinterpret_cast<const int2*>(b->d_ranges.as<int32_t>() + tile_table_at);
+    D.row_tile_frame = b->d_ranges.as<int32_t>() + tile_table_at + 2 * cand_tiles;
     /* 32-bit byte offsets into a frame's part of every table the neighbourhood kernel touches (4-byte entries of the
      * mesh's neighbour table and of the output table, 16-byte rows of the tile-local table), unless one is too large */
     D.wide_offsets = (widest_mesh >= (1ull << 30) || (uint64_t(max_cand) + 1) * uint64_t(std::max(nb_stride, 4)) >= (1ull << 30) || g_debug_wide_offsets.load()) ? 1 : 0;

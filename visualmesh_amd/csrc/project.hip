@@ -80,17 +80,21 @@ __device__ __forceinline__ int cand_to_global(const VmFrame& F, int p) {
 }
 
 /* The same for the 64 consecutive slots of a wave (p = the wave's first slot + lane): the range of the first slot is
- * found once, by a search on wave-uniform values that the scalar unit carries out; a lane then steps forward over the
- * range boundaries that lie between the first slot and its own - rarely more than one or two. */
-__device__ __forceinline__ int cand_to_global_wave(const VmFrame& F, int p, int lane) {
-    const int p0 = __builtin_amdgcn_readfirstlane(p - lane);
-    int lo = 0, hi = F.n_ranges - 1;
-    while (lo < hi) {
-        const int mid = (lo + hi + 1) >> 1;
-        if (F.range_prefix[mid] <= p0) lo = mid;
-        else hi = mid - 1;
+ * taken from the batch's tile table or found once, by a search on wave-uniform values that the scalar unit carries out;
+ * a lane then steps forward over the range boundaries that lie between that slot and its own - rarely more than one or two. */
+__device__ __forceinline__ int cand_to_global_wave(const VmFrame& F, int p, int lane, int tile_range) {
+    int lo = tile_range; /* the range of the tile's first slot, if the batch was staged with its tile tables */
+    if (tile_range < 0) {
+        const int p0 = __builtin_amdgcn_readfirstlane(p - lane);
+        int hi = F.n_ranges - 1;
+        lo = 0;
+        while (lo < hi) {
+            const int mid = (lo + hi + 1) >> 1;
+            if (F.range_prefix[mid] <= p0) lo = mid;
+            else hi = mid - 1;
+        }
+        lo = __builtin_amdgcn_readfirstlane(lo);
     }
-    lo = __builtin_amdgcn_readfirstlane(lo);
     const VM_GLOBAL int32_t* const prefix = in_device_memory(F.range_prefix);
     const int n_ranges = F.n_ranges;
     int start = prefix[lo];
@@ -443,18 +447,27 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_lookup_export_kernel(VmBatchDev
 __global__ __launch_bounds__(VMHIP_TILE) void vm_project_kernel(VmBatchDev B) {
     __shared__ int wave_count[VMHIP_TILE / 64];
     const int tile = blockIdx.x;
-    const int f = find_frame_by_cand_tile(B.frames, B.n_frames, tile);
+    int f, tile_range = -1;
+    if (B.cand_tile_info) {
+        const int2 info = B.cand_tile_info[tile];
+        f = info.x, tile_range = info.y;
+    }
+    else {
+        f = find_frame_by_cand_tile(B.frames, B.n_frames, tile);
+    }
     const VmFrame& F = B.frames[f];
-    const int p = (tile - F.cand_tile0) * VMHIP_TILE + threadIdx.x;
+    /* the frame's placement as values: read through F again after a store, it would be fetched again */
+    const int cand_base = F.cand_base, cand_tile0 = F.cand_tile0;
+    const int p = (tile - cand_tile0) * VMHIP_TILE + threadIdx.x;
     const bool valid = p < F.n_cand;
 
     bool keep = false;
     float2 px = make_float2(0.0f, 0.0f);
     if (valid) {
         /* the host's overruling decisions for this wave's candidates: read ahead of the arithmetic they do not depend on */
-        const size_t word = (size_t) (F.cand_base + p) >> 6;
+        const size_t word = (size_t) (cand_base + p) >> 6;
         const uint64_t force_valid = in_device_memory(F.force_valid)[word];
-        const int g = cand_to_global_wave(F, p, threadIdx.x & 63);
+        const int g = cand_to_global_wave(F, p, threadIdx.x & 63, tile_range);
         const VM_GLOBAL float* r = in_device_memory(F.rays) + (size_t) g * 3;
         px = project_ray(F, r[0], r[1], r[2]);
         px.x += B.px_error, px.y += B.px_error; /* zero outside tests of the edge guard */
@@ -473,14 +486,14 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_project_kernel(VmBatchDev B) {
             const int slot = atomicAdd(&B.amb_count[f], 1);
             if (slot < VMHIP_AMB_CAP) B.amb_list[(size_t) f * VMHIP_AMB_CAP + slot] = make_int2(p, keep ? 1 : 0);
         }
-        B.cand_px[(size_t) F.cand_base + p] = px;
-        B.cand_g[(size_t) F.cand_base + p] = g;
+        B.cand_px[(size_t) cand_base + p] = px;
+        B.cand_g[(size_t) cand_base + p] = g;
     }
 
     const uint64_t mask = __ballot(keep);
     const int wave = threadIdx.x >> 6;
     if ((threadIdx.x & 63) == 0) {
-        B.cand_keep[((size_t) F.cand_base >> 6) + (size_t) (tile - F.cand_tile0) * (VMHIP_TILE / 64) + wave] = mask;
+        B.cand_keep[((size_t) cand_base >> 6) + (size_t) (tile - cand_tile0) * (VMHIP_TILE / 64) + wave] = mask;
         wave_count[wave] = __popcll(mask);
     }
     __syncthreads();
@@ -620,7 +633,7 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_compact_kernel(VmBatchDev B, fl
     __shared__ int partial[VMHIP_TILE / 64];
     __shared__ int wave_count[VMHIP_TILE / 64];
     const int tile = blockIdx.x;
-    const int f = find_frame_by_cand_tile(B.frames, B.n_frames, tile);
+    const int f = B.cand_tile_info ? B.cand_tile_info[tile].x : find_frame_by_cand_tile(B.frames, B.n_frames, tile);
     const VmFrame& F = B.frames[f];
     const int t_local = tile - F.cand_tile0;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -684,7 +697,7 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_neighbourhood_kernel(VmBatchDev
     __shared__ __align__(16) uint16_t nbl_rows[VMHIP_TILE][VMHIP_NBL_STRIDE]; /* the tile's positions, stored row by row at the end */
 
     const int tile = blockIdx.x;
-    const int f = find_frame_by_row_tile(B.frames, B.n_frames, tile);
+    const int f = B.row_tile_frame ? B.row_tile_frame[tile] : find_frame_by_row_tile(B.frames, B.n_frames, tile);
     const VmFrame& F = B.frames[f];
     const int V = B.frame_V[f];
     /* the frame's fields as values: read through F again after a store, they would be fetched again */

@@ -93,6 +93,9 @@ struct VmBatchDev {
     int32_t n_frames;
     int32_t n_cand_tiles, n_row_tiles;
     uint32_t* epoch;      /* device word: the run's stamp for the reverse lookup; the reset kernel increments it */
+    /* where a tile belongs, worked out when the batch is staged so that no block has to search for it (null: the blocks search) */
+    const int2* cand_tile_info;     /* [n_cand_tiles] {frame, index of the range that holds the tile's first candidate} */
+    const int32_t* row_tile_frame;  /* [n_row_tiles] frame */
     int32_t uniform_nn;     /* neighbours per node if every frame of the batch has the same number, else 0 */
     int32_t wide_offsets;   /* a frame's part of a table reaches 4 GiB: the neighbourhood kernel addresses with 64-bit offsets */
     int32_t stamp_row_bits; /* a reverse-lookup entry is (stamp << stamp_row_bits) | local row: 24 bits of row unless a frame
