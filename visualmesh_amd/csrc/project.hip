@@ -635,15 +635,30 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_compact_kernel(VmBatchDev B, fl
     const int tile = blockIdx.x;
     const int f = B.cand_tile_info ? B.cand_tile_info[tile].x : find_frame_by_cand_tile(B.frames, B.n_frames, tile);
     const VmFrame& F = B.frames[f];
-    const int t_local = tile - F.cand_tile0;
+    /* the frame's placement as values: read through F again after a store, it would be fetched again */
+    const int cand_base = F.cand_base, cand_tile0 = F.cand_tile0, cand_tiles = F.cand_tiles, row_base = F.row_base;
+    const int t_local = tile - cand_tile0;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+
+    /* What a kept candidate brings along does not depend on where it lands: its node, its pixel and the image sample are
+     * read and worked out first, so that these reads are under way while the block counts the kept candidates before it. */
+    const uint64_t mask = B.cand_keep[((size_t) cand_base >> 6) + (size_t) t_local * (VMHIP_TILE / 64) + wave];
+    const bool kept = (mask >> lane) & 1ull;
+    const int p = t_local * VMHIP_TILE + threadIdx.x;
+    int g = 0;
+    float2 px = make_float2(0.0f, 0.0f);
+    float4 sample = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    if (kept) {
+        g = B.cand_g[(size_t) cand_base + p];
+        px = B.cand_px[(size_t) cand_base + p];
+        if (classify) sample = sample_image(F, px);
+    }
 
     /* kept candidates in this frame's earlier tiles */
     int sum = 0;
-    for (int i = threadIdx.x; i < t_local; i += VMHIP_TILE) sum += B.tile_count[F.cand_tile0 + i];
+    for (int i = threadIdx.x; i < t_local; i += VMHIP_TILE) sum += B.tile_count[cand_tile0 + i];
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
-    const uint64_t mask = B.cand_keep[((size_t) F.cand_base >> 6) + (size_t) t_local * (VMHIP_TILE / 64) + wave];
     if (lane == 0) {
         partial[wave] = sum;
         wave_count[wave] = __popcll(mask);
@@ -657,22 +672,19 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_compact_kernel(VmBatchDev B, fl
         total += wave_count[w];
     }
 
-    const int p = t_local * VMHIP_TILE + threadIdx.x;
-    if ((mask >> lane) & 1ull) {
+    if (kept) {
         const int local = base + before + __popcll(mask & ((1ull << lane) - 1ull));
-        const size_t row = (size_t) F.row_base + local;
-        const int g = B.cand_g[(size_t) F.cand_base + p];
-        const float2 px = B.cand_px[(size_t) F.cand_base + p];
+        const size_t row = (size_t) row_base + local;
         B.row_px[row] = px;
         B.row_gidx[row] = g;
         in_device_memory(F.r_lookup)[g] = (*B.epoch << B.stamp_row_bits) | (uint32_t) local;
-        if (classify) feat[row] = sample_image(F, px);
+        if (classify) feat[row] = sample;
     }
-    if (t_local == F.cand_tiles - 1 && threadIdx.x == 0) {
+    if (t_local == cand_tiles - 1 && threadIdx.x == 0) {
         const int V = base + total;
         B.frame_V[f] = V;
         /* the off-screen row, engine/cpu/engine.hpp:205-206 */
-        if (classify) feat[(size_t) F.row_base + V] = make_float4(-1.0f, -1.0f, -1.0f, -1.0f);
+        if (classify) feat[(size_t) row_base + V] = make_float4(-1.0f, -1.0f, -1.0f, -1.0f);
     }
 }
 
