@@ -300,8 +300,18 @@ int vmhip_batch_profile_read(vmhip_batch* batch, int32_t max_slots, int32_t* n_s
  *   VMHIP_DEBUG_EDGE_BAND         width in pixels of the band along the screen edges inside which nodes are re-decided
  *                                 on the host (read when a batch is staged; <= 0 restores the default, 1/64)
  *   VMHIP_DEBUG_WIDE_OFFSETS      non-zero: the neighbourhood kernel addresses its tables with 64-bit offsets, as it does by
- *                                 itself for a batch with a table of 4 GiB or more (read when a batch is staged; 0 = off) */
-enum { VMHIP_DEBUG_FLOW_POLL_LIMIT = 0, VMHIP_DEBUG_PROJECTION_ERROR = 1, VMHIP_DEBUG_EDGE_BAND = 2, VMHIP_DEBUG_WIDE_OFFSETS = 3 };
+ *                                 itself for a batch with a table of 4 GiB or more (read when a batch is staged; 0 = off)
+ *   VMHIP_DEBUG_STAMP_ROW_BITS    24..31: the entries of the reverse lookup keep at least that many bits for the row, as
+ *                                 they do by themselves for a frame of 2^24 candidates or more, and so fewer for the run
+ *                                 stamp: the table is then cleared every 2^(32 - bits) - 1 runs (read when a batch is
+ *                                 staged; 0 = off) */
+enum {
+    VMHIP_DEBUG_FLOW_POLL_LIMIT = 0,
+    VMHIP_DEBUG_PROJECTION_ERROR = 1,
+    VMHIP_DEBUG_EDGE_BAND = 2,
+    VMHIP_DEBUG_WIDE_OFFSETS = 3,
+    VMHIP_DEBUG_STAMP_ROW_BITS = 4
+};
 int vmhip_debug_set(int32_t what, double value);
 /* What the edge guard did in the runs of a batch since it was staged: near-edge nodes the device listed (summed over
  * frames and passes), the most it listed for one frame in one pass, device decisions the host overruled, passes

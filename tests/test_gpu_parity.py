@@ -96,10 +96,22 @@ def test_device_libm_matches_host(oracle):
         assert bad.size == 0, "%s: %d of %d differ, e.g. x=%r device=%r host=%r" % (name, bad.size, x.size, x[bad[0]], y[bad[0]], want[bad[0]])
 
 
-def test_reverse_lookup_across_a_restart_of_the_run_stamp(oracle):
+@pytest.mark.parametrize("row_bits,runs", [(0, 600), (30, 40), (31, 12)], ids=["8-bit stamp", "2-bit stamp", "1-bit stamp"])
+def test_reverse_lookup_across_a_restart_of_the_run_stamp(oracle, row_bits, runs):
     """A reverse-lookup entry holds an 8-bit run stamp above the row, and an engine's table is cleared when the stamps
-    start again after 255 runs. One view stamps its nodes, then another view runs 600 times on the same engine: no run
-    may take an entry of the first view (or of itself, 255 runs earlier) for current."""
+    start again after 255 runs. One view stamps its nodes, then two other views take turns 600 times on the same engine:
+    no run may take an entry of the first view (or of a run 255 runs earlier) for current. A frame of 2^24 candidates
+    or more leaves fewer bits for the stamp; the knob makes ordinary frames do so (stamps start again every 3 runs, and
+    every run)."""
+    lib = native.hip()
+    native.hip_check(lib.vmhip_debug_set(native.DEBUG_STAMP_ROW_BITS, row_bits))
+    try:
+        _stamp_restart(oracle, runs)
+    finally:
+        native.hip_check(lib.vmhip_debug_set(native.DEBUG_STAMP_ROW_BITS, 0))
+
+
+def _stamp_restart(oracle, runs):
     mesh = eng.Mesh(wl.RING6, wl.SPHERE, 0.0949, 1.0, 3.0, 8.0)
     lens = native.make_lens(320, 256, wl.RECTILINEAR, 180.0, math.pi / 2)
     first_view = wl.make_hoc(1.0, math.radians(50.0), math.radians(-4.0), math.radians(1.0))
@@ -115,7 +127,7 @@ def test_reverse_lookup_across_a_restart_of_the_run_stamp(oracle):
         o = o_mesh.project(Hoc, o_lens)
         assert 100 < len(o["gidx"]) and not set(o["gidx"]) >= set(a["gidx"])  # the first view has nodes of its own
         want.append(o)
-    for run in range(600):
+    for run in range(runs):
         got = engine.project(mesh, views[run & 1], lens)
         assert np.array_equal(got["gidx"], want[run & 1]["gidx"]), "run %d: visible nodes differ" % run
         assert np.array_equal(got["nb"], want[run & 1]["nb"]), "run %d: neighbourhood differs" % run

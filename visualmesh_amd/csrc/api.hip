@@ -21,6 +21,7 @@ thread_local std::string g_error;
 /* test knobs (vmhip_debug_set); read when a batch is staged */
 std::atomic<float> g_debug_px_error{0.0f};
 std::atomic<bool> g_debug_wide_offsets{false};
+std::atomic<int> g_debug_stamp_row_bits{0};
 std::atomic<float> g_debug_edge_band{VMHIP_AMB_EPS_DEFAULT};
 
 int fail(int code, const std::string& msg) {
@@ -344,7 +345,7 @@ int batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int
     }
     /* a reverse-lookup entry: the run's stamp above the node's row. 24 bits of row serve every frame below 2^24
      * candidates and leave 255 runs between two clears of the table; a larger frame takes the bits it needs from the stamp */
-    int row_bits = 24;
+    int row_bits = std::min(std::max(24, g_debug_stamp_row_bits.load()), 31);
     while (row_bits < 31 && (max_cand >> row_bits) != 0) ++row_bits;
     if (b->d_lookup.grew || row_bits != b->stamp_row_bits) {
         /* a fresh table, or one whose entries were split differently, holds no valid stamp: zero everywhere, and the
@@ -1432,6 +1433,7 @@ int vmhip_debug_set(int32_t what, double value) {
         }
         case VMHIP_DEBUG_PROJECTION_ERROR: g_debug_px_error.store(float(value)); return VMHIP_OK;
         case VMHIP_DEBUG_WIDE_OFFSETS: g_debug_wide_offsets.store(value != 0.0); return VMHIP_OK;
+        case VMHIP_DEBUG_STAMP_ROW_BITS: g_debug_stamp_row_bits.store(int(value)); return VMHIP_OK;
         case VMHIP_DEBUG_EDGE_BAND: g_debug_edge_band.store(value <= 0.0 ? VMHIP_AMB_EPS_DEFAULT : float(value)); return VMHIP_OK;
         default: return fail(VMHIP_ERR_ARGUMENT, "debug_set: unknown knob");
     }
