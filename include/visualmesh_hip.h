@@ -280,9 +280,10 @@ int vmhip_batch_detect(vmhip_batch* batch, int32_t class_index, float threshold,
                        vmhip_detections* out);
 
 /* Per-kernel timing of vmhip_batch_run with HIP events on the stream the kernels run on.
- * enable = 1 brackets every kernel launch of later runs with events (an event pair between two
- * kernels costs a few microseconds of idle GPU); enable = 2, valid after a run made with enable = 1,
- * brackets only the launches of the kernel that took longest in that run; 0 switches timing off.
+ * enable = 1 brackets every kernel launch of later runs with events (such runs are launched kernel by kernel, and an
+ * event pair between two kernels costs a few microseconds of idle GPU); enable = 2, valid after a run made with
+ * enable = 1, brackets only the launches of the kernel that took longest in that run (such runs replay the batch's
+ * captured graph like untimed ones, with the event records as nodes of it); 0 switches timing off.
  * After a run, vmhip_batch_profile_read returns, for kernel slot i < *n_slots, its name (static string), the
  * duration in milliseconds of its launch in the last run and the rows (nodes incl. null rows) or
  * candidates it processed. Slots are in launch order (with enable = 2: the bracketed launches only). */

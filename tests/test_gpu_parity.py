@@ -476,6 +476,45 @@ def test_graph_replays_match_eager_runs(oracle, monkeypatch):
                     assert np.array_equal(got[i][key], want[i][key]), "run %d frame %d %s" % (replay, i, key)
 
 
+def test_graph_replays_with_event_records_match_eager_runs(oracle, monkeypatch):
+    """Timing mode 2 (events around the launches of the longest kernel only) keeps the pass in its captured graph: the
+    event records are nodes of it. Every replay must reproduce the eager results bit for bit, and every replay's
+    events must give a duration of that kernel that fits inside the pass's wall time."""
+    import time
+    cfg = wl.config(2, n_frames=3)
+    _, e_lens = lens_pair(cfg)
+    _, e_mesh = meshes_for(cfg, oracle)
+    frames = [dict(mesh=e_mesh, Hoc=f["Hoc"], lens=e_lens, image=f["image"], fourcc=cfg.fourcc) for f in cfg.frames]
+    monkeypatch.setenv("VMHIP_GRAPH", "0")
+    eager = eng.Engine(cfg.network, cfg.model)
+    want = eager.classify_batch(frames)
+    monkeypatch.setenv("VMHIP_GRAPH", "1")
+    timed = eng.Engine(cfg.network, cfg.model)
+    timed.stage(frames)
+    timed.profile(1)
+    timed.run()
+    every_kernel = timed.profile_read()
+    longest = max(set(name for name, ms, units in every_kernel), key=lambda k: sum(ms for name, ms, units in every_kernel if name == k))
+    timed.profile(2)
+    for replay in range(6):  # one run kernel by kernel, one that is captured, then replays
+        t0 = time.perf_counter()
+        timed.run()
+        wall_ms = (time.perf_counter() - t0) * 1e3
+        slots = timed.profile_read()
+        assert slots and all(name == longest for name, ms, units in slots)
+        assert all(ms > 0 for name, ms, units in slots) and sum(ms for name, ms, units in slots) < wall_ms
+        got = timed.fetch()
+        eager.run()  # unrelated eager work between the replays
+        for i in range(len(frames)):
+            for key in ("px", "gidx", "nb", "cls"):
+                assert np.array_equal(got[i][key], want[i][key]), "run %d frame %d %s" % (replay, i, key)
+    timed.profile(0)
+    timed.run()  # and back to the graph without events
+    got = timed.fetch()
+    for i in range(len(frames)):
+        assert np.array_equal(got[i]["cls"], want[i]["cls"])
+
+
 def _example_network():
     import json
     import os

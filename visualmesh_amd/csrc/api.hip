@@ -306,6 +306,9 @@ int batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int
     HIP_TRY(b->d_force_valid.reserve(8 * std::max<size_t>(words, 1)));
     HIP_TRY(b->d_force_keep.reserve(8 * std::max<size_t>(words, 1)));
     HIP_TRY(b->d_frame_V.reserve(8 * size_t(n_frames))); /* visible counts, then ambiguity counts */
+    /* a frame without candidates has no tile that would write its count; the ambiguity counters start from zero, and the
+     * last kernel of every pass leaves them so */
+    HIP_TRY(hipMemsetAsync(b->d_frame_V.p, 0, 8 * size_t(n_frames), E->stream));
     {
         const size_t need = 8 * size_t(n_frames) + sizeof(int2) * size_t(n_frames) * vmhip_batch::AMB_HEAD + 16;
         if (need > b->h_pin_cap) {
@@ -341,6 +344,7 @@ int batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int
     if (!b->d_epoch.p) {
         HIP_TRY(b->d_epoch.reserve(256));
         HIP_TRY(hipMemsetAsync(b->d_epoch.p, 0, 256, E->stream));
+        HIP_TRY(hipMemsetD32Async(reinterpret_cast<hipDeviceptr_t>(b->d_epoch.p), 1, 1, E->stream));
         b->epoch = 0;
     }
     /* a reverse-lookup entry: the run's stamp above the node's row. 24 bits of row serve every frame below 2^24
@@ -351,7 +355,7 @@ int batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int
         /* a fresh table, or one whose entries were split differently, holds no valid stamp: zero everywhere, and the
          * runs count from one again */
         HIP_TRY(hipMemsetAsync(b->d_lookup.p, 0, b->d_lookup.cap, E->stream));
-        HIP_TRY(hipMemsetAsync(b->d_epoch.p, 0, 4, E->stream));
+        HIP_TRY(hipMemsetD32Async(reinterpret_cast<hipDeviceptr_t>(b->d_epoch.p), 1, 1, E->stream));
         b->epoch = 0;
         b->stamp_row_bits = row_bits;
     }
@@ -505,7 +509,6 @@ int batch_enqueue(vmhip_batch* b) {
     for (const HostFrame& hf : b->frames) cands += hf.dev.n_cand;
     rows = cands + int64_t(b->frames.size());
 
-    vm_launch_reset(D, s);
     HIP_TRY(P.begin());
     vm_launch_project(D, s);
     HIP_TRY(P.end("project", cands));
@@ -565,7 +568,7 @@ int batch_request_verdict(vmhip_batch* b) {
     /* the barrier-free convolution kernel bounds its waits; a wait that ran out (never in a correct run) means
      * the results of this run cannot be trusted */
     const unsigned int* d_timeouts = (E->use_flow && b->classify) ? b->dev.flow_timeouts : nullptr;
-    vm_launch_publish(b->d_frame_V.as<int32_t>(), 2 * n, b->d_amb_list.as<int2>(), VMHIP_AMB_CAP, HEAD, n, d_timeouts, pin_counts, pin_amb, pin_timeouts, E->stream);
+    vm_launch_publish(b->d_frame_V.as<int32_t>(), 2 * n, b->d_amb_list.as<int2>(), VMHIP_AMB_CAP, HEAD, n, d_timeouts, b->dev.epoch, pin_counts, pin_amb, pin_timeouts, E->stream);
     HIP_TRY(hipGetLastError());
     return VMHIP_OK;
 }
@@ -642,12 +645,13 @@ int batch_launch(vmhip_batch* b) {
     vmhip_engine* E = b->engine;
     if (b->epoch >= (0xffffffffu >> b->stamp_row_bits)) { /* the stamp has used all its bits: old stamps could look current again */
         HIP_TRY(hipMemsetAsync(b->d_lookup.p, 0, b->d_lookup.cap, E->stream));
-        HIP_TRY(hipMemsetAsync(b->d_epoch.p, 0, 4, E->stream));
+        HIP_TRY(hipMemsetD32Async(reinterpret_cast<hipDeviceptr_t>(b->d_epoch.p), 1, 1, E->stream));
         b->epoch = 0;
     }
-    ++b->epoch; /* the reset kernel does the same on the device */
+    ++b->epoch; /* the stamp this pass runs with: the device word holds the same (the last kernel of a pass advances it) */
     int rc = VMHIP_OK;
-    if (E->use_graph && !b->profile && b->eager_runs >= 1) {
+    /* profile mode 2 (events around the launches of one kernel only) is captured too: its event records become nodes of the graph */
+    if (E->use_graph && b->profile != 1 && b->eager_runs >= 1) {
         if (!b->graph_exec) {
             /* Capture the kernel sequence (kernels only: the clears are a kernel too, no memset nodes). The
              * first run after staging was eager, so every kernel's one-time attribute set-up is done. */
@@ -1403,6 +1407,7 @@ int vmhip_batch_profile(vmhip_batch* b, int32_t enable) {
         b->slot_wanted.assign(b->n_slots, 0);
         for (int i = 0; i < b->n_slots; ++i) b->slot_wanted[i] = longest == b->slot_names[i];
     }
+    if (b->profile != enable) b->drop_graph(); /* a captured run holds the event records of its mode, or none */
     b->profile = enable;
     return VMHIP_OK;
 }

@@ -9,13 +9,14 @@
  * node within 1/64 px of a screen edge is re-decided on the host, so the visible set cannot diverge.
  *
  * Kernels (one launch each per batch, grids over all frames of the batch):
- *   vm_reset_kernel          clears the per-frame ambiguity counters, advances the run stamp
  *   vm_project_kernel        candidate space: global index from the range table, pixel coordinate, keep
  *                            decision, per-wave keep mask (ballot), per-tile kept count, ambiguity list
  *   vm_compact_kernel        candidate space: exclusive prefix over tile counts + wave popcount prefix ->
  *                            ascending local row; writes pixel, global index, reverse lookup stamp and the
  *                            sampled 4-channel input row; the frame's last tile writes V and the null row
  *   vm_neighbourhood_kernel  row space: neighbour table through the stamped reverse lookup
+ *   vm_publish_kernel        (after the network) counts and ambiguity lists into page-locked host memory; clears the
+ *                            ambiguity counters and advances the run stamp for the next pass
  */
 #include "vmhip_internal.h"
 
@@ -180,27 +181,27 @@ __global__ __launch_bounds__(256) void vm_stream_probe_kernel(const uint4* __res
     }
 }
 
-/* What the host needs of a pass, written by the device straight into page-locked host memory (block f: the head of frame
- * f's ambiguity list; block 0 also the counts and the convolution kernel's count of waits that ran out). A copy engine is
- * not involved, so the few hundred bytes never queue behind another engine's 50 MB download. */
-__global__ __launch_bounds__(64) void vm_publish_kernel(const int32_t* __restrict__ counts, int n_counts, const int2* __restrict__ amb_list, int amb_stride,
-                                                        int amb_head, const unsigned int* __restrict__ timeouts, int32_t* host_counts, int2* host_amb,
-                                                        uint32_t* host_timeouts) {
+/* Last kernel of a pass. What the host needs of the pass is written by the device straight into page-locked host memory
+ * (block f: the head of frame f's ambiguity list; block 0 also the counts and the convolution kernel's count of waits that
+ * ran out). A copy engine is not involved, so the few hundred bytes never queue behind another engine's 50 MB download.
+ * Block 0 then prepares the next pass: the ambiguity counters (the second half of the counts) start from zero again,
+ * and the run stamp advances, so that the stamps of this pass stop matching. (As a kernel of its own at the head of a pass
+ * this cost 16 us: the pass's second kernel waited for the host to finish queueing it.) */
+__global__ __launch_bounds__(64) void vm_publish_kernel(int32_t* __restrict__ counts, int n_counts, const int2* __restrict__ amb_list, int amb_stride,
+                                                        int amb_head, const unsigned int* __restrict__ timeouts, uint32_t* __restrict__ epoch,
+                                                        int32_t* host_counts, int2* host_amb, uint32_t* host_timeouts) {
     const int f = blockIdx.x;
     for (int t = threadIdx.x; t < amb_head; t += 64) host_amb[(size_t) f * amb_head + t] = amb_list[(size_t) f * amb_stride + t];
     if (f == 0) {
-        for (int t = threadIdx.x; t < n_counts; t += 64) host_counts[t] = counts[t];
-        if (threadIdx.x == 0) *host_timeouts = timeouts ? *timeouts : 0u;
+        for (int t = threadIdx.x; t < n_counts; t += 64) {
+            host_counts[t] = counts[t];
+            if (t >= n_counts / 2) counts[t] = 0;
+        }
+        if (threadIdx.x == 0) {
+            *host_timeouts = timeouts ? *timeouts : 0u;
+            *epoch += 1;
+        }
     }
-}
-
-__global__ void vm_reset_kernel(VmBatchDev B) {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < B.n_frames) {
-        B.amb_count[i] = 0;
-        B.frame_V[i] = 0; /* a frame without candidates has no tile that would write its count */
-    }
-    if (i == 0) *B.epoch += 1; /* a new run: stamps of earlier runs stop matching */
 }
 
 /* ---- lookup on the device: the host's walk of the cone tree (cpp/visualmesh/detail/cone_tree.hpp, itself after the
@@ -882,13 +883,10 @@ void vm_launch_stream_probe(const void* src, void* dst, size_t rows, int read_by
     hipLaunchKernelGGL(vm_stream_probe_kernel, dim3(256 * 16), dim3(256), 0, stream, reinterpret_cast<const uint4*>(src), reinterpret_cast<uint4*>(dst),
                        rows / 64, read_bytes_per_row * 4, write_bytes_per_row * 4);
 }
-void vm_launch_publish(const int32_t* counts, int n_counts, const int2* amb_list, int amb_stride, int amb_head, int n_frames, const unsigned int* timeouts,
+void vm_launch_publish(int32_t* counts, int n_counts, const int2* amb_list, int amb_stride, int amb_head, int n_frames, const unsigned int* timeouts, uint32_t* epoch,
                        int32_t* host_counts, int2* host_amb, uint32_t* host_timeouts, hipStream_t stream) {
-    hipLaunchKernelGGL(vm_publish_kernel, dim3(n_frames > 0 ? n_frames : 1), dim3(64), 0, stream, counts, n_counts, amb_list, amb_stride, amb_head, timeouts, host_counts,
-                       host_amb, host_timeouts);
-}
-void vm_launch_reset(const VmBatchDev& B, hipStream_t stream) {
-    hipLaunchKernelGGL(vm_reset_kernel, dim3((B.n_frames + 63) / 64), dim3(64), 0, stream, B);
+    hipLaunchKernelGGL(vm_publish_kernel, dim3(n_frames > 0 ? n_frames : 1), dim3(64), 0, stream, counts, n_counts, amb_list, amb_stride, amb_head, timeouts, epoch,
+                       host_counts, host_amb, host_timeouts);
 }
 void vm_launch_project(const VmBatchDev& B, hipStream_t stream) {
     if (B.n_cand_tiles > 0) hipLaunchKernelGGL(vm_project_kernel, dim3(B.n_cand_tiles), dim3(VMHIP_TILE), 0, stream, B);

@@ -92,7 +92,7 @@ struct VmBatchDev {
     const VmFrame* frames;
     int32_t n_frames;
     int32_t n_cand_tiles, n_row_tiles;
-    uint32_t* epoch;      /* device word: the run's stamp for the reverse lookup; the reset kernel increments it */
+    uint32_t* epoch;      /* device word: the run's stamp for the reverse lookup, from 1; the last kernel of a pass increments it */
     /* where a tile belongs, worked out when the batch is staged so that no block has to search for it (null: the blocks search) */
     const int2* cand_tile_info;     /* [n_cand_tiles] {frame, index of the range that holds the tile's first candidate} */
     const int32_t* row_tile_frame;  /* [n_row_tiles] frame */
@@ -216,10 +216,9 @@ void vm_launch_libm(int which, const float* x, float* y, int n, hipStream_t stre
 void vm_launch_copy_probe(const void* src, void* dst, size_t bytes, hipStream_t stream);
 /* rows: a multiple of 64; bytes per row: multiples of 4 (64 rows are whole 16-byte pieces then) */
 void vm_launch_stream_probe(const void* src, void* dst, size_t rows, int read_bytes_per_row, int write_bytes_per_row, hipStream_t stream);
-void vm_launch_reset(const VmBatchDev& B, hipStream_t stream);
 /* counts[n_counts], the first amb_head entries of every frame's ambiguity list and the timeout count, stored by the device
  * into page-locked host memory (device-visible pointers) */
-void vm_launch_publish(const int32_t* counts, int n_counts, const int2* amb_list, int amb_stride, int amb_head, int n_frames, const unsigned int* timeouts,
+void vm_launch_publish(int32_t* counts, int n_counts, const int2* amb_list, int amb_stride, int amb_head, int n_frames, const unsigned int* timeouts, uint32_t* epoch,
                        int32_t* host_counts, int2* host_amb, uint32_t* host_timeouts, hipStream_t stream);
 void vm_launch_project(const VmBatchDev& B, hipStream_t stream);
 void vm_launch_compact(const VmBatchDev& B, float* feat, int classify, hipStream_t stream);
