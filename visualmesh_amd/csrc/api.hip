@@ -140,6 +140,7 @@ struct vmhip_batch {
      * every frame's ambiguity list, so that one wait per run covers everything the host normally needs */
     static constexpr int AMB_HEAD = 64;
     void* h_pin = nullptr;
+    void* h_pin_dev = nullptr; /* the same memory as the device addresses it */
     size_t h_pin_cap = 0;
     std::vector<uint64_t> h_force_valid, h_force_keep;
     /* pinned home of the frame descriptions and range tables a stage uploads: they must outlive a stage that does not
@@ -316,6 +317,7 @@ int batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int
             b->h_pin = nullptr, b->h_pin_cap = 0;
             HIP_TRY(hipHostMalloc(&b->h_pin, need, hipHostMallocDefault));
             b->h_pin_cap = need;
+            HIP_TRY(hipHostGetDevicePointer(&b->h_pin_dev, b->h_pin, 0));
         }
     }
     HIP_TRY(b->d_amb_list.reserve(sizeof(int2) * size_t(n_frames) * VMHIP_AMB_CAP));
@@ -560,9 +562,7 @@ int batch_request_verdict(vmhip_batch* b) {
     constexpr int HEAD = vmhip_batch::AMB_HEAD;
     /* a kernel stores them into the page-locked landing area: small copies would wait in the copy engine's queue behind
      * whatever another engine is downloading */
-    void* dev_view = nullptr;
-    HIP_TRY(hipHostGetDevicePointer(&dev_view, b->h_pin, 0));
-    int32_t* pin_counts = reinterpret_cast<int32_t*>(dev_view);
+    int32_t* pin_counts = reinterpret_cast<int32_t*>(b->h_pin_dev);
     int2* pin_amb = reinterpret_cast<int2*>(pin_counts + 2 * n);
     uint32_t* pin_timeouts = reinterpret_cast<uint32_t*>(pin_amb + size_t(n) * HEAD);
     /* the barrier-free convolution kernel bounds its waits; a wait that ran out (never in a correct run) means
@@ -657,17 +657,17 @@ int batch_launch(vmhip_batch* b) {
              * first run after staging was eager, so every kernel's one-time attribute set-up is done. */
             HIP_TRY(hipStreamBeginCapture(E->stream, hipStreamCaptureModeThreadLocal));
             rc = batch_enqueue(b);
+            if (rc == VMHIP_OK) rc = batch_request_verdict(b); /* the pass's last kernel is part of the graph */
             hipError_t e = hipStreamEndCapture(E->stream, &b->graph);
             if (rc != VMHIP_OK) return rc;
             HIP_TRY(e);
             HIP_TRY(hipGraphInstantiate(&b->graph_exec, b->graph, nullptr, nullptr, 0));
         }
         HIP_TRY(hipGraphLaunch(b->graph_exec, E->stream));
+        return VMHIP_OK;
     }
-    else {
-        rc = batch_enqueue(b);
-        ++b->eager_runs;
-    }
+    rc = batch_enqueue(b);
+    ++b->eager_runs;
     if (rc != VMHIP_OK) return rc;
     return batch_request_verdict(b);
 }
