@@ -196,6 +196,8 @@ def measure(cfg, engine, frames, steps, warmup, settle_s, events=True, stream_ce
         kernel_ms_per_step[name] = kernel_ms_per_step.get(name, 0.0) + ms
         launches_per_step[name] = launches_per_step.get(name, 0) + 1
     engine.profile(2 if events else 0)
+    for _ in range(2):
+        engine.run()              # untimed: the first run after a change of timing mode goes kernel by kernel, the second is captured
     kernel_ms, kernel_launches = {}, {}
     t0 = time.perf_counter()
     for _ in range(steps):
@@ -441,6 +443,7 @@ def main():
             "visible_nodes_per_batch": nodes,
             "inputs": "resident in HBM before the timed region",
             "settle_passes": m["settle_passes"],   # untimed, before the warm-up passes: the clocks settle
+            "untimed_passes_after_warmup": 3,      # one with events around every kernel, two in which the timed passes' graph is captured
             "settle_ms": m["settle_ms"],
         },
         "roofline": m["roofline"],
