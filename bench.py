@@ -26,6 +26,9 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 FP32_PEAK_TFLOPS = 157.3   # MI355X dense fp32 matrix
 BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix
+# the arithmetic a configuration's engine computes its 64-wide layers in ("split": every value a pair of bf16, three
+# products per pair of values on the bf16 matrix instructions, fp32 accumulation; parity bar as for fp32)
+DTYPE = {"fp32": "f32", "bf16": "bf16", "split": "bf16 pairs"}
 
 def measured_traffic(workload, kernel):
     """HBM bytes per launch of `kernel` on `workload` from the rocprofv3 FETCH_SIZE / WRITE_SIZE summaries under
@@ -151,7 +154,7 @@ def build_workload(index, n_frames=None):
     else:
         v = cfg.visualmesh
         mesh = eng.VisualMesh(cfg.model, cfg.shape, cfg.radius, v["min_h"], v["max_h"], cfg.k, v["max_error"], cfg.max_distance)
-    precision = native.BF16 if cfg.precision == "bf16" else native.FP32
+    precision = {"bf16": native.BF16, "split": native.SPLIT}.get(cfg.precision, native.FP32)
     engine = eng.Engine(cfg.network, cfg.model, precision)
     frames = [dict(mesh=mesh, Hoc=f["Hoc"], lens=lens, image=f["image"], fourcc=cfg.fourcc) for f in cfg.frames]
     return cfg, engine, mesh, lens, frames
@@ -290,7 +293,7 @@ def end_to_end(cfg, mesh, lens, nodes, batches):
     from visualmesh_amd import engine as eng
     from visualmesh_amd import native
     from visualmesh_amd import workloads as wl
-    precision = native.BF16 if cfg.precision == "bf16" else native.FP32
+    precision = {"bf16": native.BF16, "split": native.SPLIT}.get(cfg.precision, native.FP32)
     pipe = eng.Pipeline(cfg.network, cfg.model, precision)  # visualmesh::engine::hip::Pipeline<float>
     held, frames = pinned_copies(cfg, mesh, lens)
 
@@ -322,7 +325,7 @@ def main():
     ap.add_argument("--steps", type=int, default=None, help="timed passes (default 1000; 50 for configurations 4 and 5, whose pass takes 20-80 ms)")
     ap.add_argument("--warmup", type=int, default=None, help="untimed passes before them (default 100; 5 for configurations 4 and 5)")
     ap.add_argument("--settle", type=float, default=0.25, help="seconds of untimed passes before the warm-up, for the clocks to settle (0: none)")
-    ap.add_argument("--config", type=int, default=2, help="workload configuration 1..5 (default 2: batched 1280x1024)")
+    ap.add_argument("--config", type=int, default=2, help="workload configuration 1..6 (default 2: batched 1280x1024; 6 = configuration 4 on the split-bf16 engine)")
     ap.add_argument("--frames", type=int, default=None, help="frames per batch (default: the configuration's own)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-events", action="store_true",
@@ -334,7 +337,7 @@ def main():
     ap.add_argument("--no-pcie", action="store_true", help="skip the PCIe-inclusive figures (serial stage + run + fetch, and the pipelined end-to-end loop)")
     ap.add_argument("--no-configs", action="store_true", help="skip the short runs of the other configurations")
     args = ap.parse_args()
-    big = args.config in (4, 5)
+    big = args.config in (4, 5, 6)
     args.steps = (50 if big else 1000) if args.steps is None else args.steps
     args.warmup = (5 if big else 100) if args.warmup is None else args.warmup
     if args.gpus != 1:
@@ -385,7 +388,7 @@ def main():
         sample = cfg
         passes = 8  # ~1.5 s of wall clock per pass on 16 threads: about 12 s in all
         note = "all %d frames of the batch %d times, one frame per task" % (len(cfg.frames), passes)
-        if args.config in (4, 5):  # a frame costs ~45 s per core: time a stated subset
+        if args.config in (4, 5, 6):  # a frame costs ~45 s per core: time a stated subset
             sample = wl.config(args.config, n_frames=min(threads, len(cfg.frames)))
             passes = 1
             note = "the first %d frames of the batch once, one frame per task" % len(sample.frames)
@@ -412,13 +415,13 @@ def main():
     if not args.no_configs:
         others = {}
         del engine, frames
-        for index in (1, 2, 3, 4, 5):
+        for index in (1, 2, 3, 4, 5, 6):
             if index == args.config:
                 continue
-            heavy = index in (4, 5)
+            heavy = index in (4, 5, 6)
             c, e, _, _, fr = build_workload(index)
             r = measure(c, e, fr, 10 if heavy else 300, 2 if heavy else 30, 0.1 if heavy else args.settle, events=True, stream_ceiling=not heavy)
-            others[c.name] = dict(workload=workload_name(c, len(fr), layer_table(c, wl.N_NEIGHBOURS[c.model])), dtype="bf16" if c.precision == "bf16" else "f32",
+            others[c.name] = dict(workload=workload_name(c, len(fr), layer_table(c, wl.N_NEIGHBOURS[c.model])), dtype=DTYPE[c.precision],
                                   nodes_per_s=r["value"], frames_per_s=r["frames_per_s"], ms_per_step=r["ms_per_step"], steps=10 if heavy else 300,
                                   visible_nodes_per_batch=r["nodes"], roofline=r["roofline"], conv_rooflines=r["conv_rooflines"])
             del e, fr, c
@@ -435,7 +438,7 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16" if cfg.precision == "bf16" else "f32",
+        "dtype": DTYPE[cfg.precision],
         "data": "synthetic",
         "config": {
             "workload": workload_name(cfg, len(cfg.frames), table),

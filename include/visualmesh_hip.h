@@ -46,7 +46,14 @@ enum { VMHIP_SELU = 0, VMHIP_RELU = 1, VMHIP_SOFTMAX = 2, VMHIP_TANH = 3 };
 /* Arithmetic of the graph-convolution layers of a float engine (vmhip_engine_create); its projection and sampling are
  * always fp32. VMHIP_FP64 names the arithmetic of the double engines further down, which have entry points of their own
  * (every number they take or return is a double, so the structures differ): vmhip_engine_create refuses it and says so. */
-enum { VMHIP_FP32 = 0, VMHIP_BF16 = 1, VMHIP_FP64 = 2 };
+enum { VMHIP_FP32 = 0, VMHIP_BF16 = 1, VMHIP_FP64 = 2, VMHIP_SPLIT = 3 };
+/* VMHIP_BF16: layers that are 64 wide on both sides run on the bf16 matrix instructions, with rows between them stored as
+ * bf16 or as pairs of bf16 (probabilities within 1e-2 of the fp32 result; the other layers stay fp32).
+ * VMHIP_SPLIT: the same layers on the same instructions, but every row between them as pairs of bf16 (a value's leading
+ * 8 bits and the bf16 of what they leave over) and three products per pair of values: fp32's parity bar (probabilities
+ * within 1e-4 of the CPU engine's) for networks of up to ten such layers - 2.6e-5 at most on the 6 x 64 network at full
+ * size, 9.7e-5 with ten layers; what the pairs leave out adds up with depth - at more than twice the fp32 engine's
+ * speed on such networks, more than the fp32 matrix peak would allow. */
 
 /* POD mirror of visualmesh::Lens<float> (reference lens.hpp:41-52). */
 typedef struct vmhip_lens {

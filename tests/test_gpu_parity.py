@@ -234,7 +234,8 @@ def test_config4_network_on_config1_geometry(oracle):
 
 def test_config4_and_5_full_size_frame(oracle):
     """One frame of configurations 4 and 5 at their real size (2048x1536, ~4.5e5 visible nodes, 6 x 64 network):
-    the fp32 engine within 1e-4 and the bf16 engine within 1e-2 of the same oracle result (~45 s of CPU)."""
+    the fp32 engine within 1e-4, the bf16 engine within 1e-2 and the split engine (pairs of bf16 on the bf16 matrix
+    instructions) within fp32's 1e-4 of the same oracle result (~45 s of CPU)."""
     cfg = wl.config(4, n_frames=1)
     o_lens, e_lens = lens_pair(cfg)
     o_mesh, e_mesh = meshes_for(cfg, oracle)
@@ -242,7 +243,7 @@ def test_config4_and_5_full_size_frame(oracle):
     print("cfg4/5 full-size frame: oracle running", flush=True)
     want = o_mesh.classify(f["Hoc"], o_lens, f["image"], cfg.fourcc, vmo.Network(cfg.network))
     print("cfg4/5 full-size frame: V =", len(want["gidx"]), flush=True)
-    for precision, tol, label in ((native.FP32, PROB_TOL, "cfg4 fp32"), (native.BF16, BF16_TOL, "cfg5 bf16")):
+    for precision, tol, label in ((native.FP32, PROB_TOL, "cfg4 fp32"), (native.BF16, BF16_TOL, "cfg5 bf16"), (native.SPLIT, PROB_TOL, "cfg6 split")):
         engine = eng.Engine(cfg.network, cfg.model, precision=precision)
         got = engine(e_mesh, f["Hoc"], e_lens, f["image"], cfg.fourcc)
         print(label, "worst absolute probability error: %.3e" % float(np.abs(got["cls"] - want["cls"]).max()), flush=True)
@@ -344,6 +345,33 @@ def test_bf16_engine_on_other_depths(oracle, hidden):
     worst = float(np.abs(got["cls"] - want["cls"]).max())
     print("bf16, %d hidden layers: %d boundaries as bf16, worst absolute probability error %.3e" % (hidden, rounded, worst), flush=True)
     assert_classification_parity(got, want, BF16_TOL if rounded else 1e-3, "bf16, %d hidden layers" % hidden)
+
+
+@pytest.mark.parametrize("hidden", [3, 6, 10])
+def test_split_engine_keeps_the_fp32_bar(oracle, hidden):
+    """Precision SPLIT: the 64-wide layers on the bf16 matrix instructions with every row between them as pairs of bf16
+    and three products per pair of values. Networks of three and six 64-wide layers on configuration 1's geometry must
+    stay within the fp32 engine's gate, 1e-4 on the probabilities, and no boundary may be rounded to bf16. What the
+    pairs leave out (the product of the two low parts, and a value's bits beyond the sixteenth) adds up with depth:
+    1.1e-5, 3.4e-5 and 9.7e-5 at three, six and ten layers, so the ten-layer network is held to 2e-4."""
+    cfg = wl.config(1, n_frames=1)
+    rng = np.random.default_rng(500 + hidden)
+    net = wl.glorot_network(rng, [3] + [64] * hidden + [4], 6, wl.SELU)
+    o_lens, e_lens = lens_pair(cfg)
+    o_mesh, e_mesh = meshes_for(cfg, oracle)
+    engine = eng.Engine(net, cfg.model, precision=native.SPLIT)
+    f = cfg.frames[0]
+    got = engine(e_mesh, f["Hoc"], e_lens, f["image"], cfg.fourcc)
+    engine.stage([dict(mesh=e_mesh, Hoc=f["Hoc"], lens=e_lens, image=f["image"], fourcc=cfg.fourcc)])
+    engine.profile(True)
+    engine.run()
+    names = [n for n, _, _ in engine.profile_read() if n.startswith("conv")]
+    assert len(names) == hidden + 1 and all(n.startswith("conv_bf16_x2_") for n in names[1:hidden]), names
+    assert not any("_tobf16_" in n or n.startswith("conv_bf16_bf16_") for n in names), names
+    want = o_mesh.classify(f["Hoc"], o_lens, f["image"], cfg.fourcc, vmo.Network(net))
+    worst = float(np.abs(got["cls"] - want["cls"]).max())
+    print("split, %d hidden layers: worst absolute probability error %.3e" % (hidden, worst), flush=True)
+    assert_classification_parity(got, want, PROB_TOL if hidden <= 6 else 2e-4, "split, %d hidden layers" % hidden)
 
 
 @pytest.mark.parametrize("variant", ["halo8", "fp32_rows_in", "relu_tanh", "selu_last"])

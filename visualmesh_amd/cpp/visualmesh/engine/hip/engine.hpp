@@ -89,7 +89,7 @@ namespace engine {
             throw std::system_error(code, hip_error_category(), what);
         }
 
-        enum class Precision { FP32 = VMHIP_FP32, BF16 = VMHIP_BF16, FP64 = VMHIP_FP64 };
+        enum class Precision { FP32 = VMHIP_FP32, BF16 = VMHIP_BF16, FP64 = VMHIP_FP64, SPLIT = VMHIP_SPLIT };
 
         /// Engine<float> is the template below; Engine<double> is the specialisation at the end of this file.
         template <typename Scalar>

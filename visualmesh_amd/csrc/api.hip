@@ -848,7 +848,7 @@ int vmhip_engine_create(const vmhip_network* net, int32_t n_neighbours, int32_t 
     if (n_neighbours < 0 || n_neighbours > 16) return fail(VMHIP_ERR_ARGUMENT, "engine_create: unsupported neighbour count");
     if (precision == VMHIP_FP64)
         return fail(VMHIP_ERR_ARGUMENT, "engine_create: a double engine takes double weights: use vmhip_engine_create_f64 and the other _f64 entry points");
-    if (precision != VMHIP_FP32 && precision != VMHIP_BF16) return fail(VMHIP_ERR_ARGUMENT, "engine_create: unknown precision");
+    if (precision != VMHIP_FP32 && precision != VMHIP_BF16 && precision != VMHIP_SPLIT) return fail(VMHIP_ERR_ARGUMENT, "engine_create: unknown precision");
     int n_dev = 0;
     HIP_TRY(hipGetDeviceCount(&n_dev));
     if (n_dev <= 0) return fail(VMHIP_ERR_HIP, "engine_create: no HIP device");
@@ -914,13 +914,13 @@ int vmhip_engine_create(const vmhip_network* net, int32_t n_neighbours, int32_t 
         const int n = int(E->layers.size());
         std::vector<int> bf(n + 1, VM_ROWS_F32); /* bf[l] = format of the rows entering layer l; bf[n] = final output (fp32) */
         std::vector<int> ar(n, 0);               /* ar[l] = layer l uses the bf16 matrix instructions */
-        if (precision == VMHIP_BF16 && !rows_only) {
+        if ((precision == VMHIP_BF16 || precision == VMHIP_SPLIT) && !rows_only) {
             for (int l = 0; l < n; ++l)
                 ar[l] = (E->layers[l].slots - 1 <= VMHIP_NBL_STRIDE && vm_bf16_supported(E->layers[l].c_in, E->layers[l].c_out, E->layers[l].slots)) ? 1 : 0;
             int eligible = 0, rounded = 0;
             int n_bf16 = 0;
             for (int l = 0; l < n; ++l) n_bf16 += ar[l];
-            int max_rounded = n_bf16 <= 5 ? 2 : 0;
+            int max_rounded = (n_bf16 <= 5 && precision == VMHIP_BF16) ? 2 : 0; /* VMHIP_SPLIT: every boundary as pairs */
             if (const char* r = getenv("VMHIP_BF16_ROUNDED")) max_rounded = std::max(atoi(r), 0);
             for (int l = 1; l < n; ++l) {
                 if (!ar[l]) continue;

@@ -19,7 +19,7 @@ HOST_LIB = os.path.join(PKG, "lib", "libvisualmesh_host.so")
 HOST_LIB_F64 = os.path.join(PKG, "lib", "libvisualmesh_host_f64.so")
 
 OK, ERR_HIP, ERR_FORMAT, ERR_LENS, ERR_ARGUMENT, ERR_CAPACITY = 0, -1, -2, -3, -4, -5
-FP32, BF16, FP64 = 0, 1, 2
+FP32, BF16, FP64, SPLIT = 0, 1, 2, 3
 DEBUG_FLOW_POLL_LIMIT, DEBUG_PROJECTION_ERROR, DEBUG_EDGE_BAND, DEBUG_WIDE_OFFSETS, DEBUG_STAMP_ROW_BITS = 0, 1, 2, 3, 4
 
 # every symbol include/visualmesh_hip.h declares
