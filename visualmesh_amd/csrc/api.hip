@@ -105,7 +105,7 @@ struct HostLayer {
     float* d_w_flow = nullptr; /* w_mfma in conv_flow.hip's LDS order */
     int32_t in_bf16 = 0, out_bf16 = 0, arith_bf16 = 0;
     bool use_lds = false, use_mfma = false, use_flow = false, use_narrow = false; /* which matrix-core kernels may take the layer */
-    std::vector<float> h_w; /* kept until the row types are planned */
+    std::vector<float> h_w, h_b; /* kept until the row types are planned */
 };
 
 struct vmhip_engine {
@@ -874,6 +874,7 @@ int vmhip_engine_create(const vmhip_network* net, int32_t n_neighbours, int32_t 
             HostLayer H;
             H.c_in = width, H.c_out = L.n_out, H.slots = slots, H.activation = L.activation;
             H.h_w.assign(L.weights, L.weights + size_t(L.n_in) * L.n_out);
+            H.h_b.assign(L.biases, L.biases + size_t(L.n_out));
             if (hipMalloc(&H.d_w, 4 * size_t(L.n_in) * L.n_out) != hipSuccess || hipMalloc(&H.d_b, 4 * size_t(L.n_out)) != hipSuccess)
                 return bail(VMHIP_ERR_HIP, "engine_create: out of device memory");
             E->layers.push_back(H);
@@ -964,6 +965,21 @@ int vmhip_engine_create(const vmhip_network* net, int32_t n_neighbours, int32_t 
                     return bail(VMHIP_ERR_HIP, "engine_create: weight upload failed");
             }
             else if (H.use_mfma || H.use_lds || H.use_flow) {
+                if (H.use_lds && H.out_bf16 == VM_ROWS_BF16X2) {
+                    /* The one kernel that writes hi + lo rows without reading them keeps a lane's output values next to
+                     * each other in the row: matrix column cb * 16 + q * 4 + v stands for channel q * 4 * CB + cb * 4 + v
+                     * (conv_lds.hip), so weights and biases go to the device with their columns in that order. No other
+                     * kernel can take this layer, so none sees the biases out of order. */
+                    const int c_out = H.c_out, column_blocks = c_out / 16;
+                    auto channel_of = [&](int column) { return ((column % 16) / 4) * (4 * column_blocks) + (column / 16) * 4 + column % 4; };
+                    std::vector<float> w(H.h_w.size()), bias(H.h_b.size());
+                    for (size_t k = 0; k < H.h_w.size() / size_t(c_out); ++k)
+                        for (int column = 0; column < c_out; ++column) w[k * c_out + column] = H.h_w[k * c_out + channel_of(column)];
+                    for (int column = 0; column < c_out; ++column) bias[column] = H.h_b[channel_of(column)];
+                    H.h_w.swap(w);
+                    if (hipMemcpy(H.d_b, bias.data(), 4 * bias.size(), hipMemcpyHostToDevice) != hipSuccess)
+                        return bail(VMHIP_ERR_HIP, "engine_create: weight upload failed");
+                }
                 std::vector<unsigned char> wp(vm_mfma_weight_bytes(H.c_in, H.c_out, H.slots));
                 vm_mfma_permute_weights(H.h_w.data(), H.c_in, H.c_out, H.slots, wp.data());
                 if (hipMalloc(&H.d_w_mfma, wp.size()) != hipSuccess) return bail(VMHIP_ERR_HIP, "engine_create: out of device memory");
@@ -979,6 +995,7 @@ int vmhip_engine_create(const vmhip_network* net, int32_t n_neighbours, int32_t 
             }
             H.h_w.clear();
             H.h_w.shrink_to_fit();
+            H.h_b.clear();
         }
     }
     if (hipStreamCreateWithFlags(&E->stream, hipStreamNonBlocking) != hipSuccess) return bail(VMHIP_ERR_HIP, "engine_create: stream creation failed");
