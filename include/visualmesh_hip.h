@@ -50,10 +50,13 @@ enum { VMHIP_FP32 = 0, VMHIP_BF16 = 1, VMHIP_FP64 = 2, VMHIP_SPLIT = 3 };
 /* VMHIP_BF16: layers that are 64 wide on both sides run on the bf16 matrix instructions, with rows between them stored as
  * bf16 or as pairs of bf16 (probabilities within 1e-2 of the fp32 result; the other layers stay fp32).
  * VMHIP_SPLIT: the same layers on the same instructions, but every row between them as pairs of bf16 (a value's leading
- * 8 bits and the bf16 of what they leave over) and three products per pair of values: fp32's parity bar (probabilities
- * within 1e-4 of the CPU engine's) for networks of up to ten such layers - 2.6e-5 at most on the 6 x 64 network at full
- * size, 9.7e-5 with ten layers; what the pairs leave out adds up with depth - at more than twice the fp32 engine's
- * speed on such networks, more than the fp32 matrix peak would allow. */
+ * 8 bits and the bf16 of what they leave over) and three products per pair of values. Probabilities stay within 1e-4
+ * of the CPU engine's (fp32's parity bar) for networks of up to six such layers - 2.6e-5 at most on the 6 x 64 network
+ * at full size, 3.4e-5 on other seeds - and within 2e-4 for up to ten (9.7e-5 measured on one seed: no margin against
+ * 1e-4); what the pairs leave out adds up with depth, so an engine with more than ten such layers is refused
+ * (VMHIP_ERR_ARGUMENT): use VMHIP_FP32 there. More than twice the fp32 engine's speed on such networks, more than the
+ * fp32 matrix peak would allow. The measurement overrides VMHIP_BF16_ROUNDED / VMHIP_BF16_ROUNDED_AT are ignored for
+ * this precision: its contract has no bf16-rounded row. */
 
 /* POD mirror of visualmesh::Lens<float> (reference lens.hpp:41-52). */
 typedef struct vmhip_lens {
@@ -209,6 +212,15 @@ int vmhip_batch_run(vmhip_batch* batch);
  * and detect need the wait; the batch must not be staged or run again before it. */
 int vmhip_batch_run_async(vmhip_batch* batch);
 int vmhip_batch_wait(vmhip_batch* batch);
+/* How the passes of a batch object were put on the stream since it was made: passes captured into a HIP graph
+ * (captures), passes launched as a replay of a captured graph (graph_launches, the capturing pass included) and passes
+ * launched kernel by kernel (eager_launches). A captured pass holds addresses, launch grids and the number of frames
+ * only - the tiles in use, the frame descriptions and the range and tile tables are read from device memory - so it
+ * outlives the batch it was captured with: staging other frames keeps it, and it is captured again only when a device
+ * buffer had to grow, a batch needs larger grids or has another number of frames, or the profiling mode changes. This
+ * is what the reference's OpenCL engine does with its kernels and grow-only buffers, re-issued per frame with new
+ * arguments (engine/opencl/engine.hpp:455-489, :740-835). Any pointer may be NULL. */
+int vmhip_batch_graph_stats(const vmhip_batch* batch, int64_t* captures, int64_t* graph_launches, int64_t* eager_launches);
 /* n_visible[n_frames] of the last run */
 int vmhip_batch_counts(const vmhip_batch* batch, int32_t* n_visible);
 int vmhip_batch_fetch(vmhip_batch* batch, vmhip_result* results);

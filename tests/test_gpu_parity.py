@@ -504,6 +504,79 @@ def test_graph_replays_match_eager_runs(oracle, monkeypatch):
                     assert np.array_equal(got[i][key], want[i][key]), "run %d frame %d %s" % (replay, i, key)
 
 
+def test_a_captured_pass_outlives_the_batch_it_was_captured_with(oracle, monkeypatch):
+    """Frame after frame through one engine, the way a camera loop or the pipeline drives it (stage, run once, fetch): the
+    first pass is launched kernel by kernel, the second is captured into a HIP graph, and every batch after that - other
+    images, other poses, other visible counts, as long as it fits the grids - is a launch of that same graph, its tiles
+    in use, frame descriptions and tables read from device memory. Every result is the oracle's. A batch with another
+    number of frames, or one that outgrows the grids, is captured again; the pipeline's three engines do the same."""
+    monkeypatch.setenv("VMHIP_GRAPH", "1")
+    cfg = wl.config(2, n_frames=8)
+    o_lens, e_lens = lens_pair(cfg)
+    o_mesh, e_mesh = meshes_for(cfg, oracle)
+    net = vmo.Network(cfg.network)
+    frames = [dict(mesh=e_mesh, Hoc=f["Hoc"], lens=e_lens, image=f["image"], fourcc=cfg.fourcc) for f in cfg.frames]
+    wants = [pick(o_mesh, f["Hoc"]).classify(f["Hoc"], o_lens, f["image"], cfg.fourcc, net) for f in cfg.frames]
+    # pairs of frames in decreasing order of their candidate counts: the first batch sizes the grids, the others fit
+    probe = eng.Engine(cfg.network, cfg.model)
+    probe.stage(frames)
+    size = [sum(b - a for a, b in probe.staged_ranges(i).reshape(-1, 2)) for i in range(len(frames))]
+    order = sorted(range(len(frames)), key=lambda i: -size[i])
+    batches = [[order[0], order[1]], [order[2], order[3]], [order[5], order[4]], [order[7], order[6]]]
+    engine = eng.Engine(cfg.network, cfg.model)
+    for k, b in enumerate(batches):
+        engine.stage([frames[i] for i in b])
+        engine.run()
+        got = engine.fetch()
+        for i, r in zip(b, got):
+            assert_classification_parity(r, wants[i], PROB_TOL, "batch %d frame %d" % (k, i))
+        stats = engine.graph_stats()
+        print("after batch %d: %s" % (k, stats), flush=True)
+    assert stats == dict(captures=1, graph_launches=3, eager_launches=1), stats
+    # the same frames again, the other way round in each batch: still the one graph
+    for b in batches:
+        engine.stage([frames[i] for i in b[::-1]])
+        engine.run()
+        for i, r in zip(b[::-1], engine.fetch()):
+            assert_classification_parity(r, wants[i], PROB_TOL, "second round frame %d" % i)
+    assert engine.graph_stats() == dict(captures=1, graph_launches=7, eager_launches=1), engine.graph_stats()
+    # three frames instead of two: another graph (one pass kernel by kernel, then the capture)
+    for _ in range(2):
+        engine.stage([frames[i] for i in order[:3]])
+        engine.run()
+        for i, r in zip(order[:3], engine.fetch()):
+            assert_classification_parity(r, wants[i], PROB_TOL, "three frames, frame %d" % i)
+    stats = engine.graph_stats()
+    assert stats["captures"] == 2 and stats["eager_launches"] == 2, stats
+
+    # the pipeline: three engines, each sees every third batch; each launches its first pass kernel by kernel, captures its
+    # second and replays from then on
+    images = []
+    for f in cfg.frames:
+        held = native.pinned_empty(f["image"].shape, f["image"].dtype)
+        held[...] = f["image"]
+        images.append(held)
+    pinned = [dict(mesh=e_mesh, Hoc=f["Hoc"], lens=e_lens, image=im, fourcc=cfg.fourcc) for f, im in zip(cfg.frames, images)]
+    pipe = eng.Pipeline(cfg.network, cfg.model)
+    sequence = [[order[0], order[1]]] * 3 + [[order[2], order[3]], [order[4], order[5]], [order[6], order[7]]] * 3
+    got = []
+    for b in sequence:
+        done = pipe.submit([pinned[i] for i in b])
+        if done is not None:
+            got.append([{k: v.copy() for k, v in r.items()} for r in done])
+    while True:
+        done = pipe.flush()
+        if done is None:
+            break
+        got.append([{k: v.copy() for k, v in r.items()} for r in done])
+    assert len(got) == len(sequence)
+    for b, results in zip(sequence, got):
+        for i, r in zip(b, results):
+            assert_classification_parity(r, wants[i], PROB_TOL, "pipeline frame %d" % i)
+    stats = pipe.graph_stats()
+    assert stats == dict(captures=3, graph_launches=len(sequence) - 3, eager_launches=3), stats
+
+
 def test_graph_replays_with_event_records_match_eager_runs(oracle, monkeypatch):
     """Timing mode 2 (events around the launches of the longest kernel only) keeps the pass in its captured graph: the
     event records are nodes of it. Every replay must reproduce the eager results bit for bit, and every replay's

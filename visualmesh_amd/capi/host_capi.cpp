@@ -487,5 +487,13 @@ int vmh_pipeline_result(vmh_pipeline* p, int i, real** px, int32_t** gidx, int32
     })
 }
 int vmh_pipeline_n_classes(vmh_pipeline* p) { return p->pipe->engine(0).n_classes(); }
+/* captures, graph launches and kernel-by-kernel launches of the pipeline's three engines together */
+int vmh_pipeline_graph_stats(vmh_pipeline* p, int64_t* captures, int64_t* graph_launches, int64_t* eager_launches) {
+    GUARD({
+        const auto s = p->pipe->graph_stats();
+        *captures = s.captures, *graph_launches = s.graph_launches, *eager_launches = s.eager_launches;
+        return 0;
+    })
+}
 #endif  // !VMH_DOUBLE
 }

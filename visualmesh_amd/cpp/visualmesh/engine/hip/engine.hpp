@@ -463,6 +463,17 @@ namespace engine {
             bool device_lookup() const { return device_lookup_; }
             /// The batch object behind stage/run/fetch, for profiling hooks.
             vmhip_batch* native_batch() const { return batch_; }
+            /// How this engine's passes reached the stream so far: captured into a HIP graph, launched as a replay of a
+            /// captured graph, launched kernel by kernel. A captured pass outlives the frames it was captured with
+            /// (vmhip_batch_graph_stats), so an engine that is handed frame after frame of similar size captures once.
+            struct GraphStats {
+                int64_t captures = 0, graph_launches = 0, eager_launches = 0;
+            };
+            GraphStats graph_stats() const {
+                GraphStats s;
+                if (batch_) throw_on_error(vmhip_batch_graph_stats(batch_, &s.captures, &s.graph_launches, &s.eager_launches));
+                return s;
+            }
             /// Width of the classification rows (known once the engine has been used; -1 before).
             int n_classes() const { return engine_ ? int(vmhip_engine_n_classes(engine_)) : -1; }
 
@@ -957,6 +968,15 @@ namespace engine {
             }
             /// The engines, e.g. to set a cache limit or the lookup on the device on all three.
             Engine<Scalar>& engine(int i) { return *slots_[i % 3].engine; }
+            /// Captures and launches of the three engines together (Engine::graph_stats).
+            typename Engine<Scalar>::GraphStats graph_stats() const {
+                typename Engine<Scalar>::GraphStats total;
+                for (const Slot& s : slots_) {
+                    const typename Engine<Scalar>::GraphStats one = s.engine->graph_stats();
+                    total.captures += one.captures, total.graph_launches += one.graph_launches, total.eager_launches += one.eager_launches;
+                }
+                return total;
+            }
 
         private:
             struct Slot {

@@ -161,16 +161,37 @@ struct vmhip_batch {
     int stamp_row_bits = 0; /* how the reverse-lookup entries of the table on the device are split (VmBatchDev::stamp_row_bits) */
     /* what the edge guard did since the batch was staged (vmhip_batch_guard_stats) */
     int64_t reruns = 0, overruled = 0, amb_seen = 0, amb_most = 0;
-    /* the kernel sequence of a run, captured once per staged batch and replayed (no profiling, VMHIP_GRAPH != 0) */
+    /* The kernel sequence of a pass, captured into a HIP graph and replayed (VMHIP_GRAPH != 0, no per-kernel profiling).
+     * What a captured pass holds is addresses, launch grids and the number of frames: the tiles in use, the frame
+     * descriptions and every table are read from device memory, so the graph serves every batch staged after the one it
+     * was captured with, until a buffer grows, a batch needs a larger grid or another number of frames, or the mode changes
+     * (graph_key says what the capture was made with; batch_launch compares). */
+    struct GraphKey {
+        VmBatchDev dev;
+        const void* act[2];
+        const void* pin;
+        int32_t classify, profile;
+    };
     hipGraph_t graph = nullptr;
     hipGraphExec_t graph_exec = nullptr;
-    int eager_runs = 0; /* runs since the last stage: the first one is launched eagerly, then captured */
+    GraphKey graph_key;
+    int eager_runs = 0; /* passes launched kernel by kernel since the batch was made or its graph dropped: the first pass is
+                         * launched that way (every kernel's one-time attribute set-up happens there), the second is captured */
+    int64_t graph_captures = 0, graph_launches = 0, eager_launches = 0; /* vmhip_batch_graph_stats */
     void drop_graph() {
         if (graph_exec) (void) hipGraphExecDestroy(graph_exec);
         if (graph) (void) hipGraphDestroy(graph);
         graph_exec = nullptr, graph = nullptr, eager_runs = 0;
     }
-    size_t cand_total = 0, row_total = 0, lookup_total = 0;
+    size_t cand_total = 0, row_total = 0, lookup_total = 0; /* slots the candidate and row spaces are allocated for */
+    size_t cap_cand_tiles = 0, cap_row_tiles = 0;           /* the tiles the launch grids are sized for (>= the tiles in use) */
+    VmBatchLive live{0, 0};                                  /* the tiles in use */
+    /* the batch as the kernels outside the captured pass see it: grids of exactly the tiles in use */
+    VmBatchDev dev_exact() const {
+        VmBatchDev d = dev;
+        d.n_cand_tiles = live.n_cand_tiles, d.n_row_tiles = live.n_row_tiles;
+        return d;
+    }
 
     VmBatchDev dev{};
     DevBuf d_frames, d_ranges, d_images, d_cand_px, d_cand_g, d_cand_keep, d_tile_count, d_force_valid, d_force_keep, d_frame_V,
@@ -290,15 +311,35 @@ int batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int
         nb_stride = std::max(nb_stride, in.mesh->nn);
         uniform_nn = (f == 0 || uniform_nn == in.mesh->nn) ? in.mesh->nn : 0;
     }
+    /* Launch grids and table offsets are sized for at least the tiles in use. An engine that replays captured passes
+     * keeps them when a later batch fits (a batch that does not gets an eighth of slack, so that a stream of frames
+     * settles after a few batches); kernel-by-kernel launches take exactly the tiles in use. */
+    auto grown = [&](size_t have, size_t need) {
+        if (!E->use_graph) return need;
+        if (need <= have) return have;
+        return have == 0 ? need : (need + need / 8 + 7) / 8 * 8;
+    };
+    b->cap_cand_tiles = std::min<size_t>(grown(b->cap_cand_tiles, cand_tiles), 0x7fffff);
+    b->cap_row_tiles = std::min<size_t>(grown(b->cap_row_tiles, row_tiles), 0x7fffff);
+    b->live.n_cand_tiles = int32_t(cand_tiles), b->live.n_row_tiles = int32_t(row_tiles);
+    cand_tiles = b->cap_cand_tiles, row_tiles = b->cap_row_tiles; /* from here on: what is allocated and launched */
     b->cand_total = cand_tiles * VMHIP_TILE;
     b->row_total = row_tiles * VMHIP_TILE;
     const size_t words = b->cand_total / 64;
+    if (classify && E->use_bf16 && max_cand + 1 >= (size_t(1) << 24))
+        return fail(VMHIP_ERR_CAPACITY, "stage: a frame of 2^24 rows or more is too large for the bf16 layers (32-bit byte offsets into a frame's rows)");
 
     /* device workspace */
-    HIP_TRY(b->d_frames.reserve(sizeof(VmFrame) * n_frames));
-    /* the range tables, then the tile tables: {frame, first range} per candidate tile (on an 8-byte boundary), frame per row tile */
-    const size_t tile_table_at = align_up(std::max<size_t>(range_ints, 1), 2), n_table_ints = tile_table_at + 2 * cand_tiles + row_tiles;
-    HIP_TRY(b->d_ranges.reserve(sizeof(int32_t) * n_table_ints));
+    /* the tiles in use, then the frame descriptions */
+    constexpr size_t LIVE_BYTES = 64;
+    static_assert(sizeof(VmBatchLive) <= LIVE_BYTES, "the frame descriptions follow the live counts");
+    HIP_TRY(b->d_frames.reserve(LIVE_BYTES + sizeof(VmFrame) * n_frames));
+    /* the tile tables ({frame, first range} per candidate tile, frame per row tile: at offsets that depend on the grid
+     * sizes only), then the range tables */
+    const size_t ranges_at = align_up(2 * cand_tiles + row_tiles, 2), n_table_ints = ranges_at + std::max<size_t>(range_ints, 1);
+    /* the number of ranges varies from frame to frame with nothing to bound it: room for twice as many, so that the
+     * tables rarely move (their address is part of a captured pass) */
+    HIP_TRY(b->d_ranges.reserve(sizeof(int32_t) * (n_table_ints + (E->use_graph ? range_ints + 1024 : 0))));
     HIP_TRY(b->d_images.reserve(std::max<size_t>(image_bytes, 256)));
     HIP_TRY(b->d_cand_px.reserve(sizeof(float2) * std::max<size_t>(b->cand_total, 1)));
     HIP_TRY(b->d_cand_g.reserve(4 * std::max<size_t>(b->cand_total, 1)));
@@ -361,11 +402,10 @@ int batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int
         b->epoch = 0;
         b->stamp_row_bits = row_bits;
     }
-    b->drop_graph(); /* pointers and sizes baked into a captured run are no longer valid */
 
     /* fill in device pointers and upload */
     {
-        const size_t need = align_up(sizeof(VmFrame) * size_t(n_frames), 64) + 4 * n_table_ints;
+        const size_t need = LIVE_BYTES + align_up(sizeof(VmFrame) * size_t(n_frames), 64) + 4 * n_table_ints;
         if (need > b->h_stage_cap) {
             if (b->h_stage) HIP_TRY(hipHostFree(b->h_stage));
             b->h_stage = nullptr, b->h_stage_cap = 0;
@@ -373,9 +413,10 @@ int batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int
             b->h_stage_cap = need + need / 4;
         }
     }
-    VmFrame* h_frames = static_cast<VmFrame*>(b->h_stage);
-    int32_t* h_ranges = reinterpret_cast<int32_t*>(static_cast<char*>(b->h_stage) + align_up(sizeof(VmFrame) * size_t(n_frames), 64));
-    size_t range_off = 0, image_off = 0, lookup_off = 0;
+    *static_cast<VmBatchLive*>(b->h_stage) = b->live;
+    VmFrame* h_frames = reinterpret_cast<VmFrame*>(static_cast<char*>(b->h_stage) + LIVE_BYTES);
+    int32_t* h_ranges = reinterpret_cast<int32_t*>(static_cast<char*>(b->h_stage) + LIVE_BYTES + align_up(sizeof(VmFrame) * size_t(n_frames), 64));
+    size_t range_off = ranges_at, image_off = 0, lookup_off = 0;
     const uint8_t* run_src = nullptr; /* the run of adjoining images not yet copied */
     size_t run_dst = 0, run_bytes = 0;
     for (int f = 0; f < n_frames; ++f) {
@@ -411,17 +452,17 @@ int batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int
         d.force_keep = b->d_force_keep.as<uint64_t>();
         h_frames[f] = d;
         /* the tiles of this frame: a candidate tile's first candidate lies in range r, prefix[r] <= first < prefix[r + 1] */
-        int32_t* const cand_info = h_ranges + tile_table_at + 2 * size_t(d.cand_tile0);
+        int32_t* const cand_info = h_ranges + 2 * size_t(d.cand_tile0);
         int r = 0;
         for (int t = 0; t < d.cand_tiles; ++t) {
             while (r + 1 < R && hf.prefix[size_t(r) + 1] <= int64_t(t) * VMHIP_TILE) ++r;
             cand_info[2 * t] = f;
             cand_info[2 * t + 1] = r;
         }
-        std::fill_n(h_ranges + tile_table_at + 2 * cand_tiles + size_t(d.row_tile0), size_t(d.row_tiles), f);
+        std::fill_n(h_ranges + 2 * cand_tiles + size_t(d.row_tile0), size_t(d.row_tiles), f);
     }
     if (run_bytes > 0) HIP_TRY(hipMemcpyAsync(b->d_images.as<uint8_t>() + run_dst, run_src, run_bytes, hipMemcpyHostToDevice, E->stream));
-    HIP_TRY(hipMemcpyAsync(b->d_frames.p, h_frames, sizeof(VmFrame) * n_frames, hipMemcpyHostToDevice, E->stream));
+    HIP_TRY(hipMemcpyAsync(b->d_frames.p, b->h_stage, LIVE_BYTES + sizeof(VmFrame) * n_frames, hipMemcpyHostToDevice, E->stream));
     HIP_TRY(hipMemcpyAsync(b->d_ranges.p, h_ranges, sizeof(int32_t) * n_table_ints, hipMemcpyHostToDevice, E->stream));
     HIP_TRY(hipMemsetAsync(b->d_force_valid.p, 0, 8 * std::max<size_t>(words, 1), E->stream));
     HIP_TRY(hipMemsetAsync(b->d_force_keep.p, 0, 8 * std::max<size_t>(words, 1), E->stream));
@@ -434,7 +475,9 @@ int batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int
     b->stage_pending = !wait;
 
     VmBatchDev& D = b->dev;
-    D.frames = b->d_frames.as<VmFrame>();
+    std::memset(&D, 0, sizeof(D)); /* padding too: a captured pass is matched against this struct byte by byte */
+    D.live = b->d_frames.as<VmBatchLive>();
+    D.frames = reinterpret_cast<const VmFrame*>(b->d_frames.as<char>() + LIVE_BYTES);
     D.n_frames = n_frames;
     D.n_cand_tiles = int32_t(cand_tiles);
     D.n_row_tiles = int32_t(row_tiles);
@@ -459,8 +502,8 @@ int batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int
     D.epoch = b->d_epoch.as<uint32_t>();
     D.stamp_row_bits = b->stamp_row_bits;
     D.uniform_nn = uniform_nn;
-    D.cand_tile_info = reinterpret_cast<const int2*>(b->d_ranges.as<int32_t>() + tile_table_at);
-    D.row_tile_frame = b->d_ranges.as<int32_t>() + tile_table_at + 2 * cand_tiles;
+    D.cand_tile_info = reinterpret_cast<const int2*>(b->d_ranges.as<int32_t>());
+    D.row_tile_frame = b->d_ranges.as<int32_t>() + 2 * cand_tiles;
     /* 32-bit byte offsets into a frame's part of every table the neighbourhood kernel touches (4-byte entries of the
      * mesh's neighbour table and of the output table, 16-byte rows of the tile-local table), unless one is too large */
     D.wide_offsets = (widest_mesh >= (1ull << 30) || (uint64_t(max_cand) + 1) * uint64_t(std::max(nb_stride, 4)) >= (1ull << 30) || g_debug_wide_offsets.load()) ? 1 : 0;
@@ -648,28 +691,54 @@ int batch_launch(vmhip_batch* b) {
         HIP_TRY(hipMemsetD32Async(reinterpret_cast<hipDeviceptr_t>(b->d_epoch.p), 1, 1, E->stream));
         b->epoch = 0;
     }
-    ++b->epoch; /* the stamp this pass runs with: the device word holds the same (the last kernel of a pass advances it) */
+    /* The pass runs with stamp epoch + 1, which is what the device word holds: the last kernel of a pass advances the
+     * word, so the host's mirror advances once that kernel has been queued. */
     int rc = VMHIP_OK;
     /* profile mode 2 (events around the launches of one kernel only) is captured too: its event records become nodes of the graph */
-    if (E->use_graph && b->profile != 1 && b->eager_runs >= 1) {
-        if (!b->graph_exec) {
-            /* Capture the kernel sequence (kernels only: the clears are a kernel too, no memset nodes). The
-             * first run after staging was eager, so every kernel's one-time attribute set-up is done. */
-            HIP_TRY(hipStreamBeginCapture(E->stream, hipStreamCaptureModeThreadLocal));
-            rc = batch_enqueue(b);
-            if (rc == VMHIP_OK) rc = batch_request_verdict(b); /* the pass's last kernel is part of the graph */
-            hipError_t e = hipStreamEndCapture(E->stream, &b->graph);
-            if (rc != VMHIP_OK) return rc;
-            HIP_TRY(e);
-            HIP_TRY(hipGraphInstantiate(&b->graph_exec, b->graph, nullptr, nullptr, 0));
+    if (E->use_graph && b->profile != 1) {
+        vmhip_batch::GraphKey key;
+        std::memset(&key, 0, sizeof(key));
+        std::memcpy(&key.dev, &b->dev, sizeof(VmBatchDev));
+        key.act[0] = b->d_act[0].p, key.act[1] = b->d_act[1].p;
+        key.pin = b->h_pin_dev;
+        key.classify = b->classify, key.profile = b->profile;
+        if (b->graph_exec && std::memcmp(&key, &b->graph_key, sizeof(key)) != 0) b->drop_graph(); /* an address, a grid or the mode has changed */
+        if (b->graph_exec || b->eager_runs >= 1) {
+            if (!b->graph_exec) {
+                /* Capture the kernel sequence (kernels only: the clears are a kernel too, no memset nodes). A pass has been
+                 * launched kernel by kernel before, so every kernel's one-time attribute set-up is done. */
+                HIP_TRY(hipStreamBeginCapture(E->stream, hipStreamCaptureModeThreadLocal));
+                rc = batch_enqueue(b);
+                if (rc == VMHIP_OK) rc = batch_request_verdict(b); /* the pass's last kernel is part of the graph */
+                hipError_t e = hipStreamEndCapture(E->stream, &b->graph);
+                if (rc != VMHIP_OK || e != hipSuccess) {
+                    if (e == hipSuccess && b->graph) (void) hipGraphDestroy(b->graph);
+                    b->graph = nullptr;
+                    if (rc != VMHIP_OK) return rc;
+                    HIP_TRY(e);
+                }
+                if (hipGraphInstantiate(&b->graph_exec, b->graph, nullptr, nullptr, 0) != hipSuccess) {
+                    b->graph_exec = nullptr;
+                    b->drop_graph();
+                    return fail(VMHIP_ERR_HIP, "run: the captured pass could not be instantiated");
+                }
+                std::memcpy(&b->graph_key, &key, sizeof(key));
+                ++b->graph_captures;
+            }
+            HIP_TRY(hipGraphLaunch(b->graph_exec, E->stream));
+            ++b->graph_launches;
+            ++b->epoch;
+            return VMHIP_OK;
         }
-        HIP_TRY(hipGraphLaunch(b->graph_exec, E->stream));
-        return VMHIP_OK;
     }
     rc = batch_enqueue(b);
-    ++b->eager_runs;
     if (rc != VMHIP_OK) return rc;
-    return batch_request_verdict(b);
+    rc = batch_request_verdict(b);
+    if (rc != VMHIP_OK) return rc;
+    ++b->eager_runs;
+    ++b->eager_launches;
+    ++b->epoch;
+    return VMHIP_OK;
 }
 
 /* waits for a launched pass; repeats it (a few times at most) while the host overrules edge decisions of the device */
@@ -922,7 +991,11 @@ int vmhip_engine_create(const vmhip_network* net, int32_t n_neighbours, int32_t 
             int n_bf16 = 0;
             for (int l = 0; l < n; ++l) n_bf16 += ar[l];
             int max_rounded = (n_bf16 <= 5 && precision == VMHIP_BF16) ? 2 : 0; /* VMHIP_SPLIT: every boundary as pairs */
-            if (const char* r = getenv("VMHIP_BF16_ROUNDED")) max_rounded = std::max(atoi(r), 0);
+            /* the split engine's contract has no rounded boundary: the measurement overrides are for the bf16 engine only */
+            const bool overridable = precision == VMHIP_BF16;
+            if (precision == VMHIP_SPLIT && n_bf16 > 10)
+                return bail(VMHIP_ERR_ARGUMENT, "engine_create: VMHIP_SPLIT keeps its accuracy for up to ten 64-wide layers; use VMHIP_FP32 for this network");
+            if (const char* r = getenv("VMHIP_BF16_ROUNDED")) max_rounded = overridable ? std::max(atoi(r), 0) : max_rounded;
             for (int l = 1; l < n; ++l) {
                 if (!ar[l]) continue;
                 ++eligible;
@@ -930,7 +1003,8 @@ int vmhip_engine_create(const vmhip_network* net, int32_t n_neighbours, int32_t 
                 const bool splits = ar[l - 1] || (allow_lds && P.slots - 1 <= VMHIP_NBL_STRIDE && vm_lds_supported(P.c_in, P.c_out, P.slots, VM_ROWS_BF16X2));
                 if (!splits) continue; /* the layer before writes fp32 rows */
                 bool round_here = ar[l - 1] && eligible % 2 == 0 && rounded < max_rounded;
-                if (const char* at = getenv("VMHIP_BF16_ROUNDED_AT")) round_here = ar[l - 1] && ((strtoul(at, nullptr, 0) >> l) & 1ul);
+                if (const char* at = getenv("VMHIP_BF16_ROUNDED_AT"))
+                    if (overridable) round_here = ar[l - 1] && ((strtoul(at, nullptr, 0) >> l) & 1ul);
                 if (round_here) bf[l] = VM_ROWS_BF16, ++rounded;
                 else bf[l] = VM_ROWS_BF16X2;
             }
@@ -1238,7 +1312,7 @@ int vmhip_batch_export(vmhip_batch* b, int32_t edge_type, vmhip_lookup_export* p
     float* const vectors = reinterpret_cast<float*>(ws);
     int32_t* const graph = reinterpret_cast<int32_t*>(ws + at_graph);
     float* const pixels = reinterpret_cast<float*>(ws + at_pixels);
-    vm_launch_lookup_export(b->dev, edge_type == VMHIP_EDGE_SAME, vectors, graph, pixels, s);
+    vm_launch_lookup_export(b->dev_exact(), edge_type == VMHIP_EDGE_SAME, vectors, graph, pixels, s);
     HIP_TRY(hipGetLastError());
     for (int f = 0; f < n; ++f) {
         const VmFrame& d = b->frames[f].dev;
@@ -1266,6 +1340,13 @@ int vmhip_batch_wait(vmhip_batch* b) {
     if (!b->in_flight) return fail(VMHIP_ERR_ARGUMENT, "batch_wait: no run in flight");
     b->in_flight = false;
     return batch_complete(b);
+}
+int vmhip_batch_graph_stats(const vmhip_batch* b, int64_t* captures, int64_t* graph_launches, int64_t* eager_launches) {
+    if (!b) return fail(VMHIP_ERR_ARGUMENT, "batch_graph_stats: null batch");
+    if (captures) *captures = b->graph_captures;
+    if (graph_launches) *graph_launches = b->graph_launches;
+    if (eager_launches) *eager_launches = b->eager_launches;
+    return VMHIP_OK;
 }
 int vmhip_batch_counts(const vmhip_batch* b, int32_t* n_visible) {
     if (!b || !n_visible || !b->have_run) return fail(VMHIP_ERR_ARGUMENT, "batch_counts: no completed run");
@@ -1339,7 +1420,7 @@ int vmhip_batch_detect(vmhip_batch* b, int32_t class_index, float threshold, int
                       && std::memcmp(&b->detect_threshold, &threshold, sizeof(float)) == 0 && b->detect_arg_max == (arg_max_only != 0)
                       && b->detect_clusters == (clusters != 0);
     if (!held) {
-        vm_launch_detect(b->dev, D, clusters != 0, s);
+        vm_launch_detect(b->dev_exact(), D, clusters != 0, s);
         HIP_TRY(hipGetLastError());
         b->detect_serial = b->run_serial, b->detect_class = class_index, b->detect_threshold = threshold;
         b->detect_arg_max = arg_max_only != 0, b->detect_clusters = clusters != 0;
@@ -1373,7 +1454,7 @@ int vmhip_batch_detect(vmhip_batch* b, int32_t class_index, float threshold, int
     const size_t words = 5 * total_d + 7 * total_c;
     HIP_TRY(b->d_detect_packed.reserve(words * 4));
     HIP_TRY(pinned(words * 4));
-    vm_launch_detect_pack(b->dev, D, static_cast<uint32_t*>(b->d_detect_packed.p), int(total_d), int(total_c), s);
+    vm_launch_detect_pack(b->dev_exact(), D, static_cast<uint32_t*>(b->d_detect_packed.p), int(total_d), int(total_c), s);
     HIP_TRY(hipGetLastError());
     HIP_TRY(hipMemcpyAsync(b->h_detect, b->d_detect_packed.p, words * 4, hipMemcpyDeviceToHost, s));
     HIP_TRY(hipStreamSynchronize(s));

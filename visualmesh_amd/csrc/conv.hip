@@ -69,6 +69,7 @@ template <int C_IN, int C_OUT, int SLOTS>
 __global__ __launch_bounds__(VMHIP_TILE) void vm_conv_rows_kernel(VmBatchDev B, VmLayerDev L, const float* __restrict__ in,
                                                                   float* __restrict__ out) {
     const int tile = blockIdx.x;
+    if (tile >= vm_row_tiles(B)) return; /* the grid may be sized for more tiles than the staged batch has */
     const int f = find_frame_by_row_tile(B.frames, B.n_frames, tile);
     const VmFrame& F = B.frames[f];
     const int V = B.frame_V[f];
@@ -123,6 +124,7 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_conv_rows_kernel(VmBatchDev B, 
 __global__ __launch_bounds__(VMHIP_TILE) void vm_conv_generic_kernel(VmBatchDev B, VmLayerDev L, const float* __restrict__ in,
                                                                      float* __restrict__ out) {
     const int tile = blockIdx.x;
+    if (tile >= vm_row_tiles(B)) return; /* the grid may be sized for more tiles than the staged batch has */
     const int f = find_frame_by_row_tile(B.frames, B.n_frames, tile);
     const VmFrame& F = B.frames[f];
     const int V = B.frame_V[f];

@@ -606,6 +606,7 @@ __global__ __launch_bounds__(BT) void vm_half_tables_kernel(VmBatchDev B) {
     __shared__ __align__(16) uint16_t nbl_rows[BT][VMHIP_NBL_STRIDE];
 
     const int tile = blockIdx.x >> 1;
+    if (tile >= vm_row_tiles(B)) return; /* the grid may be sized for more tiles than the staged batch has */
     const int f = find_frame_by_row_tile(B.frames, B.n_frames, tile);
     const VmFrame& F = B.frames[f];
     const int V = B.frame_V[f];
@@ -764,7 +765,8 @@ void vm_launch_half_tables(const VmBatchDev& B, hipStream_t stream) {
 int vm_launch_conv_bf16(const VmBatchDev& B, const VmLayerDev& L, const void* in, void* out, hipStream_t stream, const char** kernel_name) {
     if (B.n_row_tiles <= 0) return 0;
     if (!B.row_nbl_h || !B.tile_note_h || !B.active_h || !L.w_mfma || !vm_bf16_supported(L.c_in, L.c_out, L.slots)) return -1;
-    /* the kernel addresses a frame's input rows with 32-bit byte offsets; a frame never has 2^24 rows */
+    /* the kernel addresses a frame's input rows with 32-bit byte offsets: a batch with a frame of 2^24 rows or more is
+     * refused when it is staged for an engine with such layers (api.hip) */
 #define Z(FI, FO, ACT, NAME)                                                       \
     if (L.in_bf16 == FI && L.out_bf16 == FO && L.activation == ACT) {              \
         if (kernel_name) *kernel_name = NAME;                                      \

@@ -221,7 +221,7 @@ __global__ __launch_bounds__(FLOW_WAVES * 64) void vm_conv_flow_kernel(VmBatchDe
     const int lw = wave; /* which loader this wave is, if it is one */
     uint32_t* const slot = counters + 8 + SLOT_WORDS * (wave % LOADERS); /* a loader's notes on the tile it stages next */
 
-    const int n_tiles = B.n_row_tiles;
+    const int n_tiles = vm_row_tiles(B);
     const int xcd = blockIdx.x & 7, lb = blockIdx.x >> 3, gx = gridDim.x >> 3;
     const int per_xcd = (n_tiles + 7) >> 3;
     const int t_end = min(n_tiles, (xcd + 1) * per_xcd);

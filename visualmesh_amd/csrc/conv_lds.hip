@@ -134,7 +134,7 @@ __global__ __launch_bounds__(NW * 64, 4) void vm_conv_lds_kernel(VmBatchDev B, V
     const int q = lane >> 4, r16 = lane & 15;
     const int activation = L.activation;
 
-    const int n_tiles = B.n_row_tiles;
+    const int n_tiles = vm_row_tiles(B);
     const int xcd = blockIdx.x & 7, lb = blockIdx.x >> 3, gx = gridDim.x >> 3;
     const int per_xcd = (n_tiles + 7) >> 3;
     const int t_end = min(n_tiles, (xcd + 1) * per_xcd);

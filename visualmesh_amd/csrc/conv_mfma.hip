@@ -169,7 +169,7 @@ __global__ __launch_bounds__(NW * 64) void vm_conv_mfma_kernel(VmBatchDev B, VmL
     }
 
     /* persistent, XCD-aware walk over the tiles */
-    const int n_tiles = B.n_row_tiles;
+    const int n_tiles = vm_row_tiles(B);
     const int xcd = blockIdx.x & 7, lb = blockIdx.x >> 3, gx = gridDim.x >> 3;
     const int per_xcd = (n_tiles + 7) >> 3;
     const int t_end = min(n_tiles, (xcd + 1) * per_xcd);

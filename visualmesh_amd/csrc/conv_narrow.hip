@@ -115,7 +115,7 @@ __global__ __launch_bounds__(NW * 64) void vm_conv_narrow_kernel(VmBatchDev B, V
     const int o_lane = lane & 3;
     const int activation = L.activation;
 
-    const int n_tiles = B.n_row_tiles;
+    const int n_tiles = vm_row_tiles(B);
     const int xcd = blockIdx.x & 7, lb = blockIdx.x >> 3, gx = gridDim.x >> 3;
     const int per_xcd = (n_tiles + 7) >> 3;
     const int t_end = min(n_tiles, (xcd + 1) * per_xcd);

@@ -114,6 +114,7 @@ __device__ __forceinline__ void unite(int32_t* parent, int a, int b) {
 
 __global__ __launch_bounds__(VMHIP_TILE) void vm_cluster_union_kernel(VmBatchDev B, VmDetectDev D) {
     const int tile = blockIdx.x;
+    if (tile >= vm_row_tiles(B)) return; /* the grid may be sized for more tiles than the staged batch has */
     const int f = frame_of_row_tile(B.frames, B.n_frames, tile);
     const VmFrame& F = B.frames[f];
     const int V = F.n_cand > 0 ? B.frame_V[f] : 0; /* a frame without candidates has no rows */

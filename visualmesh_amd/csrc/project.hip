@@ -417,6 +417,7 @@ __global__ __launch_bounds__(LOOKUP_THREADS) void vm_lookup_kernel(const VmLooku
 __global__ __launch_bounds__(VMHIP_TILE) void vm_lookup_export_kernel(VmBatchDev B, int same_edges, float* __restrict__ vectors,
                                                                        int32_t* __restrict__ graph, float2* __restrict__ pixels) {
     const int tile = blockIdx.x;
+    if (tile >= vm_cand_tiles(B)) return; /* the grid may be sized for more tiles than the staged batch has */
     const int f = find_frame_by_cand_tile(B.frames, B.n_frames, tile);
     const VmFrame& F = B.frames[f];
     const int p = (tile - F.cand_tile0) * VMHIP_TILE + threadIdx.x;
@@ -448,6 +449,7 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_lookup_export_kernel(VmBatchDev
 __global__ __launch_bounds__(VMHIP_TILE) void vm_project_kernel(VmBatchDev B) {
     __shared__ int wave_count[VMHIP_TILE / 64];
     const int tile = blockIdx.x;
+    if (tile >= vm_cand_tiles(B)) return; /* the grid may be sized for more tiles than the staged batch has */
     int f, tile_range = -1;
     if (B.cand_tile_info) {
         const int2 info = B.cand_tile_info[tile];
@@ -634,6 +636,7 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_compact_kernel(VmBatchDev B, fl
     __shared__ int partial[VMHIP_TILE / 64];
     __shared__ int wave_count[VMHIP_TILE / 64];
     const int tile = blockIdx.x;
+    if (tile >= vm_cand_tiles(B)) return;
     const int f = B.cand_tile_info ? B.cand_tile_info[tile].x : find_frame_by_cand_tile(B.frames, B.n_frames, tile);
     const VmFrame& F = B.frames[f];
     /* the frame's placement as values: read through F again after a store, it would be fetched again */
@@ -710,6 +713,7 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_neighbourhood_kernel(VmBatchDev
     __shared__ __align__(16) uint16_t nbl_rows[VMHIP_TILE][VMHIP_NBL_STRIDE]; /* the tile's positions, stored row by row at the end */
 
     const int tile = blockIdx.x;
+    if (tile >= vm_row_tiles(B)) return;
     const int f = B.row_tile_frame ? B.row_tile_frame[tile] : find_frame_by_row_tile(B.frames, B.n_frames, tile);
     const VmFrame& F = B.frames[f];
     const int V = B.frame_V[f];

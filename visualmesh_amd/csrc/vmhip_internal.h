@@ -88,10 +88,19 @@ struct VmFrame {
     const uint64_t* force_keep;
 };
 
+/* What changes from one staged batch to the next while every address and launch grid stays the same: the tiles in use.
+ * It lives in device memory (uploaded with the frame descriptions), so that a pass captured into a HIP graph with one
+ * batch serves the batches staged after it. */
+struct VmBatchLive {
+    int32_t n_cand_tiles, n_row_tiles;
+};
+
 struct VmBatchDev {
     const VmFrame* frames;
     int32_t n_frames;
+    /* the tiles the launch grids are sized for: at least the tiles in use, which kernels read through `live` */
     int32_t n_cand_tiles, n_row_tiles;
+    const VmBatchLive* live; /* null: the two counts above are the tiles in use */
     uint32_t* epoch;      /* device word: the run's stamp for the reverse lookup, from 1; the last kernel of a pass increments it */
     /* where a tile belongs, worked out when the batch is staged so that no block has to search for it (null: the blocks search) */
     const int2* cand_tile_info;     /* [n_cand_tiles] {frame, index of the range that holds the tile's first candidate} */
@@ -131,6 +140,9 @@ struct VmBatchDev {
      * differs from the host's (vmhip_debug_set) */
     float amb_eps, px_error;
 };
+/* the tiles in use, on the device (uniform: scalar loads) */
+__device__ __forceinline__ int vm_cand_tiles(const VmBatchDev& B) { return B.live ? B.live->n_cand_tiles : B.n_cand_tiles; }
+__device__ __forceinline__ int vm_row_tiles(const VmBatchDev& B) { return B.live ? B.live->n_row_tiles : B.n_row_tiles; }
 #define VMHIP_AMB_EPS_DEFAULT 0.015625f /* 1/64 px: far above any device/host libm difference, far below node spacing */
 
 /* Lookup on the device (project.hip: vm_lookup_kernel): the cone tree over a mesh's nodes and what a frame's walk of it

@@ -305,6 +305,10 @@ class Engine:
     def native_batch(self):
         return C.c_void_p(self._lib.vmh_engine_native_batch(self.ptr))
 
+    def graph_stats(self):
+        """dict(captures, graph_launches, eager_launches): how this engine's passes reached the stream so far"""
+        return native.graph_stats(self.native_batch())
+
     def detect(self, class_index, threshold, arg_max_only=False, clusters=True):
         """The nodes of one class among the results of the last run, picked (probability >= threshold, optionally only
         where the class is the arg max) and grouped into connected components of the neighbourhood graph on the
@@ -401,6 +405,12 @@ class Pipeline:
         self._neighbours.append([m.n_neighbours for m in meshes])
         self._keep.append(images)
         return self._results(native.host_check(self._lib.vmh_pipeline_submit(self.ptr, n, mesh_ptrs, _fp(H), lenses, image_ptrs, fccs)), arrays)
+
+    def graph_stats(self):
+        """dict(captures, graph_launches, eager_launches) of the three engines together"""
+        v = [C.c_int64(0) for _ in range(3)]
+        native.host_check(self._lib.vmh_pipeline_graph_stats(self.ptr, *[C.byref(x) for x in v]))
+        return dict(captures=v[0].value, graph_launches=v[1].value, eager_launches=v[2].value)
 
     def flush(self, arrays=True):
         if not self._neighbours:

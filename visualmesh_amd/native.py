@@ -27,7 +27,7 @@ HIP_SYMBOLS = [
     "vmhip_last_error", "vmhip_engine_create", "vmhip_engine_destroy", "vmhip_engine_n_classes", "vmhip_mesh_upload",
     "vmhip_mesh_release", "vmhip_project", "vmhip_classify", "vmhip_classify_batch", "vmhip_batch_create",
     "vmhip_batch_destroy", "vmhip_mesh_attach_tree", "vmhip_batch_stage", "vmhip_batch_stage_async", "vmhip_batch_ranges", "vmhip_batch_export", "vmhip_batch_run", "vmhip_batch_run_async", "vmhip_batch_wait", "vmhip_batch_counts", "vmhip_batch_fetch", "vmhip_batch_fetch_async", "vmhip_batch_fetch_wait", "vmhip_batch_fetch_packed_size", "vmhip_batch_fetch_packed_async", "vmhip_batch_detect", "vmhip_host_alloc", "vmhip_host_free",
-    "vmhip_batch_profile", "vmhip_batch_profile_read", "vmhip_selftest_libm", "vmhip_selftest_copy", "vmhip_selftest_stream", "vmhip_project_noalloc", "vmhip_debug_set", "vmhip_batch_guard_stats",
+    "vmhip_batch_profile", "vmhip_batch_profile_read", "vmhip_selftest_libm", "vmhip_selftest_copy", "vmhip_selftest_stream", "vmhip_project_noalloc", "vmhip_debug_set", "vmhip_batch_guard_stats", "vmhip_batch_graph_stats",
     "vmhip_engine_create_f64", "vmhip_engine_destroy_f64", "vmhip_engine_n_classes_f64", "vmhip_mesh_upload_f64", "vmhip_mesh_release_f64",
     "vmhip_project_f64", "vmhip_classify_f64", "vmhip_engine_guard_stats_f64",
 ]
@@ -222,6 +222,7 @@ def hip():
     L.vmhip_selftest_stream.argtypes = [C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.POINTER(C.c_float)]
     L.vmhip_debug_set.argtypes = [C.c_int32, C.c_double]
     L.vmhip_batch_guard_stats.argtypes = [vp, C.POINTER(C.c_int64), C.POINTER(C.c_int64), C.POINTER(C.c_int64), C.POINTER(C.c_int64)]
+    L.vmhip_batch_graph_stats.argtypes = [vp, C.POINTER(C.c_int64), C.POINTER(C.c_int64), C.POINTER(C.c_int64)]
     L.vmhip_project_noalloc.argtypes = [vp, C.POINTER(C.c_float), C.POINTER(Lens), C.POINTER(C.c_int32), C.c_int32, C.c_int32,
                                         C.POINTER(ProjectionDevice), vp]
     dp = C.POINTER(C.c_double)
@@ -250,6 +251,13 @@ def guard_stats(batch_ptr):
     v = [C.c_int64(0) for _ in range(4)]
     hip_check(hip().vmhip_batch_guard_stats(batch_ptr, *[C.byref(x) for x in v]))
     return dict(listed=v[0].value, most_listed=v[1].value, overruled=v[2].value, reruns=v[3].value)
+
+
+def graph_stats(batch_ptr):
+    """dict(captures, graph_launches, eager_launches): how the passes of a vmhip_batch were put on the stream since it was made"""
+    v = [C.c_int64(0) for _ in range(3)]
+    hip_check(hip().vmhip_batch_graph_stats(batch_ptr, *[C.byref(x) for x in v]))
+    return dict(captures=v[0].value, graph_launches=v[1].value, eager_launches=v[2].value)
 
 
 def copy_probe(nbytes=1 << 30, repeats=5):
@@ -348,6 +356,7 @@ def host():
     L.vmh_pipeline_submit.argtypes = [vp, C.c_int, C.POINTER(vp), C.POINTER(C.c_float), C.POINTER(Lens), C.POINTER(vp), C.POINTER(C.c_uint32)]
     L.vmh_pipeline_result.argtypes = [vp, C.c_int, fpp, ipp, ipp, fpp]
     L.vmh_pipeline_n_classes.argtypes = [vp]
+    L.vmh_pipeline_graph_stats.argtypes = [vp, C.POINTER(C.c_int64), C.POINTER(C.c_int64), C.POINTER(C.c_int64)]
     _host = L
     return L
 
