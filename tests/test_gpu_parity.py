@@ -480,6 +480,41 @@ def test_rows_beyond_the_halo_capacity(oracle, index, kernel, monkeypatch):
     assert_classification_parity(got, want, PROB_TOL, "halo cap 8, cfg%d, %s" % (index, kernel))
 
 
+@pytest.mark.parametrize("halo_cap", [None, 8], ids=["full halo", "8 halo slots"])
+@pytest.mark.parametrize("index", [1, 2, 3])
+def test_first_layer_inside_the_neighbourhood_kernel(oracle, index, halo_cap, monkeypatch):
+    """The first layer of configurations 1, 2 and 3 (4 -> 16 on Ring6, 4 -> 24 on NMGrid8) is computed by the blocks of the
+    neighbourhood kernel for their own tiles; with only 8 halo slots per tile most neighbours outside a tile are read
+    from global memory through the table the block has just written. Same results as the oracle, and as the engine
+    with the layer as a launch of its own."""
+    if halo_cap is not None:
+        monkeypatch.setenv("VMHIP_HALO_CAP", str(halo_cap))
+    cfg = wl.config(index, n_frames=2 if index == 2 else 1)
+    o_lens, e_lens = lens_pair(cfg)
+    o_mesh, e_mesh = meshes_for(cfg, oracle)
+    engine = eng.Engine(cfg.network, cfg.model)
+    frames = [dict(mesh=e_mesh, Hoc=f["Hoc"], lens=e_lens, image=f["image"], fourcc=cfg.fourcc) for f in cfg.frames]
+    results = engine.classify_batch(frames)
+    monkeypatch.setenv("VMHIP_FUSE_FIRST", "0")  # read when an engine is first used
+    apart = eng.Engine(cfg.network, cfg.model)
+    engine.profile(True)
+    engine.run()
+    names = [n for n, _, _ in engine.profile_read()]
+    first = "neighbourhood_conv_4x%ds%d" % (cfg.network[0][0][0].shape[1], 7 if index != 3 else 9)
+    assert first in names and "neighbourhood" not in names and len([n for n in names if n.startswith("conv")]) == len(cfg.network) - 1, names
+    others = apart.classify_batch(frames)
+    apart.profile(True)
+    apart.run()
+    names = [n for n, _, _ in apart.profile_read()]
+    assert "neighbourhood" in names and len([n for n in names if n.startswith("conv")]) == len(cfg.network), names
+    for i, f in enumerate(cfg.frames):
+        want = pick(o_mesh, f["Hoc"]).classify(f["Hoc"], o_lens, f["image"], cfg.fourcc, vmo.Network(cfg.network))
+        assert_classification_parity(results[i], want, PROB_TOL, "first layer with the neighbourhood, frame %d" % i)
+        assert_classification_parity(others[i], want, PROB_TOL, "first layer apart, frame %d" % i)
+        for key in ("px", "gidx", "nb"):
+            assert np.array_equal(results[i][key], others[i][key]), key
+
+
 def test_graph_replays_match_eager_runs(oracle, monkeypatch):
     """A staged batch launches its first run kernel by kernel, captures the second into a HIP graph and replays it
     afterwards. Every replay, with eager work of another engine and synchronisations in between, must reproduce
@@ -655,8 +690,9 @@ def test_reference_example_network_on_its_dataset_poses(oracle):
     results = engine.classify_batch(frames)
     engine.profile(True)
     engine.run()
-    names = [n for n, _, _ in engine.profile_read() if n.startswith("conv")]
-    assert len(names) == 13 and all(n.startswith("conv_lds_") for n in names), names
+    names = [n for n, _, _ in engine.profile_read() if "conv" in n]
+    # the first layer rides on the neighbourhood kernel, the other twelve gather from LDS
+    assert len(names) == 13 and names[0] == "neighbourhood_conv_4x16s7" and all(n.startswith("conv_lds_") for n in names[1:]), names
     for (H, ol, _, p), im, got in zip(chosen, images, results):
         want = pick(o_mesh, H).classify(H, ol, im, wl.fourcc("BGRA"), vmo.Network(network))
         print("example pose", p["number"], "V =", len(want["gidx"]), flush=True)

@@ -105,6 +105,7 @@ struct HostLayer {
     float* d_w_flow = nullptr; /* w_mfma in conv_flow.hip's LDS order */
     int32_t in_bf16 = 0, out_bf16 = 0, arith_bf16 = 0;
     bool use_lds = false, use_mfma = false, use_flow = false, use_narrow = false; /* which matrix-core kernels may take the layer */
+    bool fuse_first = false; /* the network's first layer, computed by the neighbourhood kernel's blocks for their own tiles */
     std::vector<float> h_w, h_b; /* kept until the row types are planned */
 };
 
@@ -560,18 +561,34 @@ int batch_enqueue(vmhip_batch* b) {
     HIP_TRY(P.begin());
     vm_launch_compact(D, b->d_act[0].as<float>(), b->classify, s);
     HIP_TRY(P.end(b->classify ? "compact_sample" : "compact", cands));
-    HIP_TRY(P.begin());
-    vm_launch_neighbourhood(D, s);
-    HIP_TRY(P.end("neighbourhood", rows));
+    /* the neighbourhood table - and, where the first layer is a thin one over the sampled rows, that layer with it */
+    int first_layer = 0, cur = 0;
+    bool fused = false;
+    if (b->classify && !E->layers.empty() && E->layers[0].fuse_first && D.row_nbl) {
+        const HostLayer& L = E->layers[0];
+        VmLayerDev ld{L.c_in, L.c_out, L.slots, L.activation, L.d_w, L.d_b, L.d_w_mfma, L.in_bf16, L.out_bf16, L.arith_bf16, L.d_w_flow};
+        const char* name = "neighbourhood";
+        HIP_TRY(P.begin());
+        fused = vm_launch_neighbourhood_conv(D, ld, b->d_act[0].as<float>(), b->d_act[1].as<float>(), s, &name) == 0;
+        if (fused) {
+            HIP_TRY(P.end(name, rows));
+            first_layer = 1, cur = 1;
+        }
+    }
+    if (!fused) {
+        HIP_TRY(P.begin()); /* (a second begin of the same slot records its start event again) */
+        vm_launch_neighbourhood(D, s);
+        HIP_TRY(P.end("neighbourhood", rows));
+    }
     if (b->classify && D.row_nbl_h) {
         HIP_TRY(P.begin());
         vm_launch_half_tables(D, s);
         HIP_TRY(P.end("half_tables", rows));
     }
 
-    int cur = 0;
     if (b->classify) {
-        for (const HostLayer& L : E->layers) {
+        for (size_t li = size_t(first_layer); li < E->layers.size(); ++li) {
+            const HostLayer& L = E->layers[li];
             VmLayerDev ld{L.c_in, L.c_out, L.slots, L.activation, L.d_w, L.d_b, L.d_w_mfma, L.in_bf16, L.out_bf16, L.arith_bf16, L.d_w_flow};
             const char* name = "conv";
             HIP_TRY(P.begin());
@@ -1030,6 +1047,12 @@ int vmhip_engine_create(const vmhip_network* net, int32_t n_neighbours, int32_t 
             H.use_narrow = allow_lds && !force_lds && plain && H.slots - 1 <= VMHIP_NBL_STRIDE
                            && vm_narrow_supported(H.c_in, H.c_out, H.slots);
             E->use_lds = E->use_lds || H.use_lds || H.use_flow || H.use_narrow;
+            /* the first layer inside the neighbourhood kernel (VMHIP_FUSE_FIRST=0: as a launch of its own, for comparisons) */
+            {
+                const char* fuse = getenv("VMHIP_FUSE_FIRST");
+                H.fuse_first = l == 0 && plain && H.use_lds && !pick && !(fuse && atoi(fuse) == 0) && n_neighbours <= VMHIP_NBL_STRIDE
+                               && vm_neighbourhood_conv_supported(H.c_in, H.c_out, H.slots, H.activation);
+            }
             E->use_flow = E->use_flow || H.use_flow;
             if (H.arith_bf16) {
                 std::vector<unsigned char> wp(vm_bf16_weight_bytes(H.c_in, H.c_out, H.slots));

@@ -702,15 +702,37 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_compact_kernel(VmBatchDev B, fl
  *
  * WIDE = false addresses the frame's tables with 32-bit byte offsets from wave-uniform bases (an address is then a
  * scalar register pair plus one vector register, and the 64-bit vector arithmetic that was a third of this kernel's
- * instructions is gone); the host picks WIDE = true for a batch with a table of 4 GiB or more. */
+ * instructions is gone); the host picks WIDE = true for a batch with a table of 4 GiB or more.
+ *
+ * CB > 0: the block also computes the network's first layer for its tile (reference engine/cpu/engine.hpp:213-264 for the
+ * group's first dense layer: gather of [self, neighbours] over the 4-channel sampled rows, dense, bias, activation),
+ * CB column blocks of 16 output channels. At this point the tile's neighbour rows are in registers and the rows it
+ * gathers are 16 bytes each: the layer's 28 (36) input values per row are requested as soon as the neighbours are known
+ * and arrive while the block builds its tile-local tables, so the layer costs neither a launch of its own nor a second
+ * read of the neighbour table. v_mfma_f32_16x16x4_f32: A = weights (lane l: W[4 slot + l / 16][16 cb + l % 16], the order
+ * vm_mfma_permute_weights stores), B = one gathered row per step (lane l: channel l / 16 of the row's source), D: lane l
+ * holds channels 16 cb + 4 (l / 16) + {0..3} of row l % 16, one 16-byte store. */
 #define NB_HASH 2048 /* >= the most out-of-tile neighbours a tile can have (256 rows x 8) */
-template <bool WIDE, int NN>
-__global__ __launch_bounds__(VMHIP_TILE) void vm_neighbourhood_kernel(VmBatchDev B) {
+typedef float nbc_v4f __attribute__((ext_vector_type(4)));
+typedef uint32_t nbc_v4u __attribute__((ext_vector_type(4)));
+/* selu as the convolution kernels compute it: hardware exponential on the negative branch (<= 3e-7 absolute error) */
+__device__ __forceinline__ float nbc_selu(float s) {
+    const float lambda = 1.0507009873554804934193349852946f;
+    const float alpha = 1.6732632423543772848170429916717f;
+    return lambda * (s >= 0.0f ? s : __builtin_fmaf(alpha, __builtin_amdgcn_exp2f(s * 1.44269504088896340736f), -alpha));
+}
+template <bool WIDE, int NN, int CB>
+__global__ __launch_bounds__(VMHIP_TILE, CB == 1 ? (NN <= 6 ? 8 : 6) : CB == 2 ? 5 : 1) void vm_neighbourhood_kernel(VmBatchDev B, VmLayerDev L, const float* __restrict__ feat, float* __restrict__ layer_out) {
+    static_assert(CB == 0 || (NN > 0 && NN <= VMHIP_NBL_STRIDE), "the fused first layer knows its neighbour count");
     using Off = typename std::conditional<WIDE, size_t, uint32_t>::type;
     __shared__ __align__(16) uint32_t h_key[NB_HASH];
-    __shared__ uint16_t h_dense[NB_HASH];
     __shared__ int wave_total[VMHIP_TILE / 64];
+    __shared__ uint16_t h_dense[NB_HASH];
     __shared__ __align__(16) uint16_t nbl_rows[VMHIP_TILE][VMHIP_NBL_STRIDE]; /* the tile's positions, stored row by row at the end */
+    /* CB > 0: the frame-local row of every halo slot. The sampled rows the layer gathers (the tile's 256, then its halo
+     * rows, 16 bytes each) are staged where the hash table lay, once nothing reads it any more. */
+    __shared__ uint32_t halo_list[CB > 0 ? VMHIP_HALO_MAX : 1];
+    static_assert(sizeof(h_key) >= (VMHIP_TILE + VMHIP_HALO_MAX) * 16, "the staged rows fit the hash table's memory");
 
     const int tile = blockIdx.x;
     if (tile >= vm_row_tiles(B)) return;
@@ -750,7 +772,7 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_neighbourhood_kernel(VmBatchDev
     const uint32_t nn_magic = nn > 1 ? 0xffffffffu / (uint32_t) nn + 1u : 0u;
     auto row_of = [&](int it) { return NN > 0 ? it / (NN > 0 ? NN : 1) : nn > 1 ? (int) __umulhi((uint32_t) it, nn_magic) : it; };
     constexpr int MAX_ITEMS = NN > 0 ? NN : VMHIP_NBL_STRIDE;
-    int item_row[MAX_ITEMS], item_slot[MAX_ITEMS], outs[MAX_ITEMS];
+    int outs[MAX_ITEMS];
 
     /* Items k0 .. k0 + MAX_ITEMS - 1 of this thread. The three dependent reads of an item (row -> node, node -> neighbour
      * node, neighbour node -> its row) go level by level over all the items, so that the items' reads are in flight together
@@ -759,6 +781,7 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_neighbourhood_kernel(VmBatchDev
     auto resolve = [&](int k0) {
         bool live[MAX_ITEMS];
         uint32_t stamp[MAX_ITEMS];
+        int item_row[MAX_ITEMS], item_slot[MAX_ITEMS];
 #pragma unroll
         for (int k = 0; k < MAX_ITEMS; ++k) {
             const int it = threadIdx.x + (k0 + k) * VMHIP_TILE;
@@ -793,6 +816,18 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_neighbourhood_kernel(VmBatchDev
         return;
     }
     resolve(0);
+
+    /* ---- first layer, part one: request what the contraction will read ---- */
+    constexpr int RBS = 4; /* row blocks of 16 per wave: a wave owns 64 rows of the tile */
+    constexpr int SLOTS = NN + 1;
+    float a[CB > 0 ? SLOTS : 1][CB > 0 ? CB : 1]; /* [slot][column block]: the lane's weight */
+    nbc_v4u own_row = {0u, 0u, 0u, 0u}, halo_row = {0u, 0u, 0u, 0u};
+    /* the frame's sampled rows 0..V, 16 bytes each; offsets beyond read zeros */
+    auto sampled_rows = [&] {
+        return __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(feat + (size_t) row_base * 4), 0, (int) min((uint64_t) (V + 1) * 16ull, 0xffffffffull), 0x00020000);
+    };
+    if constexpr (CB > 0) own_row = __builtin_amdgcn_raw_buffer_load_b128(sampled_rows(), (row0 + min((int) threadIdx.x, n_rows - 1)) * 16, 0, 0);
+
 #pragma unroll
     for (int k = 0; k < MAX_ITEMS; ++k) {
         const int out = outs[k];
@@ -839,13 +874,24 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_neighbourhood_kernel(VmBatchDev
         for (int k = 0; k < PER; ++k) {
             if (keys[k] != EMPTY) {
                 h_dense[threadIdx.x * PER + k] = (uint16_t) min(before, 0xffff);
-                if (before < cap) tile_halo[before] = (uint32_t) row_base + keys[k];
+                if (before < cap) {
+                    tile_halo[before] = (uint32_t) row_base + keys[k];
+                    if constexpr (CB > 0) halo_list[before] = keys[k];
+                }
                 ++before;
             }
         }
     }
     if (threadIdx.x == 0) B.tile_desc[tile] = make_int4(row_base + row0, n_rows, min(total, cap), row_base);
     __syncthreads();
+    if constexpr (CB > 0) { /* the halo rows, one per thread, and the layer's weights */
+        halo_row = __builtin_amdgcn_raw_buffer_load_b128(sampled_rows(), (int) threadIdx.x < min(total, cap) ? halo_list[threadIdx.x] * 16u : 0xffffffffu, 0, 0);
+        const VM_GLOBAL float* const w = in_device_memory(reinterpret_cast<const float*>(L.w_mfma));
+#pragma unroll
+        for (int s = 0; s < SLOTS; ++s)
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) a[s][cb] = w[(s * CB + cb) * 64 + (threadIdx.x & 63)];
+    }
 
 #pragma unroll
     for (int k = 0; k < MAX_ITEMS; ++k) {
@@ -861,7 +907,10 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_neighbourhood_kernel(VmBatchDev
                 const int dense = h_dense[slot];
                 local = dense < cap ? (uint32_t) (VMHIP_TILE + dense) : VMHIP_NBL_FAR;
             }
-            nbl_rows[item_row[k] - row0][item_slot[k]] = (uint16_t) local;
+            /* the item's row of the tile and neighbour number, worked out again rather than kept in registers all the way */
+            const int it = threadIdx.x + k * VMHIP_TILE;
+            const int r = row_of(it);
+            nbl_rows[r][it - r * nn] = (uint16_t) local;
         }
     }
     __syncthreads();
@@ -870,6 +919,74 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_neighbourhood_kernel(VmBatchDev
         uint16_t* const nbl_out = B.row_nbl + (size_t) row_base * VMHIP_NBL_STRIDE;
         typedef unsigned int row_words __attribute__((ext_vector_type(4)));
         write_element(reinterpret_cast<row_words*>(nbl_out), (Off) (row0 + threadIdx.x), *reinterpret_cast<const row_words*>(nbl_rows[threadIdx.x]));
+    }
+
+    /* ---- first layer, part two: contraction, activation, store ---- */
+    if constexpr (CB > 0) {
+        const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, q = lane >> 4, r16 = lane & 15;
+        const int c_out = L.c_out, activation = L.activation;
+        /* the rows the tile gathers, where the hash table was (every thread has passed the barrier after its last look at it) */
+        nbc_v4u* const staged = reinterpret_cast<nbc_v4u*>(h_key);
+        staged[threadIdx.x] = own_row;
+        staged[VMHIP_TILE + threadIdx.x] = halo_row;
+        __syncthreads();
+        const float* const staged_f = reinterpret_cast<const float*>(h_key);
+        float x[RBS][SLOTS]; /* [row block][slot]: the lane's channel of the slot's source row */
+#pragma unroll
+        for (int rb = 0; rb < RBS; ++rb) {
+            const int row_t = min(wave * 64 + rb * 16 + r16, n_rows - 1); /* lanes past the tile's rows repeat its last row and store nothing */
+            const nbc_v4u positions = *reinterpret_cast<const nbc_v4u*>(nbl_rows[row_t]);
+            x[rb][0] = staged_f[row_t * 4 + q];
+#pragma unroll
+            for (int s = 0; s < NN; ++s) {
+                const uint32_t word = (s >> 1) == 0 ? positions.x : (s >> 1) == 1 ? positions.y : (s >> 1) == 2 ? positions.z : positions.w;
+                const uint32_t at = (s & 1) ? (word >> 16) : (word & 0xffffu);
+                if (at != VMHIP_NBL_FAR) {
+                    x[rb][s + 1] = staged_f[at * 4 + q];
+                }
+                else { /* more halo rows than slots (rare): the row's number from the table this block has just written */
+                    const int g = read_element(nb_out, (Off) (row0 + row_t) * nb_stride + (Off) s);
+                    x[rb][s + 1] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(sampled_rows(), g * 16 + q * 4, 0, 0));
+                }
+            }
+        }
+        const VM_GLOBAL float* const bias = in_device_memory(L.b);
+        nbc_v4f acc[RBS][CB];
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) {
+            nbc_v4f b4 = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (cb * 16 + q * 4 < c_out) b4 = *reinterpret_cast<const VM_GLOBAL nbc_v4f*>(bias + cb * 16 + q * 4); /* c_out is a multiple of 4 */
+#pragma unroll
+            for (int rb = 0; rb < RBS; ++rb) acc[rb][cb] = b4;
+        }
+#pragma unroll
+        for (int s = 0; s < SLOTS; ++s)
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+                for (int rb = 0; rb < RBS; ++rb) acc[rb][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[s][cb], x[rb][s], acc[rb][cb], 0, 0, 0);
+#pragma unroll
+        for (int rb = 0; rb < RBS; ++rb)
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const float t = acc[rb][cb][v];
+                    acc[rb][cb][v] = activation == VMHIP_SELU ? nbc_selu(t) : activation == VMHIP_RELU ? fmaxf(t, 0.0f) : tanhf(t);
+                }
+        /* the tile's output rows; a lane without a row, or a column block's padding, gets an offset the hardware drops */
+        const __amdgpu_buffer_rsrc_t out_rsrc =
+          __builtin_amdgcn_make_buffer_rsrc(layer_out + ((size_t) row_base + row0) * c_out, 0, VMHIP_TILE * c_out * 4, 0x00020000);
+#pragma unroll
+        for (int rb = 0; rb < RBS; ++rb) {
+            const int row_t = wave * 64 + rb * 16 + r16;
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) {
+                const int o = cb * 16 + q * 4;
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(nbc_v4u, acc[rb][cb]), out_rsrc,
+                                                       (row_t < n_rows && o < c_out) ? (uint32_t) (row_t * c_out + o) * 4u : 0xffffffffu, 0, 0);
+            }
+        }
     }
 }
 
@@ -913,15 +1030,46 @@ void vm_launch_lookup(const VmLookupFrame* frames, int n_frames, hipStream_t str
 template <bool WIDE>
 static void launch_neighbourhood(const VmBatchDev& B, hipStream_t stream) {
     const dim3 grid(B.n_row_tiles), block(VMHIP_TILE);
+    const VmLayerDev none{};
     switch (B.uniform_nn) {
-        case 4: hipLaunchKernelGGL((vm_neighbourhood_kernel<WIDE, 4>), grid, block, 0, stream, B); break;
-        case 6: hipLaunchKernelGGL((vm_neighbourhood_kernel<WIDE, 6>), grid, block, 0, stream, B); break;
-        case 8: hipLaunchKernelGGL((vm_neighbourhood_kernel<WIDE, 8>), grid, block, 0, stream, B); break;
-        default: hipLaunchKernelGGL((vm_neighbourhood_kernel<WIDE, 0>), grid, block, 0, stream, B); break;
+        case 4: hipLaunchKernelGGL((vm_neighbourhood_kernel<WIDE, 4, 0>), grid, block, 0, stream, B, none, nullptr, nullptr); break;
+        case 6: hipLaunchKernelGGL((vm_neighbourhood_kernel<WIDE, 6, 0>), grid, block, 0, stream, B, none, nullptr, nullptr); break;
+        case 8: hipLaunchKernelGGL((vm_neighbourhood_kernel<WIDE, 8, 0>), grid, block, 0, stream, B, none, nullptr, nullptr); break;
+        default: hipLaunchKernelGGL((vm_neighbourhood_kernel<WIDE, 0, 0>), grid, block, 0, stream, B, none, nullptr, nullptr); break;
     }
 }
 void vm_launch_neighbourhood(const VmBatchDev& B, hipStream_t stream) {
     if (B.n_row_tiles <= 0) return;
     if (B.wide_offsets) launch_neighbourhood<true>(B, stream);
     else launch_neighbourhood<false>(B, stream);
+}
+
+bool vm_neighbourhood_conv_supported(int c_in, int c_out, int slots, int activation) {
+    return c_in == 4 && c_out >= 4 && c_out <= 32 && c_out % 4 == 0 && (slots == 5 || slots == 7 || slots == 9) && activation != VMHIP_SOFTMAX;
+}
+template <bool WIDE, int NN>
+static void launch_neighbourhood_conv(const VmBatchDev& B, const VmLayerDev& L, const float* in, float* out, hipStream_t stream) {
+    const dim3 grid(B.n_row_tiles), block(VMHIP_TILE);
+    if (L.c_out <= 16) hipLaunchKernelGGL((vm_neighbourhood_kernel<WIDE, NN, 1>), grid, block, 0, stream, B, L, in, out);
+    else hipLaunchKernelGGL((vm_neighbourhood_kernel<WIDE, NN, 2>), grid, block, 0, stream, B, L, in, out);
+}
+int vm_launch_neighbourhood_conv(const VmBatchDev& B, const VmLayerDev& L, const float* in, float* out, hipStream_t stream, const char** kernel_name) {
+    if (!vm_neighbourhood_conv_supported(L.c_in, L.c_out, L.slots, L.activation) || !B.row_nbl || !L.w_mfma || !L.b || L.in_bf16 || L.out_bf16 || L.arith_bf16
+        || B.uniform_nn != L.slots - 1)
+        return -1;
+    if (kernel_name) *kernel_name = vm_kernel_name("neighbourhood_conv", L.c_in, L.c_out, L.slots);
+    if (B.n_row_tiles <= 0) return 0;
+#define X(NN)                                                                             \
+    case NN:                                                                              \
+        if (B.wide_offsets) launch_neighbourhood_conv<true, NN>(B, L, in, out, stream);   \
+        else launch_neighbourhood_conv<false, NN>(B, L, in, out, stream);                 \
+        break;
+    switch (B.uniform_nn) {
+        X(4)
+        X(6)
+        X(8)
+        default: return -1;
+    }
+#undef X
+    return 0;
 }

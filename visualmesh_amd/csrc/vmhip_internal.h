@@ -235,6 +235,11 @@ void vm_launch_publish(int32_t* counts, int n_counts, const int2* amb_list, int 
 void vm_launch_project(const VmBatchDev& B, hipStream_t stream);
 void vm_launch_compact(const VmBatchDev& B, float* feat, int classify, hipStream_t stream);
 void vm_launch_neighbourhood(const VmBatchDev& B, hipStream_t stream); /* also the tile-local tables if B.row_nbl */
+/* the same launch with the network's first layer (4 sampled channels in, up to 32 out) computed by the blocks for their
+ * own tiles: `in` = the sampled rows, `out` = the layer's rows; a negative value if the layer or the batch does not fit
+ * (then nothing was launched) */
+bool vm_neighbourhood_conv_supported(int c_in, int c_out, int slots, int activation);
+int vm_launch_neighbourhood_conv(const VmBatchDev& B, const VmLayerDev& L, const float* in, float* out, hipStream_t stream, const char** kernel_name);
 /* in -> out over the row space; returns 0 or a negative status if the shape is unsupported */
 int vm_launch_conv(const VmBatchDev& B, const VmLayerDev& L, const float* in, float* out, hipStream_t stream,
                    const char** kernel_name);
