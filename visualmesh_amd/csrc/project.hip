@@ -932,21 +932,37 @@ __global__ __launch_bounds__(VMHIP_TILE, CB == 1 ? (NN <= 6 ? 8 : 6) : CB == 2 ?
         __syncthreads();
         const float* const staged_f = reinterpret_cast<const float*>(h_key);
         float x[RBS][SLOTS]; /* [row block][slot]: the lane's channel of the slot's source row */
+        /* block-uniform: every halo row of the tile has a slot (nearly always). The code is compiled for both cases,
+         * so that the usual one carries no test per position. */
+        const bool all_staged = total <= cap;
+        auto gather = [&](auto checked_tag) {
+            constexpr bool CHECKED = decltype(checked_tag)::value;
 #pragma unroll
-        for (int rb = 0; rb < RBS; ++rb) {
-            const int row_t = min(wave * 64 + rb * 16 + r16, n_rows - 1); /* lanes past the tile's rows repeat its last row and store nothing */
-            const nbc_v4u positions = *reinterpret_cast<const nbc_v4u*>(nbl_rows[row_t]);
-            x[rb][0] = staged_f[row_t * 4 + q];
+            for (int rb = 0; rb < RBS; ++rb) {
+                const int row_t = min(wave * 64 + rb * 16 + r16, n_rows - 1); /* lanes past the tile's rows repeat its last row and store nothing */
+                const nbc_v4u positions = *reinterpret_cast<const nbc_v4u*>(nbl_rows[row_t]);
+                x[rb][0] = staged_f[row_t * 4 + q];
 #pragma unroll
-            for (int s = 0; s < NN; ++s) {
-                const uint32_t word = (s >> 1) == 0 ? positions.x : (s >> 1) == 1 ? positions.y : (s >> 1) == 2 ? positions.z : positions.w;
-                const uint32_t at = (s & 1) ? (word >> 16) : (word & 0xffffu);
-                if (at != VMHIP_NBL_FAR) {
-                    x[rb][s + 1] = staged_f[at * 4 + q];
+                for (int s = 0; s < NN; ++s) {
+                    const uint32_t word = (s >> 1) == 0 ? positions.x : (s >> 1) == 1 ? positions.y : (s >> 1) == 2 ? positions.z : positions.w;
+                    const uint32_t at = (s & 1) ? (word >> 16) : (word & 0xffffu);
+                    /* a position that is not staged reads slot 0 here and is patched below */
+                    x[rb][s + 1] = staged_f[(CHECKED && at == VMHIP_NBL_FAR ? 0u : at) * 4 + q];
                 }
-                else { /* more halo rows than slots (rare): the row's number from the table this block has just written */
-                    const int g = read_element(nb_out, (Off) (row0 + row_t) * nb_stride + (Off) s);
-                    x[rb][s + 1] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(sampled_rows(), g * 16 + q * 4, 0, 0));
+            }
+        };
+        if (all_staged) gather(std::false_type());
+        else gather(std::true_type());
+        if (!all_staged) { /* more halo rows than slots: those rows' numbers from the table this block has just written */
+#pragma unroll
+            for (int rb = 0; rb < RBS; ++rb) {
+                const int row_t = min(wave * 64 + rb * 16 + r16, n_rows - 1);
+#pragma unroll
+                for (int s = 0; s < NN; ++s) {
+                    if (nbl_rows[row_t][s] == VMHIP_NBL_FAR) {
+                        const int g = read_element(nb_out, (Off) (row0 + row_t) * nb_stride + (Off) s);
+                        x[rb][s + 1] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(sampled_rows(), g * 16 + q * 4, 0, 0));
+                    }
                 }
             }
         }
@@ -965,15 +981,18 @@ __global__ __launch_bounds__(VMHIP_TILE, CB == 1 ? (NN <= 6 ? 8 : 6) : CB == 2 ?
             for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
                 for (int rb = 0; rb < RBS; ++rb) acc[rb][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[s][cb], x[rb][s], acc[rb][cb], 0, 0, 0);
+        /* one uniform branch for all the values */
+        auto for_each_value = [&](auto fn) {
 #pragma unroll
-        for (int rb = 0; rb < RBS; ++rb)
+            for (int rb = 0; rb < RBS; ++rb)
 #pragma unroll
-            for (int cb = 0; cb < CB; ++cb)
+                for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    const float t = acc[rb][cb][v];
-                    acc[rb][cb][v] = activation == VMHIP_SELU ? nbc_selu(t) : activation == VMHIP_RELU ? fmaxf(t, 0.0f) : tanhf(t);
-                }
+                    for (int v = 0; v < 4; ++v) acc[rb][cb][v] = fn(acc[rb][cb][v]);
+        };
+        if (activation == VMHIP_SELU) for_each_value([](float t) { return nbc_selu(t); });
+        else if (activation == VMHIP_RELU) for_each_value([](float t) { return fmaxf(t, 0.0f); });
+        else for_each_value([](float t) { return tanhf(t); });
         /* the tile's output rows; a lane without a row, or a column block's padding, gets an offset the hardware drops */
         const __amdgpu_buffer_rsrc_t out_rsrc =
           __builtin_amdgcn_make_buffer_rsrc(layer_out + ((size_t) row_base + row0) * c_out, 0, VMHIP_TILE * c_out * 4, 0x00020000);
