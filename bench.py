@@ -23,6 +23,13 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
+# Every engine owns a HIP stream, and the HIP runtime spreads a process's streams over GPU_MAX_HW_QUEUES hardware queues
+# (4 unless the environment says otherwise). This process has up to five streams alive at a time (the engine of the timed
+# passes, three engines in rotation for the end-to-end figure, the default stream); two streams on one hardware queue
+# take turns, and the rotation then needs 2.55 ms per batch instead of 1.82 (measured both ways, and with 2 queues and no
+# extra engine: 2.55 ms as well). Read by the runtime when it starts, so it is set before anything touches HIP.
+os.environ.setdefault("GPU_MAX_HW_QUEUES", "8")
+
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 FP32_PEAK_TFLOPS = 157.3   # MI355X dense fp32 matrix
 BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix
@@ -85,6 +92,11 @@ def conv_roofline(name, avg_ms, rows):
     s_in = 2 if name.startswith("conv_bf16_bf16_") else 4
     s_out = 2 if "_tobf16_" in name else 4
     bytes_per_row = c_in * s_in + 4 * (slots - 1) + c_out * s_out
+    if name.startswith("neighbourhood_conv_"):
+        # the neighbourhood kernel with the first layer in it: the mesh's neighbour table read, the reverse-lookup gathers
+        # and the row's table written (4 bytes per neighbour each), then the layer's input and output rows; the table
+        # the layer gathers through is the one just written, so it is counted once
+        bytes_per_row = 12 * (slots - 1) + c_in * 4 + c_out * 4
     flops_per_row = 2 * slots * c_in * c_out
     intensity = flops_per_row / bytes_per_row
     matrix_peak = BF16_PEAK_TFLOPS if bf16_arith else FP32_PEAK_TFLOPS
@@ -202,6 +214,7 @@ def measure(cfg, engine, frames, steps, warmup, settle_s, events=True, stream_ce
     for _ in range(2):
         engine.run()              # untimed: the first run after a change of timing mode goes kernel by kernel, the second is captured
     kernel_ms, kernel_launches = {}, {}
+    dominant_ms_total = 0.0
     t0 = time.perf_counter()
     for _ in range(steps):
         engine.run()              # launches the whole path and waits for it
@@ -242,7 +255,7 @@ def measure(cfg, engine, frames, steps, warmup, settle_s, events=True, stream_ce
     # every graph-convolution kernel against its own roofline, from the one fully bracketed (untimed) pass
     conv_rooflines = {}
     for name, ms in sorted(kernel_ms_per_step.items()):
-        if name.startswith("conv"):
+        if name.startswith(("conv", "neighbourhood_conv")):
             entry = conv_roofline(name, ms / launches_per_step[name], rows)[0]
             conv_rooflines[name] = dict(bound=entry["bound"], achieved=entry["achieved"], unit=entry["unit"], frac=entry["frac"],
                                         avg_launch_ms=ms / launches_per_step[name])
@@ -252,7 +265,7 @@ def measure(cfg, engine, frames, steps, warmup, settle_s, events=True, stream_ce
     if stream_ceiling:
         from visualmesh_amd import native
         for name, entry in conv_rooflines.items():
-            if entry["bound"] != "hbm":
+            if entry["bound"] != "hbm" or name.startswith("neighbourhood_conv"):
                 continue
             shape = name.split("_")[-1]
             c_in, rest = shape.split("x")
@@ -264,9 +277,11 @@ def measure(cfg, engine, frames, steps, warmup, settle_s, events=True, stream_ce
             ceiling = (read_b + write_b) * ((rows + 63) // 64 * 64) / (ms * 1e-3) / 1e9
             entry["stream_ceiling_GBps"] = ceiling
             entry["frac_of_stream_ceiling"] = entry["achieved"] / ceiling
+    # the dominant kernel's launches inside the timed passes themselves, per pass: never more than ms_per_step
+    dominant_ms_total = sum(kernel_ms.values()) / steps if kernel_ms else None
     return dict(value=nodes * steps / elapsed, frames_per_s=len(frames) * steps / elapsed, ms_per_step=elapsed * 1e3 / steps, nodes=nodes,
                 settle_passes=settle_passes, settle_ms=settle_ms, roofline=roofline, kernel_ms_per_step=dict(sorted(kernel_ms_per_step.items())),
-                conv_rooflines=conv_rooflines)
+                conv_rooflines=conv_rooflines, dominant_kernel_ms_per_step_in_timed_passes=dominant_ms_total)
 
 
 def pinned_copies(cfg, mesh, lens):
@@ -282,6 +297,24 @@ def pinned_copies(cfg, mesh, lens):
         held.append(a)
         at += n
     return held, [dict(mesh=mesh, Hoc=f["Hoc"], lens=lens, image=a, fourcc=cfg.fourcc) for f, a in zip(cfg.frames, held)]
+
+
+def call_latency(index, repeats):
+    """One call of the reference's interface, engine(mesh, Hoc, lens, image, fourcc) -> ClassifiedMesh by value, on the
+    first frame of configuration `index`: host lookup, upload of the image, every kernel, download of the whole
+    classified mesh, timed inside the C++ host library (reference example/benchmark.cpp:50-58 times this call per frame).
+    From an image in ordinary (pageable) memory, as the reference's callers hold it, and from a page-locked one."""
+    from visualmesh_amd import native
+    cfg, engine, mesh, lens, frames = build_workload(index, 1)
+    f = cfg.frames[0]
+    pageable_ms, visible = engine.time_calls(mesh, f["Hoc"], lens, f["image"], cfg.fourcc, repeats)
+    held = native.pinned_empty(f["image"].shape, f["image"].dtype)
+    held[...] = f["image"]
+    locked_ms, _ = engine.time_calls(mesh, f["Hoc"], lens, held, cfg.fourcc, repeats)
+    stats = engine.graph_stats()
+    return dict(pageable_image_ms=pageable_ms, page_locked_image_ms=locked_ms, visible_nodes=visible, calls=repeats,
+                image_bytes=int(f["image"].nbytes), passes_as_graph_launches=stats["graph_launches"], passes_kernel_by_kernel=stats["eager_launches"],
+                what="one engine(mesh, Hoc, lens, image, fourcc) call on one frame: lookup + upload + kernels + download, results by value")
 
 
 def end_to_end(cfg, mesh, lens, nodes, batches):
@@ -336,6 +369,7 @@ def main():
     ap.add_argument("--no-copy-probe", action="store_true", help="skip the plain copy kernel")
     ap.add_argument("--no-pcie", action="store_true", help="skip the PCIe-inclusive figures (serial stage + run + fetch, and the pipelined end-to-end loop)")
     ap.add_argument("--no-configs", action="store_true", help="skip the short runs of the other configurations")
+    ap.add_argument("--no-calls", action="store_true", help="skip the single-call latencies (one engine(...) call per frame, configurations 1-5)")
     args = ap.parse_args()
     big = args.config in (4, 5, 6)
     args.steps = (50 if big else 1000) if args.steps is None else args.steps
@@ -349,12 +383,9 @@ def main():
     from visualmesh_amd import workloads as wl
 
     cfg, engine, mesh, lens, frames = build_workload(args.config, args.frames)
-    # PCIe-inclusive figures (never `value`), measured before anything else runs in this process: with an engine alive
-    # that ran a few passes before the rotation's engines were made, the rotation below takes 2.5-2.6 ms per batch instead
-    # of 1.86 ms on the same box (not a graph, event or stream-count effect; engines made the other way round, or that
-    # engine destroyed first, and it is gone), so these figures are taken with only their own engines alive.
-    # Serial: images in page-locked host memory -> stage + run + fetch of the whole classified mesh into one page-locked
-    # block, one engine, the three steps one after the other. Pipelined: end_to_end() above.
+    # PCIe-inclusive figures (never `value`). Serial: images in page-locked host memory -> stage + run + fetch of the whole
+    # classified mesh into one page-locked block, one engine, the three steps one after the other. Pipelined: end_to_end()
+    # above, with the serial figure's engine still alive beside the rotation's three (see GPU_MAX_HW_QUEUES at the top).
     pcie, e2e = None, None
     if not args.no_pcie:
         held, pinned_frames = pinned_copies(cfg, mesh, lens)
@@ -368,9 +399,8 @@ def main():
         dt = (time.perf_counter() - t0) / passes
         pcie = dict(ms_per_batch=dt * 1e3, nodes_per_s=nodes / dt, frames_per_s=len(frames) / dt,
                     what="stage from page-locked images + run + fetch (all frames' arrays gathered on the device, one copy into a page-locked block), one engine, serial")
-        del held, pinned_frames, engine
+        del held, pinned_frames
         e2e = end_to_end(cfg, mesh, lens, nodes, 12 if big else 60)
-        cfg, engine, mesh, lens, frames = build_workload(args.config, args.frames)
 
     nn = wl.N_NEIGHBOURS[cfg.model]
     m = measure(cfg, engine, frames, args.steps, args.warmup, args.settle, events=not args.no_events)
@@ -410,6 +440,11 @@ def main():
             pass
         cpu = dict(value=nps, unit="nodes/s", cores=threads, kind=kind, cpu_model=model, one_thread=one, frames_per_s=fps, seconds=dt, sample=note)
 
+    # the reference's own interface: one call per frame
+    calls = None
+    if not args.no_calls:
+        calls = {"cfg%d" % index: call_latency(index, 8 if index in (4, 5) else 50) for index in (1, 2, 3, 4, 5)}
+
     # the other configurations, briefly (device-resident like `value`; each one's dominant kernel against its roofline)
     others = None
     if not args.no_configs:
@@ -423,7 +458,9 @@ def main():
             r = measure(c, e, fr, 10 if heavy else 300, 2 if heavy else 30, 0.1 if heavy else args.settle, events=True, stream_ceiling=not heavy)
             others[c.name] = dict(workload=workload_name(c, len(fr), layer_table(c, wl.N_NEIGHBOURS[c.model])), dtype=DTYPE[c.precision],
                                   nodes_per_s=r["value"], frames_per_s=r["frames_per_s"], ms_per_step=r["ms_per_step"], steps=10 if heavy else 300,
-                                  visible_nodes_per_batch=r["nodes"], roofline=r["roofline"], conv_rooflines=r["conv_rooflines"])
+                                  visible_nodes_per_batch=r["nodes"], roofline=r["roofline"], conv_rooflines=r["conv_rooflines"],
+                                  dominant_kernel_ms_per_step_in_timed_passes=r["dominant_kernel_ms_per_step_in_timed_passes"],
+                                  kernel_ms_per_step_of_one_bracketed_pass=r["kernel_ms_per_step"])
             del e, fr, c
 
     out = {
@@ -448,13 +485,26 @@ def main():
             "settle_passes": m["settle_passes"],   # untimed, before the warm-up passes: the clocks settle
             "untimed_passes_after_warmup": 3,      # one with events around every kernel, two in which the timed passes' graph is captured
             "settle_ms": m["settle_ms"],
+            # the metric as the whole job sees it, beside `value` (which starts with the inputs resident in HBM):
+            "end_to_end_ms_per_batch": e2e["ms_per_batch"] if e2e else None,      # host images -> classified mesh in host arrays, three engines in rotation
+            "end_to_end_nodes_per_s": e2e["nodes_per_s"] if e2e else None,
+            "end_to_end_frames_per_s": e2e["frames_per_s"] if e2e else None,
+            "cpu_one_thread_nodes_per_s": cpu["one_thread"]["value"] if cpu and cpu.get("one_thread") else None,
+            "cpu_nodes_per_s": cpu["value"] if cpu else None,
+            "cpu_threads": cpu["cores"] if cpu else None,
+            # the layers bound by memory, as fractions of the 8 TB/s HBM peak by algorithmic bytes
+            "memory_bound_layers_frac_of_hbm_peak": {k: round(v["frac"], 4) for k, v in m["conv_rooflines"].items() if v["bound"] == "hbm"},
+            "matrix_bound_layers_frac_of_fp32_mfma_peak": {k: round(v["frac"], 4) for k, v in m["conv_rooflines"].items() if v["bound"] == "mfma"},
+            "call_ms": {k: {"pageable": round(v["pageable_image_ms"], 4), "page_locked": round(v["page_locked_image_ms"], 4)} for k, v in calls.items()} if calls else None,
+            "dominant_kernel_ms_per_step_in_timed_passes": m["dominant_kernel_ms_per_step_in_timed_passes"],
         },
         "roofline": m["roofline"],
         "cpu_baseline": cpu,
         "copy_kernel_GBps": copy_gbs,
         "end_to_end": e2e,
         "pcie_inclusive": pcie,
-        "kernel_ms_per_step": m["kernel_ms_per_step"],   # from the one fully profiled, untimed pass
+        "call_latency": calls,
+        "kernel_ms_per_step": m["kernel_ms_per_step"],   # from the one fully profiled, untimed pass (kernel by kernel, events around each: a few per cent slower than a timed pass)
         "conv_rooflines": m["conv_rooflines"],
         "configs": others,
     }

@@ -10,6 +10,7 @@
  * (libvisualmesh_host_f64.so: the same names with `real` = double and the _f64 structures of visualmesh_hip.h; the
  * parts of Engine<float> that Engine<double> does not offer - staged batches, lookup graphs, model files - are left out).
  */
+#include <chrono>
 #include <cstring>
 #include <memory>
 #include <stdexcept>
@@ -266,6 +267,26 @@ int vmh_engine_classify(vmh_engine* e, const vmh_mesh* m, const real* Hoc16, con
         const int V = export_result(r, cap, px, nb, gidx);
         if (V > 0 && cls) std::memcpy(cls, r.classifications.data(), sizeof(real) * r.classifications.size());
         return V;
+    })
+}
+
+/* Average wall-clock milliseconds of `repeats` calls of engine(mesh, Hoc, lens, image, fourcc), results returned by value
+ * and dropped: what one call of the reference's interface costs a C++ caller (reference example/benchmark.cpp:50-58
+ * times exactly this). One untimed call comes first. */
+int vmh_engine_time_calls(vmh_engine* e, const vmh_mesh* m, const real* Hoc16, const vmh_lens_t* lens, const void* image,
+                          uint32_t fourcc, int repeats, double* ms_per_call) {
+    GUARD({
+        size_t visible = 0;
+        const auto Hoc = to_hoc(Hoc16);
+        const auto L = to_lens(lens);
+        std::chrono::steady_clock::time_point t0;
+        for (int i = -1; i < repeats; ++i) {
+            if (i == 0) t0 = std::chrono::steady_clock::now();
+            if (m->r6) visible += (*e->engine)(*m->r6, Hoc, L, image, fourcc).global_indices.size();
+            else visible += (*e->engine)(*m->g8, Hoc, L, image, fourcc).global_indices.size();
+        }
+        *ms_per_call = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count() / (repeats > 0 ? repeats : 1);
+        return int(visible / size_t(repeats + 1));
     })
 }
 

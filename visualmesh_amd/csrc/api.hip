@@ -23,6 +23,7 @@ std::atomic<float> g_debug_px_error{0.0f};
 std::atomic<bool> g_debug_wide_offsets{false};
 std::atomic<int> g_debug_stamp_row_bits{0};
 std::atomic<float> g_debug_edge_band{VMHIP_AMB_EPS_DEFAULT};
+std::atomic<int> g_live_engines{0}; /* engines alive in the process, each with a stream of its own */
 
 int fail(int code, const std::string& msg) {
     g_error = msg;
@@ -121,6 +122,7 @@ struct vmhip_engine {
     int32_t max_width = 4;
     std::vector<HostLayer> layers;
     hipStream_t stream = nullptr;
+    bool counted = false;           /* in g_live_engines */
     vmhip_batch* scratch = nullptr; /* used by the one-call entry points */
 };
 
@@ -1096,6 +1098,19 @@ int vmhip_engine_create(const vmhip_network* net, int32_t n_neighbours, int32_t 
         }
     }
     if (hipStreamCreateWithFlags(&E->stream, hipStreamNonBlocking) != hipSuccess) return bail(VMHIP_ERR_HIP, "engine_create: stream creation failed");
+    /* Every engine owns a stream, and the runtime spreads the process's streams over GPU_MAX_HW_QUEUES hardware queues (4
+     * unless the environment says otherwise). Streams that share a queue take turns: three engines in rotation lose 40 %
+     * (2.55 ms per batch instead of 1.82) when a fourth engine's stream makes two of them share. Said once. */
+    {
+        const char* q = getenv("GPU_MAX_HW_QUEUES");
+        const int queues = q && atoi(q) > 0 ? atoi(q) : 4;
+        static std::atomic<bool> said{false};
+        if (++g_live_engines + 1 > queues && !said.exchange(true)) /* + 1: the default stream */
+            fprintf(stderr, "libvisualmesh_hip: %d engines are alive, each with a stream of its own, on %d hardware queues: engines that work at the same "
+                            "time will take turns; set GPU_MAX_HW_QUEUES to at least the number of engines + 1 before the process starts\n",
+                    g_live_engines.load(), queues);
+    }
+    E->counted = true;
     *out = E;
     return VMHIP_OK;
 }
@@ -1110,6 +1125,7 @@ void vmhip_engine_destroy(vmhip_engine* E) {
         if (L.d_w_flow) (void) hipFree(L.d_w_flow);
     }
     if (E->stream) (void) hipStreamDestroy(E->stream);
+    if (E->counted) --g_live_engines;
     delete E;
 }
 

@@ -143,6 +143,16 @@ class Engine:
             return self.project(mesh, Hoc, lens)
         return self.classify(mesh, Hoc, lens, image, fcc)
 
+    def time_calls(self, mesh, Hoc, lens, image, fcc, repeats=50):
+        """(average milliseconds of one C++ call engine(mesh, Hoc, lens, image, fourcc) with its results returned by value,
+        visible nodes): the calls are made and timed inside the C++ host library, one untimed call first"""
+        m = self._pick(mesh, Hoc)
+        H = np.ascontiguousarray(Hoc, dtype=np.float32)
+        img = np.ascontiguousarray(image)
+        ms = C.c_double(0.0)
+        V = native.host_check(self._lib.vmh_engine_time_calls(self.ptr, m.ptr, _fp(H), C.byref(lens), img.ctypes.data, fcc, repeats, C.byref(ms)))
+        return float(ms.value), V
+
     # ---- staged batches
     def stage(self, frames, wait=True):
         """frames: list of dict(mesh=Mesh|VisualMesh, Hoc, lens, image, fourcc); copies the inputs to the device.

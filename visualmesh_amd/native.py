@@ -323,6 +323,7 @@ def host():
                                      C.POINTER(C.c_int32), C.POINTER(C.c_int32)]
     L.vmh_engine_classify.argtypes = [vp, vp, C.POINTER(C.c_float), C.POINTER(Lens), vp, C.c_uint32, C.c_int,
                                       C.POINTER(C.c_float), C.POINTER(C.c_int32), C.POINTER(C.c_int32), C.POINTER(C.c_float)]
+    L.vmh_engine_time_calls.argtypes = [vp, vp, C.POINTER(C.c_float), C.POINTER(Lens), vp, C.c_uint32, C.c_int, C.POINTER(C.c_double)]
     L.vmh_engine_stage.argtypes = [vp, C.c_int, C.POINTER(vp), C.POINTER(C.c_float), C.POINTER(Lens), C.POINTER(vp),
                                    C.POINTER(C.c_uint32), C.c_int]
     L.vmh_engine_run.argtypes = [vp]
