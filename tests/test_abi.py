@@ -110,11 +110,13 @@ def test_engine_can_be_compiled_out():
     assert done.returncode == 0, done.stdout[-2000:]
 
 
-def test_bf16_kernels_with_weights_in_accumulation_registers_do_not_spill(tmp_path):
-    """conv_bf16.hip places the weights of most instantiations in accumulation registers (an "a" constraint); the ones that
-    spill to scratch memory gave wrong results that way and are excluded in the source (tanh, fp32 rows in). The excluded
-    set must cover every instantiation that spills: compile the file to assembly with the library's flags and check each
-    kernel's scratch segment against where its matrix instructions read the weights from."""
+def test_bf16_kernels_do_not_spill(tmp_path):
+    """conv_bf16.hip places the weights of nearly all instantiations in accumulation registers (an "a" constraint). A
+    kernel that spills with its weights placed like that gets wrong results from this compiler: a weight's four
+    registers go to scratch as three words plus one word parked in a vector register, and only the three come back
+    before the matrix instruction reads all four. So no instantiation may have a scratch segment at all, pinned or not
+    (the hand-counted waits of the kernel also assume that the compiler adds no memory traffic of its own): compile the
+    file to assembly with the library's flags and check every kernel, and that the weights are where the source says."""
     import subprocess
     from visualmesh_amd import build as vm_build
     out = tmp_path / "conv_bf16.s"
@@ -124,14 +126,14 @@ def test_bf16_kernels_with_weights_in_accumulation_registers_do_not_spill(tmp_pa
     text = out.read_text()
     checked = 0
     for m in re.finditer(r"\n(_ZN12_GLOBAL__N_119vm_conv_bf16_kernelILi7ELi(\d)ELi(\d)ELi(\d)EEEv\S+?):", text):
-        name, rows_in, activation = m.group(1), int(m.group(2)), int(m.group(4))
+        name, rows_in, rows_out, activation = m.group(1), int(m.group(2)), int(m.group(3)), int(m.group(4))
         body = text[m.end():text.index(".Lfunc_end", m.end())]
         from_agprs = sum(1 for line in body.splitlines() if line.strip().startswith("v_mfma") and line.split(",")[1].strip().startswith("a["))
         total = sum(1 for line in body.splitlines() if line.strip().startswith("v_mfma"))
         scratch = int(re.search(r"\.private_segment_fixed_size:\s+(\d+)", text[text.index(".name:           " + name):]).group(1))
-        expected_in_agprs = rows_in != 0 and activation != 3
+        expected_in_agprs = not (rows_in == 0 and rows_out == 2 and activation in (0, 3))
         assert (from_agprs > total // 2) == expected_in_agprs, (name, from_agprs, total)
-        if expected_in_agprs:
-            assert scratch == 0, name + " spills with its weights in accumulation registers"
+        assert scratch == 0, name + " spills"
+        assert "Folded Reload" not in body and "scratch_" not in body, name
         checked += 1
     assert checked == 36

@@ -414,6 +414,38 @@ def test_bf16_layer_variants(oracle, variant, monkeypatch):
         assert_classification_parity(got, want, BF16_TOL, "bf16 " + variant)
 
 
+@pytest.mark.parametrize("variant", ["fp32_rows_in", "relu_tanh", "tanh_only"])
+def test_bf16_layer_variants_without_a_rounded_boundary(oracle, variant, monkeypatch):
+    """The same less travelled instantiations with every boundary between the bf16 layers as hi + lo pairs
+    (VMHIP_BF16_ROUNDED=0): nothing is rounded to bf16 then, so the results must be within 1e-3 of the fp32 oracle - a
+    gate that a residual error of a kernel (a wrong operand, a lost register) could not hide behind the way it could
+    behind the 1e-2 of a rounded boundary. tanh_only: tanh after every layer, through kernels that read fp32 rows, hi + lo
+    rows and write both."""
+    monkeypatch.setenv("VMHIP_BF16_ROUNDED", "0")
+    if variant == "fp32_rows_in":
+        monkeypatch.setenv("VMHIP_CONV_KERNEL", "mfma")
+    cfg = wl.config(1, n_frames=1)
+    rng = np.random.default_rng(78)
+    net = wl.glorot_network(rng, [3, 64, 64, 64, 64, 4], 6, wl.SELU)
+    if variant == "relu_tanh":
+        net = [[(w, b, a if a == wl.SOFTMAX else (wl.RELU if i % 2 == 0 else wl.TANH)) for (w, b, a) in g] for i, g in enumerate(net)]
+    if variant == "tanh_only":
+        net = [[(w, b, a if a == wl.SOFTMAX else wl.TANH) for (w, b, a) in g] for g in net]
+    o_lens, e_lens = lens_pair(cfg)
+    o_mesh, e_mesh = meshes_for(cfg, oracle)
+    engine = eng.Engine(net, cfg.model, precision=native.BF16)
+    f = cfg.frames[0]
+    got = engine(e_mesh, f["Hoc"], e_lens, f["image"], cfg.fourcc)
+    engine.profile(True)
+    engine.run()
+    names = [n for n, _, _ in engine.profile_read() if n.startswith("conv")]
+    assert sum(n.startswith("conv_bf16_") for n in names) == 3 and not any("_tobf16_" in n or "_bf16_bf16_" in n for n in names), names
+    want = o_mesh.classify(f["Hoc"], o_lens, f["image"], cfg.fourcc, vmo.Network(net))
+    worst = float(np.abs(got["cls"] - want["cls"]).max())
+    print("bf16 %s without a rounded boundary, worst absolute error: %.3e" % (variant, worst), flush=True)
+    assert_classification_parity(got, want, 1e-3, "bf16 " + variant + ", no rounded boundary")
+
+
 def test_bf16_engine_keeps_narrow_networks_in_fp32(oracle):
     """Rows narrower than 64 channels are not worth bf16 storage (one rounding already costs ~1e-2 on a 3-class
     softmax): a bf16 engine built on configuration 2's network meets the fp32 gate."""

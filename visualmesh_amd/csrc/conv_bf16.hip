@@ -100,6 +100,15 @@ __device__ __forceinline__ float selu(float s) {
     return lambda * (s >= 0.0f ? s : __builtin_fmaf(alpha, __builtin_amdgcn_exp2f(s * 1.44269504088896340736f), -alpha));
 }
 
+/* tanh(x) = 1 - 2 / (e^(2x) + 1) with the hardware exponential and reciprocal: within ~3e-7 absolute of the correctly
+ * rounded result over the whole range (e^(2x) overflows to infinity and underflows to zero where tanh is +-1), in a
+ * handful of instructions and two registers - the library routine's polynomial needs enough of both to push the kernel's
+ * working set out of the register file */
+__device__ __forceinline__ float fast_tanh(float x) {
+    const float t = __builtin_amdgcn_exp2f(x * 2.88539008177792681472f); /* 2 log2 e */
+    return __builtin_fmaf(-2.0f, __builtin_amdgcn_rcpf(t + 1.0f), 1.0f);
+}
+
 /* two floats -> two bf16 in one word, round to nearest even (v_cvt_pk_bf16_f32) */
 __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
     typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
@@ -236,11 +245,16 @@ __global__ __launch_bounds__(256) void vm_conv_bf16_kernel(VmBatchDev B, VmLayer
      * say where the weights live: in accumulation registers ("a"), from which the matrix instruction reads them as well
      * as from vector registers. Left to itself the compiler keeps the 224 weight registers in the vector file and moves
      * everything else in and out of accumulation registers around each use (822 such moves in the kernel against 176, a
-     * sixth of its instructions; 4-5 % of its time). Only the instantiations that fit the register file get this: the
-     * ones that spill to scratch memory (tanh, fp32 rows in) gave wrong results with it and keep the weights where the
-     * compiler puts them; tests/test_abi.py checks that no instantiation with weights in accumulation registers has a
-     * scratch segment. */
-    constexpr bool WEIGHTS_IN_AGPRS = IN_FMT != VM_ROWS_F32 && ACT != VMHIP_TANH;
+     * sixth of its instructions; 4-5 % of its time).
+     * No instantiation may spill to scratch memory. With the weights placed like this the compiler (ROCm 7.2's clang)
+     * spills a weight's four registers as three words to scratch plus one word kept in a spare vector register, and at
+     * the use reloads the three words only (scratch_load_dwordx3 v[24:26], then v_mfma ... v[24:27]): the matrix
+     * instruction multiplies with whatever the fourth register last held, and the results are garbage, NaNs included.
+     * That is what instantiations with a library tanh did (its polynomial's registers pushed 18 to 30 values out); with
+     * fast_tanh above they all fit. The two that still do not (fp32 rows in, hi + lo rows out, selu or tanh: the splitting of
+     * rows in registers on top of the widest epilogue) keep the weights where the compiler puts them, and fit that way.
+     * tests/test_abi.py compiles this file and checks that none of the 36 kernels has a scratch segment. */
+    constexpr bool WEIGHTS_IN_AGPRS = !(IN_FMT == VM_ROWS_F32 && OUT_FMT == VM_ROWS_BF16X2 && (ACT == VMHIP_SELU || ACT == VMHIP_TANH));
 #pragma unroll
     for (int s = 0; s < SLOTS; ++s)
 #pragma unroll
@@ -364,7 +378,7 @@ __global__ __launch_bounds__(256) void vm_conv_bf16_kernel(VmBatchDev B, VmLayer
             if constexpr (ACT != VMHIP_SOFTMAX) {
                 const int rb = i >> 4, v = i & 15;
                 const float x = a[rb][v];
-                a[rb][v] = ACT == VMHIP_SELU ? selu(x) : ACT == VMHIP_RELU ? fmaxf(x, 0.0f) : tanhf(x);
+                a[rb][v] = ACT == VMHIP_SELU ? selu(x) : ACT == VMHIP_RELU ? fmaxf(x, 0.0f) : fast_tanh(x);
             }
         }
         else if (i < N_SLICES) {
