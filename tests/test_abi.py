@@ -100,6 +100,28 @@ def test_engine_header_compiles_against_the_references_own_headers():
     assert "visualmesh_amd/cpp/visualmesh/mesh.hpp" not in deps, deps
 
 
+@pytest.mark.skipif(not os.path.isdir(os.path.join(REFERENCE_CPP, "visualmesh")), reason="the reference tree is not mounted here")
+def test_converting_constructors_match_the_references(tmp_path):
+    """Mesh<float>(Mesh<double>), Mesh<double>(Mesh<float>) and VisualMesh<float>(VisualMesh<double>) (reference
+    mesh.hpp:476-488, visualmesh.hpp:104-110): one source compiled against the host headers here and against the
+    reference's; nodes, neighbours and the lookup ranges of the converted meshes must come out the same, bit for bit."""
+    import subprocess
+    from visualmesh_amd import build as vm_build
+    src = os.path.join(ROOT, "tests", "native", "convert_scalar.cpp")
+    printed = []
+    for name, include in (("ours", os.path.join(ROOT, "visualmesh_amd", "cpp")), ("reference", REFERENCE_CPP)):
+        exe = str(tmp_path / ("convert_" + name))
+        flags = [f for f in vm_build.HOST_EXACT_FLAGS if f not in ("-fPIC", "-Wall", "-Wextra")]
+        subprocess.run(["g++"] + flags + ["-I" + include, src, "-o", exe], check=True)
+        printed.append(subprocess.run([exe], stdout=subprocess.PIPE, universal_newlines=True, check=True).stdout)
+    assert printed[0] == printed[1]
+    lines = printed[0].splitlines()
+    assert len(lines) == 30 and all("ranges 0:" not in line for line in lines if "lens 0" in line), printed[0]
+    # a converted mesh keeps the node count of the mesh it came from, not of one generated in its own scalar type
+    count = {line.split(" nodes ")[0]: int(line.split(" nodes ")[1].split()[0]) for line in lines if " nodes " in line}
+    assert count["double->float"] == count["double"] and count["float->double"] == count["float"]
+
+
 def test_engine_can_be_compiled_out():
     """VISUALMESH_DISABLE_HIP (what cmake/HipEngine.cmake defines when BUILD_HIP_ENGINE is off, as the reference does for
     its OpenCL and Vulkan engines) leaves an empty header: nothing of the HIP library is needed then."""

@@ -89,6 +89,72 @@ def test_multi_layer_groups_and_all_activations(oracle):
         assert_classification_parity(got, want, PROB_TOL, name)
 
 
+def test_a_four_neighbour_model_runs_on_the_matrix_cores(oracle):
+    """The reference's four-neighbour models (model/ring4.hpp, xygrid4.hpp, xmgrid4.hpp, nmgrid4.hpp) gather five slots.
+    A mesh with four columns of neighbours (the first four of a Ring6 mesh's, so that neighbours stay close) goes through
+    vmhip_classify with a network whose layers land on the fused first layer (4 -> 16), the LDS-gather kernel (16 -> 40,
+    12 -> 5) and the register-gather kernel (40 -> 12), all in their five-slot instantiations. Checked against the
+    definition (engine/cpu/engine.hpp:205-264): the neighbourhood table from the visible set, the sampled inputs from the
+    oracle's interpolate on the returned pixels, the layers in float64."""
+    import ctypes as C
+    L = native.hip()
+    rng = np.random.default_rng(44)
+    mesh = eng.Mesh(wl.RING6, wl.SPHERE, 0.0949, 1.0, 4.0, 8.0)
+    rays, nbr6 = mesh.arrays()
+    nn = 4
+    nbr = np.ascontiguousarray(nbr6[:, :nn])
+    W, H = 320, 256
+    lens = native.make_lens(W, H, wl.EQUISOLID, 105.0, math.pi)
+    Hoc = np.ascontiguousarray(wl.make_hoc(1.0, math.radians(40.0), 0.02, 0.3), dtype=np.float32)
+    ranges = np.ascontiguousarray(mesh.lookup(Hoc, lens), dtype=np.int32)
+    n_cand = int((ranges[:, 1] - ranges[:, 0]).sum())
+    Rco = np.ascontiguousarray(Hoc[:3, :3].T)
+    image = wl.random_image(rng, W, H, 4)
+    groups = wl.glorot_network(rng, [3, 16, 40, 12, 5], nn, wl.SELU)
+    net = native.Network(groups)
+    engine, handle = C.c_void_p(), C.c_void_p()
+    native.hip_check(L.vmhip_engine_create(C.byref(net.c), nn, native.FP32, C.byref(engine)))
+    native.hip_check(L.vmhip_mesh_upload(rays.ctypes.data_as(C.POINTER(C.c_float)), nbr.ctypes.data_as(C.POINTER(C.c_int32)), mesh.n_nodes, nn, C.byref(handle)))
+    px = np.zeros((n_cand, 2), np.float32)
+    gidx = np.zeros(n_cand, np.int32)
+    nb = np.full((n_cand + 1, nn), -1, np.int32)
+    cls = np.zeros((n_cand + 1, 5), np.float32)
+    frame = native.Frame(handle, (C.c_float * 9)(*Rco.ravel()), lens, ranges.ctypes.data_as(C.POINTER(C.c_int32)), len(ranges),
+                         image.ctypes.data, wl.fourcc("RGBA"), None)
+    result = native.Result(n_cand, 0, px.ctypes.data_as(C.POINTER(C.c_float)), gidx.ctypes.data_as(C.POINTER(C.c_int32)),
+                           nb.ctypes.data_as(C.POINTER(C.c_int32)), cls.ctypes.data_as(C.POINTER(C.c_float)))
+    native.hip_check(L.vmhip_classify(engine, C.byref(frame), C.byref(result)))
+    V = result.n_visible
+    assert V > 500
+    row_of = np.full(mesh.n_nodes + 1, V, np.int32)
+    row_of[gidx[:V]] = np.arange(V, dtype=np.int32)
+    want_nb = np.concatenate([row_of[nbr[gidx[:V]]], np.full((1, nn), V, np.int32)])
+    assert np.array_equal(nb[:V + 1], want_nb)
+    # the network by its definition, in float64
+    x = np.concatenate([np.stack([oracle.fn_interpolate(px[i], image, W, H, wl.fourcc("RGBA")) for i in range(V)]), -np.ones((1, 4), np.float32)]).astype(np.float64)
+    for (w, b, act), in groups:
+        gathered = np.concatenate([x] + [x[want_nb[:, j]] for j in range(nn)], axis=1)
+        x = gathered @ w.astype(np.float64) + b.astype(np.float64)
+        if act == wl.SELU:
+            x = 1.0507009873554804934193349852946 * np.where(x >= 0, x, 1.6732632423543772848170429916717 * np.exp(x) - 1.6732632423543772848170429916717)
+        else:
+            x = np.exp(x) / np.exp(x).sum(axis=1, keepdims=True)
+    worst = float(np.abs(cls[:V + 1] - x).max())
+    print("four-neighbour model: V = %d, worst absolute probability error %.3e" % (V, worst), flush=True)
+    assert worst <= 1e-4
+    # which kernels ran: a staged batch of the same frame with profiling on
+    batch = C.c_void_p()
+    native.hip_check(L.vmhip_batch_create(engine, C.byref(batch)))
+    native.hip_check(L.vmhip_batch_stage(batch, C.byref(frame), 1, 1))
+    native.hip_check(L.vmhip_batch_profile(batch, 1))
+    native.hip_check(L.vmhip_batch_run(batch))
+    names = [n for n, _, _ in native.profile_read(batch)]
+    assert names[2:6] == ["neighbourhood_conv_4x16s5", "conv_lds_16x40s5", "conv_mfma_40x12s5", "conv_lds_12x5s5"], names
+    L.vmhip_batch_destroy(batch)
+    L.vmhip_mesh_release(handle)
+    L.vmhip_engine_destroy(engine)
+
+
 def test_frames_that_see_nothing(oracle):
     """engine/cpu/engine.hpp:193: nothing visible is not an error, the result is empty - for the single calls, and for
     such a frame at the start, in the middle and at the end of a batch whose other frames are ordinary."""

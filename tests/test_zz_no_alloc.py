@@ -137,3 +137,87 @@ def test_projection_without_allocation_matches_vmhip_project():
     for h in handles:
         L.vmhip_mesh_release(h)
     L.vmhip_engine_destroy(engine)
+
+
+def test_projection_without_allocation_inside_a_captured_graph():
+    """The use the entry point names first: one call captured into a HIP graph on a stream of the caller's, replayed
+    past the point where the 8-bit run stamp starts again (255 calls), with eager calls on another input and waits
+    between the replays. Every replay checked leaves vmhip_project's outputs; a frame without candidates leaves a
+    visible count of zero and its null row."""
+    hip_runtime = C.CDLL("libamdhip64.so")
+    for fn in ("hipStreamCreate", "hipStreamBeginCapture", "hipStreamEndCapture", "hipGraphInstantiate", "hipGraphLaunch", "hipStreamSynchronize",
+               "hipGraphExecDestroy", "hipGraphDestroy", "hipStreamDestroy"):
+        getattr(hip_runtime, fn).restype = C.c_int
+    hip_runtime.hipStreamBeginCapture.argtypes = [C.c_void_p, C.c_int]
+    hip_runtime.hipStreamEndCapture.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
+    hip_runtime.hipGraphInstantiate.argtypes = [C.POINTER(C.c_void_p), C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]
+    hip_runtime.hipGraphLaunch.argtypes = [C.c_void_p, C.c_void_p]
+    hip_runtime.hipStreamSynchronize.argtypes = [C.c_void_p]
+    hip_runtime.hipGraphExecDestroy.argtypes = [C.c_void_p]
+    hip_runtime.hipGraphDestroy.argtypes = [C.c_void_p]
+    hip_runtime.hipStreamDestroy.argtypes = [C.c_void_p]
+
+    L = native.hip()
+    empty = native.Network([])
+    engine = C.c_void_p()
+    native.hip_check(L.vmhip_engine_create(C.byref(empty.c), 6, native.FP32, C.byref(engine)))
+    mesh = eng.Mesh(wl.RING6, wl.SPHERE, 0.0949, 1.0, 3.0, 8.0)
+    other = eng.Mesh(wl.RING6, wl.SPHERE, 0.0949, 1.2, 4.0, 10.0)
+    handles = []
+    for m in (mesh, other):
+        rays, nbr = m.arrays()
+        h = C.c_void_p()
+        native.hip_check(L.vmhip_mesh_upload(_fp(rays), _ip(nbr), m.n_nodes, m.n_neighbours, C.byref(h)))
+        handles.append(h)
+    lens = native.make_lens(320, 256, wl.RECTILINEAR, 180.0, math.pi / 2)
+    Hoc = wl.make_hoc(1.0, math.radians(50.0), math.radians(-4.0), math.radians(1.0))
+    Hoc_other = wl.make_hoc(1.2, math.radians(35.0), math.radians(2.0), math.radians(-3.0))
+    want, got, (ranges, n_cand) = _both_ways(L, engine, handles[0], mesh, Hoc, lens)
+    _assert_same(want, got, "eager call")
+    V = want["V"]
+    assert V > 100
+
+    nn = mesh.n_neighbours
+    d_ranges = native.pinned_empty(ranges.shape, np.int32)
+    d_ranges[...] = ranges
+    d_V = native.pinned_empty((1,), np.int32)
+    d_px = native.pinned_empty((n_cand, 2), np.float32)
+    d_gidx = native.pinned_empty((n_cand,), np.int32)
+    d_nb = native.pinned_empty((n_cand + 1, nn), np.int32)
+    out = ProjectionDevice(n_cand, _ip(d_V), _fp(d_px), _ip(d_gidx), _ip(d_nb))
+    Rco = np.ascontiguousarray(np.asarray(Hoc, np.float32)[:3, :3].T)
+
+    stream, graph, graph_exec = C.c_void_p(), C.c_void_p(), C.c_void_p()
+    assert hip_runtime.hipStreamCreate(C.byref(stream)) == 0
+    assert hip_runtime.hipStreamBeginCapture(stream, 1) == 0  # hipStreamCaptureModeThreadLocal
+    rc = L.vmhip_project_noalloc(handles[0], _fp(Rco), C.byref(lens), _ip(d_ranges), len(ranges), n_cand, C.byref(out), stream)
+    assert hip_runtime.hipStreamEndCapture(stream, C.byref(graph)) == 0
+    native.hip_check(rc)
+    assert hip_runtime.hipGraphInstantiate(C.byref(graph_exec), graph, None, None, 0) == 0
+    for replay in range(300):
+        checked = replay < 4 or replay % 50 == 0 or 250 <= replay < 262 or replay == 299
+        if checked:
+            d_V[0] = -7
+            d_px[...] = np.nan
+            d_gidx[...] = -1
+            d_nb[...] = -1
+        assert hip_runtime.hipGraphLaunch(graph_exec, stream) == 0
+        assert hip_runtime.hipStreamSynchronize(stream) == 0
+        if checked:
+            got = dict(V=int(d_V[0]), px=d_px[:V].copy(), gidx=d_gidx[:V].copy(), nb=d_nb[:V + 1].copy())
+            _assert_same(want, got, "replay %d" % replay)
+            # an eager call on another mesh and view between the replays: it shares the workspace, not the outputs
+            w2, g2, _ = _both_ways(L, engine, handles[1], other, Hoc_other, lens)
+            _assert_same(w2, g2, "eager call after replay %d" % replay)
+    assert hip_runtime.hipGraphExecDestroy(graph_exec) == 0 and hip_runtime.hipGraphDestroy(graph) == 0 and hip_runtime.hipStreamDestroy(stream) == 0
+
+    # no candidates at all: a visible count of zero and the null row, nothing else
+    d_V[0] = -7
+    d_nb[...] = -1
+    native.hip_check(L.vmhip_project_noalloc(handles[0], _fp(Rco), C.byref(lens), _ip(d_ranges), 0, 0, C.byref(out), None))
+    _device_wait()
+    assert int(d_V[0]) == 0 and (d_nb[0] == 0).all() and (d_nb[1:] == -1).all()
+
+    for h in handles:
+        L.vmhip_mesh_release(h)
+    L.vmhip_engine_destroy(engine)

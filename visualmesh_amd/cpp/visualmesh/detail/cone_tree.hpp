@@ -65,6 +65,23 @@ namespace detail {
 
         const std::vector<Element>& elements() const { return elements_; }
 
+        ConeTreeT() = default;
+        /// The same tree over another scalar type: ranges and children as they are, every cone's axis, cosine and sine
+        /// converted value by value (what reference mesh.hpp:476-488 does with its bsp entries).
+        template <typename U>
+        explicit ConeTreeT(const ConeTreeT<U>& other) {
+            elements_.reserve(other.elements().size());
+            for (const typename ConeTreeT<U>::Element& e : other.elements()) {
+                Element mine;
+                mine.first = e.first, mine.last = e.last;
+                mine.child[0] = e.child[0], mine.child[1] = e.child[1];
+                mine.cone.axis = vec3<T>{{static_cast<T>(e.cone.axis[0]), static_cast<T>(e.cone.axis[1]), static_cast<T>(e.cone.axis[2])}};
+                mine.cone.c = static_cast<T>(e.cone.c);
+                mine.cone.s = static_cast<T>(e.cone.s);
+                elements_.push_back(mine);
+            }
+        }
+
         /// What a walk of the tree compares an element against, for one camera pose: the field-of-view cone and the
         /// four cones (or planes) along the screen edges. visible_ranges() works these out for itself; a walk that
         /// runs elsewhere (on the device) is handed them.

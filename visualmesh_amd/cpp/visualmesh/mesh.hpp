@@ -52,6 +52,21 @@ public:
         }
     }
 
+    /// A mesh of another scalar type converted to this one (reference mesh.hpp:476-488): same nodes in the same order with
+    /// their unit vectors converted value by value, same neighbours, same tree with converted cones. Note that this is
+    /// not the mesh that generating in this scalar type would give (ring sizes come from ceil() of quotients in Scalar).
+    template <typename U>
+    Mesh(const Mesh<U, Model>& other)
+      : h(static_cast<Scalar>(other.h)), max_distance(static_cast<Scalar>(other.max_distance)), tree_(other.tree()) {
+        nodes.reserve(other.nodes.size());
+        for (const auto& n : other.nodes) {
+            node_type mine;
+            mine.ray = vec3<Scalar>{{static_cast<Scalar>(n.ray[0]), static_cast<Scalar>(n.ray[1]), static_cast<Scalar>(n.ray[2])}};
+            for (int t = 0; t < N_NEIGHBOURS; ++t) mine.neighbours[t] = n.neighbours[t];
+            nodes.push_back(mine);
+        }
+    }
+
     /// Index ranges [first, last) of nodes that may be on screen, ascending and disjoint.
     std::vector<std::pair<int, int>> lookup(const mat4<Scalar>& Hoc, const Lens<Scalar>& lens) const {
         return tree_.visible_ranges([this](int i) -> const vec3<Scalar>& { return nodes[i].ray; }, Hoc, lens);

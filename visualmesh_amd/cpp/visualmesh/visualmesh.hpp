@@ -46,6 +46,13 @@ public:
         }
     }
 
+    /// A VisualMesh of another scalar type converted to this one (reference visualmesh.hpp:104-110): every height and
+    /// every mesh converted (Mesh's converting constructor).
+    template <typename U>
+    VisualMesh(const VisualMesh<U, Model>& other) {
+        for (const auto& entry : other.meshes()) luts.emplace(static_cast<Scalar>(entry.first), Mesh<Scalar, Model>(entry.second));
+    }
+
     /// The mesh generated for the height closest to `height`; ties go to the lower mesh.
     const Mesh<Scalar, Model>& height(const Scalar& height) const {
         auto it = luts.lower_bound(height);

@@ -508,7 +508,9 @@ int launch_lds(const VmBatchDev& B, const VmLayerDev& L, const float* in, float*
  * instantiations that know the input width and the number of 16-channel column blocks, and read the exact number of
  * output channels at run time (reference engine/opencl/operation/make_network.hpp:43-214 generates a kernel for any
  * shape). X(C_in, column blocks, slots). */
-#define VM_LDS_ANY_WIDTHS(X, CI) X(CI, 1, 7) X(CI, 2, 7) X(CI, 3, 7) X(CI, 4, 7) X(CI, 1, 9) X(CI, 2, 9) X(CI, 3, 9) X(CI, 4, 9)
+/* 7 and 9 gather slots: the six- and eight-neighbour models (Ring6, NMGrid8 ...); 5: the four-neighbour ones
+ * (reference model/ring4.hpp, xygrid4.hpp, xmgrid4.hpp, nmgrid4.hpp) */
+#define VM_LDS_ANY_WIDTHS(X, CI) X(CI, 1, 7) X(CI, 2, 7) X(CI, 3, 7) X(CI, 4, 7) X(CI, 1, 9) X(CI, 2, 9) X(CI, 3, 9) X(CI, 4, 9) X(CI, 1, 5) X(CI, 2, 5) X(CI, 3, 5) X(CI, 4, 5)
 #define VM_FOR_EACH_LDS_ANY_SHAPE(X) \
     VM_LDS_ANY_WIDTHS(X, 4)          \
     VM_LDS_ANY_WIDTHS(X, 8)          \
@@ -524,7 +526,7 @@ bool vm_lds_supported(int c_in, int c_out, int slots, int out_fmt) {
     if (c_in == CI && c_out == CO && slots == SL) return true;
     if (out_fmt == VM_ROWS_F32) {
         VM_FOR_EACH_LDS_SHAPE(X)
-        return c_in % 4 == 0 && c_in >= 4 && c_in <= 32 && c_out >= 1 && c_out <= 64 && (slots == 7 || slots == 9);
+        return c_in % 4 == 0 && c_in >= 4 && c_in <= 32 && c_out >= 1 && c_out <= 64 && (slots == 5 || slots == 7 || slots == 9);
     }
     else if (out_fmt == VM_ROWS_BF16X2) {
         VM_FOR_EACH_LDS_SPLIT_SHAPE(X)

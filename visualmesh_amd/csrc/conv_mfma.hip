@@ -423,7 +423,7 @@ void vm_mfma_permute_weights(const float* w, int c_in, int c_out, int slots, voi
 /* Every other shape with input rows of 36 to 64 channels (whole 16-byte pieces) and up to 64 output channels:
  * instantiations that know the input width and the number of 16-channel column blocks and read the exact number of
  * output channels at run time; narrower input rows are conv_lds.hip's. X(C_in, column blocks, slots). */
-#define VM_MFMA_ANY_WIDTHS(X, CI) X(CI, 1, 7) X(CI, 2, 7) X(CI, 3, 7) X(CI, 4, 7) X(CI, 1, 9) X(CI, 2, 9) X(CI, 3, 9) X(CI, 4, 9)
+#define VM_MFMA_ANY_WIDTHS(X, CI) X(CI, 1, 7) X(CI, 2, 7) X(CI, 3, 7) X(CI, 4, 7) X(CI, 1, 9) X(CI, 2, 9) X(CI, 3, 9) X(CI, 4, 9) X(CI, 1, 5) X(CI, 2, 5) X(CI, 3, 5) X(CI, 4, 5)
 #define VM_FOR_EACH_MFMA_ANY_SHAPE(X) \
     VM_MFMA_ANY_WIDTHS(X, 36)         \
     VM_MFMA_ANY_WIDTHS(X, 40)         \
@@ -439,7 +439,7 @@ bool vm_mfma_supported(int c_in, int c_out, int slots) {
     if (c_in == CI && c_out == CO && slots == SL) return true;
     VM_FOR_EACH_MFMA_VARIANT(X)
 #undef X
-    return c_in % 4 == 0 && c_in >= 36 && c_in <= 64 && c_out >= 1 && c_out <= 64 && (slots == 7 || slots == 9);
+    return c_in % 4 == 0 && c_in >= 36 && c_in <= 64 && c_out >= 1 && c_out <= 64 && (slots == 5 || slots == 7 || slots == 9);
 }
 
 int vm_launch_conv_mfma(const VmBatchDev& B, const VmLayerDev& L, const void* in, void* out, hipStream_t stream, const char** kernel_name) {

@@ -6,8 +6,8 @@
  * grows with the batch lives here in one array of fixed size inside the library's device image.
  *
  * The array exists once per device and keeps its contents between calls: the reverse lookup table is validated by a
- * run stamp that the first kernel of every call advances (so it is never cleared, except when the 32-bit stamp wraps,
- * which a kernel of every call checks for), everything else is rewritten by the call before it is read. Calls that
+ * run stamp that the first kernel of every call advances (so it is never cleared, except when the 8-bit stamp starts
+ * again after 255 calls, which a kernel of every call checks for), everything else is rewritten by the call before it is read. Calls that
  * overlap on one device race on the array.
  */
 #include <atomic>
@@ -69,7 +69,7 @@ constexpr int PREPARE_THREADS = 1024;
  * A rejected table leaves a frame without candidates and -1 in *n_visible; the kernels that follow then write nothing. */
 __global__ __launch_bounds__(PREPARE_THREADS) void vm_noalloc_prepare_kernel(VmFrame F, const int32_t* __restrict__ ranges, int n_candidates,
                                                                                Header* header, VmFrame* frame_out, int32_t* range_first,
-                                                                               int32_t* range_prefix, int32_t* n_visible) {
+                                                                               int32_t* range_prefix, int32_t* n_visible, int32_t* neighbourhood) {
     __shared__ int wave_total[PREPARE_THREADS / 64];
     __shared__ int bad;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -123,6 +123,9 @@ __global__ __launch_bounds__(PREPARE_THREADS) void vm_noalloc_prepare_kernel(VmF
         F.row_base = 0, F.row_tile0 = 0, F.row_tiles = n > 0 ? (n + 1 + VMHIP_TILE - 1) / VMHIP_TILE : 0;
         *frame_out = F;
         *n_visible = ok ? 0 : -1;
+        /* a frame without candidates has no tile that would write its null row (row 0 then: every neighbour is row 0) */
+        if (ok && n == 0)
+            for (int j = 0; j < F.nn; ++j) neighbourhood[j] = 0;
     }
 }
 
@@ -233,7 +236,7 @@ extern "C" int vmhip_project_noalloc(const vmhip_mesh* mesh, const float* Rco, c
     B.px_error = 0.0f;
 
     hipLaunchKernelGGL(vm_noalloc_prepare_kernel, dim3(1), dim3(PREPARE_THREADS), 0, s, F, ranges, n_candidates, header, d_frame, range_first,
-                       range_prefix, out->n_visible);
+                       range_prefix, out->n_visible, out->neighbourhood);
     hipLaunchKernelGGL(vm_noalloc_wrap_kernel, dim3(256), dim3(256), 0, s, header, lookup, size_t(MAX_NODES) + 1);
     vm_launch_project(B, s);
     vm_launch_compact(B, nullptr, 0, s);
