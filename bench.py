@@ -229,7 +229,7 @@ def measure(cfg, engine, frames, steps, warmup, settle_s, events=True, stream_ce
     # roofline of the dominant kernel: a graph-convolution kernel, or (small single-frame workloads) one of the
     # kernels before the network, which move bytes only
     rows = nodes + len(frames)    # visible nodes + one null row per frame
-    conv = {k: v for k, v in kernel_ms.items() if k.startswith("conv")}
+    conv = {k: v for k, v in kernel_ms.items() if k.startswith(("conv", "neighbourhood_conv"))}
     dominant = max(conv, key=conv.get) if conv else None
     roofline = None
     if not dominant and kernel_ms:

@@ -298,17 +298,23 @@ __global__ __launch_bounds__(NW * 64) void vm_conv_narrow_kernel(VmBatchDev B, V
         request_halo_rows(min(NBUFS == 2 ? t3 : t2, t_last));
         __builtin_amdgcn_sched_barrier(0);
 
-        /* activation: the lane holds its row's channels 0..3 */
+        /* activation: the lane holds its row's channels 0..3. Softmax as the reference computes it (exp, then the division
+         * by the row's sum, no shift by the maximum: apply_activation.hpp:57-64), with the hardware's exponential and
+         * reciprocal: e^x = 2^(x log2 e) is off by at most |x| 1e-7 relative (the product's rounding) plus an ulp, the
+         * reciprocal by an ulp - 3e-6 on a probability for logits up to 30, against a gate of 1e-4 - and the two take
+         * a dozen instructions per row where the library's expf and an IEEE division take 150, which was a third of this
+         * kernel's vector work per tile. */
         if (activation == VMHIP_SOFTMAX) {
             float sum = 0.0f;
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
-                const float e = v < C_OUT ? expf(acc[v]) : 0.0f;
+                const float e = v < C_OUT ? __builtin_amdgcn_exp2f(acc[v] * 1.44269504088896340736f) : 0.0f;
                 acc[v] = e;
                 sum += e;
             }
+            const float scale = __builtin_amdgcn_rcpf(sum);
 #pragma unroll
-            for (int v = 0; v < 4; ++v) acc[v] = acc[v] / sum;
+            for (int v = 0; v < 4; ++v) acc[v] = acc[v] * scale;
         }
         else {
 #pragma unroll
