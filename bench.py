@@ -27,8 +27,12 @@ if ROOT not in sys.path:
 # (4 unless the environment says otherwise). This process has up to five streams alive at a time (the engine of the timed
 # passes, three engines in rotation for the end-to-end figure, the default stream); two streams on one hardware queue
 # take turns, and the rotation then needs 2.55 ms per batch instead of 1.82 (measured both ways, and with 2 queues and no
-# extra engine: 2.55 ms as well). Read by the runtime when it starts, so it is set before anything touches HIP.
-os.environ.setdefault("GPU_MAX_HW_QUEUES", "8")
+# extra engine: 2.55 ms as well). Read by the runtime when it starts, so it is set before anything touches HIP - unless a
+# profiler has already started the runtime's lower layers in this process with the value it found (rocprofv3's preloaded
+# tool does; a different value afterwards crashes it in the first graph launch): then the environment is left alone, and
+# a command line that wants the setting exports it before the profiler.
+if not any(k.startswith(("ROCPROF", "ROCP_")) for k in os.environ) and "rocprof" not in os.environ.get("LD_PRELOAD", ""):
+    os.environ.setdefault("GPU_MAX_HW_QUEUES", "8")
 
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 FP32_PEAK_TFLOPS = 157.3   # MI355X dense fp32 matrix

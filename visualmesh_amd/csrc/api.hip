@@ -319,7 +319,7 @@ int batch_stage(vmhip_batch* b, const vmhip_frame* frames, int32_t n_frames, int
      * settles after a few batches); kernel-by-kernel launches take exactly the tiles in use. */
     auto grown = [&](size_t have, size_t need) {
         if (!E->use_graph) return need;
-        if (need <= have) return have;
+        if (need <= have) return need * 2 < have ? need : have; /* far smaller batches do not launch the old one's grids */
         return have == 0 ? need : (need + need / 8 + 7) / 8 * 8;
     };
     b->cap_cand_tiles = std::min<size_t>(grown(b->cap_cand_tiles, cand_tiles), 0x7fffff);
