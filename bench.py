@@ -32,7 +32,12 @@ if ROOT not in sys.path:
 # tool does; a different value afterwards crashes it in the first graph launch): then the environment is left alone, and
 # a command line that wants the setting exports it before the profiler.
 if not any(k.startswith(("ROCPROF", "ROCP_")) for k in os.environ) and "rocprof" not in os.environ.get("LD_PRELOAD", ""):
-    os.environ.setdefault("GPU_MAX_HW_QUEUES", "8")
+    try:
+        queues_now = int(os.environ.get("GPU_MAX_HW_QUEUES", "4"))
+    except ValueError:
+        queues_now = 4
+    if queues_now < 8:  # an environment that names the runtime's default of 4 is raised too: five streams need five queues
+        os.environ["GPU_MAX_HW_QUEUES"] = "8"
 
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 FP32_PEAK_TFLOPS = 157.3   # MI355X dense fp32 matrix
