@@ -11,7 +11,7 @@
  * the 16-column instruction, which spends 5.3 times more on a 3-channel layer.
  *
  * Staging follows conv_flow.hip: rows travel from global memory straight into LDS (buffer_load ... lds), tile-local tables, XCD-aware persistent tile walk, a side path for
- * neighbours that are not staged. A lane reads its whole source row from LDS per gather slot.
+ * neighbours that are not staged. A lane reads its whole source row from LDS per gather slot, a quarter at a time.
  */
 #include <cstdlib>
 #include <type_traits>
@@ -220,62 +220,69 @@ __global__ __launch_bounds__(NW * 64) void vm_conv_narrow_kernel(VmBatchDev B, V
         }
         const bool any_far = __any(far);
 
-        v4f acc = *reinterpret_cast<const v4f*>(b_lds); /* the four channels' biases */
+        /* Two accumulators, even and odd input channels: a matrix instruction that adds to the result of the one right
+         * before it waits for that result (the compiler puts two idle cycles between them); alternating, each finds its
+         * operand ready. The first starts from the four channels' biases, the sum of the two is the row's result. */
+        v4f accs[2] = {*reinterpret_cast<const v4f*>(b_lds), v4f{0.0f, 0.0f, 0.0f, 0.0f}};
 
-        /* per slot: the lane's whole source row and the slot's weights for its channel, then one matrix instruction
-         * per input channel; the next slot's operands are requested before this slot's instructions */
+        /* The operands come from LDS a quarter slot (four input channels) at a time: 16 bytes of the lane's source row and
+         * 16 bytes of the slot's weights for its channel, four matrix instructions. A ring of Q4 quarters keeps the reads
+         * one slot ahead of their use in half the registers of two whole slots. */
         auto contract = [&](auto far_tag) {
             constexpr bool FAR = decltype(far_tag)::value;
-            auto gather = [&](int sl, float (&x)[C_IN]) {
-                const uint32_t at = (FAR && li[sl] >= FAR_FROM) ? 0u : li[sl];
-#pragma unroll
-                for (int k4 = 0; k4 < Q4; ++k4) {
-                    float t[4];
-                    load_floats<4>(rows + at * RS + ((SWZ ? (k4 ^ (int) ((at >> 2) & 3)) : k4) << 2), t);
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) x[k4 * 4 + e] = t[e];
-                }
-                if constexpr (FAR && NN > 0) {
-                    if (sl > 0 && li[sl] >= FAR_FROM) {
-                        const int g = B.row_nb[(size_t) (d_cur.x + li[0]) * B.nb_stride + (sl - 1)];
-                        load_floats<C_IN>(in + (size_t) (d_cur.w + g) * C_IN, x);
-                    }
-                }
-            };
-            auto weights = [&](int sl, float (&a)[C_IN]) {
-#pragma unroll
-                for (int k4 = 0; k4 < Q4; ++k4) {
-                    float t[4];
-                    load_floats<4>(w_lds + ((sl * Q4 + k4) * 4 + o_lane) * 4, t);
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) a[k4 * 4 + e] = t[e];
-                }
-            };
-            constexpr int NBUF = FAR ? 1 : 2;
-            float x[NBUF][C_IN], a[NBUF][C_IN];
             if constexpr (!FAR) {
-                gather(0, x[0]);
-                weights(0, a[0]);
+                constexpr int NQ = SLOTS * Q4, RING = Q4;
+                float x[RING][4], a[RING][4];
+                auto fetch = [&](int q, float (&xq)[4], float (&aq)[4]) {
+                    const int sl = q / Q4, k4 = q % Q4;
+                    const uint32_t at = li[sl];
+                    load_floats<4>(rows + at * RS + ((SWZ ? (k4 ^ (int) ((at >> 2) & 3)) : k4) << 2), xq);
+                    load_floats<4>(w_lds + ((sl * Q4 + k4) * 4 + o_lane) * 4, aq);
+                };
+#pragma unroll
+                for (int r = 0; r < RING; ++r) fetch(r, x[r], a[r]);
+#pragma unroll
+                for (int q = 0; q < NQ; ++q) {
+                    const int r = q % RING;
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) accs[e & 1] = __builtin_amdgcn_mfma_f32_4x4x1f32(a[r][e], x[r][e], accs[e & 1], 0, 0, 0);
+                    if (q + RING < NQ) fetch(q + RING, x[r], a[r]);
+                }
             }
+            else {
+                /* a tile with neighbours that are not staged: those lanes read their operands from global memory, slot by
+                 * slot; same order of additions as above */
+                float x[C_IN], a[C_IN];
 #pragma unroll
-            for (int sl = 0; sl < SLOTS; ++sl) {
-                const int b = FAR ? 0 : (sl & 1);
-                if constexpr (FAR) {
-                    gather(sl, x[0]);
-                    weights(sl, a[0]);
-                }
-                else if (sl + 1 < SLOTS) {
-                    gather(sl + 1, x[b ^ 1]);
-                    weights(sl + 1, a[b ^ 1]);
-                }
-                __builtin_amdgcn_sched_barrier(0);
+                for (int sl = 0; sl < SLOTS; ++sl) {
+                    const uint32_t at = li[sl] >= FAR_FROM ? 0u : li[sl];
 #pragma unroll
-                for (int k = 0; k < C_IN; ++k) acc = __builtin_amdgcn_mfma_f32_4x4x1f32(a[b][k], x[b][k], acc, 0, 0, 0);
-                if constexpr (FAR) __builtin_amdgcn_sched_barrier(0);
+                    for (int k4 = 0; k4 < Q4; ++k4) {
+                        float t[4];
+                        load_floats<4>(rows + at * RS + ((SWZ ? (k4 ^ (int) ((at >> 2) & 3)) : k4) << 2), t);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) x[k4 * 4 + e] = t[e];
+                        load_floats<4>(w_lds + ((sl * Q4 + k4) * 4 + o_lane) * 4, t);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) a[k4 * 4 + e] = t[e];
+                    }
+                    if constexpr (NN > 0) {
+                        if (sl > 0 && li[sl] >= FAR_FROM) {
+                            const int g = B.row_nb[(size_t) (d_cur.x + li[0]) * B.nb_stride + (sl - 1)];
+                            load_floats<C_IN>(in + (size_t) (d_cur.w + g) * C_IN, x);
+                        }
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int k = 0; k < C_IN; ++k) accs[k & 1] = __builtin_amdgcn_mfma_f32_4x4x1f32(a[k], x[k], accs[k & 1], 0, 0, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
         };
         if (any_far) contract(std::true_type());
         else contract(std::false_type());
+        v4f acc = accs[0] + accs[1];
 
         /* ---- every wave is done reading this buffer (with two buffers also: the next tile is complete and visible,
          * see conv_flow.hip) ---- */
