@@ -715,6 +715,7 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_compact_kernel(VmBatchDev B, fl
 #define NB_HASH 2048 /* >= the most out-of-tile neighbours a tile can have (256 rows x 8) */
 typedef float nbc_v4f __attribute__((ext_vector_type(4)));
 typedef uint32_t nbc_v4u __attribute__((ext_vector_type(4)));
+typedef int nbc_v2i __attribute__((ext_vector_type(2)));
 /* selu as the convolution kernels compute it: hardware exponential on the negative branch (<= 3e-7 absolute error) */
 __device__ __forceinline__ float nbc_selu(float s) {
     const float lambda = 1.0507009873554804934193349852946f;
@@ -815,7 +816,48 @@ __global__ __launch_bounds__(VMHIP_TILE, CB == 1 ? (NN <= 6 ? 8 : 6) : CB == 2 ?
         for (int k0 = 0; k0 < nn; k0 += MAX_ITEMS) resolve(k0);
         return;
     }
-    resolve(0);
+    /* With the tables, and the neighbour count known at compile time, a thread takes one row and all its neighbours
+     * (PER_ROW): the row's node is read once, its neighbours are NN consecutive words of the mesh's table (read and
+     * written two at a time), no item needs a division to find its row, and the row's eight table entries are packed in
+     * registers and stored with one instruction. A wave's reads and writes of the two tables are contiguous either way.
+     * Threads past the tile's rows redo its last row and store nothing. */
+    constexpr bool PER_ROW = NN > 0 && NN % 2 == 0;
+    const bool have_row = (int) threadIdx.x < n_rows;
+    if constexpr (PER_ROW) {
+        const int row = row0 + min((int) threadIdx.x, n_rows - 1);
+        uint32_t stamp[NN];
+#pragma unroll
+        for (int k = 0; k < NN; ++k) stamp[k] = 0u; /* zero carries no run's stamp: runs count from one */
+        if (V > 0) {
+            const int node = read_element(gidx, (Off) min(row, V - 1));
+            int nb[NN];
+#pragma unroll
+            for (int j = 0; j < NN / 2; ++j) {
+                const nbc_v2i two = read_element(reinterpret_cast<const nbc_v2i*>(nbr), (Off) node * (Off) (NN / 2) + (Off) j);
+                nb[2 * j] = min(two.x, n_nodes), nb[2 * j + 1] = min(two.y, n_nodes);
+            }
+#pragma unroll
+            for (int k = 0; k < NN; ++k) stamp[k] = read_element(lookup, (Off) nb[k]);
+        }
+#pragma unroll
+        for (int k = 0; k < NN; ++k) {
+            const bool found = row < V && (stamp[k] >> B.stamp_row_bits) == epoch;
+            outs[k] = have_row ? (found ? (int) (stamp[k] & row_mask) : V) : -1;
+        }
+        if (have_row) {
+            if (B.nb_stride == NN) {
+#pragma unroll
+                for (int j = 0; j < NN / 2; ++j) write_element(reinterpret_cast<nbc_v2i*>(nb_out), (Off) row * (Off) (NN / 2) + (Off) j, nbc_v2i{outs[2 * j], outs[2 * j + 1]});
+            }
+            else {
+#pragma unroll
+                for (int k = 0; k < NN; ++k) write_element(nb_out, (Off) row * nb_stride + (Off) k, outs[k]);
+            }
+        }
+    }
+    else {
+        resolve(0);
+    }
 
     /* ---- first layer, part one: request what the contraction will read ---- */
     constexpr int RBS = 4; /* row blocks of 16 per wave: a wave owns 64 rows of the tile */
@@ -828,9 +870,11 @@ __global__ __launch_bounds__(VMHIP_TILE, CB == 1 ? (NN <= 6 ? 8 : 6) : CB == 2 ?
     };
     if constexpr (CB > 0) own_row = __builtin_amdgcn_raw_buffer_load_b128(sampled_rows(), (row0 + min((int) threadIdx.x, n_rows - 1)) * 16, 0, 0);
 
+    uint32_t h_slot[MAX_ITEMS]; /* where the item's row went in the hash table */
 #pragma unroll
     for (int k = 0; k < MAX_ITEMS; ++k) {
         const int out = outs[k];
+        h_slot[k] = 0u;
         if (out >= 0 && (out < row0 || out >= row0 + VMHIP_TILE)) {
             uint32_t slot = hash((uint32_t) out);
             while (true) {
@@ -838,6 +882,7 @@ __global__ __launch_bounds__(VMHIP_TILE, CB == 1 ? (NN <= 6 ? 8 : 6) : CB == 2 ?
                 if (prev == EMPTY || prev == (uint32_t) out) break;
                 slot = (slot + 1) & (NB_HASH - 1);
             }
+            h_slot[k] = slot;
         }
     }
     __syncthreads();
@@ -893,32 +938,39 @@ __global__ __launch_bounds__(VMHIP_TILE, CB == 1 ? (NN <= 6 ? 8 : 6) : CB == 2 ?
             for (int cb = 0; cb < CB; ++cb) a[s][cb] = w[(s * CB + cb) * 64 + (threadIdx.x & 63)];
     }
 
+    typedef unsigned int row_words __attribute__((ext_vector_type(4)));
+    uint16_t* const nbl_out = B.row_nbl + (size_t) row_base * VMHIP_NBL_STRIDE;
+    auto position_of = [&](int out, uint32_t slot) {
+        if (out >= row0 && out < row0 + VMHIP_TILE) return (uint32_t) (out - row0);
+        const int dense = h_dense[slot];
+        return dense < cap ? (uint32_t) (VMHIP_TILE + dense) : (uint32_t) VMHIP_NBL_FAR;
+    };
+    if constexpr (PER_ROW) {
+        /* the row's entries packed two to a word (entries past nn are never read) */
+        uint32_t words[4] = {0u, 0u, 0u, 0u};
 #pragma unroll
-    for (int k = 0; k < MAX_ITEMS; ++k) {
-        const int out = outs[k];
-        if (out >= 0) {
-            uint32_t local;
-            if (out >= row0 && out < row0 + VMHIP_TILE) {
-                local = (uint32_t) (out - row0);
-            }
-            else {
-                uint32_t slot = hash((uint32_t) out);
-                while (h_key[slot] != (uint32_t) out) slot = (slot + 1) & (NB_HASH - 1);
-                const int dense = h_dense[slot];
-                local = dense < cap ? (uint32_t) (VMHIP_TILE + dense) : VMHIP_NBL_FAR;
-            }
-            /* the item's row of the tile and neighbour number, worked out again rather than kept in registers all the way */
-            const int it = threadIdx.x + k * VMHIP_TILE;
-            const int r = row_of(it);
-            nbl_rows[r][it - r * nn] = (uint16_t) local;
+        for (int k = 0; k < NN; ++k) words[k >> 1] |= (have_row ? position_of(outs[k], h_slot[k]) : 0u) << (16 * (k & 1));
+        const row_words packed = {words[0], words[1], words[2], words[3]};
+        if (have_row) write_element(reinterpret_cast<row_words*>(nbl_out), (Off) (row0 + threadIdx.x), packed);
+        if constexpr (CB > 0) {
+            *reinterpret_cast<row_words*>(nbl_rows[threadIdx.x]) = packed;
+            __syncthreads();
         }
     }
-    __syncthreads();
-    /* one 16-byte store per row (entries past nn are never read) */
-    if ((int) threadIdx.x < n_rows) {
-        uint16_t* const nbl_out = B.row_nbl + (size_t) row_base * VMHIP_NBL_STRIDE;
-        typedef unsigned int row_words __attribute__((ext_vector_type(4)));
-        write_element(reinterpret_cast<row_words*>(nbl_out), (Off) (row0 + threadIdx.x), *reinterpret_cast<const row_words*>(nbl_rows[threadIdx.x]));
+    else {
+#pragma unroll
+        for (int k = 0; k < MAX_ITEMS; ++k) {
+            const int out = outs[k];
+            if (out >= 0) {
+                /* the item's row of the tile and neighbour number, worked out again rather than kept in registers all the way */
+                const int it = threadIdx.x + k * VMHIP_TILE;
+                const int r = row_of(it);
+                nbl_rows[r][it - r * nn] = (uint16_t) position_of(out, h_slot[k]);
+            }
+        }
+        __syncthreads();
+        /* one 16-byte store per row (entries past nn are never read) */
+        if (have_row) write_element(reinterpret_cast<row_words*>(nbl_out), (Off) (row0 + threadIdx.x), *reinterpret_cast<const row_words*>(nbl_rows[threadIdx.x]));
     }
 
     /* ---- first layer, part two: contraction, activation, store ---- */
