@@ -695,10 +695,10 @@ __global__ __launch_bounds__(VMHIP_TILE) void vm_compact_kernel(VmBatchDev B, fl
 /* reference engine/cpu/engine.hpp:127-143: one thread per (row, neighbour).
  *
  * When the batch carries tile-local tables the block also builds them for its tile: the neighbours that live in
- * other tiles are deduplicated through an open-addressing hash in LDS, numbered densely in table order (the
- * halo slots), and every neighbour is rewritten as a position in "own tile rows, then halo slots". Which row
- * gets which halo slot depends on the order the atomics land in and may differ from run to run; the rows that a
- * slot stands for, and so every result computed through the tables, do not.
+ * other tiles are deduplicated through an open-addressing hash in LDS, the thread that enters a row first takes the
+ * next halo slot from a counter, and every neighbour is rewritten as a position in "own tile rows, then halo
+ * slots". Which row gets which halo slot depends on the order the atomics land in and differs from run to run;
+ * the rows that a slot stands for, and so every result computed through the tables, do not.
  *
  * WIDE = false addresses the frame's tables with 32-bit byte offsets from wave-uniform bases (an address is then a
  * scalar register pair plus one vector register, and the 64-bit vector arithmetic that was a third of this kernel's
@@ -727,7 +727,7 @@ __global__ __launch_bounds__(VMHIP_TILE, CB == 1 ? (NN <= 6 ? 8 : 6) : CB == 2 ?
     static_assert(CB == 0 || (NN > 0 && NN <= VMHIP_NBL_STRIDE), "the fused first layer knows its neighbour count");
     using Off = typename std::conditional<WIDE, size_t, uint32_t>::type;
     __shared__ __align__(16) uint32_t h_key[NB_HASH];
-    __shared__ int wave_total[VMHIP_TILE / 64];
+    __shared__ int halo_count; /* halo slots handed out so far */
     __shared__ uint16_t h_dense[NB_HASH];
     __shared__ __align__(16) uint16_t nbl_rows[VMHIP_TILE][VMHIP_NBL_STRIDE]; /* the tile's positions, stored row by row at the end */
     /* CB > 0: the frame-local row of every halo slot. The sampled rows the layer gathers (the tile's 256, then its halo
@@ -754,6 +754,7 @@ __global__ __launch_bounds__(VMHIP_TILE, CB == 1 ? (NN <= 6 ? 8 : 6) : CB == 2 ?
     auto hash = [](uint32_t key) { return (key * 2654435761u) >> 21; }; /* 11 bits */
     if (tables) {
         for (int e = threadIdx.x * 4; e < NB_HASH; e += VMHIP_TILE * 4) *reinterpret_cast<uint4*>(&h_key[e]) = make_uint4(EMPTY, EMPTY, EMPTY, EMPTY);
+        if (threadIdx.x == 0) halo_count = 0;
         __syncthreads();
     }
 
@@ -864,12 +865,15 @@ __global__ __launch_bounds__(VMHIP_TILE, CB == 1 ? (NN <= 6 ? 8 : 6) : CB == 2 ?
     constexpr int SLOTS = NN + 1;
     float a[CB > 0 ? SLOTS : 1][CB > 0 ? CB : 1]; /* [slot][column block]: the lane's weight */
     nbc_v4u own_row = {0u, 0u, 0u, 0u}, halo_row = {0u, 0u, 0u, 0u};
+    nbc_v4f bias4[CB > 0 ? CB : 1]; /* the lane's four output channels' biases, per column block */
     /* the frame's sampled rows 0..V, 16 bytes each; offsets beyond read zeros */
     auto sampled_rows = [&] {
         return __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(feat + (size_t) row_base * 4), 0, (int) min((uint64_t) (V + 1) * 16ull, 0xffffffffull), 0x00020000);
     };
     if constexpr (CB > 0) own_row = __builtin_amdgcn_raw_buffer_load_b128(sampled_rows(), (row0 + min((int) threadIdx.x, n_rows - 1)) * 16, 0, 0);
 
+    const int cap = B.halo_cap;
+    uint32_t* const tile_halo = B.tile_halo + (size_t) tile * VMHIP_HALO_MAX;
     uint32_t h_slot[MAX_ITEMS]; /* where the item's row went in the hash table */
 #pragma unroll
     for (int k = 0; k < MAX_ITEMS; ++k) {
@@ -879,56 +883,24 @@ __global__ __launch_bounds__(VMHIP_TILE, CB == 1 ? (NN <= 6 ? 8 : 6) : CB == 2 ?
             uint32_t slot = hash((uint32_t) out);
             while (true) {
                 const uint32_t prev = atomicCAS(&h_key[slot], EMPTY, (uint32_t) out);
-                if (prev == EMPTY || prev == (uint32_t) out) break;
+                if (prev == EMPTY) { /* the row is new to the tile: it gets the next halo slot */
+                    const int dense = atomicAdd(&halo_count, 1);
+                    h_dense[slot] = (uint16_t) min(dense, 0xffff);
+                    if (dense < cap) {
+                        tile_halo[dense] = (uint32_t) row_base + (uint32_t) out;
+                        if constexpr (CB > 0) halo_list[dense] = (uint32_t) out;
+                    }
+                    break;
+                }
+                if (prev == (uint32_t) out) break;
                 slot = (slot + 1) & (NB_HASH - 1);
             }
             h_slot[k] = slot;
         }
     }
     __syncthreads();
-
-    /* dense numbering of the occupied hash entries, in table order: 16 entries per thread, block-wide scan */
-    constexpr int PER = NB_HASH / VMHIP_TILE;
-    uint32_t keys[PER];
-#pragma unroll
-    for (int k = 0; k < PER; k += 4) {
-        const uint4 t = *reinterpret_cast<const uint4*>(&h_key[threadIdx.x * PER + k]);
-        keys[k] = t.x, keys[k + 1] = t.y, keys[k + 2] = t.z, keys[k + 3] = t.w;
-    }
-    int mine = 0;
-#pragma unroll
-    for (int k = 0; k < PER; ++k) mine += keys[k] != EMPTY;
-    int scan = mine;
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-        const int up = __shfl_up(scan, d);
-        if ((int) (threadIdx.x & 63) >= d) scan += up;
-    }
-    if ((threadIdx.x & 63) == 63) wave_total[threadIdx.x >> 6] = scan;
-    __syncthreads();
-    int before = scan - mine, total = 0;
-#pragma unroll
-    for (int w = 0; w < VMHIP_TILE / 64; ++w) {
-        if (w < (int) (threadIdx.x >> 6)) before += wave_total[w];
-        total += wave_total[w];
-    }
-    const int cap = B.halo_cap;
-    uint32_t* const tile_halo = B.tile_halo + (size_t) tile * VMHIP_HALO_MAX;
-    if (mine > 0) {
-#pragma unroll
-        for (int k = 0; k < PER; ++k) {
-            if (keys[k] != EMPTY) {
-                h_dense[threadIdx.x * PER + k] = (uint16_t) min(before, 0xffff);
-                if (before < cap) {
-                    tile_halo[before] = (uint32_t) row_base + keys[k];
-                    if constexpr (CB > 0) halo_list[before] = keys[k];
-                }
-                ++before;
-            }
-        }
-    }
+    const int total = halo_count;
     if (threadIdx.x == 0) B.tile_desc[tile] = make_int4(row_base + row0, n_rows, min(total, cap), row_base);
-    __syncthreads();
     if constexpr (CB > 0) { /* the halo rows, one per thread, and the layer's weights */
         halo_row = __builtin_amdgcn_raw_buffer_load_b128(sampled_rows(), (int) threadIdx.x < min(total, cap) ? halo_list[threadIdx.x] * 16u : 0xffffffffu, 0, 0);
         const VM_GLOBAL float* const w = in_device_memory(reinterpret_cast<const float*>(L.w_mfma));
@@ -936,6 +908,13 @@ __global__ __launch_bounds__(VMHIP_TILE, CB == 1 ? (NN <= 6 ? 8 : 6) : CB == 2 ?
         for (int s = 0; s < SLOTS; ++s)
 #pragma unroll
             for (int cb = 0; cb < CB; ++cb) a[s][cb] = w[(s * CB + cb) * 64 + (threadIdx.x & 63)];
+        const VM_GLOBAL float* const bias = in_device_memory(L.b);
+        const int q4 = ((threadIdx.x & 63) >> 4) * 4;
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) {
+            bias4[cb] = nbc_v4f{0.0f, 0.0f, 0.0f, 0.0f};
+            if (cb * 16 + q4 < L.c_out) bias4[cb] = *reinterpret_cast<const VM_GLOBAL nbc_v4f*>(bias + cb * 16 + q4); /* c_out is a multiple of 4 */
+        }
     }
 
     typedef unsigned int row_words __attribute__((ext_vector_type(4)));
@@ -1018,15 +997,11 @@ __global__ __launch_bounds__(VMHIP_TILE, CB == 1 ? (NN <= 6 ? 8 : 6) : CB == 2 ?
                 }
             }
         }
-        const VM_GLOBAL float* const bias = in_device_memory(L.b);
         nbc_v4f acc[RBS][CB];
 #pragma unroll
-        for (int cb = 0; cb < CB; ++cb) {
-            nbc_v4f b4 = {0.0f, 0.0f, 0.0f, 0.0f};
-            if (cb * 16 + q * 4 < c_out) b4 = *reinterpret_cast<const VM_GLOBAL nbc_v4f*>(bias + cb * 16 + q * 4); /* c_out is a multiple of 4 */
+        for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
-            for (int rb = 0; rb < RBS; ++rb) acc[rb][cb] = b4;
-        }
+            for (int rb = 0; rb < RBS; ++rb) acc[rb][cb] = bias4[cb];
 #pragma unroll
         for (int s = 0; s < SLOTS; ++s)
 #pragma unroll
