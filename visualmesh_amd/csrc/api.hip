@@ -1058,7 +1058,7 @@ int vmhip_engine_create(const vmhip_network* net, int32_t n_neighbours, int32_t 
             E->use_flow = E->use_flow || H.use_flow;
             if (H.arith_bf16) {
                 std::vector<unsigned char> wp(vm_bf16_weight_bytes(H.c_in, H.c_out, H.slots));
-                vm_bf16_permute_weights(H.h_w.data(), H.c_in, H.c_out, H.slots, wp.data());
+                vm_bf16_permute_weights(H.h_w.data(), H.c_in, H.c_out, H.slots, H.out_bf16, wp.data());
                 if (hipMalloc(&H.d_w_mfma, wp.size()) != hipSuccess) return bail(VMHIP_ERR_HIP, "engine_create: out of device memory");
                 if (hipMemcpy(H.d_w_mfma, wp.data(), wp.size(), hipMemcpyHostToDevice) != hipSuccess)
                     return bail(VMHIP_ERR_HIP, "engine_create: weight upload failed");

@@ -170,12 +170,18 @@ __host__ __device__ constexpr size_t bf16_lds_bytes(int in_fmt) { return 2 * siz
 constexpr int FILL_EVERY = 3;
 constexpr int slice_of_item(int item, int n_fill) { return item - (item / FILL_EVERY + 1 < n_fill ? item / FILL_EVERY + 1 : n_fill); }
 /* stores (pieces 32.., of which with fp32 or bf16 rows out only the even ones store) issued after the last load */
-constexpr int stores_after_fills(int n_fill, int n_slices, bool two_stores) {
+/* whether piece sl of a half tile's results stores: pieces 32 + 2 u and 33 + 2 u belong to unit u = (row block, g). fp32
+ * rows out: the first piece of every unit (four channels, 16 bytes); bf16 rows out: the first piece of the units with even
+ * g (eight channels, 16 bytes); hi + lo rows out: both pieces of those units (the hi parts, then the lo parts) */
+constexpr bool slice_stores(int sl, int out_fmt) {
+    if (sl < 32) return false;
+    const int g = ((sl - 32) >> 1) & 3, part = (sl - 32) & 1;
+    return out_fmt == VM_ROWS_F32 ? part == 0 : out_fmt == VM_ROWS_BF16 ? (g % 2 == 0 && part == 0) : g % 2 == 0;
+}
+constexpr int stores_after_fills(int n_fill, int n_slices, int out_fmt) {
     int n = 0;
-    for (int item = FILL_EVERY * (n_fill - 1) + 1; slice_of_item(item, n_fill) < n_slices; ++item) {
-        const int sl = slice_of_item(item, n_fill);
-        if (sl >= 32 && (two_stores || (sl - 32) % 2 == 0)) ++n;
-    }
+    for (int item = FILL_EVERY * (n_fill - 1) + 1; slice_of_item(item, n_fill) < n_slices; ++item)
+        if (slice_stores(slice_of_item(item, n_fill), out_fmt)) ++n;
     return n;
 }
 
@@ -206,7 +212,7 @@ __global__ __launch_bounds__(256) void vm_conv_bf16_kernel(VmBatchDev B, VmLayer
     constexpr int BUF = bf16_buf_bytes(IN_FMT);
     constexpr int NBL_AT = BROWS * ROWB;      /* the half tile's neighbour table follows its rows */
     constexpr bool WIDE = IN_FMT != VM_ROWS_BF16; /* inputs come as hi + lo */
-    constexpr int N_STORES = OUT_FMT == VM_ROWS_BF16X2 ? 16 : 8; /* vector stores of a wave per half tile */
+    constexpr int N_STORES = OUT_FMT == VM_ROWS_BF16 ? 4 : 8; /* vector stores of a wave per half tile */
     constexpr int N_FILL = NR + 2;            /* loads of a wave per half tile: rows, neighbour table */
     static_assert(N_STORES + N_FILL + 3 < 64, "what a wave has in flight must fit the vmcnt counter");
 
@@ -346,11 +352,11 @@ __global__ __launch_bounds__(256) void vm_conv_bf16_kernel(VmBatchDev B, VmLayer
         for (int v = 0; v < 16; ++v) acc_done[rb][v] = 0.0f;
     }
 
-    /* Activation and stores of a finished half tile (lane holds channels cb*32 + g*8 + h*4 + {0..3} of its rows), cut
+    /* Activation and stores of a finished half tile (lane holds channels cb*32 + h*16 + g*4 + {0..3} of its rows), cut
      * into N_SLICES pieces of a few vector instructions each, so that one piece can follow each matrix instruction of
      * the half tile after: pieces 0..31 apply the activation to one value each, pieces 32..47 convert and store -
-     * piece 32 + 2u and 33 + 2u the four channels of unit u = (row block, g). The softmax needs the sums of whole
-     * rows first, which lie in two waves: prepare_softmax does that part in one go. */
+     * pieces 32 + 2u and 33 + 2u belong to unit u = (row block, g), and slice_stores says which of them store. The
+     * softmax needs the sums of whole rows first, which lie in two waves: prepare_softmax does that part in one go. */
     constexpr int N_SLICES = 48;
     auto prepare_softmax = [&](v16f (&a)[2]) {
 #pragma unroll
@@ -384,26 +390,34 @@ __global__ __launch_bounds__(256) void vm_conv_bf16_kernel(VmBatchDev B, VmLayer
         else if (i < N_SLICES) {
             const int u = (i - 32) >> 1, part = (i - 32) & 1;
             const int rb = u >> 2, g = u & 3;
-            const int o = cb * 32 + g * 8 + h * 4;
-            const float v0 = a[rb][g * 4 + 0], v1 = a[rb][g * 4 + 1], v2 = a[rb][g * 4 + 2], v3 = a[rb][g * 4 + 3];
+            /* What one store instruction writes of a row should be as long a run as two lanes can make it: 32 bytes. fp32
+             * rows out: matrix column 8 g + 4 h + v is channel 8 g + 4 h + v, a lane's four values of unit g are 16 bytes
+             * and the row's other lane holds the next 16. bf16 and hi + lo rows out: the host gives matrix column
+             * 8 g + 4 h + v the weights of channel 16 (g / 2) + 8 h + 4 (g % 2) + v, so that a lane's eight values of
+             * units g and g + 1 are eight consecutive channels, 16 bytes, and again the other lane holds the next 16
+             * (with the columns left as they are a lane had 8 bytes per instruction, the pair 16, and twice the
+             * instructions). */
+            const int o = cb * 32 + (OUT_FMT == VM_ROWS_F32 ? g * 8 + h * 4 : (g >> 1) * 16 + h * 8);
             if constexpr (OUT_FMT == VM_ROWS_F32) {
-                if (part == 0)
+                if (part == 0) {
+                    const float v0 = a[rb][g * 4 + 0], v1 = a[rb][g * 4 + 1], v2 = a[rb][g * 4 + 2], v3 = a[rb][g * 4 + 3];
                     __builtin_amdgcn_raw_buffer_store_b128(v4u{__float_as_uint(v0), __float_as_uint(v1), __float_as_uint(v2), __float_as_uint(v3)}, rs,
                                                            t.valid[rb] ? t.own[rb] * OUTB + o * 4 : OOR, 0, 0);
-            }
-            else if constexpr (OUT_FMT == VM_ROWS_BF16) {
-                if (part == 0)
-                    __builtin_amdgcn_raw_buffer_store_b64(v2u{pack_bf16(v0, v1), pack_bf16(v2, v3)}, rs, t.valid[rb] ? t.own[rb] * OUTB + o * 2 : OOR, 0, 0);
-            }
-            else {
-                const uint32_t at = t.valid[rb] ? t.own[rb] * OUTB + o * 2 : OOR;
-                const uint32_t h0 = pack_bf16(v0, v1), h1 = pack_bf16(v2, v3);
-                if (part == 0) {
-                    __builtin_amdgcn_raw_buffer_store_b64(v2u{h0, h1}, rs, at, 0, 0);
                 }
-                else {
-                    const uint32_t l0 = pack_bf16(v0 - bf16_low(h0), v1 - bf16_high(h0)), l1 = pack_bf16(v2 - bf16_low(h1), v3 - bf16_high(h1));
-                    __builtin_amdgcn_raw_buffer_store_b64(v2u{l0, l1}, rs, t.valid[rb] ? at + CH * 2 : OOR, 0, 0);
+            }
+            else if (g % 2 == 0) { /* eight channels: units g and g + 1 */
+                float v[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) v[e] = a[rb][g * 4 + e];
+                const uint32_t h0 = pack_bf16(v[0], v[1]), h1 = pack_bf16(v[2], v[3]), h2 = pack_bf16(v[4], v[5]), h3 = pack_bf16(v[6], v[7]);
+                const uint32_t at = t.valid[rb] ? t.own[rb] * OUTB + o * 2 : OOR;
+                if (part == 0) {
+                    __builtin_amdgcn_raw_buffer_store_b128(v4u{h0, h1, h2, h3}, rs, at, 0, 0);
+                }
+                else if constexpr (OUT_FMT == VM_ROWS_BF16X2) {
+                    const uint32_t l0 = pack_bf16(v[0] - bf16_low(h0), v[1] - bf16_high(h0)), l1 = pack_bf16(v[2] - bf16_low(h1), v[3] - bf16_high(h1));
+                    const uint32_t l2 = pack_bf16(v[4] - bf16_low(h2), v[5] - bf16_high(h2)), l3 = pack_bf16(v[6] - bf16_low(h3), v[7] - bf16_high(h3));
+                    __builtin_amdgcn_raw_buffer_store_b128(v4u{l0, l1, l2, l3}, rs, t.valid[rb] ? at + CH * 2 : OOR, 0, 0);
                 }
             }
         }
@@ -418,7 +432,7 @@ __global__ __launch_bounds__(256) void vm_conv_bf16_kernel(VmBatchDev B, VmLayer
         /* my loads of half tile k and the note of k+1 have landed once nothing but the stores issued after them can
          * be in flight (vector memory operations complete in order); before the first stores: once nothing is */
         if (k == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(stores_after_fills(N_FILL, 48, OUT_FMT == VM_ROWS_BF16X2)) : "memory");
+        else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(stores_after_fills(N_FILL, 48, OUT_FMT)) : "memory");
         __syncthreads(); /* everyone's have landed; everyone has read the last of half tile k-1 */
         const int4 d_cur = d_next;
         d_next = read_note();
@@ -455,7 +469,7 @@ __global__ __launch_bounds__(256) void vm_conv_bf16_kernel(VmBatchDev B, VmLayer
         v16f acc[2];
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-            const v4f b4 = *reinterpret_cast<const v4f*>(b_lds + cb * 32 + g * 8 + h * 4);
+            const v4f b4 = *reinterpret_cast<const v4f*>(b_lds + cb * 32 + (OUT_FMT == VM_ROWS_F32 ? g * 8 + h * 4 : (g >> 1) * 16 + h * 8 + (g & 1) * 4));
 #pragma unroll
             for (int rb = 0; rb < 2; ++rb) acc[rb][g * 4 + 0] = b4[0], acc[rb][g * 4 + 1] = b4[1], acc[rb][g * 4 + 2] = b4[2], acc[rb][g * 4 + 3] = b4[3];
         }
@@ -744,9 +758,11 @@ uint16_t bf16_round(float f) {
 }  // namespace
 
 /* Weight layout the kernel consumes: [channel block cb][slot][step j][part: hi, lo][lane = h*32 + o][e = 0..7] bf16 of
- * W[slot*64 + (4h + j)*8 + e][cb*32 + o]. */
+ * W[slot*64 + (4h + j)*8 + e][cb*32 + channel(o)]. The matrix instruction leaves a lane columns 8 g + 4 h' + v (g = 0..3,
+ * v = 0..3) of its row; for a layer that writes fp32 rows channel(o) = o, for one that writes bf16 or hi + lo rows
+ * channel(8 g + 4 h' + v) = 16 (g / 2) + 8 h' + 4 (g % 2) + v (the kernel's store says why). */
 size_t vm_bf16_weight_bytes(int c_in, int c_out, int slots) { return size_t(slots) * (c_in / 16) * (c_out / 32) * 2 * 64 * 16; }
-void vm_bf16_permute_weights(const float* w, int c_in, int c_out, int slots, void* wp) {
+void vm_bf16_permute_weights(const float* w, int c_in, int c_out, int slots, int out_fmt, void* wp) {
     uint16_t* dst = reinterpret_cast<uint16_t*>(wp);
     const int steps = c_in / 16, cbs = c_out / 32;
     for (int cb = 0; cb < cbs; ++cb)
@@ -756,7 +772,9 @@ void vm_bf16_permute_weights(const float* w, int c_in, int c_out, int slots, voi
                     for (int o = 0; o < 32; ++o)
                         for (int e = 0; e < 8; ++e) {
                             const int k = s * c_in + (h * steps + j) * 8 + e;
-                            const float v = w[size_t(k) * c_out + cb * 32 + o];
+                            const int g = o >> 3, hh = (o >> 2) & 1, vv = o & 3;
+                            const int channel = out_fmt == VM_ROWS_F32 ? o : (g >> 1) * 16 + hh * 8 + (g & 1) * 4 + vv;
+                            const float v = w[size_t(k) * c_out + cb * 32 + channel];
                             const uint16_t hi = bf16_round(v);
                             const uint32_t hi_bits = uint32_t(hi) << 16;
                             float hi_f;

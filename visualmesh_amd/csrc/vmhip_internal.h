@@ -255,7 +255,7 @@ int vm_launch_conv_mfma(const VmBatchDev& B, const VmLayerDev& L, const void* in
  * of half tiles staged in LDS. vm_launch_half_tables builds the half-tile tables from the neighbour table of the run. */
 bool vm_bf16_supported(int c_in, int c_out, int slots);
 size_t vm_bf16_weight_bytes(int c_in, int c_out, int slots);
-void vm_bf16_permute_weights(const float* w, int c_in, int c_out, int slots, void* wp);
+void vm_bf16_permute_weights(const float* w, int c_in, int c_out, int slots, int out_fmt, void* wp);
 void vm_launch_half_tables(const VmBatchDev& B, hipStream_t stream);
 int vm_launch_conv_bf16(const VmBatchDev& B, const VmLayerDev& L, const void* in, void* out, hipStream_t stream,
                         const char** kernel_name);
