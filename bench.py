@@ -348,14 +348,20 @@ def end_to_end(cfg, mesh, lens, nodes, batches):
         assert returned == n
 
     rotate(6)  # buffers allocated
-    t0 = time.perf_counter()
-    rotate(batches)
-    dt = (time.perf_counter() - t0) / batches
+    # Three timed stretches of `batches` batches each; the figure is the fastest, all three are in the result: the bus
+    # and the host's memory are shared with whatever else the machine is doing, and a stretch that meets other traffic
+    # has been seen to read four times slower with nothing of this program's changed.
+    stretches = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        rotate(batches)
+        stretches.append((time.perf_counter() - t0) / batches)
+    dt = min(stretches)
     nn = wl.N_NEIGHBOURS[cfg.model]
     classes = cfg.network[-1][-1][0].shape[1]
     h2d = sum(int(f["image"].nbytes) for f in cfg.frames)
     d2h = nodes * (8 + 4) + (nodes + len(cfg.frames)) * 4 * (nn + classes)
-    return dict(ms_per_batch=dt * 1e3, nodes_per_s=nodes / dt, frames_per_s=len(cfg.frames) / dt, engines=3, batches=batches,
+    return dict(ms_per_batch=dt * 1e3, ms_per_batch_of_each_stretch=[x * 1e3 for x in stretches], nodes_per_s=nodes / dt, frames_per_s=len(cfg.frames) / dt, engines=3, batches=batches,
                 h2d_bytes_per_batch=h2d, d2h_bytes_per_batch=d2h, pcie_GBps_each_way=[h2d / dt / 1e9, d2h / dt / 1e9],
                 what="host lookup + upload from page-locked images + all kernels + download of the whole classified mesh into "
                      "page-locked arrays; three engines in rotation (one staging, one running, one copying out)")
