@@ -265,9 +265,16 @@ def measure(cfg, engine, frames, steps, warmup, settle_s, events=True, stream_ce
     conv_rooflines = {}
     for name, ms in sorted(kernel_ms_per_step.items()):
         if name.startswith(("conv", "neighbourhood_conv")):
-            entry = conv_roofline(name, ms / launches_per_step[name], rows)[0]
+            entry, bytes_per_row, flops_per_row = conv_roofline(name, ms / launches_per_step[name], rows)
             conv_rooflines[name] = dict(bound=entry["bound"], achieved=entry["achieved"], unit=entry["unit"], frac=entry["frac"],
-                                        avg_launch_ms=ms / launches_per_step[name])
+                                        avg_launch_ms=ms / launches_per_step[name], algorithmic_bytes_per_row=bytes_per_row,
+                                        flops_per_row=flops_per_row)
+            if name.startswith("neighbourhood_conv"):
+                nn = int(name.split("s")[-1]) - 1
+                conv_rooflines[name]["bytes_per_row_is"] = (
+                    "%d for the neighbourhood stage (mesh neighbours, reverse-lookup gathers and the table written, 4 bytes per "
+                    "neighbour each) + %d for the layer (input row, neighbour table, output row) - %d: the layer gathers through "
+                    "the table the same kernel has just written" % (12 * nn, bytes_per_row - 12 * nn + 4 * nn, 4 * nn))
     # The layers bound by memory, against what the memory system gives a kernel that does nothing but read and write
     # their bytes (same rows, same bytes per row in and out, whole cache lines, no gather, no arithmetic): the ceiling
     # that a copy-like kernel of that shape reaches on this device, next to the 8 TB/s on the data sheet.
