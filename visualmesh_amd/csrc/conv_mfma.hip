@@ -149,7 +149,18 @@ __global__ __launch_bounds__(NW * 64) void vm_conv_mfma_kernel(VmBatchDev B, VmL
     typedef typename OP::op_t op_t;
 
     extern __shared__ float4 w_lds4[];
-    for (int i = threadIdx.x; i < W_BYTES / 16; i += NW * 64) w_lds4[i] = reinterpret_cast<const float4*>(L.w_mfma)[i];
+    /* G consecutive steps of a lane's weights lie next to each other in LDS, so that one read brings G of them */
+    constexpr int G = (PARTS == 1 && sizeof(areg_t) == 4 && STEPS % 4 == 0) ? 4 : 1;
+    if constexpr (G == 1) {
+        for (int i = threadIdx.x; i < W_BYTES / 16; i += NW * 64) w_lds4[i] = reinterpret_cast<const float4*>(L.w_mfma)[i];
+    }
+    else {
+        float* const w = reinterpret_cast<float*>(w_lds4);
+        for (int i = threadIdx.x; i < W_BYTES / 4; i += NW * 64) {
+            const int e = i % G, l = (i / G) % 64, cb = (i / (G * 64)) % CB, jg = (i / (G * 64 * CB)) % (STEPS / G), sl = i / (STEPS * 64 * CB);
+            w[i] = reinterpret_cast<const float*>(L.w_mfma)[((sl * STEPS + jg * G + e) * CB + cb) * 64 + l];
+        }
+    }
     __syncthreads();
     const areg_t* w_lds = reinterpret_cast<const areg_t*>(w_lds4);
 
@@ -275,15 +286,30 @@ __global__ __launch_bounds__(NW * 64) void vm_conv_mfma_kernel(VmBatchDev B, VmL
             op_t b[RB][STEPS];
 #pragma unroll
             for (int rb = 0; rb < RB; ++rb) OP::prepare(x[cur_buf][rb], b[rb]);
+            if constexpr (G == 1) {
 #pragma unroll
-            for (int j = 0; j < STEPS; ++j) {
+                for (int j = 0; j < STEPS; ++j) {
 #pragma unroll
-                for (int cb = 0; cb < CB; ++cb) {
+                    for (int cb = 0; cb < CB; ++cb) {
 #pragma unroll
-                    for (int part = 0; part < PARTS; ++part) {
-                        const areg_t a = w_lds[(((s * STEPS + j) * CB + cb) * PARTS + part) * 64 + lane];
+                        for (int part = 0; part < PARTS; ++part) {
+                            const areg_t a = w_lds[(((s * STEPS + j) * CB + cb) * PARTS + part) * 64 + lane];
 #pragma unroll
-                        for (int rb = 0; rb < RB; ++rb) acc[rb][cb] = OP::accumulate(part, a, b[rb][j], acc[rb][cb]);
+                            for (int rb = 0; rb < RB; ++rb) acc[rb][cb] = OP::accumulate(part, a, b[rb][j], acc[rb][cb]);
+                        }
+                    }
+                }
+            }
+            else {
+#pragma unroll
+                for (int jg = 0; jg < STEPS / G; ++jg) {
+#pragma unroll
+                    for (int cb = 0; cb < CB; ++cb) {
+                        const v4f a4 = *reinterpret_cast<const v4f*>(reinterpret_cast<const float*>(w_lds) + ((((s * (STEPS / G) + jg) * CB + cb) * 64 + lane) * G));
+#pragma unroll
+                        for (int e = 0; e < G; ++e)
+#pragma unroll
+                            for (int rb = 0; rb < RB; ++rb) acc[rb][cb] = OP::accumulate(0, a4[e], b[rb][jg * G + e], acc[rb][cb]);
                     }
                 }
             }
