@@ -150,7 +150,7 @@ __global__ __launch_bounds__(NW * 64) void vm_conv_mfma_kernel(VmBatchDev B, VmL
 
     extern __shared__ float4 w_lds4[];
     /* G consecutive steps of a lane's weights lie next to each other in LDS, so that one read brings G of them */
-    constexpr int G = (PARTS == 1 && sizeof(areg_t) == 4 && STEPS % 4 == 0) ? 4 : 1;
+    constexpr int G = (PARTS == 1 && sizeof(areg_t) == 4) ? (STEPS % 4 == 0 ? 4 : STEPS % 2 == 0 ? 2 : 1) : 1;
     if constexpr (G == 1) {
         for (int i = threadIdx.x; i < W_BYTES / 16; i += NW * 64) w_lds4[i] = reinterpret_cast<const float4*>(L.w_mfma)[i];
     }
@@ -305,11 +305,12 @@ __global__ __launch_bounds__(NW * 64) void vm_conv_mfma_kernel(VmBatchDev B, VmL
                 for (int jg = 0; jg < STEPS / G; ++jg) {
 #pragma unroll
                     for (int cb = 0; cb < CB; ++cb) {
-                        const v4f a4 = *reinterpret_cast<const v4f*>(reinterpret_cast<const float*>(w_lds) + ((((s * (STEPS / G) + jg) * CB + cb) * 64 + lane) * G));
+                        float a[G];
+                        load_words<float, G>(reinterpret_cast<const float*>(w_lds) + ((((s * (STEPS / G) + jg) * CB + cb) * 64 + lane) * G), a);
 #pragma unroll
                         for (int e = 0; e < G; ++e)
 #pragma unroll
-                            for (int rb = 0; rb < RB; ++rb) acc[rb][cb] = OP::accumulate(0, a4[e], b[rb][jg * G + e], acc[rb][cb]);
+                            for (int rb = 0; rb < RB; ++rb) acc[rb][cb] = OP::accumulate(0, a[e], b[rb][jg * G + e], acc[rb][cb]);
                     }
                 }
             }
